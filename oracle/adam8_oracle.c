@@ -1,0 +1,277 @@
+/*
+ * CPU oracle for the blockwise 8-bit AdamW step.  TEST INFRASTRUCTURE ONLY: nothing in the
+ * shipped library or the Python package may link, load or call this file; it exists so that the
+ * tests, the smoke check and the benchmark's cpu_baseline leg have something to compare with
+ * and to time.
+ *
+ * It is a scalar restatement, one individually rounded fp32 operation per line, of
+ *   - EriDiffusion's Adam8bit::step          src/trainers/adam8bit_enhanced.rs:202-291  (mode ERI)
+ *   - EriDiffusion's functional Adam8bit::update  src/trainers/adam8bit.rs:101-208      (mode L2)
+ * with the state held in the blockwise format the optimizer is specified to use: uint8 codes
+ * into the signed (first moment) and unsigned (second moment) 256-entry dynamic maps of
+ * bitsandbytes (functional.py: create_dynamic_map), one fp32 absmax per 2048-element block.
+ * The reference tree has no blockwise quantiser and no golden vectors for any optimizer, so the
+ * quantiser half of this file restates the published bitsandbytes blockwise algorithm
+ * (quantize_blockwise / dequantize_blockwise: code -> map[code] * absmax, value -> nearest map
+ * entry of value / absmax); what pins it is listed next to each function.
+ *
+ * Pinning status (tests/test_oracle_*.py):
+ *   eri_oracle_bf16_*          all 65,536 high halves against torch.bfloat16        pinned
+ *   eri_oracle_nearest_index   brute-force argmin over 256 entries, round trip      pinned
+ *   eri_oracle_hyper_pack      closed forms at t = 1, f64 restatement               pinned
+ *   eri_oracle_step_tensor     closed forms (zero grad, first step), torch.optim.Adam with the
+ *                              quantiser bypassed, block-max brute force, and bit-for-bit
+ *                              agreement with the independent NumPy restatement
+ *                              (oracle/adam8_numpy.py)                              pinned
+ *   bit-level equality with the reference's own legacy per-tensor linear format
+ *   (adam8bit.rs:211-241, flame-core's to_dtype(U8)/round semantics are absent)     parity unpinned
+ *
+ * Build: see oracle/Makefile (gcc -O2 -ffp-contract=off, no fast-math: every fp32 operation
+ * below must round exactly once).
+ */
+#include <math.h>
+#include <stdint.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define ERI_ORACLE_BLOCK 2048
+
+enum { ERI_ORACLE_MODE_ERI = 0, ERI_ORACLE_MODE_L2 = 1 };
+enum { ERI_ORACLE_F32 = 0, ERI_ORACLE_BF16 = 2 };
+
+typedef struct EriOracleHyper {
+    float beta1;        /* (float)beta1                                   adam8bit_enhanced.rs:256 */
+    float beta2;        /* (float)beta2                                   :260 */
+    float omb1;         /* ERI: 1.0f - (float)beta1 (fp32 subtraction)    :256
+                           L2 : (float)(1.0 - beta1)  (f64 subtraction)   adam8bit.rs:142 */
+    float omb2;         /* same for beta2                                 :260 / adam8bit.rs:151 */
+    float eps;          /* (float)eps                                     :263 / adam8bit.rs:186 */
+    float weight_decay; /* (float)wd                                      :268 / adam8bit.rs:117 */
+    float step_size;    /* ERI: (float)(lr*sqrt(bc2)/bc1)                 :213-215,:274
+                           L2 : (float)lr                                 adam8bit.rs:193 */
+    float bc1;          /* L2 : (float)(1 - beta1^s), s = max(step,1)     adam8bit.rs:164-168 */
+    float bc2;          /* L2 : (float)(1 - beta2^s)                      adam8bit.rs:175 */
+    float grad_scale;   /* multiplies every gradient first (clip factor / per-layer LR multiplier,
+                           pipeline_flux_lora_sequential.rs:759-766,1198-1213); 1.0f = off */
+    int32_t mode;
+    int32_t use_grad_scale;
+} EriOracleHyper;
+
+/* ---- bf16 <-> fp32 -------------------------------------------------------------------- */
+
+float eri_oracle_bf16_to_f32(uint16_t h) {
+    uint32_t u = (uint32_t)h << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+/* round-to-nearest-even; NaN stays NaN (quiet bit forced) */
+uint16_t eri_oracle_f32_to_bf16(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+/* ---- quantiser ------------------------------------------------------------------------ */
+
+/* mid[j] = (map[j] + map[j+1]) * 0.5f, j = 0..254, in fp32 */
+void eri_oracle_midpoints(const float *map, float *mid) {
+    for (int j = 0; j < 255; ++j) {
+        float s = map[j] + map[j + 1];
+        mid[j] = s * 0.5f;
+    }
+}
+
+/* Number of midpoints strictly below x: the nearest map entry, the lower index on an exact tie.
+ * NaN compares false everywhere and lands on code 0. */
+int eri_oracle_nearest_index(const float *mid, float x) {
+    int lo = 0, hi = 255; /* answer in [lo, hi] */
+    while (lo < hi) {
+        int c = (lo + hi) >> 1;
+        if (x > mid[c]) lo = c + 1; else hi = c;
+    }
+    return lo;
+}
+
+/* ---- per-step scalars ----------------------------------------------------------------- */
+
+/* step = the optimizer's counter AFTER its increment for ERI (adam8bit_enhanced.rs:203), the
+ * counter as it stands when update() is called for L2 (adam8bit.rs:164, bumped later by step()). */
+void eri_oracle_hyper_pack(double lr, double beta1, double beta2, double eps, double wd,
+                           uint64_t step, int mode, EriOracleHyper *h) {
+    memset(h, 0, sizeof(*h));
+    h->mode = mode;
+    h->beta1 = (float)beta1;
+    h->beta2 = (float)beta2;
+    h->eps = (float)eps;
+    h->weight_decay = (float)wd;
+    h->grad_scale = 1.0f;
+    h->use_grad_scale = 0;
+    if (mode == ERI_ORACLE_MODE_L2) {
+        uint64_t s = step < 1 ? 1 : step;
+        h->omb1 = (float)(1.0 - beta1);
+        h->omb2 = (float)(1.0 - beta2);
+        h->bc1 = (float)(1.0 - pow(beta1, (double)(int32_t)s));
+        h->bc2 = (float)(1.0 - pow(beta2, (double)(int32_t)s));
+        h->step_size = (float)lr;
+    } else {
+        double t = (double)step;
+        double bc1 = 1.0 - pow(beta1, t);
+        double bc2 = 1.0 - pow(beta2, t);
+        h->omb1 = 1.0f - h->beta1;
+        h->omb2 = 1.0f - h->beta2;
+        h->bc1 = (float)bc1;
+        h->bc2 = (float)bc2;
+        h->step_size = (float)(lr * (sqrt(bc2) / bc1));
+    }
+}
+
+/* ---- one block ------------------------------------------------------------------------ */
+
+static inline float load_elem(const void *base, uint64_t i, int dtype) {
+    if (dtype == ERI_ORACLE_F32) return ((const float *)base)[i];
+    return eri_oracle_bf16_to_f32(((const uint16_t *)base)[i]);
+}
+
+static void step_block(void *p, const void *g, uint8_t *mc, uint8_t *vc, float *am, float *av,
+                       uint64_t base, int n, int dtype, const EriOracleHyper *h,
+                       const float *map_s, const float *map_u, const float *mid_s,
+                       const float *mid_u) {
+    float mbuf[ERI_ORACLE_BLOCK], vbuf[ERI_ORACLE_BLOCK];
+    const float a_m = *am, a_v = *av;
+    float new_am = 0.0f, new_av = 0.0f;
+    for (int i = 0; i < n; ++i) {
+        const uint64_t e = base + (uint64_t)i;
+        float m_old = map_s[mc[e]] * a_m;
+        float v_old = map_u[vc[e]] * a_v;
+        float gr = load_elem(g, e, dtype);
+        float pf = load_elem(p, e, dtype);
+        if (h->use_grad_scale) gr = gr * h->grad_scale;
+        if (h->mode == ERI_ORACLE_MODE_L2 && h->weight_decay > 0.0f) {
+            float pw = pf * h->weight_decay;            /* adam8bit.rs:113-120 */
+            gr = gr + pw;
+        }
+        float t1 = m_old * h->beta1;                    /* adam8bit_enhanced.rs:256 */
+        float t2 = gr * h->omb1;
+        float m = t1 + t2;
+        float gg = gr * gr;                             /* :259 */
+        float t3 = v_old * h->beta2;                    /* :260 */
+        float t4 = gg * h->omb2;
+        float v = t3 + t4;
+        mbuf[i] = m;
+        vbuf[i] = v;
+        new_am = fmaxf(new_am, fabsf(m));
+        new_av = fmaxf(new_av, fabsf(v));
+
+        float pn;
+        if (h->mode == ERI_ORACLE_MODE_L2) {
+            float mh = m / h->bc1;                      /* adam8bit.rs:170 */
+            float vh = v / h->bc2;                      /* :178 */
+            vh = fmaxf(vh, 0.0f);                       /* :181-182 */
+            float den = sqrtf(vh) + h->eps;             /* :187 */
+            float upd = mh / den;
+            float us = upd * h->step_size;              /* :196 */
+            if (dtype == ERI_ORACLE_BF16)               /* :197-198 update cast to the param dtype */
+                us = eri_oracle_bf16_to_f32(eri_oracle_f32_to_bf16(us));
+            pn = pf - us;                               /* :205 */
+        } else {
+            float den = sqrtf(v) + h->eps;              /* adam8bit_enhanced.rs:263 */
+            float r = m / den;                          /* :264 */
+            float u = r;
+            if (h->weight_decay > 0.0f) {               /* :267-271 */
+                float pw = pf * h->weight_decay;
+                u = r + pw;
+            }
+            float us = u * h->step_size;                /* :274 */
+            pn = pf - us;                               /* :275 apply_update: p <- p - x */
+        }
+        if (dtype == ERI_ORACLE_F32) ((float *)p)[e] = pn;
+        else ((uint16_t *)p)[e] = eri_oracle_f32_to_bf16(pn);
+    }
+    for (int i = 0; i < n; ++i) {
+        const uint64_t e = base + (uint64_t)i;
+        float xm = (new_am == 0.0f) ? 0.0f : mbuf[i] / new_am;
+        float xv = (new_av == 0.0f) ? 0.0f : vbuf[i] / new_av;
+        mc[e] = (uint8_t)eri_oracle_nearest_index(mid_s, xm);
+        vc[e] = (uint8_t)eri_oracle_nearest_index(mid_u, xv);
+    }
+    *am = new_am;
+    *av = new_av;
+}
+
+/*
+ * One step over one tensor.  Returns 0, or -1 for an empty tensor (the reference refuses to
+ * quantise an empty tensor, adam8bit_enhanced.rs:46-50), -2 for an unsupported dtype.
+ * threads <= 1 runs serially; otherwise blocks are split statically over that many threads.
+ */
+int eri_oracle_step_tensor(void *p, const void *g, uint8_t *m, uint8_t *v, float *absmax_m,
+                           float *absmax_v, uint64_t numel, int dtype, const EriOracleHyper *h,
+                           const float *map_s, const float *map_u, int threads) {
+    if (numel == 0) return -1;
+    if (dtype != ERI_ORACLE_F32 && dtype != ERI_ORACLE_BF16) return -2;
+    float mid_s[255], mid_u[255];
+    eri_oracle_midpoints(map_s, mid_s);
+    eri_oracle_midpoints(map_u, mid_u);
+    const int64_t nblocks = (int64_t)((numel + ERI_ORACLE_BLOCK - 1) / ERI_ORACLE_BLOCK);
+    (void)threads;
+#ifdef _OPENMP
+#pragma omp parallel for schedule(static) num_threads(threads > 1 ? threads : 1)
+#endif
+    for (int64_t b = 0; b < nblocks; ++b) {
+        uint64_t base = (uint64_t)b * ERI_ORACLE_BLOCK;
+        uint64_t left = numel - base;
+        int n = left < ERI_ORACLE_BLOCK ? (int)left : ERI_ORACLE_BLOCK;
+        step_block(p, g, m, v, absmax_m + b, absmax_v + b, base, n, dtype, h, map_s, map_u, mid_s,
+                   mid_u);
+    }
+    return 0;
+}
+
+/* Fresh state: the codes of 0.0 with absmax 0, what quantising a zeros tensor gives
+ * (the reference initialises from Tensor::zeros, adam8bit_enhanced.rs:179-197). */
+void eri_oracle_state_init(uint8_t *m, uint8_t *v, float *absmax_m, float *absmax_v,
+                           uint64_t numel) {
+    uint64_t nblocks = (numel + ERI_ORACLE_BLOCK - 1) / ERI_ORACLE_BLOCK;
+    memset(m, 127, numel);
+    memset(v, 0, numel);
+    for (uint64_t b = 0; b < nblocks; ++b) { absmax_m[b] = 0.0f; absmax_v[b] = 0.0f; }
+}
+
+/* Blockwise dequantisation of a state to fp32 (checkpoint export, adam8bit.rs:296-308). */
+void eri_oracle_dequantize(const uint8_t *codes, const float *absmax, const float *map,
+                           uint64_t numel, float *out) {
+    for (uint64_t i = 0; i < numel; ++i) out[i] = map[codes[i]] * absmax[i / ERI_ORACLE_BLOCK];
+}
+
+/* Blockwise quantisation of an fp32 tensor (checkpoint import, adam8bit.rs:316-329). */
+void eri_oracle_quantize(const float *x, const float *map, uint64_t numel, uint8_t *codes,
+                         float *absmax) {
+    float mid[255];
+    eri_oracle_midpoints(map, mid);
+    uint64_t nblocks = (numel + ERI_ORACLE_BLOCK - 1) / ERI_ORACLE_BLOCK;
+    for (uint64_t b = 0; b < nblocks; ++b) {
+        uint64_t base = b * ERI_ORACLE_BLOCK;
+        uint64_t n = numel - base < ERI_ORACLE_BLOCK ? numel - base : ERI_ORACLE_BLOCK;
+        float a = 0.0f;
+        for (uint64_t i = 0; i < n; ++i) a = fmaxf(a, fabsf(x[base + i]));
+        for (uint64_t i = 0; i < n; ++i) {
+            float q = (a == 0.0f) ? 0.0f : x[base + i] / a;
+            codes[base + i] = (uint8_t)eri_oracle_nearest_index(mid, q);
+        }
+        absmax[b] = a;
+    }
+}
+
+int eri_oracle_num_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
