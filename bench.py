@@ -1,0 +1,207 @@
+#!/usr/bin/env python3
+"""Benchmark of the blockwise 8-bit AdamW step on one MI355X.
+
+A step = one pass of the multi-tensor optimizer step over the whole parameter set, every input
+already resident in HBM.  Default workload: the FLUX-12B-shaped full fine-tune set (780 bf16
+tensors, 11,901,408,320 parameters, 8-bit m/v + fp32 absmax per 2048-block, ~72 GB resident).
+Prints one JSON line: params/s, the HBM roofline fraction of the step kernel (algorithmic bytes /
+measured launch duration / 8 TB/s) and, beside it, the CPU oracle timed on this host's cores.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBPS = 8000.0
+# algorithmic bytes per parameter: read p, g, m, v and write p, m, v, plus 16 bytes of absmax per block
+BYTES_PER_PARAM = {"bf16": 2 + 2 + 1 + 1 + 2 + 1 + 1 + 16.0 / 2048, "f32": 4 + 4 + 1 + 1 + 4 + 1 + 1 + 16.0 / 2048}
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--config", default="c5_flux12b_full")
+    ap.add_argument("--flags", type=int, default=0, help="ERI_ADAM8_FLAG_* bits for the step")
+    ap.add_argument("--cpu-sample", type=int, default=512 << 20, help="parameters in the CPU baseline sample (0 = skip)")
+    ap.add_argument("--traffic-json", default=os.path.join(ROOT, "profiles", "traffic.json"),
+                    help="HBM bytes per launch derived from rocprofv3 --pmc runs, if present")
+    return ap.parse_args()
+
+
+def align(n, a=256):
+    return (n + a - 1) // a * a
+
+
+class Arena:
+    """One flat device allocation per kind of buffer; every tensor starts on a 256-byte boundary."""
+
+    def __init__(self, torch, sizes_bytes):
+        self.offsets = []
+        total = 0
+        for b in sizes_bytes:
+            self.offsets.append(total)
+            total += align(b)
+        self.buf = torch.empty(max(total, 256), dtype=torch.uint8, device="cuda:0")
+        self.base = self.buf.data_ptr()
+
+    def ptr(self, i):
+        return self.base + self.offsets[i]
+
+    def view(self, i, nbytes):
+        return self.buf[self.offsets[i]:self.offsets[i] + nbytes]
+
+
+def cpu_baseline(tensors, bf16, sample_params, hyper_args):
+    """Times the C oracle (oracle/liberi_oracle.so) on a prefix of the same tensor list."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import numpy as np
+
+    import oracle_c as oc
+    from eridiffusion_amd.workloads import numel
+
+    threads = max(1, min(16, os.cpu_count() or 1))
+    sizes, total = [], 0
+    for _, shape in tensors:
+        n = numel(shape)
+        if total + n > sample_params and sizes:
+            break
+        n = min(n, sample_params)
+        sizes.append(n)
+        total += n
+    rng = np.random.default_rng(7)
+    tile = 1 << 22
+    base_p = (rng.standard_normal(tile) * 0.02).astype(np.float32)
+    base_g = (rng.standard_normal(tile) * 1e-3).astype(np.float32)
+    if bf16:
+        from oracle import adam8_numpy as onp
+        base_p, base_g = onp.f32_to_bf16(base_p), onp.f32_to_bf16(base_g)
+    maps = oc.load_maps()
+    bufs = []
+    for n in sizes:
+        reps = (n + tile - 1) // tile
+        bufs.append((np.tile(base_p, reps)[:n].copy(), np.tile(base_g, reps)[:n].copy(), list(oc.state_init(n))))
+    dt_tag = oc.DT_BF16 if bf16 else oc.DT_F32
+    best = None
+    for rep in range(2):  # first pass warms the pages and gives the states real contents
+        h = oc.hyper_pack(*hyper_args[:5], rep + 1)
+        t0 = time.perf_counter()
+        for p, g, st in bufs:
+            oc.step_tensor(p, g, *st, h, maps, dt_tag, threads)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    return {"value": total / best, "unit": "params/s", "cores": threads, "kind": "port",
+            "sample": "first %d tensors of the workload (%d params), one step, C oracle with OpenMP over blocks, "
+                      "best of 2" % (len(sizes), total)}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the 8-bit AdamW step has no cross-GPU exchange and this build runs on "
+              "a single MI355X; rerun with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from eridiffusion_amd import _lib as L
+    from eridiffusion_amd import workloads as W
+
+    fn, dt_name = W.CONFIGS[args.config]
+    tensors = fn()
+    bf16 = dt_name == "bf16"
+    esz = 2 if bf16 else 4
+    sizes = [W.numel(s) for _, s in tensors]
+    n_params = sum(sizes)
+    n_blocks = sum((n + L.BLOCK - 1) // L.BLOCK for n in sizes)
+    torch.cuda.set_device(0)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    a_p = Arena(torch, [n * esz for n in sizes])
+    a_g = Arena(torch, [n * esz for n in sizes])
+    a_m = Arena(torch, sizes)
+    a_v = Arena(torch, sizes)
+    a_am = Arena(torch, [((n + 2047) // 2048) * 4 for n in sizes])
+    a_av = Arena(torch, [((n + 2047) // 2048) * 4 for n in sizes])
+    tdt = torch.bfloat16 if bf16 else torch.float32
+    gen = torch.Generator(device="cuda:0")
+    gen.manual_seed(0xE21D + 5)
+    p_std, g_std = (0.02, 1e-3)
+    for i, n in enumerate(sizes):  # synthetic data: p ~ N(0, 0.02), g ~ N(0, 1e-3)
+        a_p.view(i, n * esz).view(tdt).copy_(torch.randn(n, device="cuda:0", generator=gen).mul_(p_std).to(tdt))
+        a_g.view(i, n * esz).view(tdt).copy_(torch.randn(n, device="cuda:0", generator=gen).mul_(g_std).to(tdt))
+        L.check(L.lib().eri_adam8_state_init(a_m.ptr(i), a_v.ptr(i), a_am.ptr(i), a_av.ptr(i), n, stream), "state_init")
+    rows = (L.TensorRow * len(sizes))()
+    start = 0
+    for i, n in enumerate(sizes):
+        r = rows[i]
+        r.p, r.g, r.m, r.v, r.absmax_m, r.absmax_v = a_p.ptr(i), a_g.ptr(i), a_m.ptr(i), a_v.ptr(i), a_am.ptr(i), a_av.ptr(i)
+        r.numel, r.block_start, r.dtype_tag, r.grad_scale = n, start, (L.DTYPE_BF16 if bf16 else L.DTYPE_F32), 1.0
+        start += (n + L.BLOCK - 1) // L.BLOCK
+    table = C.c_void_p()
+    L.check(L.lib().eri_adam8_table_create(rows, len(rows), stream, C.byref(table)), "table_create")
+    hyper_args = (1e-4, 0.9, 0.999, 1e-8, 0.01)
+
+    def step(t):
+        h = L.hyper_pack(*hyper_args, t, L.MODE_ERI, args.flags)
+        L.check(L.lib().eri_adam8_step_table(table, C.byref(h), stream), "step_table")
+
+    t = 0
+    for _ in range(args.warmup):
+        t += 1
+        step(t)
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        t += 1
+        ev[k][0].record()
+        step(t)
+        ev[k][1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    launch_ms = [a.elapsed_time(b) for a, b in ev]
+    avg_launch_s = sum(launch_ms) / len(launch_ms) / 1e3
+
+    algo_bytes = BYTES_PER_PARAM[dt_name] * n_params
+    achieved = algo_bytes / avg_launch_s / 1e9
+    traffic = None
+    if os.path.exists(args.traffic_json):
+        try:
+            with open(args.traffic_json) as f:
+                traffic = json.load(f).get(args.config)
+        except Exception:
+            traffic = None
+    out = {
+        "metric": "params/sec per 8-bit AdamW step",
+        "value": n_params * args.steps / wall,
+        "unit": "params/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": wall / args.steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": args.config, "tensors": len(sizes), "params": n_params, "blocks": n_blocks,
+                   "param_dtype": dt_name, "state": "uint8 m/v + fp32 absmax per 2048-block", "flags": args.flags,
+                   "resident_gb": round((n_params * (2 * esz + 2) + n_blocks * 8) / 1e9, 2)},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                     "frac": achieved / PEAK_HBM_GBPS, "traffic": traffic,
+                     "kernel_ms": avg_launch_s * 1e3, "algorithmic_bytes": algo_bytes},
+    }
+    L.lib().eri_adam8_table_destroy(table)
+    if args.cpu_sample > 0:
+        out["cpu_baseline"] = cpu_baseline(tensors, bf16, args.cpu_sample, hyper_args)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

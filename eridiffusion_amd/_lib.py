@@ -1,0 +1,99 @@
+"""ctypes binding of liberi_optim8.so (the C ABI declared in include/eri_optim8.h).
+
+The library is built in-tree by `make -C eridiffusion_amd/csrc` (or __graft_entry__.build()).
+There is no fallback: if the shared object is missing or a call fails, this module raises.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "liberi_optim8.so")
+
+BLOCK = 2048
+DTYPE_F32, DTYPE_F16, DTYPE_BF16, DTYPE_I32 = 0, 1, 2, 3
+MODE_ERI, MODE_L2 = 0, 1
+FLAG_GRAD_SCALE, FLAG_EXACT_PARAM, FLAG_BSEARCH = 1, 2, 4
+
+
+class Hyper(C.Structure):
+    _fields_ = [("beta1", C.c_float), ("beta2", C.c_float), ("omb1", C.c_float), ("omb2", C.c_float),
+                ("eps", C.c_float), ("weight_decay", C.c_float), ("step_size", C.c_float),
+                ("bc1", C.c_float), ("bc2", C.c_float), ("grad_scale", C.c_float),
+                ("mode", C.c_int32), ("flags", C.c_uint32)]
+
+
+class TensorRow(C.Structure):
+    _fields_ = [("p", C.c_void_p), ("g", C.c_void_p), ("m", C.c_void_p), ("v", C.c_void_p),
+                ("absmax_m", C.c_void_p), ("absmax_v", C.c_void_p), ("numel", C.c_uint64),
+                ("block_start", C.c_uint64), ("dtype_tag", C.c_int32), ("grad_scale", C.c_float)]
+
+
+class EriError(RuntimeError):
+    def __init__(self, what, code, message):
+        super().__init__("%s failed with code %d: %s" % (what, code, message))
+        self.code = code
+        self.message = message
+
+
+EXPORTS = {
+    # name: (restype, argtypes)
+    "eri_last_error": (C.c_char_p, []),
+    "eri_hip_device_count": (C.c_int, [C.POINTER(C.c_int)]),
+    "eri_hip_set_device": (C.c_int, [C.c_int]),
+    "eri_hip_malloc_zeroed": (C.c_int, [C.c_int, C.c_size_t, C.POINTER(C.c_void_p)]),
+    "eri_hip_free": (C.c_int, [C.c_void_p]),
+    "eri_hip_host_alloc": (C.c_void_p, [C.c_size_t]),
+    "eri_hip_host_free": (C.c_int, [C.c_void_p]),
+    "eri_hip_memcpy_async": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]),
+    "eri_hip_memset_async": (C.c_int, [C.c_void_p, C.c_int, C.c_size_t, C.c_void_p]),
+    "eri_hip_stream_create": (C.c_int, [C.POINTER(C.c_void_p)]),
+    "eri_hip_stream_sync": (C.c_int, [C.c_void_p]),
+    "eri_hip_stream_destroy": (C.c_int, [C.c_void_p]),
+    "eri_hip_mem_info": (C.c_int, [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
+    "eri_adam8_init": (C.c_int, []),
+    "eri_adam8_get_maps": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "eri_adam8_table_image": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_size_t), C.POINTER(C.c_uint32)]),
+    "eri_adam8_hyper_pack": (C.c_int, [C.c_double] * 5 + [C.c_uint64, C.c_int, C.c_uint32, C.POINTER(Hyper)]),
+    "eri_adam8_state_init": (C.c_int, [C.c_void_p] * 4 + [C.c_uint64, C.c_void_p]),
+    "eri_adam8_table_create": (C.c_int, [C.POINTER(TensorRow), C.c_uint32, C.c_void_p, C.POINTER(C.c_void_p)]),
+    "eri_adam8_table_update": (C.c_int, [C.c_void_p, C.POINTER(TensorRow), C.c_uint32, C.c_void_p]),
+    "eri_adam8_table_destroy": (C.c_int, [C.c_void_p]),
+    "eri_adam8_table_info": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
+    "eri_adam8_step_table": (C.c_int, [C.c_void_p, C.POINTER(Hyper), C.c_void_p]),
+    "eri_adam8_step_multi": (C.c_int, [C.POINTER(TensorRow), C.c_uint32, C.POINTER(Hyper), C.c_void_p]),
+    "eri_adam8_dequantize": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_uint64, C.c_void_p, C.c_void_p]),
+    "eri_adam8_quantize": (C.c_int, [C.c_void_p, C.c_int, C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p]),
+}
+
+_lib = None
+
+
+def lib():
+    """The loaded library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("%s is missing: build it with `make -C eridiffusion_amd/csrc` "
+                               "(there is no CPU or PyTorch fallback)" % LIB_PATH)
+        L = C.CDLL(LIB_PATH)
+        for name, (res, args) in EXPORTS.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def check(code, what):
+    if code != 0:
+        raise EriError(what, code, lib().eri_last_error().decode("utf-8", "replace"))
+
+
+def hyper_pack(lr, beta1, beta2, eps, weight_decay, step, mode=MODE_ERI, flags=0, grad_scale=None):
+    h = Hyper()
+    check(lib().eri_adam8_hyper_pack(lr, beta1, beta2, eps, weight_decay, step, mode, flags, C.byref(h)),
+          "eri_adam8_hyper_pack")
+    if grad_scale is not None:
+        h.grad_scale = grad_scale
+        h.flags |= FLAG_GRAD_SCALE
+    return h

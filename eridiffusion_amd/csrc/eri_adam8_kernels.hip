@@ -1,0 +1,517 @@
+/*
+ * gfx950 kernels of the blockwise 8-bit AdamW step.
+ *
+ * Work decomposition: one 64-lane wavefront owns one 2048-element quantisation block from its
+ * first load to its last store, so the per-block absmax needs nothing but a DPP reduction inside
+ * the wave -- no barrier, no cross-wave exchange.  A block is read in four 512-element passes;
+ * lane l of pass c holds elements c*512 + 8*l .. +7, which makes every access a contiguous
+ * 128-bit (params, grads) or 64-bit (codes) load per lane.  The fp32 moments of the whole block
+ * stay in registers (32 + 32 per lane) between the update and the requantisation, so each byte of
+ * p, g, m, v crosses HBM once in each direction.
+ *
+ * The grid is persistent: workgroups stage the lookup tables into LDS once, then their waves walk
+ * the global block list with a grid-sized stride, so consecutive waves touch consecutive blocks.
+ * The tensor that owns a block is found by a scalar binary search over the launch table.
+ *
+ * Arithmetic: every fp32 operation of the update is written as its own statement and the file is
+ * compiled with -ffp-contract=off, because the reference runs each as a separate tensor op
+ * (src/trainers/adam8bit_enhanced.rs:252-275).  fmaf appears only inside the exactly rounded
+ * division below.
+ */
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "eri_adam8_device.h"
+
+namespace eri {
+
+// ------------------------------------------------------------------------------------------
+// small device helpers
+// ------------------------------------------------------------------------------------------
+
+__device__ __forceinline__ uint32_t f2u(float x) { return __builtin_bit_cast(uint32_t, x); }
+__device__ __forceinline__ float u2f(uint32_t x) { return __builtin_bit_cast(float, x); }
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_mov(float x) {
+    return u2f((uint32_t)__builtin_amdgcn_update_dpp((int)f2u(x), (int)f2u(x), CTRL, ROW_MASK, 0xf, false));
+}
+
+/* Maximum over the 64 lanes of non-negative, NaN-free values, returned wave-uniform. */
+__device__ __forceinline__ float wave_max(float x) {
+    x = fmaxf(x, dpp_mov<0xB1, 0xf>(x));  // quad_perm [1,0,3,2]
+    x = fmaxf(x, dpp_mov<0x4E, 0xf>(x));  // quad_perm [2,3,0,1]
+    x = fmaxf(x, dpp_mov<0x141, 0xf>(x)); // row_half_mirror
+    x = fmaxf(x, dpp_mov<0x140, 0xf>(x)); // row_mirror: every lane now holds its row's maximum
+    x = fmaxf(x, dpp_mov<0x142, 0xa>(x)); // row_bcast:15 into rows 1 and 3
+    x = fmaxf(x, dpp_mov<0x143, 0xc>(x)); // row_bcast:31 into rows 2 and 3
+    return u2f((uint32_t)__builtin_amdgcn_readlane((int)f2u(x), 63));
+}
+
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return u2f(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return u2f(w & 0xffff0000u); }
+
+/* fp32 -> bf16 bits, round to nearest even, NaN kept quiet. */
+__device__ __forceinline__ uint32_t bf16_bits(float f) {
+    __bf16 b = (__bf16)f;
+    return (uint32_t)__builtin_bit_cast(uint16_t, b);
+}
+__device__ __forceinline__ float bf16_round(float f) { return u2f(bf16_bits(f) << 16); }
+
+/*
+ * m / a for a divisor shared by a whole block.  With ra = RN(1/a), q0 = RN(m*ra) is within an
+ * ulp or two of the quotient, the remainder m - q0*a is exact in one fma, and one correction
+ * gives the correctly rounded quotient (Markstein); `fast` excludes the divisors for which that
+ * argument needs care (zero, subnormal-range or huge values, an all-ones significand), and those
+ * blocks use the hardware-assisted IEEE division instead.  Both produce the same bits.
+ */
+struct BlockDiv {
+    float a, ra;
+    bool fast;
+    __device__ __forceinline__ explicit BlockDiv(float a_) : a(a_) {
+        fast = (a_ >= 0x1p-60f) && (a_ <= 0x1p60f) && ((f2u(a_) & 0x7fffffu) != 0x7fffffu);
+        ra = fast ? 1.0f / a_ : 0.0f;
+    }
+    __device__ __forceinline__ float div_fast(float m) const {
+        float q0 = m * ra;
+        float r = __builtin_fmaf(-q0, a, m);
+        return __builtin_fmaf(r, ra, q0);
+    }
+    __device__ __forceinline__ float div_slow(float m) const { return a == 0.0f ? 0.0f : m / a; }
+};
+
+struct Lds {
+    const float *map_s, *map_u, *mid_s, *mid_u;
+    const KeySlot *key_s, *key_u;
+};
+
+__device__ __forceinline__ uint32_t code_signed_key(float x, const KeySlot *key_s) {
+    const uint32_t b = f2u(x);
+    uint32_t k = (b & 0x7fffffffu) >> kSShift;
+    k = __builtin_elementwise_sub_sat(k, kSBase);
+    k = min(k, kSSlots);
+    k += (b >> 31) * kSPerSign;
+    const KeySlot s = key_s[k];
+    return s.lo + (x > s.mid ? 1u : 0u);
+}
+
+__device__ __forceinline__ uint32_t code_unsigned_key(float x, const KeySlot *key_u) {
+    uint32_t k = f2u(x) >> kUShift; // x >= 0, or NaN with either sign (clamped to the NaN slot)
+    k = __builtin_elementwise_sub_sat(k, kUBase);
+    k = min(k, kUSlots);
+    const KeySlot s = key_u[k];
+    return s.lo + (x > s.mid ? 1u : 0u);
+}
+
+/* Number of midpoints below x by binary search of the 255-entry LDS table (entry 255 is +inf). */
+__device__ __forceinline__ uint32_t code_bsearch(float x, const float *mid) {
+    uint32_t idx = 0;
+#pragma unroll
+    for (uint32_t s = 128; s >= 1; s >>= 1) idx += (x > mid[idx + s - 1]) ? s : 0u;
+    return idx;
+}
+
+// ------------------------------------------------------------------------------------------
+// the update of one element
+// ------------------------------------------------------------------------------------------
+
+template <int MODE, bool EXACT, bool BF16, bool WD, bool GS>
+__device__ __forceinline__ void adam_elem(float p, float g, float m_old, float v_old, const EriAdam8Hyper &h,
+                                          float gscale, const BlockDiv &dbc1, const BlockDiv &dbc2, float &m,
+                                          float &v, float &pn) {
+    if (GS) g = g * gscale;
+    if (MODE == ERI_ADAM8_MODE_L2 && WD) { // adam8bit.rs:113-120
+        float pw = p * h.weight_decay;
+        g = g + pw;
+    }
+    float t1 = m_old * h.beta1; // adam8bit_enhanced.rs:256
+    float t2 = g * h.omb1;
+    m = t1 + t2;
+    float gg = g * g; // :259-260
+    float t3 = v_old * h.beta2;
+    float t4 = gg * h.omb2;
+    v = t3 + t4;
+    if (MODE == ERI_ADAM8_MODE_L2) {
+        float mh = dbc1.fast ? dbc1.div_fast(m) : m / dbc1.a; // adam8bit.rs:170
+        float vh = dbc2.fast ? dbc2.div_fast(v) : v / dbc2.a; // :178
+        vh = fmaxf(vh, 0.0f);                                  // :181-182
+        float upd;
+        if (EXACT) {
+            float den = sqrtf(vh) + h.eps; // :187
+            upd = mh / den;
+        } else {
+            float den = __builtin_amdgcn_sqrtf(vh) + h.eps;
+            upd = mh * __builtin_amdgcn_rcpf(den);
+        }
+        float us = upd * h.step_size; // :196
+        if (BF16) us = bf16_round(us); // :197-198
+        pn = p - us;                   // :205
+    } else {
+        float r;
+        if (EXACT) {
+            float den = sqrtf(v) + h.eps; // adam8bit_enhanced.rs:263
+            r = m / den;                  // :264
+        } else {
+            float den = __builtin_amdgcn_sqrtf(v) + h.eps;
+            r = m * __builtin_amdgcn_rcpf(den);
+        }
+        float u = r;
+        if (WD) { // :267-271
+            float pw = p * h.weight_decay;
+            u = r + pw;
+        }
+        float us = u * h.step_size; // :274
+        pn = p - us;                // :275
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// 8 consecutive elements per lane: loads and stores
+// ------------------------------------------------------------------------------------------
+
+template <bool BF16>
+__device__ __forceinline__ void load8(const void *base, uint32_t elem, float (&out)[8]) {
+    if (BF16) {
+        const uint4 w = *reinterpret_cast<const uint4 *>(static_cast<const uint16_t *>(base) + elem);
+        out[0] = bf16_lo(w.x); out[1] = bf16_hi(w.x); out[2] = bf16_lo(w.y); out[3] = bf16_hi(w.y);
+        out[4] = bf16_lo(w.z); out[5] = bf16_hi(w.z); out[6] = bf16_lo(w.w); out[7] = bf16_hi(w.w);
+    } else {
+        const float4 *q = reinterpret_cast<const float4 *>(static_cast<const float *>(base) + elem);
+        const float4 a = q[0], b = q[1];
+        out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w;
+        out[4] = b.x; out[5] = b.y; out[6] = b.z; out[7] = b.w;
+    }
+}
+
+template <bool BF16>
+__device__ __forceinline__ void store8(void *base, uint32_t elem, const float (&v)[8]) {
+    if (BF16) {
+        uint4 w;
+        w.x = bf16_bits(v[0]) | (bf16_bits(v[1]) << 16);
+        w.y = bf16_bits(v[2]) | (bf16_bits(v[3]) << 16);
+        w.z = bf16_bits(v[4]) | (bf16_bits(v[5]) << 16);
+        w.w = bf16_bits(v[6]) | (bf16_bits(v[7]) << 16);
+        *reinterpret_cast<uint4 *>(static_cast<uint16_t *>(base) + elem) = w;
+    } else {
+        float4 *q = reinterpret_cast<float4 *>(static_cast<float *>(base) + elem);
+        q[0] = make_float4(v[0], v[1], v[2], v[3]);
+        q[1] = make_float4(v[4], v[5], v[6], v[7]);
+    }
+}
+
+__device__ __forceinline__ uint32_t byte_of(const uint2 w, int k) {
+    const uint32_t d = k < 4 ? w.x : w.y;
+    return (d >> (8 * (k & 3))) & 0xffu;
+}
+
+// ------------------------------------------------------------------------------------------
+// a full 2048-element block, one wavefront
+// ------------------------------------------------------------------------------------------
+
+template <bool FAST_DIV, bool KEYTAB>
+__device__ __forceinline__ void requant8(const float *mf, const float *vf, const BlockDiv &dm, const BlockDiv &dv,
+                                         const Lds &L, uint2 &mw, uint2 &vw) {
+    uint32_t cm[8], cv[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const float xm = FAST_DIV ? dm.div_fast(mf[k]) : dm.div_slow(mf[k]);
+        const float xv = FAST_DIV ? dv.div_fast(vf[k]) : dv.div_slow(vf[k]);
+        cm[k] = KEYTAB ? code_signed_key(xm, L.key_s) : code_bsearch(xm, L.mid_s);
+        cv[k] = KEYTAB ? code_unsigned_key(xv, L.key_u) : code_bsearch(xv, L.mid_u);
+    }
+    mw.x = cm[0] | (cm[1] << 8) | (cm[2] << 16) | (cm[3] << 24);
+    mw.y = cm[4] | (cm[5] << 8) | (cm[6] << 16) | (cm[7] << 24);
+    vw.x = cv[0] | (cv[1] << 8) | (cv[2] << 16) | (cv[3] << 24);
+    vw.y = cv[4] | (cv[5] << 8) | (cv[6] << 16) | (cv[7] << 24);
+}
+
+template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB>
+__device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint32_t lane, const EriAdam8Hyper &h,
+                                           float gscale, const BlockDiv &dbc1, const BlockDiv &dbc2, const Lds &L) {
+    const size_t e0 = (size_t)lb * kBlock;
+    const size_t esz = BF16 ? 2 : 4;
+    char *p = static_cast<char *>(t.p) + e0 * esz;
+    const char *g = static_cast<const char *>(t.g) + e0 * esz;
+    uint8_t *mc = t.m + e0;
+    uint8_t *vc = t.v + e0;
+    const float a_m = t.absmax_m[lb];
+    const float a_v = t.absmax_v[lb];
+
+    float mf[32], vf[32];
+    float lm = 0.0f, lv = 0.0f;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const uint32_t o = c * 512 + lane * 8;
+        float pv[8], gv[8], pn[8];
+        load8<BF16>(p, o, pv);
+        load8<BF16>(g, o, gv);
+        const uint2 mw = *reinterpret_cast<const uint2 *>(mc + o);
+        const uint2 vw = *reinterpret_cast<const uint2 *>(vc + o);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const float m_old = L.map_s[byte_of(mw, k)] * a_m;
+            const float v_old = L.map_u[byte_of(vw, k)] * a_v;
+            float m, v;
+            adam_elem<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], m_old, v_old, h, gscale, dbc1, dbc2, m, v, pn[k]);
+            mf[c * 8 + k] = m;
+            vf[c * 8 + k] = v;
+            lm = fmaxf(lm, __builtin_fabsf(m));
+            lv = fmaxf(lv, __builtin_fabsf(v));
+        }
+        store8<BF16>(p, o, pn);
+    }
+    const float nam = wave_max(lm);
+    const float nav = wave_max(lv);
+    if (lane == 0) {
+        t.absmax_m[lb] = nam;
+        t.absmax_v[lb] = nav;
+    }
+    const BlockDiv dm(nam), dv(nav);
+    if (dm.fast && dv.fast) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t o = c * 512 + lane * 8;
+            uint2 mw, vw;
+            requant8<true, KEYTAB>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
+            *reinterpret_cast<uint2 *>(mc + o) = mw;
+            *reinterpret_cast<uint2 *>(vc + o) = vw;
+        }
+    } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t o = c * 512 + lane * 8;
+            uint2 mw, vw;
+            requant8<false, KEYTAB>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
+            *reinterpret_cast<uint2 *>(mc + o) = mw;
+            *reinterpret_cast<uint2 *>(vc + o) = vw;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// the last, partial block of a tensor: element-wise, bounds-checked, moments recomputed in the
+// second sweep instead of being held (n < 2048 elements, once per tensor at most)
+// ------------------------------------------------------------------------------------------
+
+template <bool BF16>
+__device__ __forceinline__ float load1(const void *base, size_t i) {
+    if (BF16) return u2f((uint32_t)static_cast<const uint16_t *>(base)[i] << 16);
+    return static_cast<const float *>(base)[i];
+}
+
+template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB>
+__device__ __noinline__ void tail_block(const DevTensor &t, uint32_t lb, uint32_t n, uint32_t lane,
+                                        const EriAdam8Hyper &h, float gscale, const BlockDiv &dbc1,
+                                        const BlockDiv &dbc2, const Lds &L) {
+    const size_t e0 = (size_t)lb * kBlock;
+    const float a_m = t.absmax_m[lb];
+    const float a_v = t.absmax_v[lb];
+    float lm = 0.0f, lv = 0.0f;
+    for (uint32_t i = lane; i < n; i += kWave) {
+        const size_t e = e0 + i;
+        float m, v, pn;
+        adam_elem<MODE, EXACT, BF16, WD, GS>(load1<BF16>(t.p, e), load1<BF16>(t.g, e), L.map_s[t.m[e]] * a_m,
+                                             L.map_u[t.v[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn);
+        lm = fmaxf(lm, __builtin_fabsf(m));
+        lv = fmaxf(lv, __builtin_fabsf(v));
+    }
+    const float nam = wave_max(lm);
+    const float nav = wave_max(lv);
+    const BlockDiv dm(nam), dv(nav);
+    for (uint32_t i = lane; i < n; i += kWave) {
+        const size_t e = e0 + i;
+        float m, v, pn;
+        adam_elem<MODE, EXACT, BF16, WD, GS>(load1<BF16>(t.p, e), load1<BF16>(t.g, e), L.map_s[t.m[e]] * a_m,
+                                             L.map_u[t.v[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn);
+        const float xm = dm.div_slow(m);
+        const float xv = dv.div_slow(v);
+        t.m[e] = (uint8_t)(KEYTAB ? code_signed_key(xm, L.key_s) : code_bsearch(xm, L.mid_s));
+        t.v[e] = (uint8_t)(KEYTAB ? code_unsigned_key(xv, L.key_u) : code_bsearch(xv, L.mid_u));
+        if (BF16) static_cast<uint16_t *>(t.p)[e] = (uint16_t)bf16_bits(pn);
+        else static_cast<float *>(t.p)[e] = pn;
+    }
+    if (lane == 0) {
+        t.absmax_m[lb] = nam;
+        t.absmax_v[lb] = nav;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// the step kernel
+// ------------------------------------------------------------------------------------------
+
+extern __shared__ uint4 lds_raw[];
+
+template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB>
+__global__ __launch_bounds__(1024) void adam8_step_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
+                                                          uint32_t total_blocks, EriAdam8Hyper h,
+                                                          const uint4 *__restrict__ lds_image) {
+    for (uint32_t i = threadIdx.x; i < kLdsImageBytes / 16; i += blockDim.x) lds_raw[i] = lds_image[i];
+    __syncthreads();
+    const char *base = reinterpret_cast<const char *>(lds_raw);
+    Lds L;
+    L.map_s = reinterpret_cast<const float *>(base + kOffMapS);
+    L.map_u = reinterpret_cast<const float *>(base + kOffMapU);
+    L.mid_s = reinterpret_cast<const float *>(base + kOffMidS);
+    L.mid_u = reinterpret_cast<const float *>(base + kOffMidU);
+    L.key_s = reinterpret_cast<const KeySlot *>(base + kOffKeyS);
+    L.key_u = reinterpret_cast<const KeySlot *>(base + kOffKeyU);
+
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t waves_per_wg = blockDim.x / kWave;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
+    const uint32_t stride = gridDim.x * waves_per_wg;
+    const BlockDiv dbc1(h.bc1), dbc2(h.bc2);
+
+    uint32_t ti = 0; // rows[ti].block_start <= blk; blk only grows, so the search restarts from ti
+    for (uint32_t blk = wave; blk < total_blocks; blk += stride) {
+        uint32_t lo = ti, hi = n_rows; // answer in [lo, hi)
+        while (hi - lo > 1) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (rows[mid].block_start <= blk) lo = mid; else hi = mid;
+        }
+        ti = lo;
+        const DevTensor t = rows[ti];
+        const uint32_t lb = blk - t.block_start;
+        const uint64_t left = t.numel - (uint64_t)lb * kBlock;
+        const float gscale = GS ? h.grad_scale * t.grad_scale : 1.0f;
+        if (left >= kBlock)
+            full_block<BF16, MODE, EXACT, WD, GS, KEYTAB>(t, lb, lane, h, gscale, dbc1, dbc2, L);
+        else
+            tail_block<BF16, MODE, EXACT, WD, GS, KEYTAB>(t, lb, (uint32_t)left, lane, h, gscale, dbc1, dbc2, L);
+    }
+}
+
+template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB>
+static int launch_one(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
+                      const void *lds_image, uint32_t grid, uint32_t wg, hipStream_t s) {
+    auto k = adam8_step_kernel<BF16, MODE, EXACT, WD, GS, KEYTAB>;
+    static bool attr_set = false; // the table image exceeds the 64 KiB default only if it ever grows
+    if (!attr_set) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)kLdsImageBytes);
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(k, dim3(grid), dim3(wg), kLdsImageBytes, s, rows, n_rows, total_blocks, h,
+                       static_cast<const uint4 *>(lds_image));
+    return (int)hipGetLastError();
+}
+
+template <bool BF16, int MODE, bool EXACT>
+static int launch_flags(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
+                        const void *img, uint32_t grid, uint32_t wg, hipStream_t s) {
+    const bool wd = h.weight_decay > 0.0f;
+    const bool gs = (h.flags & ERI_ADAM8_FLAG_GRAD_SCALE) != 0;
+    const bool bs = (h.flags & ERI_ADAM8_FLAG_BSEARCH) != 0;
+#define ERI_GO(W, G, K) return launch_one<BF16, MODE, EXACT, W, G, K>(rows, n_rows, total_blocks, h, img, grid, wg, s)
+    if (bs) { // cross-check path: only the two decay variants are built for it
+        if (wd) { if (gs) ERI_GO(true, true, false); ERI_GO(true, false, false); }
+        if (gs) ERI_GO(false, true, false);
+        ERI_GO(false, false, false);
+    }
+    if (wd) { if (gs) ERI_GO(true, true, true); ERI_GO(true, false, true); }
+    if (gs) ERI_GO(false, true, true);
+    ERI_GO(false, false, true);
+#undef ERI_GO
+}
+
+int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, int dtype_tag,
+                const EriAdam8Hyper &h, const void *lds_image, uint32_t grid, uint32_t wg, void *stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool exact = (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0;
+    if (dtype_tag == ERI_DTYPE_F32) {
+        if (h.mode == ERI_ADAM8_MODE_L2)
+            return launch_flags<false, ERI_ADAM8_MODE_L2, true>(rows, n_rows, total_blocks, h, lds_image, grid, wg, s);
+        return launch_flags<false, ERI_ADAM8_MODE_ERI, true>(rows, n_rows, total_blocks, h, lds_image, grid, wg, s);
+    }
+    if (h.mode == ERI_ADAM8_MODE_L2) {
+        if (exact) return launch_flags<true, ERI_ADAM8_MODE_L2, true>(rows, n_rows, total_blocks, h, lds_image, grid, wg, s);
+        return launch_flags<true, ERI_ADAM8_MODE_L2, false>(rows, n_rows, total_blocks, h, lds_image, grid, wg, s);
+    }
+    if (exact) return launch_flags<true, ERI_ADAM8_MODE_ERI, true>(rows, n_rows, total_blocks, h, lds_image, grid, wg, s);
+    return launch_flags<true, ERI_ADAM8_MODE_ERI, false>(rows, n_rows, total_blocks, h, lds_image, grid, wg, s);
+}
+
+// ------------------------------------------------------------------------------------------
+// state initialisation and blockwise (de)quantisation for checkpoint traffic
+// ------------------------------------------------------------------------------------------
+
+__global__ void state_init_kernel(uint8_t *m, uint8_t *v, float *am, float *av, uint64_t numel, uint64_t nblocks) {
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint64_t n = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = tid; i < numel; i += n) {
+        m[i] = 127;
+        v[i] = 0;
+    }
+    for (uint64_t b = tid; b < nblocks; b += n) {
+        am[b] = 0.0f;
+        av[b] = 0.0f;
+    }
+}
+
+int launch_state_init(uint8_t *m, uint8_t *v, float *absmax_m, float *absmax_v, uint64_t numel, void *stream) {
+    const uint64_t nblocks = (numel + kBlock - 1) / kBlock;
+    uint64_t grid = (numel + 255) / 256;
+    if (grid > 8192) grid = 8192;
+    hipLaunchKernelGGL(state_init_kernel, dim3((uint32_t)grid), dim3(256), 0, static_cast<hipStream_t>(stream), m,
+                       v, absmax_m, absmax_v, numel, nblocks);
+    return (int)hipGetLastError();
+}
+
+__global__ void dequantize_kernel(const uint8_t *codes, const float *absmax, uint64_t numel, float *out,
+                                  const float *map) {
+    __shared__ float lmap[256];
+    lmap[threadIdx.x] = map[threadIdx.x];
+    __syncthreads();
+    const uint64_t n = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < numel; i += n)
+        out[i] = lmap[codes[i]] * absmax[i / kBlock];
+}
+
+int launch_dequantize(const uint8_t *codes, const float *absmax, int signed_map, uint64_t numel, float *out,
+                      const void *lds_image, void *stream) {
+    const float *map = reinterpret_cast<const float *>(static_cast<const char *>(lds_image) +
+                                                       (signed_map ? kOffMapS : kOffMapU));
+    uint64_t grid = (numel + 255) / 256;
+    if (grid > 16384) grid = 16384;
+    hipLaunchKernelGGL(dequantize_kernel, dim3((uint32_t)grid), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       codes, absmax, numel, out, map);
+    return (int)hipGetLastError();
+}
+
+/* One wavefront per block: absmax by DPP, then the nearest code by binary search. */
+__global__ void quantize_kernel(const float *x, uint64_t numel, uint64_t nblocks, uint8_t *codes, float *absmax,
+                                const float *mid) {
+    __shared__ float lmid[256];
+    lmid[threadIdx.x] = mid[threadIdx.x];
+    __syncthreads();
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint64_t wave = (uint64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+    const uint64_t nw = (uint64_t)gridDim.x * (blockDim.x / kWave);
+    for (uint64_t b = wave; b < nblocks; b += nw) {
+        const uint64_t e0 = b * kBlock;
+        const uint32_t n = (uint32_t)((numel - e0) < kBlock ? (numel - e0) : kBlock);
+        float a = 0.0f;
+        for (uint32_t i = lane; i < n; i += kWave) a = fmaxf(a, __builtin_fabsf(x[e0 + i]));
+        a = wave_max(a);
+        for (uint32_t i = lane; i < n; i += kWave) {
+            const float q = a == 0.0f ? 0.0f : x[e0 + i] / a;
+            codes[e0 + i] = (uint8_t)code_bsearch(q, lmid);
+        }
+        if (lane == 0) absmax[b] = a;
+    }
+}
+
+int launch_quantize(const float *x, int signed_map, uint64_t numel, uint8_t *codes, float *absmax,
+                    const void *lds_image, void *stream) {
+    const float *mid = reinterpret_cast<const float *>(static_cast<const char *>(lds_image) +
+                                                       (signed_map ? kOffMidS : kOffMidU));
+    const uint64_t nblocks = (numel + kBlock - 1) / kBlock;
+    uint64_t grid = (nblocks + 3) / 4;
+    if (grid > 8192) grid = 8192;
+    hipLaunchKernelGGL(quantize_kernel, dim3((uint32_t)grid), dim3(256), 0, static_cast<hipStream_t>(stream), x,
+                       numel, nblocks, codes, absmax, mid);
+    return (int)hipGetLastError();
+}
+
+} // namespace eri

@@ -1,0 +1,603 @@
+/*
+ * Host side of the C ABI declared in include/eri_optim8.h: device storage over the HIP runtime,
+ * construction and self-check of the quantisation tables, validation and upload of the launch
+ * table, and the step dispatch.  No torch, no CUDA shim; the only dependency is libamdhip64.
+ */
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <limits>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "eri_adam8_device.h"
+#include "eri_dynamic_maps.inc"
+
+namespace {
+
+thread_local std::string g_err;
+
+int fail(int code, const std::string &msg) {
+    g_err = msg;
+    return code;
+}
+
+int hip_fail(hipError_t e, const char *what) {
+    g_err = std::string(what) + ": " + hipGetErrorString(e);
+    return (int)e;
+}
+
+#define ERI_HIP(call)                                        \
+    do {                                                     \
+        hipError_t e_ = (call);                              \
+        if (e_ != hipSuccess) return hip_fail(e_, #call);    \
+    } while (0)
+
+inline float bits_to_float(uint32_t u) {
+    float f;
+    std::memcpy(&f, &u, 4);
+    return f;
+}
+
+// ---------------------------------------------------------------------------------------------
+// quantisation tables
+// ---------------------------------------------------------------------------------------------
+
+struct Tables {
+    float map_s[256], map_u[256];
+    float mid_s[256], mid_u[256]; // 255 midpoints + inf
+    std::vector<unsigned char> image;
+    bool ok = false;
+    std::string why;
+};
+
+uint32_t count_below(const float *mid, float x) { // the definition the slots must reproduce
+    uint32_t n = 0;
+    for (int j = 0; j < 255; ++j) n += (x > mid[j]) ? 1u : 0u;
+    return n;
+}
+
+/* Fills `slots` for one sign of one map and checks that no slot spans more than one midpoint. */
+bool build_slots(const float *mid, uint32_t shift, uint32_t base, uint32_t nslots, bool negative,
+                 eri::KeySlot *slots, std::string &why) {
+    const uint32_t sign = negative ? 0x80000000u : 0u;
+    for (uint32_t k = 0; k < nslots; ++k) {
+        uint32_t lo_bits = (k + base) << shift;
+        uint32_t hi_bits = lo_bits | ((1u << shift) - 1u);
+        if (k == 0) lo_bits = 0;                // saturating subtraction folds everything smaller in here
+        if (k == nslots - 1) hi_bits = lo_bits; // x == 1.0 exactly
+        // extreme values of the slot in value order
+        const float x_small = bits_to_float((negative ? hi_bits : lo_bits) | sign);
+        const float x_large = bits_to_float((negative ? lo_bits : hi_bits) | sign);
+        const uint32_t c0 = count_below(mid, x_small);
+        const uint32_t c1 = count_below(mid, x_large);
+        if (c1 < c0 || c1 - c0 > 1) {
+            why = "a lookup slot spans more than one quantisation midpoint";
+            return false;
+        }
+        slots[k].lo = c0;
+        slots[k].mid = (c1 == c0) ? std::numeric_limits<float>::infinity() : mid[c0];
+    }
+    slots[nslots].lo = 0; // NaN slot: every comparison of a search is false
+    slots[nslots].mid = std::numeric_limits<float>::infinity();
+    return true;
+}
+
+const Tables &tables() {
+    static Tables t;
+    static std::once_flag once;
+    std::call_once(once, [] {
+        for (int i = 0; i < 256; ++i) {
+            t.map_s[i] = bits_to_float(ERI_DYNAMIC_MAP_SIGNED_BITS[i]);
+            t.map_u[i] = bits_to_float(ERI_DYNAMIC_MAP_UNSIGNED_BITS[i]);
+        }
+        for (int j = 0; j < 255; ++j) {
+            float s = t.map_s[j] + t.map_s[j + 1];
+            t.mid_s[j] = s * 0.5f;
+            float u = t.map_u[j] + t.map_u[j + 1];
+            t.mid_u[j] = u * 0.5f;
+        }
+        t.mid_s[255] = t.mid_u[255] = std::numeric_limits<float>::infinity();
+        for (int j = 0; j < 255; ++j) {
+            if (!(t.map_s[j] < t.map_s[j + 1]) || !(t.map_u[j] < t.map_u[j + 1])) {
+                t.why = "quantisation map is not strictly increasing";
+                return;
+            }
+        }
+        if (t.map_s[127] != 0.0f || t.map_u[0] != 0.0f || t.map_s[255] != 1.0f || t.map_u[255] != 1.0f) {
+            t.why = "quantisation map lost its fixed points";
+            return;
+        }
+        t.image.assign(eri::kLdsImageBytes, 0);
+        std::memcpy(&t.image[eri::kOffMapS], t.map_s, 1024);
+        std::memcpy(&t.image[eri::kOffMapU], t.map_u, 1024);
+        std::memcpy(&t.image[eri::kOffMidS], t.mid_s, 1024);
+        std::memcpy(&t.image[eri::kOffMidU], t.mid_u, 1024);
+        auto *ks = reinterpret_cast<eri::KeySlot *>(&t.image[eri::kOffKeyS]);
+        auto *ku = reinterpret_cast<eri::KeySlot *>(&t.image[eri::kOffKeyU]);
+        if (!build_slots(t.mid_s, eri::kSShift, eri::kSBase, eri::kSSlots, false, ks, t.why)) return;
+        if (!build_slots(t.mid_s, eri::kSShift, eri::kSBase, eri::kSSlots, true, ks + eri::kSPerSign, t.why)) return;
+        if (!build_slots(t.mid_u, eri::kUShift, eri::kUBase, eri::kUSlots, false, ku, t.why)) return;
+        t.ok = true;
+    });
+    return t;
+}
+
+// ---------------------------------------------------------------------------------------------
+// per-device context
+// ---------------------------------------------------------------------------------------------
+
+constexpr int kMaxDevices = 16;
+
+struct DeviceCtx {
+    void *image = nullptr; // device copy of the LDS image
+    uint32_t cus = 0;
+    uint32_t wg = 512;       // threads per workgroup
+    uint32_t wg_per_cu = 2;  // persistent workgroups per compute unit
+    bool ready = false;
+};
+
+DeviceCtx g_ctx[kMaxDevices];
+std::mutex g_ctx_mu;
+
+int env_u32(const char *name, uint32_t lo, uint32_t hi, uint32_t dflt) {
+    const char *s = std::getenv(name);
+    if (!s || !*s) return (int)dflt;
+    long v = std::strtol(s, nullptr, 10);
+    if (v < (long)lo || v > (long)hi) return (int)dflt;
+    return (int)v;
+}
+
+int get_ctx(DeviceCtx **out) {
+    int dev = 0;
+    ERI_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(ERI_ERR_ARG, "device index out of range");
+    std::lock_guard<std::mutex> lk(g_ctx_mu);
+    DeviceCtx &c = g_ctx[dev];
+    if (!c.ready) {
+        const Tables &t = tables();
+        if (!t.ok) return fail(ERI_ERR_INTERNAL, "quantisation tables failed their self-check: " + t.why);
+        hipDeviceProp_t prop;
+        ERI_HIP(hipGetDeviceProperties(&prop, dev));
+        c.cus = (uint32_t)prop.multiProcessorCount;
+        c.wg = (uint32_t)env_u32("ERI_ADAM8_WG", 64, 1024, 512) & ~63u;
+        c.wg_per_cu = (uint32_t)env_u32("ERI_ADAM8_WG_PER_CU", 1, 16, 2);
+        ERI_HIP(hipMalloc(&c.image, eri::kLdsImageBytes));
+        ERI_HIP(hipMemcpy(c.image, t.image.data(), eri::kLdsImageBytes, hipMemcpyHostToDevice));
+        c.ready = true;
+    }
+    *out = &c;
+    return 0;
+}
+
+uint64_t blocks_of(uint64_t numel) { return (numel + eri::kBlock - 1) / eri::kBlock; }
+
+} // namespace
+
+// ---------------------------------------------------------------------------------------------
+// launch table
+// ---------------------------------------------------------------------------------------------
+
+struct EriAdam8Table {
+    struct Group {
+        int dtype = 0;
+        uint32_t n = 0;
+        uint32_t total_blocks = 0;
+        eri::DevTensor *dev = nullptr;
+        eri::DevTensor *pinned = nullptr;
+        std::vector<uint32_t> src; // index into the caller's rows
+    };
+    int device = 0;
+    uint32_t n = 0;
+    uint64_t total_numel = 0;
+    uint64_t total_blocks = 0;
+    Group groups[2]; // F32, BF16
+    std::vector<uint64_t> numel;
+    std::vector<int32_t> dtype;
+    hipEvent_t uploaded = nullptr;
+    bool upload_pending = false;
+};
+
+namespace {
+
+int validate_rows(const EriAdam8Tensor *rows, uint32_t n) {
+    if (!rows) return fail(ERI_ERR_NULL, "rows is NULL");
+    if (n == 0) return fail(ERI_ERR_ARG, "launch table has no rows");
+    uint64_t running = 0;
+    char buf[160];
+    for (uint32_t i = 0; i < n; ++i) {
+        const EriAdam8Tensor &r = rows[i];
+        if (!r.p || !r.g || !r.m || !r.v || !r.absmax_m || !r.absmax_v) {
+            std::snprintf(buf, sizeof buf, "row %u: NULL pointer", i);
+            return fail(ERI_ERR_NULL, buf);
+        }
+        if (r.numel == 0) {
+            std::snprintf(buf, sizeof buf, "row %u: Empty tensor for quantization", i);
+            return fail(ERI_ERR_EMPTY, buf);
+        }
+        if (r.dtype_tag != ERI_DTYPE_F32 && r.dtype_tag != ERI_DTYPE_BF16) {
+            std::snprintf(buf, sizeof buf, "row %u: unsupported dtype tag %d (F32=0 and BF16=2 are supported)", i,
+                          r.dtype_tag);
+            return fail(ERI_ERR_DTYPE, buf);
+        }
+        const uintptr_t wide = (uintptr_t)r.p | (uintptr_t)r.g | (uintptr_t)r.m | (uintptr_t)r.v;
+        const uintptr_t narrow = (uintptr_t)r.absmax_m | (uintptr_t)r.absmax_v;
+        if ((wide & 15u) || (narrow & 3u)) {
+            std::snprintf(buf, sizeof buf, "row %u: p/g/m/v must be 16-byte aligned, absmax 4-byte aligned", i);
+            return fail(ERI_ERR_ALIGN, buf);
+        }
+        if (r.block_start != running) {
+            std::snprintf(buf, sizeof buf, "row %u: block_start %llu, expected %llu", i,
+                          (unsigned long long)r.block_start, (unsigned long long)running);
+            return fail(ERI_ERR_BLOCK_START, buf);
+        }
+        running += blocks_of(r.numel);
+    }
+    if (running > 0x7fffffffull) return fail(ERI_ERR_TOO_LARGE, "more than 2^31 - 1 blocks in one table");
+    return 0;
+}
+
+void fill_group(EriAdam8Table::Group &g, const EriAdam8Tensor *rows) {
+    uint32_t start = 0;
+    for (uint32_t j = 0; j < g.n; ++j) {
+        const EriAdam8Tensor &r = rows[g.src[j]];
+        eri::DevTensor &d = g.pinned[j];
+        d.p = r.p;
+        d.g = r.g;
+        d.m = r.m;
+        d.v = r.v;
+        d.absmax_m = r.absmax_m;
+        d.absmax_v = r.absmax_v;
+        d.numel = r.numel;
+        d.block_start = start;
+        d.grad_scale = r.grad_scale;
+        start += (uint32_t)blocks_of(r.numel);
+    }
+    g.total_blocks = start;
+}
+
+int upload(EriAdam8Table *t, void *stream) {
+    for (auto &g : t->groups) {
+        if (g.n == 0) continue;
+        ERI_HIP(hipMemcpyAsync(g.dev, g.pinned, sizeof(eri::DevTensor) * g.n, hipMemcpyHostToDevice,
+                               static_cast<hipStream_t>(stream)));
+    }
+    ERI_HIP(hipEventRecord(t->uploaded, static_cast<hipStream_t>(stream)));
+    t->upload_pending = true;
+    return 0;
+}
+
+void destroy_table(EriAdam8Table *t) {
+    if (!t) return;
+    for (auto &g : t->groups) {
+        if (g.dev) (void)hipFree(g.dev);
+        if (g.pinned) (void)hipHostFree(g.pinned);
+    }
+    if (t->uploaded) (void)hipEventDestroy(t->uploaded);
+    delete t;
+}
+
+} // namespace
+
+extern "C" {
+
+const char *eri_last_error(void) { return g_err.c_str(); }
+
+// ---- storage --------------------------------------------------------------------------------
+
+int eri_hip_device_count(int *count) {
+    if (!count) return fail(ERI_ERR_NULL, "count is NULL");
+    ERI_HIP(hipGetDeviceCount(count));
+    return 0;
+}
+
+int eri_hip_set_device(int device) {
+    ERI_HIP(hipSetDevice(device));
+    return 0;
+}
+
+int eri_hip_malloc_zeroed(int device, size_t bytes, void **out) {
+    if (!out) return fail(ERI_ERR_NULL, "out is NULL");
+    *out = nullptr;
+    if (bytes == 0) return fail(ERI_ERR_ARG, "zero-byte allocation");
+    int prev = 0;
+    ERI_HIP(hipGetDevice(&prev));
+    if (prev != device) ERI_HIP(hipSetDevice(device));
+    void *p = nullptr;
+    hipError_t e = hipMalloc(&p, bytes);
+    if (e == hipSuccess) e = hipMemset(p, 0, bytes);
+    if (prev != device) (void)hipSetDevice(prev);
+    if (e != hipSuccess) {
+        if (p) (void)hipFree(p);
+        return hip_fail(e, "hipMalloc/hipMemset");
+    }
+    *out = p;
+    return 0;
+}
+
+int eri_hip_free(void *ptr) {
+    if (!ptr) return 0;
+    ERI_HIP(hipFree(ptr));
+    return 0;
+}
+
+void *eri_hip_host_alloc(size_t bytes) {
+    void *p = nullptr;
+    hipError_t e = hipHostMalloc(&p, bytes, hipHostMallocPortable);
+    if (e != hipSuccess) {
+        hip_fail(e, "hipHostMalloc");
+        return nullptr;
+    }
+    return p;
+}
+
+int eri_hip_host_free(void *ptr) {
+    if (!ptr) return 0;
+    ERI_HIP(hipHostFree(ptr));
+    return 0;
+}
+
+int eri_hip_memcpy_async(void *dst, const void *src, size_t bytes, int kind, void *stream) {
+    if (bytes == 0) return 0;
+    if (!dst || !src) return fail(ERI_ERR_NULL, "memcpy with NULL pointer");
+    hipMemcpyKind k = hipMemcpyDefault;
+    if (kind == 1) k = hipMemcpyHostToDevice;
+    else if (kind == 2) k = hipMemcpyDeviceToHost;
+    else if (kind == 3) k = hipMemcpyDeviceToDevice;
+    ERI_HIP(hipMemcpyAsync(dst, src, bytes, k, static_cast<hipStream_t>(stream)));
+    return 0;
+}
+
+int eri_hip_memset_async(void *dst, int value, size_t bytes, void *stream) {
+    if (bytes == 0) return 0;
+    if (!dst) return fail(ERI_ERR_NULL, "memset with NULL pointer");
+    ERI_HIP(hipMemsetAsync(dst, value, bytes, static_cast<hipStream_t>(stream)));
+    return 0;
+}
+
+int eri_hip_stream_create(void **stream) {
+    if (!stream) return fail(ERI_ERR_NULL, "stream is NULL");
+    hipStream_t s = nullptr;
+    ERI_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *stream = s;
+    return 0;
+}
+
+int eri_hip_stream_sync(void *stream) {
+    ERI_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    return 0;
+}
+
+int eri_hip_stream_destroy(void *stream) {
+    if (!stream) return 0;
+    ERI_HIP(hipStreamDestroy(static_cast<hipStream_t>(stream)));
+    return 0;
+}
+
+int eri_hip_mem_info(size_t *free_bytes, size_t *total_bytes) {
+    size_t f = 0, t = 0;
+    ERI_HIP(hipMemGetInfo(&f, &t));
+    if (free_bytes) *free_bytes = f;
+    if (total_bytes) *total_bytes = t;
+    return 0;
+}
+
+// ---- optimizer ------------------------------------------------------------------------------
+
+int eri_adam8_init(void) {
+    DeviceCtx *c = nullptr;
+    return get_ctx(&c);
+}
+
+int eri_adam8_get_maps(float *signed256, float *unsigned256) {
+    const Tables &t = tables();
+    if (!t.ok) return fail(ERI_ERR_INTERNAL, "quantisation tables failed their self-check: " + t.why);
+    if (signed256) std::memcpy(signed256, t.map_s, 1024);
+    if (unsigned256) std::memcpy(unsigned256, t.map_u, 1024);
+    return 0;
+}
+
+int eri_adam8_table_image(void *out, size_t cap, size_t *bytes, uint32_t offsets[6]) {
+    const Tables &t = tables();
+    if (!t.ok) return fail(ERI_ERR_INTERNAL, "quantisation tables failed their self-check: " + t.why);
+    if (bytes) *bytes = t.image.size();
+    if (offsets) {
+        const uint32_t o[6] = {eri::kOffMapS, eri::kOffMapU, eri::kOffMidS, eri::kOffMidU, eri::kOffKeyS, eri::kOffKeyU};
+        std::memcpy(offsets, o, sizeof o);
+    }
+    if (out) {
+        if (cap < t.image.size()) return fail(ERI_ERR_ARG, "table image does not fit the buffer");
+        std::memcpy(out, t.image.data(), t.image.size());
+    }
+    return 0;
+}
+
+int eri_adam8_hyper_pack(double lr, double beta1, double beta2, double eps, double weight_decay, uint64_t step,
+                         int mode, uint32_t flags, EriAdam8Hyper *out) {
+    if (!out) return fail(ERI_ERR_NULL, "out is NULL");
+    if (mode != ERI_ADAM8_MODE_ERI && mode != ERI_ADAM8_MODE_L2) return fail(ERI_ERR_ARG, "unknown mode");
+    std::memset(out, 0, sizeof(*out));
+    out->mode = mode;
+    out->flags = flags;
+    out->beta1 = (float)beta1;
+    out->beta2 = (float)beta2;
+    out->eps = (float)eps;
+    out->weight_decay = (float)weight_decay;
+    out->grad_scale = 1.0f;
+    if (mode == ERI_ADAM8_MODE_L2) {
+        const uint64_t s = step < 1 ? 1 : step;               // adam8bit.rs:164
+        out->omb1 = (float)(1.0 - beta1);                      // :142  f64 subtraction, then the cast
+        out->omb2 = (float)(1.0 - beta2);                      // :151
+        out->bc1 = (float)(1.0 - std::pow(beta1, (double)(int32_t)s)); // :167 powi
+        out->bc2 = (float)(1.0 - std::pow(beta2, (double)(int32_t)s)); // :175
+        out->step_size = (float)lr;                            // :193
+    } else {
+        const double t = (double)step;                         // adam8bit_enhanced.rs:210
+        const double bc1 = 1.0 - std::pow(beta1, t);           // :213
+        const double bc2 = 1.0 - std::pow(beta2, t);           // :214
+        out->omb1 = 1.0f - out->beta1;                         // :256  `1.0 - beta1 as f32`
+        out->omb2 = 1.0f - out->beta2;                         // :260
+        out->bc1 = (float)bc1;
+        out->bc2 = (float)bc2;
+        out->step_size = (float)(lr * (std::sqrt(bc2) / bc1)); // :215, cast at :274
+    }
+    return 0;
+}
+
+int eri_adam8_state_init(uint8_t *m, uint8_t *v, float *absmax_m, float *absmax_v, uint64_t numel, void *stream) {
+    if (!m || !v || !absmax_m || !absmax_v) return fail(ERI_ERR_NULL, "state pointer is NULL");
+    if (numel == 0) return fail(ERI_ERR_EMPTY, "Empty tensor for quantization");
+    int rc = eri::launch_state_init(m, v, absmax_m, absmax_v, numel, stream);
+    if (rc) return hip_fail((hipError_t)rc, "state_init launch");
+    return 0;
+}
+
+int eri_adam8_table_create(const EriAdam8Tensor *rows, uint32_t n, void *stream, EriAdam8Table **out) {
+    if (!out) return fail(ERI_ERR_NULL, "out is NULL");
+    *out = nullptr;
+    int rc = validate_rows(rows, n);
+    if (rc) return rc;
+    DeviceCtx *ctx = nullptr;
+    rc = get_ctx(&ctx);
+    if (rc) return rc;
+    EriAdam8Table *t = new EriAdam8Table();
+    t->n = n;
+    (void)hipGetDevice(&t->device);
+    t->groups[0].dtype = ERI_DTYPE_F32;
+    t->groups[1].dtype = ERI_DTYPE_BF16;
+    t->numel.resize(n);
+    t->dtype.resize(n);
+    for (uint32_t i = 0; i < n; ++i) {
+        t->numel[i] = rows[i].numel;
+        t->dtype[i] = rows[i].dtype_tag;
+        t->total_numel += rows[i].numel;
+        t->total_blocks += blocks_of(rows[i].numel);
+        t->groups[rows[i].dtype_tag == ERI_DTYPE_F32 ? 0 : 1].src.push_back(i);
+    }
+    hipError_t e = hipEventCreateWithFlags(&t->uploaded, hipEventDisableTiming);
+    for (auto &g : t->groups) {
+        g.n = (uint32_t)g.src.size();
+        if (g.n == 0 || e != hipSuccess) continue;
+        e = hipMalloc((void **)&g.dev, sizeof(eri::DevTensor) * g.n);
+        if (e == hipSuccess) e = hipHostMalloc((void **)&g.pinned, sizeof(eri::DevTensor) * g.n, hipHostMallocDefault);
+        if (e == hipSuccess) fill_group(g, rows);
+    }
+    if (e != hipSuccess) {
+        destroy_table(t);
+        return hip_fail(e, "launch table allocation");
+    }
+    rc = upload(t, stream);
+    if (rc) {
+        destroy_table(t);
+        return rc;
+    }
+    *out = t;
+    return 0;
+}
+
+int eri_adam8_table_update(EriAdam8Table *t, const EriAdam8Tensor *rows, uint32_t n, void *stream) {
+    if (!t) return fail(ERI_ERR_NULL, "table is NULL");
+    int rc = validate_rows(rows, n);
+    if (rc) return rc;
+    if (n != t->n) return fail(ERI_ERR_ARG, "table_update: row count differs from the table's");
+    for (uint32_t i = 0; i < n; ++i)
+        if (rows[i].numel != t->numel[i] || rows[i].dtype_tag != t->dtype[i])
+            return fail(ERI_ERR_ARG, "table_update: numel or dtype differs from the table's");
+    if (t->upload_pending) { // the pinned mirror may still be the source of the previous copy
+        ERI_HIP(hipEventSynchronize(t->uploaded));
+        t->upload_pending = false;
+    }
+    for (auto &g : t->groups)
+        if (g.n) fill_group(g, rows);
+    return upload(t, stream);
+}
+
+int eri_adam8_table_destroy(EriAdam8Table *t) {
+    destroy_table(t);
+    return 0;
+}
+
+int eri_adam8_table_info(const EriAdam8Table *t, uint64_t *total_numel, uint64_t *total_blocks) {
+    if (!t) return fail(ERI_ERR_NULL, "table is NULL");
+    if (total_numel) *total_numel = t->total_numel;
+    if (total_blocks) *total_blocks = t->total_blocks;
+    return 0;
+}
+
+int eri_adam8_step_table(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream) {
+    if (!t || !h) return fail(ERI_ERR_NULL, "table or hyper is NULL");
+    if (h->mode != ERI_ADAM8_MODE_ERI && h->mode != ERI_ADAM8_MODE_L2) return fail(ERI_ERR_ARG, "unknown mode");
+    DeviceCtx *ctx = nullptr;
+    int rc = get_ctx(&ctx);
+    if (rc) return rc;
+    for (auto &g : t->groups) {
+        if (g.n == 0) continue;
+        const uint32_t waves_per_wg = ctx->wg / eri::kWave;
+        uint32_t grid = ctx->cus * ctx->wg_per_cu;
+        const uint32_t need = (g.total_blocks + waves_per_wg - 1) / waves_per_wg;
+        if (grid > need) grid = need;
+        if (grid == 0) grid = 1;
+        rc = eri::launch_step(g.dev, g.n, g.total_blocks, g.dtype, *h, ctx->image, grid, ctx->wg, stream);
+        if (rc) return hip_fail((hipError_t)rc, "adam8 step launch");
+    }
+    return 0;
+}
+
+int eri_adam8_step_multi(const EriAdam8Tensor *rows, uint32_t n, const EriAdam8Hyper *h, void *stream) {
+    struct Cache {
+        EriAdam8Table *table = nullptr;
+        std::vector<EriAdam8Tensor> last;
+        ~Cache() { destroy_table(table); }
+    };
+    thread_local Cache cache;
+    if (!rows || !h) return fail(ERI_ERR_NULL, "rows or hyper is NULL");
+    int dev = 0;
+    ERI_HIP(hipGetDevice(&dev));
+    bool same_shape = cache.table && cache.table->n == n && cache.table->device == dev;
+    if (same_shape)
+        for (uint32_t i = 0; i < n && same_shape; ++i)
+            same_shape = rows[i].numel == cache.table->numel[i] && rows[i].dtype_tag == cache.table->dtype[i];
+    int rc = 0;
+    if (!same_shape) {
+        destroy_table(cache.table);
+        cache.table = nullptr;
+        cache.last.clear();
+        rc = eri_adam8_table_create(rows, n, stream, &cache.table);
+        if (rc) return rc;
+        cache.last.assign(rows, rows + n);
+    } else if (std::memcmp(cache.last.data(), rows, sizeof(EriAdam8Tensor) * n) != 0) {
+        rc = eri_adam8_table_update(cache.table, rows, n, stream);
+        if (rc) return rc;
+        cache.last.assign(rows, rows + n);
+    }
+    return eri_adam8_step_table(cache.table, h, stream);
+}
+
+int eri_adam8_dequantize(const uint8_t *codes, const float *absmax, int signed_map, uint64_t numel, float *out,
+                         void *stream) {
+    if (!codes || !absmax || !out) return fail(ERI_ERR_NULL, "dequantize with NULL pointer");
+    if (numel == 0) return fail(ERI_ERR_EMPTY, "Empty quantized data");
+    DeviceCtx *ctx = nullptr;
+    int rc = get_ctx(&ctx);
+    if (rc) return rc;
+    rc = eri::launch_dequantize(codes, absmax, signed_map, numel, out, ctx->image, stream);
+    if (rc) return hip_fail((hipError_t)rc, "dequantize launch");
+    return 0;
+}
+
+int eri_adam8_quantize(const float *x, int signed_map, uint64_t numel, uint8_t *codes, float *absmax, void *stream) {
+    if (!x || !codes || !absmax) return fail(ERI_ERR_NULL, "quantize with NULL pointer");
+    if (numel == 0) return fail(ERI_ERR_EMPTY, "Empty tensor for quantization");
+    DeviceCtx *ctx = nullptr;
+    int rc = get_ctx(&ctx);
+    if (rc) return rc;
+    rc = eri::launch_quantize(x, signed_map, numel, codes, absmax, ctx->image, stream);
+    if (rc) return hip_fail((hipError_t)rc, "quantize launch");
+    return 0;
+}
+
+} // extern "C"

@@ -1,0 +1,169 @@
+/*
+ * eri_optim8 -- C ABI of the MI355X (gfx950) blockwise 8-bit AdamW step for EriDiffusion.
+ *
+ * Everything EriDiffusion's optimizer path needs from native code crosses this header: device
+ * storage (hipMalloc / hipMemcpyAsync, no CUDA shim), the multi-tensor launch table, and the
+ * single-pass step kernel.  Plain pointers and sizes only; a Rust `extern "C"` block, ctypes or
+ * cgo can bind it as it stands.
+ *
+ * Conventions, taken from the reference's own Rust<->C seam:
+ *   - every call returns int: 0 on success, a positive hipError_t from the runtime, or a negative
+ *     EriStatus for argument errors.  The reference's launchers return 0 or the raw cudaError_t
+ *     (crates/core/cuda/narrow_strided.cu:93-97) and its Rust side turns non-zero into
+ *     Err(TensorOp("... failed with code N")) (crates/core/src/tensor_narrow.rs:221-227).
+ *   - streams are passed as void* and NULL means the default stream
+ *     (crates/core/src/device.rs:69-71, tensor_narrow.rs:197-201).
+ *   - dtype tags are F32=0, F16=1, BF16=2, I32=3 (crates/core/src/cuda/dtype_tag.rs:3-19);
+ *     the optimizer accepts F32 and BF16 parameters/gradients.
+ *   - nothing here synchronises the device unless its name says so; the step is stream-ordered.
+ *   - the library never takes ownership of parameter, gradient or state memory.
+ */
+#ifndef ERI_OPTIM8_H
+#define ERI_OPTIM8_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ERI_ADAM8_BLOCK 2048u /* elements per quantisation block */
+
+typedef enum EriDTypeTag { ERI_DTYPE_F32 = 0, ERI_DTYPE_F16 = 1, ERI_DTYPE_BF16 = 2, ERI_DTYPE_I32 = 3 } EriDTypeTag;
+
+typedef enum EriStatus {
+    ERI_OK = 0,
+    ERI_ERR_NULL = -1,        /* a required pointer is NULL */
+    ERI_ERR_ALIGN = -2,       /* p/g/m/v not 16-byte aligned, absmax not 4-byte aligned */
+    ERI_ERR_EMPTY = -3,       /* numel == 0 ("Empty tensor for quantization", adam8bit_enhanced.rs:46-50) */
+    ERI_ERR_DTYPE = -4,       /* dtype tag other than F32 / BF16 */
+    ERI_ERR_BLOCK_START = -5, /* block_start is not the running sum of ceil(numel / 2048) */
+    ERI_ERR_ARG = -6,         /* any other bad argument (mode, count, size, kind) */
+    ERI_ERR_TOO_LARGE = -7,   /* more than 2^31 - 1 blocks in one table */
+    ERI_ERR_INTERNAL = -8     /* the lookup tables failed their self-check */
+} EriStatus;
+
+/* Message for the last failing call on this thread ("" if none).  Never NULL. */
+const char *eri_last_error(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * Device storage.  Replaces the cudarc-backed seam of the reference:
+ *   cuda_malloc_zeroed(dev, size) -> *mut u8          crates/core/src/cuda/mod.rs:47-66
+ *   MemoryPool::allocate_raw_memory                    crates/core/src/memory.rs:289-311
+ *   cuda_alloc_pinned_host / cuda_free_pinned_host /
+ *   cuda_memcpy_async(dst, src, bytes, kind, stream)   crates/core/cuda/utils_pinned.cu:4-20
+ * `kind` keeps the reference's encoding: 1 = host->device, 2 = device->host, 3 = device->device,
+ * anything else = let the runtime infer it.
+ * ------------------------------------------------------------------------------------------- */
+int eri_hip_device_count(int *count);
+int eri_hip_set_device(int device);
+int eri_hip_malloc_zeroed(int device, size_t bytes, void **out); /* 256-byte aligned, zero-filled */
+int eri_hip_free(void *ptr);
+void *eri_hip_host_alloc(size_t bytes);                          /* pinned; NULL on failure */
+int eri_hip_host_free(void *ptr);
+int eri_hip_memcpy_async(void *dst, const void *src, size_t bytes, int kind, void *stream);
+int eri_hip_memset_async(void *dst, int value, size_t bytes, void *stream);
+int eri_hip_stream_create(void **stream);                        /* default priority */
+int eri_hip_stream_sync(void *stream);
+int eri_hip_stream_destroy(void *stream);
+int eri_hip_mem_info(size_t *free_bytes, size_t *total_bytes);
+
+/* ---------------------------------------------------------------------------------------------
+ * The optimizer step.
+ * ------------------------------------------------------------------------------------------- */
+
+/* Which reference function the arithmetic follows. */
+typedef enum EriAdam8Mode {
+    ERI_ADAM8_MODE_ERI = 0, /* Adam8bit::step,   src/trainers/adam8bit_enhanced.rs:202-291:
+                               p -= step_size * (m / (sqrt(v) + eps) + wd * p) */
+    ERI_ADAM8_MODE_L2 = 1   /* Adam8bit::update, src/trainers/adam8bit.rs:101-208:
+                               g += wd * p; p -= cast(lr * (m/bc1) / (sqrt(max(v/bc2, 0)) + eps)) */
+} EriAdam8Mode;
+
+enum {
+    ERI_ADAM8_FLAG_GRAD_SCALE = 1u << 0,  /* multiply gradients by hyper.grad_scale * tensor.grad_scale */
+    ERI_ADAM8_FLAG_EXACT_PARAM = 1u << 1, /* IEEE sqrt and divide on the parameter update of BF16
+                                             tensors too (F32 tensors always use them) */
+    ERI_ADAM8_FLAG_BSEARCH = 1u << 2      /* requantise by binary search of the LDS midpoint table
+                                             instead of the float-keyed slot table (same codes) */
+};
+
+/* Per-step scalars, already cast where the reference casts them.  Fill with eri_adam8_hyper_pack. */
+typedef struct EriAdam8Hyper {
+    float beta1, beta2; /* (float)beta                               adam8bit_enhanced.rs:256,260 */
+    float omb1, omb2;   /* ERI: 1.0f - (float)beta; L2: (float)(1.0 - beta)    :256,260 / adam8bit.rs:142,151 */
+    float eps;          /* (float)eps                                :263 */
+    float weight_decay; /* (float)wd                                 :268 */
+    float step_size;    /* ERI: (float)(lr * sqrt(bc2) / bc1), f64 inside      :213-215,274; L2: (float)lr */
+    float bc1, bc2;     /* L2: (float)(1 - beta^max(step,1))         adam8bit.rs:164-178 */
+    float grad_scale;   /* used with ERI_ADAM8_FLAG_GRAD_SCALE       pipeline_flux_lora_sequential.rs:1198-1213 */
+    int32_t mode;       /* EriAdam8Mode */
+    uint32_t flags;     /* ERI_ADAM8_FLAG_* */
+} EriAdam8Hyper;
+
+/* `step` is the optimizer's counter after its increment for ERI (adam8bit_enhanced.rs:203) and the
+ * counter as it stands when update() runs for L2 (adam8bit.rs:164; step() bumps it afterwards). */
+int eri_adam8_hyper_pack(double lr, double beta1, double beta2, double eps, double weight_decay,
+                         uint64_t step, int mode, uint32_t flags, EriAdam8Hyper *out);
+
+/* One row of the launch table: a parameter tensor, its gradient and its 8-bit state.
+ * m/v hold numel codes, absmax_* hold ceil(numel / 2048) floats.  All device pointers. */
+typedef struct EriAdam8Tensor {
+    void *p;              /* parameters, updated in place */
+    const void *g;        /* gradients, same dtype as p */
+    uint8_t *m;           /* first-moment codes (signed dynamic map) */
+    uint8_t *v;           /* second-moment codes (unsigned dynamic map) */
+    float *absmax_m;      /* per-block scale of m */
+    float *absmax_v;      /* per-block scale of v */
+    uint64_t numel;
+    uint64_t block_start; /* index of this tensor's first block = sum of the blocks before it */
+    int32_t dtype_tag;    /* ERI_DTYPE_F32 or ERI_DTYPE_BF16 */
+    float grad_scale;     /* per-layer multiplier (pipeline_flux_lora_sequential.rs:759-766);
+                             read only with ERI_ADAM8_FLAG_GRAD_SCALE */
+} EriAdam8Tensor;
+
+typedef struct EriAdam8Table EriAdam8Table; /* device-resident copy of a launch table */
+
+/* Loads the quantisation tables onto the current device.  Optional: the first table does it. */
+int eri_adam8_init(void);
+
+/* The two 256-entry maps (code -> value in [-1, 1] / [0, 1]) the states are expressed in. */
+int eri_adam8_get_maps(float *signed256, float *unsigned256);
+
+/* Codes of 0.0 (127 / 0) and absmax 0: the state of a zeros tensor (adam8bit_enhanced.rs:179-197). */
+int eri_adam8_state_init(uint8_t *m, uint8_t *v, float *absmax_m, float *absmax_v, uint64_t numel,
+                         void *stream);
+
+/* Validates `rows` and uploads them.  The steady-state step then allocates nothing. */
+int eri_adam8_table_create(const EriAdam8Tensor *rows, uint32_t n, void *stream, EriAdam8Table **out);
+/* Same tensors (count, numel, dtype), new pointers / grad_scale -- e.g. fresh gradient buffers. */
+int eri_adam8_table_update(EriAdam8Table *table, const EriAdam8Tensor *rows, uint32_t n, void *stream);
+int eri_adam8_table_destroy(EriAdam8Table *table);
+int eri_adam8_table_info(const EriAdam8Table *table, uint64_t *total_numel, uint64_t *total_blocks);
+
+/* One optimizer step over every tensor of the table: one kernel launch per dtype present. */
+int eri_adam8_step_table(EriAdam8Table *table, const EriAdam8Hyper *hyper, void *stream);
+
+/* Convenience for callers that keep no handle: keeps one cached table per calling thread and
+ * re-uploads it only when `rows` changed since that thread's last call. */
+int eri_adam8_step_multi(const EriAdam8Tensor *rows, uint32_t n, const EriAdam8Hyper *hyper, void *stream);
+
+/* Copies the host image of the kernel's lookup tables (the bytes every workgroup stages into LDS)
+ * into `out` (capacity `cap`) and reports its size and the byte offsets of its six parts:
+ * signed map, unsigned map, signed midpoints, unsigned midpoints, signed slots, unsigned slots.
+ * No device is touched; the CPU tests replay the kernel's slot lookup against it. */
+int eri_adam8_table_image(void *out, size_t cap, size_t *bytes, uint32_t offsets[6]);
+
+/* Blockwise state <-> fp32, for checkpoints that store unquantised moments
+ * (get_state_as_tensors / load_state_from_tensors, src/trainers/adam8bit.rs:296-329).
+ * signed_map != 0 selects the first-moment map. */
+int eri_adam8_dequantize(const uint8_t *codes, const float *absmax, int signed_map, uint64_t numel,
+                         float *out, void *stream);
+int eri_adam8_quantize(const float *x, int signed_map, uint64_t numel, uint8_t *codes, float *absmax,
+                       void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ERI_OPTIM8_H */

@@ -1,0 +1,212 @@
+"""GPU parity: the HIP step, called through the C ABI, against the CPU oracle on the same inputs.
+
+The bar, written out: absmax bit-exact; state codes bit-exact (any +-1 neighbour is counted, and
+the counts are asserted to be zero here because the kernel and the oracle share the tie rule);
+fp32 parameters bit-exact; bf16 parameters bit-exact with ERI_ADAM8_FLAG_EXACT_PARAM and within
+one bf16 ulp (counted) on the default approximate square root / reciprocal path.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import harness as hs
+import oracle_c as oc
+
+pytestmark = pytest.mark.gpu
+
+LR, B1, B2, EPS, WD = 1e-4, 0.9, 0.999, 1e-8, 0.01
+
+
+def _lib():
+    from eridiffusion_amd import _lib
+    return _lib
+
+
+def _stream():
+    import torch
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _sync():
+    import torch
+    torch.cuda.synchronize()
+
+
+def gpu_steps(gt, steps_grads, first_step, mode=0, flags=0, wd=WD, lr=LR, grad_scale=None, tensor_scales=None,
+              use_multi=False):
+    """Runs len(steps_grads) steps on the device; the first uses the gradients already uploaded."""
+    L = _lib()
+    rows = gt.rows(tensor_scales)
+    table = C.c_void_p()
+    if not use_multi:
+        L.check(L.lib().eri_adam8_table_create(rows, len(rows), _stream(), C.byref(table)), "table_create")
+    for k, gs in enumerate(steps_grads):
+        if gs is not None:
+            gt.set_grads(gs)
+        step = first_step + k
+        h = L.hyper_pack(lr, B1, B2, EPS, wd, step if mode == 0 else step - 1, mode, flags, grad_scale)
+        if use_multi:
+            L.check(L.lib().eri_adam8_step_multi(rows, len(rows), C.byref(h), _stream()), "step_multi")
+        else:
+            L.check(L.lib().eri_adam8_step_table(table, C.byref(h), _stream()), "step_table")
+    _sync()
+    if not use_multi:
+        L.lib().eri_adam8_table_destroy(table)
+
+
+def run_case(sizes, bf16, seed, steps=3, mode=0, flags=0, wd=WD, p_std=0.02, g_std=1e-3, prior=0,
+             grad_scale=None, use_multi=False, label=""):
+    ps, gs = hs.make_inputs(sizes, bf16, seed, p_std, g_std)
+    states = hs.oracle_states(sizes)
+    omode = oc.MODE_ERI if mode == 0 else oc.MODE_L2
+    for t in range(1, prior + 1):  # seed the states with a few oracle steps
+        g_t = hs.fresh_grads(sizes, bf16, seed * 1000 + t, g_std)
+        hs.oracle_step(ps, g_t, states, (LR, B1, B2, EPS, wd, t if mode == 0 else t - 1), bf16, omode, grad_scale)
+    gt = hs.GpuTensors(ps, gs, states, bf16)
+    all_g = [gs] + [hs.fresh_grads(sizes, bf16, seed * 7777 + k, g_std) for k in range(1, steps)]
+    for k, g_k in enumerate(all_g):
+        t = prior + 1 + k
+        hs.oracle_step(ps, g_k, states, (LR, B1, B2, EPS, wd, t if mode == 0 else t - 1), bf16, omode, grad_scale)
+    gpu_steps(gt, [None] + all_g[1:], prior + 1, mode, flags, wd, grad_scale=grad_scale, use_multi=use_multi)
+    got_p, got_st = gt.fetch()
+    exact = (not bf16) or bool(flags & 2)
+    stats = hs.compare(got_p, got_st, ps, states, bf16, exact, label)
+    print("%s: params=%d code_mismatch=%d param_1ulp=%d" % (label, stats["params"], stats["code_mismatch"],
+                                                              stats["param_1ulp"]), flush=True)
+    assert stats["code_mismatch"] == 0
+    return stats
+
+
+def test_config1_flat_fp32_after_ten_prior_steps():
+    # BASELINE configuration 1: 2**20 fp32 params ~N(0, 0.02), grads ~N(0, 1e-3), states from ten
+    # prior steps, block 2048, lr 1e-4, betas (0.9, 0.999), eps 1e-8, wd 0.01; one step
+    run_case([1 << 20], False, 0xE21D + 1, steps=1, prior=10, label="c1")
+
+
+def test_config1_all_eleven_steps_on_the_device():
+    run_case([1 << 20], False, 0xE21D + 1, steps=11, prior=0, label="c1-11")
+
+
+@pytest.mark.parametrize("flags", [0, 2, 4, 6])
+def test_bf16_ragged_multi_tensor(flags):
+    sizes = [2048 * 3 + 5, 1, 7, 320, 2047, 2048, 2049, 16 * 640, 1280 * 16, 4, 100000]
+    run_case(sizes, True, 100 + flags, steps=4, flags=flags, label="bf16-ragged-flags%d" % flags)
+
+
+@pytest.mark.parametrize("flags", [0, 4])
+def test_fp32_ragged_multi_tensor(flags):
+    sizes = [2048 * 2 + 1234, 1, 7, 320, 2047, 2049, 65536 + 3]
+    run_case(sizes, False, 200 + flags, steps=4, flags=flags, label="fp32-ragged-flags%d" % flags)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("wd", [0.0, 0.01])
+def test_l2_mode_follows_the_functional_update(bf16, wd):
+    sizes = [2048 * 5 + 77, 320, 2048, 9]
+    run_case(sizes, bf16, 300 + bf16, steps=3, mode=1, flags=2, wd=wd, label="l2-bf16%d-wd%g" % (bf16, wd))
+
+
+def test_no_weight_decay_variant():
+    run_case([2048 * 9 + 3, 640], True, 400, steps=3, wd=0.0, flags=2, label="wd0")
+    run_case([2048 * 9 + 3, 640], False, 401, steps=3, wd=0.0, label="wd0-fp32")
+
+
+def test_grad_scale_folded_into_the_step():
+    run_case([2048 * 4 + 3, 640], True, 500, steps=3, flags=2, grad_scale=0.37, label="gscale")
+    run_case([2048 * 4 + 3, 640], False, 501, steps=2, grad_scale=0.37, label="gscale-fp32")
+
+
+def test_step_multi_convenience_entry_point():
+    run_case([2048 * 4 + 3, 640, 5000], True, 600, steps=3, flags=2, use_multi=True, label="step_multi")
+
+
+def test_lora_scale_values_bf16():
+    # LoRA-B-like: params and updates of the same magnitude (heavy cancellation in p - update)
+    run_case([16 * 5120, 1280 * 16, 16 * 320], True, 700, steps=5, p_std=1e-4, g_std=1e-4, flags=2, label="lora-exact")
+    run_case([16 * 5120, 1280 * 16, 16 * 320], True, 700, steps=5, p_std=1e-4, g_std=1e-4, flags=0, label="lora-fast")
+
+
+def test_scaled_model_shapes_bf16():
+    from eridiffusion_amd import workloads as w
+    for name, tensors in (("c2", w.c2_sdxl_lora(pairs=60, scale=4)), ("c3", w.c3_flux_lora(scale=16)),
+                          ("c4", w.c4_sdxl_full(scale=8)), ("c5", w.c5_flux_full(scale=32))):
+        sizes = [w.numel(s) for _, s in tensors]
+        if name in ("c3", "c5"):
+            sizes = sizes[::6]
+        run_case(sizes, True, 800 + len(sizes), steps=2, label=name + "-scaled")
+
+
+def test_zero_gradients_and_zero_state():
+    sizes = [2048 * 2 + 9]
+    ps, gs = hs.make_inputs(sizes, False, 900)
+    gs = [np.zeros_like(g) for g in gs]
+    states = hs.oracle_states(sizes)
+    gt = hs.GpuTensors(ps, gs, states, False)
+    hs.oracle_step(ps, gs, states, (LR, B1, B2, EPS, WD, 1), False)
+    gpu_steps(gt, [None], 1)
+    got_p, got_st = gt.fetch()
+    hs.compare(got_p, got_st, ps, states, False, True, "zero")
+    assert np.all(got_st[0][0] == 127) and np.all(got_st[0][1] == 0) and np.all(got_st[0][2] == 0)
+
+
+def test_extreme_and_non_finite_gradients():
+    sizes = [2048 * 4]
+    ps, gs = hs.make_inputs(sizes, False, 901)
+    g = gs[0]
+    g[0:2048] *= 1e-30           # absmax of v far below 2^-60: the IEEE-division branch
+    g[2048:4096] *= 1e18         # huge moments
+    g[4096 + 5] = np.nan         # one NaN inside a block
+    g[6144 + 9] = np.inf         # one Inf inside a block
+    states = hs.oracle_states(sizes)
+    gt = hs.GpuTensors(ps, gs, states, False)
+    g2 = hs.fresh_grads(sizes, False, 902)
+    with np.errstate(all="ignore"):
+        hs.oracle_step(ps, gs, states, (LR, B1, B2, EPS, WD, 1), False)
+        hs.oracle_step(ps, g2, states, (LR, B1, B2, EPS, WD, 2), False)
+    gpu_steps(gt, [None, g2], 1)
+    got_p, got_st = gt.fetch()
+    # absmax may be NaN/Inf here; compare bit patterns of finite entries and the NaN pattern
+    for k in (2, 3):
+        a, b = got_st[0][k], states[0][k]
+        assert np.array_equal(np.isnan(a), np.isnan(b))
+        assert np.array_equal(a[~np.isnan(a)].view(np.uint32), b[~np.isnan(b)].view(np.uint32))
+    for k in (0, 1):
+        assert np.array_equal(got_st[0][k], states[0][k])
+    nan = np.isnan(ps[0])
+    assert np.array_equal(nan, np.isnan(got_p[0]))
+    assert np.array_equal(got_p[0][~nan].view(np.uint32), ps[0][~nan].view(np.uint32))
+
+
+def test_state_init_and_quantize_round_trip():
+    import torch
+    L = _lib()
+    n = 2048 * 3 + 17
+    dev = torch.device("cuda:0")
+    m = torch.full((n,), 9, dtype=torch.uint8, device=dev)
+    v = torch.full((n,), 9, dtype=torch.uint8, device=dev)
+    am = torch.full((4,), 3.0, device=dev)
+    av = torch.full((4,), 3.0, device=dev)
+    L.check(L.lib().eri_adam8_state_init(m.data_ptr(), v.data_ptr(), am.data_ptr(), av.data_ptr(), n, _stream()), "init")
+    _sync()
+    assert bool((m == 127).all()) and bool((v == 0).all()) and bool((am == 0).all()) and bool((av == 0).all())
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    x[2048:4096] = 0
+    for signed, table in ((1, hs.MAPS[0]), (0, hs.MAPS[1])):
+        xs = x if signed else np.abs(x)
+        xd = torch.from_numpy(xs).to(dev)
+        codes = torch.empty(n, dtype=torch.uint8, device=dev)
+        absmax = torch.empty(4, dtype=torch.float32, device=dev)
+        back = torch.empty(n, dtype=torch.float32, device=dev)
+        L.check(L.lib().eri_adam8_quantize(xd.data_ptr(), signed, n, codes.data_ptr(), absmax.data_ptr(), _stream()), "q")
+        L.check(L.lib().eri_adam8_dequantize(codes.data_ptr(), absmax.data_ptr(), signed, n, back.data_ptr(), _stream()), "dq")
+        _sync()
+        wc = np.empty(n, np.uint8)
+        wa = np.empty(4, np.float32)
+        wb = np.empty(n, np.float32)
+        oc.lib().eri_oracle_quantize(oc.ptr(xs), oc.ptr(table), n, oc.ptr(wc), oc.ptr(wa))
+        oc.lib().eri_oracle_dequantize(oc.ptr(wc), oc.ptr(wa), oc.ptr(table), n, oc.ptr(wb))
+        assert np.array_equal(codes.cpu().numpy(), wc)
+        assert np.array_equal(absmax.cpu().numpy().view(np.uint32), wa.view(np.uint32))
+        assert np.array_equal(back.cpu().numpy().view(np.uint32), wb.view(np.uint32))
