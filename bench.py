@@ -30,6 +30,9 @@ def parse():
     ap.add_argument("--config", default="c5_flux12b_full")
     ap.add_argument("--flags", type=int, default=0, help="ERI_ADAM8_FLAG_* bits for the step")
     ap.add_argument("--cpu-sample", type=int, default=512 << 20, help="parameters in the CPU baseline sample (0 = skip)")
+    ap.add_argument("--calibrate-copy", type=int, default=0,
+                    help="instead of the benchmark, run a plain device copy of this many bytes three times "
+                         "(the known-size kernel the rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by)")
     ap.add_argument("--traffic-json", default=os.path.join(ROOT, "profiles", "traffic.json"),
                     help="HBM bytes per launch derived from rocprofv3 --pmc runs, if present")
     return ap.parse_args()
@@ -108,6 +111,15 @@ def main():
               "a single MI355X; rerun with --gpus 1", file=sys.stderr)
         sys.exit(2)
     import torch
+
+    if args.calibrate_copy > 0:
+        src = torch.empty(args.calibrate_copy // 4, dtype=torch.float32, device="cuda:0").fill_(1.0)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_bytes": src.numel() * 4, "launches": 3}))
+        return
 
     from eridiffusion_amd import _lib as L
     from eridiffusion_amd import workloads as W
@@ -195,7 +207,8 @@ def main():
                    "resident_gb": round((n_params * (2 * esz + 2) + n_blocks * 8) / 1e9, 2)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                      "frac": achieved / PEAK_HBM_GBPS, "traffic": traffic,
-                     "kernel_ms": avg_launch_s * 1e3, "algorithmic_bytes": algo_bytes},
+                     "kernel_ms": avg_launch_s * 1e3, "kernel_ms_min": min(launch_ms), "kernel_ms_max": max(launch_ms),
+                     "algorithmic_bytes": algo_bytes},
     }
     L.lib().eri_adam8_table_destroy(table)
     if args.cpu_sample > 0:

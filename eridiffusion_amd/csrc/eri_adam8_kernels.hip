@@ -29,6 +29,19 @@ namespace eri {
 // small device helpers
 // ------------------------------------------------------------------------------------------
 
+/* Pointers read from the launch table have no known address space; every one of them is device
+ * memory, and saying so turns flat_load/flat_store (which also tick the LDS counter and so
+ * serialise with the table lookups) into global_load/global_store. */
+#define ERI_GLOBAL __attribute__((address_space(1)))
+template <typename T>
+__device__ __forceinline__ ERI_GLOBAL T *as_global(T *p) {
+    return (ERI_GLOBAL T *)p;
+}
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
 __device__ __forceinline__ uint32_t f2u(float x) { return __builtin_bit_cast(uint32_t, x); }
 __device__ __forceinline__ float u2f(uint32_t x) { return __builtin_bit_cast(float, x); }
 
@@ -55,6 +68,13 @@ __device__ __forceinline__ float bf16_hi(uint32_t w) { return u2f(w & 0xffff0000
 __device__ __forceinline__ uint32_t bf16_bits(float f) {
     __bf16 b = (__bf16)f;
     return (uint32_t)__builtin_bit_cast(uint16_t, b);
+}
+/* Two fp32 -> one dword of two bf16 (lo in the low half): a single v_cvt_pk_bf16_f32. */
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t bf16_pair(float lo, float hi) {
+    const f32x2 f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
 }
 __device__ __forceinline__ float bf16_round(float f) { return u2f(bf16_bits(f) << 16); }
 
@@ -169,37 +189,53 @@ __device__ __forceinline__ void adam_elem(float p, float g, float m_old, float v
 // 8 consecutive elements per lane: loads and stores
 // ------------------------------------------------------------------------------------------
 
+/* Eight consecutive elements of one lane as they come from memory: one 128-bit word of bf16, or
+ * two of fp32.  Loading and unpacking are separate so that a block's loads can all be issued
+ * before the first value is needed. */
 template <bool BF16>
-__device__ __forceinline__ void load8(const void *base, uint32_t elem, float (&out)[8]) {
-    if (BF16) {
-        const uint4 w = *reinterpret_cast<const uint4 *>(static_cast<const uint16_t *>(base) + elem);
+struct Raw8;
+template <>
+struct Raw8<true> {
+    u32x4 w;
+    __device__ __forceinline__ void load(const void *base, uint32_t elem) {
+        w = *as_global(reinterpret_cast<const u32x4 *>(static_cast<const uint16_t *>(base) + elem));
+    }
+    __device__ __forceinline__ void unpack(float (&out)[8]) const {
         out[0] = bf16_lo(w.x); out[1] = bf16_hi(w.x); out[2] = bf16_lo(w.y); out[3] = bf16_hi(w.y);
         out[4] = bf16_lo(w.z); out[5] = bf16_hi(w.z); out[6] = bf16_lo(w.w); out[7] = bf16_hi(w.w);
-    } else {
-        const float4 *q = reinterpret_cast<const float4 *>(static_cast<const float *>(base) + elem);
-        const float4 a = q[0], b = q[1];
+    }
+};
+template <>
+struct Raw8<false> {
+    f32x4 a, b;
+    __device__ __forceinline__ void load(const void *base, uint32_t elem) {
+        ERI_GLOBAL const f32x4 *q = as_global(reinterpret_cast<const f32x4 *>(static_cast<const float *>(base) + elem));
+        a = q[0];
+        b = q[1];
+    }
+    __device__ __forceinline__ void unpack(float (&out)[8]) const {
         out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w;
         out[4] = b.x; out[5] = b.y; out[6] = b.z; out[7] = b.w;
     }
-}
+};
 
 template <bool BF16>
 __device__ __forceinline__ void store8(void *base, uint32_t elem, const float (&v)[8]) {
     if (BF16) {
-        uint4 w;
-        w.x = bf16_bits(v[0]) | (bf16_bits(v[1]) << 16);
-        w.y = bf16_bits(v[2]) | (bf16_bits(v[3]) << 16);
-        w.z = bf16_bits(v[4]) | (bf16_bits(v[5]) << 16);
-        w.w = bf16_bits(v[6]) | (bf16_bits(v[7]) << 16);
-        *reinterpret_cast<uint4 *>(static_cast<uint16_t *>(base) + elem) = w;
+        u32x4 w;
+        w.x = bf16_pair(v[0], v[1]);
+        w.y = bf16_pair(v[2], v[3]);
+        w.z = bf16_pair(v[4], v[5]);
+        w.w = bf16_pair(v[6], v[7]);
+        *as_global(reinterpret_cast<u32x4 *>(static_cast<uint16_t *>(base) + elem)) = w;
     } else {
-        float4 *q = reinterpret_cast<float4 *>(static_cast<float *>(base) + elem);
-        q[0] = make_float4(v[0], v[1], v[2], v[3]);
-        q[1] = make_float4(v[4], v[5], v[6], v[7]);
+        ERI_GLOBAL f32x4 *q = as_global(reinterpret_cast<f32x4 *>(static_cast<float *>(base) + elem));
+        q[0] = f32x4{v[0], v[1], v[2], v[3]};
+        q[1] = f32x4{v[4], v[5], v[6], v[7]};
     }
 }
 
-__device__ __forceinline__ uint32_t byte_of(const uint2 w, int k) {
+__device__ __forceinline__ uint32_t byte_of(const u32x2 w, int k) {
     const uint32_t d = k < 4 ? w.x : w.y;
     return (d >> (8 * (k & 3))) & 0xffu;
 }
@@ -210,7 +246,7 @@ __device__ __forceinline__ uint32_t byte_of(const uint2 w, int k) {
 
 template <bool FAST_DIV, bool KEYTAB>
 __device__ __forceinline__ void requant8(const float *mf, const float *vf, const BlockDiv &dm, const BlockDiv &dv,
-                                         const Lds &L, uint2 &mw, uint2 &vw) {
+                                         const Lds &L, u32x2 &mw, u32x2 &vw) {
     uint32_t cm[8], cv[8];
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
@@ -234,56 +270,71 @@ __device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint
     const char *g = static_cast<const char *>(t.g) + e0 * esz;
     uint8_t *mc = t.m + e0;
     uint8_t *vc = t.v + e0;
-    const float a_m = t.absmax_m[lb];
-    const float a_v = t.absmax_v[lb];
+    const float a_m = as_global(t.absmax_m)[lb];
+    const float a_v = as_global(t.absmax_v)[lb];
 
     float mf[32], vf[32];
     float lm = 0.0f, lv = 0.0f;
+    // Issue the loads of DEPTH passes before touching the first value: the wave then waits once per
+    // DEPTH passes, with 48 * DEPTH bytes per lane in flight (bf16; fp32 holds twice the registers).
+    constexpr int DEPTH = BF16 ? 4 : 2;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-        const uint32_t o = c * 512 + lane * 8;
-        float pv[8], gv[8], pn[8];
-        load8<BF16>(p, o, pv);
-        load8<BF16>(g, o, gv);
-        const uint2 mw = *reinterpret_cast<const uint2 *>(mc + o);
-        const uint2 vw = *reinterpret_cast<const uint2 *>(vc + o);
+    for (int c0 = 0; c0 < 4; c0 += DEPTH) {
+        Raw8<BF16> pr[DEPTH], gr[DEPTH];
+        u32x2 mr[DEPTH], vr[DEPTH];
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
-            const float m_old = L.map_s[byte_of(mw, k)] * a_m;
-            const float v_old = L.map_u[byte_of(vw, k)] * a_v;
-            float m, v;
-            adam_elem<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], m_old, v_old, h, gscale, dbc1, dbc2, m, v, pn[k]);
-            mf[c * 8 + k] = m;
-            vf[c * 8 + k] = v;
-            lm = fmaxf(lm, __builtin_fabsf(m));
-            lv = fmaxf(lv, __builtin_fabsf(v));
+        for (int d = 0; d < DEPTH; ++d) {
+            const uint32_t o = (c0 + d) * 512 + lane * 8;
+            pr[d].load(p, o);
+            gr[d].load(g, o);
+            mr[d] = *as_global(reinterpret_cast<const u32x2 *>(mc + o));
+            vr[d] = *as_global(reinterpret_cast<const u32x2 *>(vc + o));
         }
-        store8<BF16>(p, o, pn);
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const int c = c0 + d;
+            const uint32_t o = c * 512 + lane * 8;
+            float pv[8], gv[8], pn[8];
+            pr[d].unpack(pv);
+            gr[d].unpack(gv);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const float m_old = L.map_s[byte_of(mr[d], k)] * a_m;
+                const float v_old = L.map_u[byte_of(vr[d], k)] * a_v;
+                float m, v;
+                adam_elem<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], m_old, v_old, h, gscale, dbc1, dbc2, m, v, pn[k]);
+                mf[c * 8 + k] = m;
+                vf[c * 8 + k] = v;
+                lm = fmaxf(lm, __builtin_fabsf(m));
+                lv = fmaxf(lv, __builtin_fabsf(v));
+            }
+            store8<BF16>(p, o, pn);
+        }
     }
     const float nam = wave_max(lm);
     const float nav = wave_max(lv);
     if (lane == 0) {
-        t.absmax_m[lb] = nam;
-        t.absmax_v[lb] = nav;
+        as_global(t.absmax_m)[lb] = nam;
+        as_global(t.absmax_v)[lb] = nav;
     }
     const BlockDiv dm(nam), dv(nav);
     if (dm.fast && dv.fast) {
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             const uint32_t o = c * 512 + lane * 8;
-            uint2 mw, vw;
+            u32x2 mw, vw;
             requant8<true, KEYTAB>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
-            *reinterpret_cast<uint2 *>(mc + o) = mw;
-            *reinterpret_cast<uint2 *>(vc + o) = vw;
+            *as_global(reinterpret_cast<u32x2 *>(mc + o)) = mw;
+            *as_global(reinterpret_cast<u32x2 *>(vc + o)) = vw;
         }
     } else {
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             const uint32_t o = c * 512 + lane * 8;
-            uint2 mw, vw;
+            u32x2 mw, vw;
             requant8<false, KEYTAB>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
-            *reinterpret_cast<uint2 *>(mc + o) = mw;
-            *reinterpret_cast<uint2 *>(vc + o) = vw;
+            *as_global(reinterpret_cast<u32x2 *>(mc + o)) = mw;
+            *as_global(reinterpret_cast<u32x2 *>(vc + o)) = vw;
         }
     }
 }
@@ -295,23 +346,25 @@ __device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint
 
 template <bool BF16>
 __device__ __forceinline__ float load1(const void *base, size_t i) {
-    if (BF16) return u2f((uint32_t)static_cast<const uint16_t *>(base)[i] << 16);
-    return static_cast<const float *>(base)[i];
+    if (BF16) return u2f((uint32_t)as_global(static_cast<const uint16_t *>(base))[i] << 16);
+    return as_global(static_cast<const float *>(base))[i];
 }
 
 template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB>
-__device__ __noinline__ void tail_block(const DevTensor &t, uint32_t lb, uint32_t n, uint32_t lane,
+__device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint32_t n, uint32_t lane,
                                         const EriAdam8Hyper &h, float gscale, const BlockDiv &dbc1,
                                         const BlockDiv &dbc2, const Lds &L) {
     const size_t e0 = (size_t)lb * kBlock;
-    const float a_m = t.absmax_m[lb];
-    const float a_v = t.absmax_v[lb];
+    ERI_GLOBAL uint8_t *mc = as_global(t.m);
+    ERI_GLOBAL uint8_t *vc = as_global(t.v);
+    const float a_m = as_global(t.absmax_m)[lb];
+    const float a_v = as_global(t.absmax_v)[lb];
     float lm = 0.0f, lv = 0.0f;
     for (uint32_t i = lane; i < n; i += kWave) {
         const size_t e = e0 + i;
         float m, v, pn;
-        adam_elem<MODE, EXACT, BF16, WD, GS>(load1<BF16>(t.p, e), load1<BF16>(t.g, e), L.map_s[t.m[e]] * a_m,
-                                             L.map_u[t.v[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn);
+        adam_elem<MODE, EXACT, BF16, WD, GS>(load1<BF16>(t.p, e), load1<BF16>(t.g, e), L.map_s[mc[e]] * a_m,
+                                             L.map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn);
         lm = fmaxf(lm, __builtin_fabsf(m));
         lv = fmaxf(lv, __builtin_fabsf(v));
     }
@@ -321,18 +374,18 @@ __device__ __noinline__ void tail_block(const DevTensor &t, uint32_t lb, uint32_
     for (uint32_t i = lane; i < n; i += kWave) {
         const size_t e = e0 + i;
         float m, v, pn;
-        adam_elem<MODE, EXACT, BF16, WD, GS>(load1<BF16>(t.p, e), load1<BF16>(t.g, e), L.map_s[t.m[e]] * a_m,
-                                             L.map_u[t.v[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn);
+        adam_elem<MODE, EXACT, BF16, WD, GS>(load1<BF16>(t.p, e), load1<BF16>(t.g, e), L.map_s[mc[e]] * a_m,
+                                             L.map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn);
         const float xm = dm.div_slow(m);
         const float xv = dv.div_slow(v);
-        t.m[e] = (uint8_t)(KEYTAB ? code_signed_key(xm, L.key_s) : code_bsearch(xm, L.mid_s));
-        t.v[e] = (uint8_t)(KEYTAB ? code_unsigned_key(xv, L.key_u) : code_bsearch(xv, L.mid_u));
-        if (BF16) static_cast<uint16_t *>(t.p)[e] = (uint16_t)bf16_bits(pn);
-        else static_cast<float *>(t.p)[e] = pn;
+        mc[e] = (uint8_t)(KEYTAB ? code_signed_key(xm, L.key_s) : code_bsearch(xm, L.mid_s));
+        vc[e] = (uint8_t)(KEYTAB ? code_unsigned_key(xv, L.key_u) : code_bsearch(xv, L.mid_u));
+        if (BF16) as_global(static_cast<uint16_t *>(t.p))[e] = (uint16_t)bf16_bits(pn);
+        else as_global(static_cast<float *>(t.p))[e] = pn;
     }
     if (lane == 0) {
-        t.absmax_m[lb] = nam;
-        t.absmax_v[lb] = nav;
+        as_global(t.absmax_m)[lb] = nam;
+        as_global(t.absmax_v)[lb] = nav;
     }
 }
 
