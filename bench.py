@@ -30,6 +30,8 @@ def parse():
     ap.add_argument("--config", default="c5_flux12b_full")
     ap.add_argument("--flags", type=int, default=0, help="ERI_ADAM8_FLAG_* bits for the step")
     ap.add_argument("--cpu-sample", type=int, default=512 << 20, help="parameters in the CPU baseline sample (0 = skip)")
+    ap.add_argument("--alloc", choices=["arena", "tensor"], default="arena",
+                    help="one flat allocation per kind of buffer, or one allocation per tensor and buffer")
     ap.add_argument("--calibrate-copy", type=int, default=0,
                     help="instead of the benchmark, run a plain device copy of this many bytes three times "
                          "(the known-size kernel the rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by)")
@@ -42,23 +44,50 @@ def align(n, a=256):
     return (n + a - 1) // a * a
 
 
-class Arena:
-    """One flat device allocation per kind of buffer; every tensor starts on a 256-byte boundary."""
+class PerTensor:
+    """One device allocation per tensor (how a tensor runtime holds parameters and states)."""
 
     def __init__(self, torch, sizes_bytes):
+        self.bufs = [torch.empty(max(b, 16), dtype=torch.uint8, device="cuda:0") for b in sizes_bytes]
+
+    def ptr(self, i):
+        return self.bufs[i].data_ptr()
+
+    def fill(self, i, src, stream):
+        self.bufs[i][:src.numel() * src.element_size()].copy_(src.view(-1).view(self.bufs[i].dtype))
+
+    def free(self):
+        self.bufs = []
+
+
+class Arena:
+    """One flat device allocation per kind of buffer, from the library's allocator
+    (eri_hip_malloc_zeroed); every tensor starts on a 256-byte boundary."""
+
+    def __init__(self, torch, sizes_bytes):
+        from eridiffusion_amd import _lib as L
         self.offsets = []
         total = 0
         for b in sizes_bytes:
             self.offsets.append(total)
             total += align(b)
-        self.buf = torch.empty(max(total, 256), dtype=torch.uint8, device="cuda:0")
-        self.base = self.buf.data_ptr()
+        self.nbytes = max(total, 256)
+        out = C.c_void_p()
+        L.check(L.lib().eri_hip_malloc_zeroed(0, self.nbytes, C.byref(out)), "eri_hip_malloc_zeroed")
+        self.base = out.value
 
     def ptr(self, i):
         return self.base + self.offsets[i]
 
-    def view(self, i, nbytes):
-        return self.buf[self.offsets[i]:self.offsets[i] + nbytes]
+    def fill(self, i, src, stream):
+        """Device-to-device copy of a torch tensor's bytes into tensor i, on torch's current stream."""
+        from eridiffusion_amd import _lib as L
+        L.check(L.lib().eri_hip_memcpy_async(self.ptr(i), src.data_ptr(), src.numel() * src.element_size(), 3, stream),
+                "eri_hip_memcpy_async")
+
+    def free(self):
+        from eridiffusion_amd import _lib as L
+        L.lib().eri_hip_free(self.base)
 
 
 def cpu_baseline(tensors, bf16, sample_params, hyper_args):
@@ -134,19 +163,20 @@ def main():
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream().cuda_stream
 
-    a_p = Arena(torch, [n * esz for n in sizes])
-    a_g = Arena(torch, [n * esz for n in sizes])
-    a_m = Arena(torch, sizes)
-    a_v = Arena(torch, sizes)
-    a_am = Arena(torch, [((n + 2047) // 2048) * 4 for n in sizes])
-    a_av = Arena(torch, [((n + 2047) // 2048) * 4 for n in sizes])
+    Alloc = Arena if args.alloc == "arena" else PerTensor
+    a_p = Alloc(torch, [n * esz for n in sizes])
+    a_g = Alloc(torch, [n * esz for n in sizes])
+    a_m = Alloc(torch, sizes)
+    a_v = Alloc(torch, sizes)
+    a_am = Alloc(torch, [((n + 2047) // 2048) * 4 for n in sizes])
+    a_av = Alloc(torch, [((n + 2047) // 2048) * 4 for n in sizes])
     tdt = torch.bfloat16 if bf16 else torch.float32
     gen = torch.Generator(device="cuda:0")
     gen.manual_seed(0xE21D + 5)
     p_std, g_std = (0.02, 1e-3)
     for i, n in enumerate(sizes):  # synthetic data: p ~ N(0, 0.02), g ~ N(0, 1e-3)
-        a_p.view(i, n * esz).view(tdt).copy_(torch.randn(n, device="cuda:0", generator=gen).mul_(p_std).to(tdt))
-        a_g.view(i, n * esz).view(tdt).copy_(torch.randn(n, device="cuda:0", generator=gen).mul_(g_std).to(tdt))
+        a_p.fill(i, torch.randn(n, device="cuda:0", generator=gen).mul_(p_std).to(tdt), stream)
+        a_g.fill(i, torch.randn(n, device="cuda:0", generator=gen).mul_(g_std).to(tdt), stream)
         L.check(L.lib().eri_adam8_state_init(a_m.ptr(i), a_v.ptr(i), a_am.ptr(i), a_av.ptr(i), n, stream), "state_init")
     rows = (L.TensorRow * len(sizes))()
     start = 0
@@ -211,6 +241,8 @@ def main():
                      "algorithmic_bytes": algo_bytes},
     }
     L.lib().eri_adam8_table_destroy(table)
+    for a in (a_p, a_g, a_m, a_v, a_am, a_av):
+        a.free()
     if args.cpu_sample > 0:
         out["cpu_baseline"] = cpu_baseline(tensors, bf16, args.cpu_sample, hyper_args)
     print(json.dumps(out), flush=True)

@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(_HERE, "liberi_optim8.so")
 BLOCK = 2048
 DTYPE_F32, DTYPE_F16, DTYPE_BF16, DTYPE_I32 = 0, 1, 2, 3
 MODE_ERI, MODE_L2 = 0, 1
-FLAG_GRAD_SCALE, FLAG_EXACT_PARAM, FLAG_BSEARCH = 1, 2, 4
+FLAG_GRAD_SCALE, FLAG_EXACT_PARAM, FLAG_BSEARCH, FLAG_NO_PIPELINE = 1, 2, 4, 8
 
 
 class Hyper(C.Structure):

@@ -29,40 +29,40 @@ struct DevTensor {
 static_assert(sizeof(DevTensor) == 64, "DevTensor must stay 64 bytes");
 
 /*
- * Requantisation without a search.  For x in [-1, 1] the top bits of |x| (sign, exponent and the
- * leading kMant mantissa bits) select a slot; the slots are narrow enough that at most one
+ * Requantisation without a search.  The quotient x = value / absmax in [-1, 1] is produced
+ * already multiplied by kKeyScale (a power of two, so nothing is rounded differently), converted
+ * to binary16 with round-to-nearest-even, and the top bits of that half float -- sign, exponent
+ * and the leading mantissa bits -- select a slot.  The slots are narrow enough that at most one
  * midpoint of the map lies inside any of them, so
- *     code(x) = slot.lo + (x > slot.mid)
+ *     code(x) = slot.lo + (x * kKeyScale > slot.mid)
  * equals the number of midpoints below x, i.e. the binary search's answer, ties included.
- * Slot 0 also takes everything smaller than 2^(kExp0-127); the last slot of each sign takes NaN
- * and returns code 0, which is what a search does with NaN (every comparison false).
+ * Every binary16 pattern has a slot: there is nothing to clamp, NaN lands in slots that answer 0
+ * (a search finds every comparison false), and the scale keeps all midpoints in the normal
+ * binary16 range, so the result does not depend on how half denormals are treated.
  */
 struct KeySlot {
-    float mid;   /* the one midpoint inside the slot, +inf if there is none */
+    float mid;   /* the one midpoint inside the slot times kKeyScale, +inf if there is none */
     uint32_t lo; /* number of midpoints below every value of the slot */
 };
 
-constexpr uint32_t kKeyExp0 = 106; /* biased exponent of the first binade that gets its own slots */
-constexpr uint32_t kSMant = 6;     /* signed map: 64 slots per binade */
-constexpr uint32_t kUMant = 7;     /* unsigned map: 128 slots per binade */
-constexpr uint32_t kSShift = 23 - kSMant;
-constexpr uint32_t kUShift = 23 - kUMant;
-constexpr uint32_t kSBase = kKeyExp0 << kSMant;
-constexpr uint32_t kUBase = kKeyExp0 << kUMant;
-constexpr uint32_t kSSlots = ((127 - kKeyExp0) << kSMant) + 1; /* through x == 1.0 */
-constexpr uint32_t kUSlots = ((127 - kKeyExp0) << kUMant) + 1;
-constexpr uint32_t kSPerSign = kSSlots + 1; /* + the NaN slot */
-constexpr uint32_t kUCount = kUSlots + 1;
+constexpr float kKeyScale = 4096.0f;
+constexpr float kKeyScaleInv = 1.0f / 4096.0f;
+constexpr uint32_t kSKeyDrop = 4;   /* signed map: keep 6 mantissa bits of the half float */
+constexpr uint32_t kUKeyDrop = 3;   /* unsigned map: keep 7 */
+constexpr uint32_t kSKeyStride = 16; /* bytes between signed slots: address = half & 0xfff0 */
+constexpr uint32_t kUKeyStride = 8;  /* bytes between unsigned slots: address = half & 0x7ff8 */
+constexpr uint32_t kSKeyCount = 1u << (16 - kSKeyDrop); /* 4096, sign included */
+constexpr uint32_t kUKeyCount = 1u << (15 - kUKeyDrop); /* 4096, sign masked off */
 
 /* Byte offsets inside the LDS image. */
 constexpr uint32_t kOffMapS = 0;                              /* 256 floats: code -> value */
 constexpr uint32_t kOffMapU = kOffMapS + 1024;                /* 256 floats */
 constexpr uint32_t kOffMidS = kOffMapU + 1024;                /* 255 midpoints + one +inf */
 constexpr uint32_t kOffMidU = kOffMidS + 1024;
-constexpr uint32_t kOffKeyS = kOffMidU + 1024;                /* 2 * kSPerSign slots: positive, negative */
-constexpr uint32_t kOffKeyU = kOffKeyS + 2 * kSPerSign * 8;   /* kUCount slots */
-constexpr uint32_t kLdsImageBytesRaw = kOffKeyU + kUCount * 8;
-constexpr uint32_t kLdsImageBytes = (kLdsImageBytesRaw + 15u) & ~15u;
+constexpr uint32_t kOffKeyS = kOffMidU + 1024;                /* kSKeyCount slots, kSKeyStride apart */
+constexpr uint32_t kOffKeyU = kOffKeyS + kSKeyCount * kSKeyStride; /* kUKeyCount slots */
+constexpr uint32_t kLdsImageBytes = kOffKeyU + kUKeyCount * kUKeyStride;
+static_assert(kLdsImageBytes % 16 == 0, "the image is staged in 16-byte words");
 
 /* Launchers implemented in eri_adam8_kernels.hip; `stream` is a hipStream_t.  All return a
  * hipError_t as int.  `lds_image` is the device copy of the kLdsImageBytes table image. */

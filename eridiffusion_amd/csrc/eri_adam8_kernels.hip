@@ -79,48 +79,53 @@ __device__ __forceinline__ uint32_t bf16_pair(float lo, float hi) {
 __device__ __forceinline__ float bf16_round(float f) { return u2f(bf16_bits(f) << 16); }
 
 /*
- * m / a for a divisor shared by a whole block.  With ra = RN(1/a), q0 = RN(m*ra) is within an
- * ulp or two of the quotient, the remainder m - q0*a is exact in one fma, and one correction
- * gives the correctly rounded quotient (Markstein); `fast` excludes the divisors for which that
- * argument needs care (zero, subnormal-range or huge values, an all-ones significand), and those
- * blocks use the hardware-assisted IEEE division instead.  Both produce the same bits.
+ * SCALE * (m / a) for a divisor shared by a whole block, SCALE a power of two.  With
+ * ra = RN(1/a), q0 = RN(m*ra) is within an ulp or two of the quotient, the remainder m - q0*a is
+ * exact in one fma, and one correction gives the correctly rounded quotient (Markstein); folding
+ * the power of two into ra (and its inverse into a) scales every intermediate exactly.  `fast`
+ * excludes the divisors for which that argument needs care (zero, subnormal-range or huge values,
+ * an all-ones significand), and those blocks use the hardware-assisted IEEE division instead.
+ * Both produce the same bits.
  */
 struct BlockDiv {
-    float a, ra;
+    float a, as, ras, scale;
     bool fast;
-    __device__ __forceinline__ explicit BlockDiv(float a_) : a(a_) {
+    __device__ __forceinline__ explicit BlockDiv(float a_, float scale_ = 1.0f, float scale_inv = 1.0f)
+        : a(a_), scale(scale_) {
         fast = (a_ >= 0x1p-60f) && (a_ <= 0x1p60f) && ((f2u(a_) & 0x7fffffu) != 0x7fffffu);
-        ra = fast ? 1.0f / a_ : 0.0f;
+        const float ra = fast ? 1.0f / a_ : 0.0f;
+        ras = ra * scale_;
+        as = a_ * scale_inv;
     }
     __device__ __forceinline__ float div_fast(float m) const {
-        float q0 = m * ra;
-        float r = __builtin_fmaf(-q0, a, m);
-        return __builtin_fmaf(r, ra, q0);
+        float q0 = m * ras;
+        float r = __builtin_fmaf(-q0, as, m);
+        return __builtin_fmaf(r, ras, q0);
     }
-    __device__ __forceinline__ float div_slow(float m) const { return a == 0.0f ? 0.0f : m / a; }
+    __device__ __forceinline__ float div_slow(float m) const {
+        float q = a == 0.0f ? 0.0f : m / a;
+        return q * scale;
+    }
 };
 
 struct Lds {
     const float *map_s, *map_u, *mid_s, *mid_u;
-    const KeySlot *key_s, *key_u;
+    const char *key_s, *key_u;
 };
 
-__device__ __forceinline__ uint32_t code_signed_key(float x, const KeySlot *key_s) {
-    const uint32_t b = f2u(x);
-    uint32_t k = (b & 0x7fffffffu) >> kSShift;
-    k = __builtin_elementwise_sub_sat(k, kSBase);
-    k = min(k, kSSlots);
-    k += (b >> 31) * kSPerSign;
-    const KeySlot s = key_s[k];
-    return s.lo + (x > s.mid ? 1u : 0u);
+__device__ __forceinline__ uint32_t half_key(float xs) {
+    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)xs); // v_cvt_f16_f32, round to nearest even
 }
 
-__device__ __forceinline__ uint32_t code_unsigned_key(float x, const KeySlot *key_u) {
-    uint32_t k = f2u(x) >> kUShift; // x >= 0, or NaN with either sign (clamped to the NaN slot)
-    k = __builtin_elementwise_sub_sat(k, kUBase);
-    k = min(k, kUSlots);
-    const KeySlot s = key_u[k];
-    return s.lo + (x > s.mid ? 1u : 0u);
+/* xs = kKeyScale * x.  The slot address is the half pattern with its low bits cleared. */
+__device__ __forceinline__ uint32_t code_signed_key(float xs, const char *key_s) {
+    const KeySlot s = *reinterpret_cast<const KeySlot *>(key_s + (half_key(xs) & 0xfff0u));
+    return s.lo + (xs > s.mid ? 1u : 0u);
+}
+
+__device__ __forceinline__ uint32_t code_unsigned_key(float xs, const char *key_u) {
+    const KeySlot s = *reinterpret_cast<const KeySlot *>(key_u + (half_key(xs) & 0x7ff8u));
+    return s.lo + (xs > s.mid ? 1u : 0u);
 }
 
 /* Number of midpoints below x by binary search of the 255-entry LDS table (entry 255 is +inf). */
@@ -227,7 +232,7 @@ __device__ __forceinline__ void store8(void *base, uint32_t elem, const float (&
         w.y = bf16_pair(v[2], v[3]);
         w.z = bf16_pair(v[4], v[5]);
         w.w = bf16_pair(v[6], v[7]);
-        *as_global(reinterpret_cast<u32x4 *>(static_cast<uint16_t *>(base) + elem)) = w;
+        __builtin_nontemporal_store(w, as_global(reinterpret_cast<u32x4 *>(static_cast<uint16_t *>(base) + elem)));
     } else {
         ERI_GLOBAL f32x4 *q = as_global(reinterpret_cast<f32x4 *>(static_cast<float *>(base) + elem));
         q[0] = f32x4{v[0], v[1], v[2], v[3]};
@@ -250,7 +255,7 @@ __device__ __forceinline__ void requant8(const float *mf, const float *vf, const
     uint32_t cm[8], cv[8];
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
-        const float xm = FAST_DIV ? dm.div_fast(mf[k]) : dm.div_slow(mf[k]);
+        const float xm = FAST_DIV ? dm.div_fast(mf[k]) : dm.div_slow(mf[k]); // times dm.scale
         const float xv = FAST_DIV ? dv.div_fast(vf[k]) : dv.div_slow(vf[k]);
         cm[k] = KEYTAB ? code_signed_key(xm, L.key_s) : code_bsearch(xm, L.mid_s);
         cv[k] = KEYTAB ? code_unsigned_key(xv, L.key_u) : code_bsearch(xv, L.mid_u);
@@ -317,7 +322,8 @@ __device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint
         as_global(t.absmax_m)[lb] = nam;
         as_global(t.absmax_v)[lb] = nav;
     }
-    const BlockDiv dm(nam), dv(nav);
+    constexpr float ks = KEYTAB ? kKeyScale : 1.0f, ksi = KEYTAB ? kKeyScaleInv : 1.0f;
+    const BlockDiv dm(nam, ks, ksi), dv(nav, ks, ksi);
     if (dm.fast && dv.fast) {
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
@@ -370,7 +376,8 @@ __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint
     }
     const float nam = wave_max(lm);
     const float nav = wave_max(lv);
-    const BlockDiv dm(nam), dv(nav);
+    constexpr float ks = KEYTAB ? kKeyScale : 1.0f, ksi = KEYTAB ? kKeyScaleInv : 1.0f;
+    const BlockDiv dm(nam, ks, ksi), dv(nav, ks, ksi);
     for (uint32_t i = lane; i < n; i += kWave) {
         const size_t e = e0 + i;
         float m, v, pn;
@@ -407,8 +414,8 @@ __global__ __launch_bounds__(1024) void adam8_step_kernel(const DevTensor *__res
     L.map_u = reinterpret_cast<const float *>(base + kOffMapU);
     L.mid_s = reinterpret_cast<const float *>(base + kOffMidS);
     L.mid_u = reinterpret_cast<const float *>(base + kOffMidU);
-    L.key_s = reinterpret_cast<const KeySlot *>(base + kOffKeyS);
-    L.key_u = reinterpret_cast<const KeySlot *>(base + kOffKeyU);
+    L.key_s = base + kOffKeyS;
+    L.key_u = base + kOffKeyU;
 
     const uint32_t lane = threadIdx.x & (kWave - 1);
     const uint32_t waves_per_wg = blockDim.x / kWave;
@@ -433,6 +440,174 @@ __global__ __launch_bounds__(1024) void adam8_step_kernel(const DevTensor *__res
         else
             tail_block<BF16, MODE, EXACT, WD, GS, KEYTAB>(t, lb, (uint32_t)left, lane, h, gscale, dbc1, dbc2, L);
     }
+}
+
+// ------------------------------------------------------------------------------------------
+// software-pipelined step kernel for bf16 tensors
+//
+// Same arithmetic as adam8_step_kernel, but a wave issues the loads of its NEXT block after the
+// update half of the current block (when the raw words of the current block are dead) and before
+// the requantisation half, so it always has 48 bytes per lane in flight while it computes.  The
+// registers of the raw words are the ones just freed, so the pipeline costs no copies; it needs
+// 48 (raw) + 64 (moments) + temporaries at its peak, hence three waves per SIMD (768 threads).
+// ------------------------------------------------------------------------------------------
+
+struct RawBlock {
+    u32x4 p[4], g[4];
+    u32x2 m[4], v[4];
+    float a_m, a_v;
+    __device__ __forceinline__ void issue(const DevTensor &t, uint32_t lb, uint32_t lane) {
+        const size_t e0 = (size_t)lb * kBlock;
+        ERI_GLOBAL const u32x4 *pp = as_global(reinterpret_cast<const u32x4 *>(static_cast<const uint16_t *>(t.p) + e0));
+        ERI_GLOBAL const u32x4 *gp = as_global(reinterpret_cast<const u32x4 *>(static_cast<const uint16_t *>(t.g) + e0));
+        ERI_GLOBAL const u32x2 *mp = as_global(reinterpret_cast<const u32x2 *>(t.m + e0));
+        ERI_GLOBAL const u32x2 *vp = as_global(reinterpret_cast<const u32x2 *>(t.v + e0));
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            p[c] = __builtin_nontemporal_load(&pp[c * 64 + lane]); // each byte is touched once per step
+            g[c] = __builtin_nontemporal_load(&gp[c * 64 + lane]);
+            m[c] = __builtin_nontemporal_load(&mp[c * 64 + lane]);
+            v[c] = __builtin_nontemporal_load(&vp[c * 64 + lane]);
+        }
+        a_m = as_global(t.absmax_m)[lb];
+        a_v = as_global(t.absmax_v)[lb];
+    }
+};
+
+/* Where a wave is in the global block list (all wave-uniform). */
+struct Cursor {
+    uint32_t blk, ti, lb, left;
+    DevTensor t;
+    bool valid;
+    __device__ __forceinline__ void locate(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks) {
+        valid = blk < total_blocks;
+        if (!valid) return;
+        uint32_t lo = ti, hi = n_rows; // rows[lo].block_start <= blk; blk only grows
+        while (hi - lo > 1) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (rows[mid].block_start <= blk) lo = mid; else hi = mid;
+        }
+        ti = lo;
+        t = rows[ti];
+        lb = blk - t.block_start;
+        const uint64_t l = t.numel - (uint64_t)lb * kBlock;
+        left = l >= kBlock ? kBlock : (uint32_t)l;
+    }
+};
+
+template <int MODE, bool EXACT, bool WD, bool GS>
+__global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTensor *__restrict__ rows,
+                                                                   uint32_t n_rows, uint32_t total_blocks,
+                                                                   EriAdam8Hyper h,
+                                                                   const uint4 *__restrict__ lds_image) {
+    for (uint32_t i = threadIdx.x; i < kLdsImageBytes / 16; i += blockDim.x) lds_raw[i] = lds_image[i];
+    __syncthreads();
+    const char *base = reinterpret_cast<const char *>(lds_raw);
+    Lds L;
+    L.map_s = reinterpret_cast<const float *>(base + kOffMapS);
+    L.map_u = reinterpret_cast<const float *>(base + kOffMapU);
+    L.mid_s = reinterpret_cast<const float *>(base + kOffMidS);
+    L.mid_u = reinterpret_cast<const float *>(base + kOffMidU);
+    L.key_s = base + kOffKeyS;
+    L.key_u = base + kOffKeyU;
+
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t waves_per_wg = blockDim.x / kWave;
+    const uint32_t stride = gridDim.x * waves_per_wg;
+    const BlockDiv dbc1(h.bc1), dbc2(h.bc2);
+
+    Cursor cur;
+    cur.blk = __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
+    cur.ti = 0;
+    cur.locate(rows, n_rows, total_blocks);
+    RawBlock raw;
+    if (cur.valid && cur.left == kBlock) raw.issue(cur.t, cur.lb, lane);
+
+    while (cur.valid) {
+        Cursor nxt;
+        nxt.blk = cur.blk + stride;
+        nxt.ti = cur.ti;
+        nxt.locate(rows, n_rows, total_blocks);
+        const bool prefetch = nxt.valid && nxt.left == kBlock;
+        const float gscale = GS ? h.grad_scale * cur.t.grad_scale : 1.0f;
+        if (cur.left == kBlock) {
+            const size_t e0 = (size_t)cur.lb * kBlock;
+            char *p = static_cast<char *>(cur.t.p) + e0 * 2;
+            uint8_t *mc = cur.t.m + e0;
+            uint8_t *vc = cur.t.v + e0;
+            float mf[32], vf[32];
+            float lm = 0.0f, lv = 0.0f;
+            const float a_m = raw.a_m, a_v = raw.a_v;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint32_t o = c * 512 + lane * 8;
+                Raw8<true> pr, gr;
+                pr.w = raw.p[c];
+                gr.w = raw.g[c];
+                float pv[8], gv[8], pn[8];
+                pr.unpack(pv);
+                gr.unpack(gv);
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    const float m_old = L.map_s[byte_of(raw.m[c], k)] * a_m;
+                    const float v_old = L.map_u[byte_of(raw.v[c], k)] * a_v;
+                    float m, v;
+                    adam_elem<MODE, EXACT, true, WD, GS>(pv[k], gv[k], m_old, v_old, h, gscale, dbc1, dbc2, m, v, pn[k]);
+                    mf[c * 8 + k] = m;
+                    vf[c * 8 + k] = v;
+                    lm = fmaxf(lm, __builtin_fabsf(m));
+                    lv = fmaxf(lv, __builtin_fabsf(v));
+                }
+                store8<true>(p, o, pn);
+            }
+            const float nam = wave_max(lm);
+            const float nav = wave_max(lv);
+            if (lane == 0) {
+                as_global(cur.t.absmax_m)[cur.lb] = nam;
+                as_global(cur.t.absmax_v)[cur.lb] = nav;
+            }
+            if (prefetch) raw.issue(nxt.t, nxt.lb, lane);
+            const BlockDiv dm(nam, kKeyScale, kKeyScaleInv), dv(nav, kKeyScale, kKeyScaleInv);
+            if (dm.fast && dv.fast) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const uint32_t o = c * 512 + lane * 8;
+                    u32x2 mw, vw;
+                    requant8<true, true>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
+                    __builtin_nontemporal_store(mw, as_global(reinterpret_cast<u32x2 *>(mc + o)));
+                    __builtin_nontemporal_store(vw, as_global(reinterpret_cast<u32x2 *>(vc + o)));
+                }
+            } else {
+                for (int c = 0; c < 4; ++c) {
+                    const uint32_t o = c * 512 + lane * 8;
+                    u32x2 mw, vw;
+                    requant8<false, true>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
+                    __builtin_nontemporal_store(mw, as_global(reinterpret_cast<u32x2 *>(mc + o)));
+                    __builtin_nontemporal_store(vw, as_global(reinterpret_cast<u32x2 *>(vc + o)));
+                }
+            }
+        } else {
+            tail_block<true, MODE, EXACT, WD, GS, true>(cur.t, cur.lb, cur.left, lane, h, gscale, dbc1, dbc2, L);
+            if (prefetch) raw.issue(nxt.t, nxt.lb, lane);
+        }
+        cur = nxt;
+    }
+}
+
+template <int MODE, bool EXACT, bool WD, bool GS>
+static int launch_pipelined(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
+                            const void *lds_image, uint32_t grid, uint32_t wg, hipStream_t s) {
+    auto k = adam8_step_pipelined_kernel<MODE, EXACT, WD, GS>;
+    static bool attr_set = false; // the table image is larger than the 64 KiB default limit
+    if (!attr_set) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)kLdsImageBytes);
+        attr_set = true;
+    }
+    if (wg > 768) wg = 768;
+    hipLaunchKernelGGL(k, dim3(grid), dim3(wg), kLdsImageBytes, s, rows, n_rows, total_blocks, h,
+                       static_cast<const uint4 *>(lds_image));
+    return (int)hipGetLastError();
 }
 
 template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB>
@@ -461,6 +636,14 @@ static int launch_flags(const DevTensor *rows, uint32_t n_rows, uint32_t total_b
         if (wd) { if (gs) ERI_GO(true, true, false); ERI_GO(true, false, false); }
         if (gs) ERI_GO(false, true, false);
         ERI_GO(false, false, false);
+    }
+    if (BF16 && (h.flags & ERI_ADAM8_FLAG_NO_PIPELINE) == 0) {
+        if (wd) {
+            if (gs) return launch_pipelined<MODE, EXACT, true, true>(rows, n_rows, total_blocks, h, img, grid, wg, s);
+            return launch_pipelined<MODE, EXACT, true, false>(rows, n_rows, total_blocks, h, img, grid, wg, s);
+        }
+        if (gs) return launch_pipelined<MODE, EXACT, false, true>(rows, n_rows, total_blocks, h, img, grid, wg, s);
+        return launch_pipelined<MODE, EXACT, false, false>(rows, n_rows, total_blocks, h, img, grid, wg, s);
     }
     if (wd) { if (gs) ERI_GO(true, true, true); ERI_GO(true, false, true); }
     if (gs) ERI_GO(false, true, true);

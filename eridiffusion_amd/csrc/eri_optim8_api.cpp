@@ -61,29 +61,85 @@ uint32_t count_below(const float *mid, float x) { // the definition the slots mu
     return n;
 }
 
-/* Fills `slots` for one sign of one map and checks that no slot spans more than one midpoint. */
-bool build_slots(const float *mid, uint32_t shift, uint32_t base, uint32_t nslots, bool negative,
-                 eri::KeySlot *slots, std::string &why) {
-    const uint32_t sign = negative ? 0x80000000u : 0u;
-    for (uint32_t k = 0; k < nslots; ++k) {
-        uint32_t lo_bits = (k + base) << shift;
-        uint32_t hi_bits = lo_bits | ((1u << shift) - 1u);
-        if (k == 0) lo_bits = 0;                // saturating subtraction folds everything smaller in here
-        if (k == nslots - 1) hi_bits = lo_bits; // x == 1.0 exactly
-        // extreme values of the slot in value order
-        const float x_small = bits_to_float((negative ? hi_bits : lo_bits) | sign);
-        const float x_large = bits_to_float((negative ? lo_bits : hi_bits) | sign);
-        const uint32_t c0 = count_below(mid, x_small);
-        const uint32_t c1 = count_below(mid, x_large);
-        if (c1 < c0 || c1 - c0 > 1) {
-            why = "a lookup slot spans more than one quantisation midpoint";
-            return false;
-        }
-        slots[k].lo = c0;
-        slots[k].mid = (c1 == c0) ? std::numeric_limits<float>::infinity() : mid[c0];
+/* binary32 -> binary16 bit pattern, round to nearest even (what v_cvt_f16_f32 does). */
+uint16_t half_bits(float f) {
+    uint32_t u;
+    std::memcpy(&u, &f, 4);
+    const uint32_t sign = (u >> 16) & 0x8000u;
+    const uint32_t abs = u & 0x7fffffffu;
+    if (abs > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);  // NaN
+    if (abs >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u); // rounds to infinity (>= 65520)
+    if (abs < 0x33000001u) return (uint16_t)sign;              // below half the smallest denormal
+    int exp = (int)(abs >> 23) - 127;
+    uint32_t mant = (abs & 0x7fffffu) | 0x800000u;
+    int shift = (exp < -14) ? (13 + (-14 - exp)) : 13; // bits to drop
+    uint32_t kept = mant >> shift;
+    const uint32_t rem = mant & ((1u << shift) - 1u);
+    const uint32_t half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (kept & 1u))) kept += 1;
+    uint32_t out;
+    if (exp < -14) out = kept; // denormal (a carry into bit 10 becomes the smallest normal)
+    else out = ((uint32_t)(exp + 15) << 10) + (kept - 0x400u); // a mantissa carry bumps the exponent
+    return (uint16_t)(sign | out);
+}
+
+/*
+ * Fills the slot table of one map.  `drop` low bits of the half pattern are ignored, `mask` is
+ * applied first (it removes the sign for the unsigned map), `stride` bytes separate slots.
+ * For each sign the magnitudes 0 .. kKeyScale are walked as bit patterns (which order floats of one
+ * sign); every maximal run of magnitudes that convert into the same slot gives the slot's extreme
+ * scaled quotients, and the slot is accepted only if at most one scaled midpoint lies between them.
+ */
+bool build_slots(const float *mid, uint32_t drop, uint32_t mask, uint32_t stride, uint32_t count,
+                 unsigned char *out, std::string &why) {
+    float smid[255];
+    for (int j = 0; j < 255; ++j) smid[j] = mid[j] * eri::kKeyScale; // exact: power of two, no underflow
+    const float inf = std::numeric_limits<float>::infinity();
+    for (uint32_t k = 0; k < count; ++k) {
+        eri::KeySlot s;
+        s.lo = 0;
+        s.mid = inf; // NaN and unreachable patterns answer code 0
+        std::memcpy(out + (size_t)k * stride, &s, sizeof s);
     }
-    slots[nslots].lo = 0; // NaN slot: every comparison of a search is false
-    slots[nslots].mid = std::numeric_limits<float>::infinity();
+    uint32_t top_bits;
+    std::memcpy(&top_bits, &eri::kKeyScale, 4);
+    const int signs = (mask & 0x8000u) ? 2 : 1;
+    for (int sg = 0; sg < signs; ++sg) {
+        const uint32_t sign = sg ? 0x80000000u : 0u;
+        auto value = [&](uint32_t mag) { return bits_to_float(mag | sign); };
+        auto slot_of = [&](uint32_t mag) { return (uint32_t)((half_bits(value(mag)) & mask) >> drop); };
+        uint32_t b_lo = 0;
+        while (b_lo <= top_bits) {
+            const uint32_t k = slot_of(b_lo);
+            uint32_t a = b_lo, b = top_bits + 1; // slot_of(a) == k; b is past the run or past the range
+            if (slot_of(top_bits) == k) a = top_bits;
+            else {
+                b = top_bits;
+                while (b - a > 1) {
+                    const uint32_t c = a + (b - a) / 2;
+                    if (slot_of(c) == k) a = c; else b = c;
+                }
+            }
+            const uint32_t b_hi = a;
+            const float x_small = sg ? value(b_hi) : value(b_lo);
+            const float x_large = sg ? value(b_lo) : value(b_hi);
+            const uint32_t c0 = count_below(smid, x_small);
+            const uint32_t c1 = count_below(smid, x_large);
+            if (k >= count) {
+                why = "a quotient converts to a half float outside the slot table";
+                return false;
+            }
+            if (c1 < c0 || c1 - c0 > 1) {
+                why = "a lookup slot spans more than one quantisation midpoint";
+                return false;
+            }
+            eri::KeySlot s;
+            s.lo = c0;
+            s.mid = (c1 == c0) ? inf : smid[c0];
+            std::memcpy(out + (size_t)k * stride, &s, sizeof s);
+            b_lo = b_hi + 1;
+        }
+    }
     return true;
 }
 
@@ -117,11 +173,8 @@ const Tables &tables() {
         std::memcpy(&t.image[eri::kOffMapU], t.map_u, 1024);
         std::memcpy(&t.image[eri::kOffMidS], t.mid_s, 1024);
         std::memcpy(&t.image[eri::kOffMidU], t.mid_u, 1024);
-        auto *ks = reinterpret_cast<eri::KeySlot *>(&t.image[eri::kOffKeyS]);
-        auto *ku = reinterpret_cast<eri::KeySlot *>(&t.image[eri::kOffKeyU]);
-        if (!build_slots(t.mid_s, eri::kSShift, eri::kSBase, eri::kSSlots, false, ks, t.why)) return;
-        if (!build_slots(t.mid_s, eri::kSShift, eri::kSBase, eri::kSSlots, true, ks + eri::kSPerSign, t.why)) return;
-        if (!build_slots(t.mid_u, eri::kUShift, eri::kUBase, eri::kUSlots, false, ku, t.why)) return;
+        if (!build_slots(t.mid_s, eri::kSKeyDrop, 0xffffu, eri::kSKeyStride, eri::kSKeyCount, &t.image[eri::kOffKeyS], t.why)) return;
+        if (!build_slots(t.mid_u, eri::kUKeyDrop, 0x7fffu, eri::kUKeyStride, eri::kUKeyCount, &t.image[eri::kOffKeyU], t.why)) return;
         t.ok = true;
     });
     return t;
@@ -136,8 +189,8 @@ constexpr int kMaxDevices = 16;
 struct DeviceCtx {
     void *image = nullptr; // device copy of the LDS image
     uint32_t cus = 0;
-    uint32_t wg = 512;       // threads per workgroup
-    uint32_t wg_per_cu = 2;  // persistent workgroups per compute unit
+    uint32_t wg = 1024;      // threads per workgroup: the table image (~100 KB of LDS) allows one per CU
+    uint32_t wg_per_cu = 1;  // persistent workgroups per compute unit
     bool ready = false;
 };
 
@@ -164,14 +217,24 @@ int get_ctx(DeviceCtx **out) {
         hipDeviceProp_t prop;
         ERI_HIP(hipGetDeviceProperties(&prop, dev));
         c.cus = (uint32_t)prop.multiProcessorCount;
-        c.wg = (uint32_t)env_u32("ERI_ADAM8_WG", 64, 1024, 512) & ~63u;
-        c.wg_per_cu = (uint32_t)env_u32("ERI_ADAM8_WG_PER_CU", 1, 16, 2);
+        c.wg = (uint32_t)env_u32("ERI_ADAM8_WG", 64, 1024, 1024) & ~63u;
+        c.wg_per_cu = (uint32_t)env_u32("ERI_ADAM8_WG_PER_CU", 1, 16, 1);
         ERI_HIP(hipMalloc(&c.image, eri::kLdsImageBytes));
         ERI_HIP(hipMemcpy(c.image, t.image.data(), eri::kLdsImageBytes, hipMemcpyHostToDevice));
         c.ready = true;
     }
     *out = &c;
     return 0;
+}
+
+constexpr size_t kRecycleThreshold = (size_t)64 << 20;
+
+bool recycle_enabled() {
+    static const bool on = [] {
+        const char *s = std::getenv("ERI_HIP_MALLOC_RECYCLE");
+        return !(s && s[0] == '0');
+    }();
+    return on;
 }
 
 uint64_t blocks_of(uint64_t numel) { return (numel + eri::kBlock - 1) / eri::kBlock; }
@@ -309,6 +372,16 @@ int eri_hip_malloc_zeroed(int device, size_t bytes, void **out) {
     if (prev != device) ERI_HIP(hipSetDevice(device));
     void *p = nullptr;
     hipError_t e = hipMalloc(&p, bytes);
+    // Placement conditioning.  On MI355X the first physical placement a large allocation receives
+    // sustains visibly less write bandwidth than the placement the same request receives once the
+    // range has been handed back to the driver (measured with a plain streaming kernel: 4.6 vs
+    // 5.5 TB/s on 24 GB buffers).  Large allocations are therefore allocated, released and
+    // allocated again.  ERI_HIP_MALLOC_RECYCLE=0 switches this off.
+    if (e == hipSuccess && bytes >= kRecycleThreshold && recycle_enabled()) {
+        e = hipFree(p);
+        p = nullptr;
+        if (e == hipSuccess) e = hipMalloc(&p, bytes);
+    }
     if (e == hipSuccess) e = hipMemset(p, 0, bytes);
     if (prev != device) (void)hipSetDevice(prev);
     if (e != hipSuccess) {
@@ -536,12 +609,17 @@ int eri_adam8_step_table(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream)
     if (rc) return rc;
     for (auto &g : t->groups) {
         if (g.n == 0) continue;
-        const uint32_t waves_per_wg = ctx->wg / eri::kWave;
-        uint32_t grid = ctx->cus * ctx->wg_per_cu;
+        // One wavefront per block.  A small table gets smaller workgroups so that its blocks still
+        // spread over every compute unit instead of filling a few of them.
+        uint32_t waves_per_wg = ctx->wg / eri::kWave;
+        const uint32_t slots = ctx->cus * ctx->wg_per_cu;
+        const uint32_t per_slot = (g.total_blocks + slots - 1) / slots;
+        if (per_slot < waves_per_wg) waves_per_wg = per_slot < 4 ? 4 : per_slot;
+        uint32_t grid = slots;
         const uint32_t need = (g.total_blocks + waves_per_wg - 1) / waves_per_wg;
         if (grid > need) grid = need;
         if (grid == 0) grid = 1;
-        rc = eri::launch_step(g.dev, g.n, g.total_blocks, g.dtype, *h, ctx->image, grid, ctx->wg, stream);
+        rc = eri::launch_step(g.dev, g.n, g.total_blocks, g.dtype, *h, ctx->image, grid, waves_per_wg * eri::kWave, stream);
         if (rc) return hip_fail((hipError_t)rc, "adam8 step launch");
     }
     return 0;

@@ -85,8 +85,10 @@ enum {
     ERI_ADAM8_FLAG_GRAD_SCALE = 1u << 0,  /* multiply gradients by hyper.grad_scale * tensor.grad_scale */
     ERI_ADAM8_FLAG_EXACT_PARAM = 1u << 1, /* IEEE sqrt and divide on the parameter update of BF16
                                              tensors too (F32 tensors always use them) */
-    ERI_ADAM8_FLAG_BSEARCH = 1u << 2      /* requantise by binary search of the LDS midpoint table
+    ERI_ADAM8_FLAG_BSEARCH = 1u << 2,     /* requantise by binary search of the LDS midpoint table
                                              instead of the float-keyed slot table (same codes) */
+    ERI_ADAM8_FLAG_NO_PIPELINE = 1u << 3  /* BF16: use the plain kernel, not the one that prefetches
+                                             the next block (same results; for A/B measurements) */
 };
 
 /* Per-step scalars, already cast where the reference casts them.  Fill with eri_adam8_hyper_pack. */

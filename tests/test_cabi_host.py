@@ -111,26 +111,25 @@ def _image():
     return buf, list(offs)
 
 
+KEY_SCALE = np.float32(4096.0)
+
+
 def _replay(x, img, offs, signed):
-    """The kernel's slot lookup (code_signed_key / code_unsigned_key), in NumPy."""
-    exp0 = 106
-    mant = 6 if signed else 7
-    shift = 23 - mant
-    base = exp0 << mant
-    slots = ((127 - exp0) << mant) + 1
-    off = offs[4] if signed else offs[5]
-    count = 2 * (slots + 1) if signed else slots + 1
-    tab = img[off:off + count * 8].view(np.uint32).reshape(count, 2)
-    b = x.view(np.uint32)
-    k = ((b & 0x7FFFFFFF) if signed else b) >> shift
-    k = np.where(k > base, k - base, 0)
-    k = np.minimum(k, slots)
-    if signed:
-        k = k + (b >> 31) * (slots + 1)
-    mid = tab[k, 0].copy().view(np.float32)
-    lo = tab[k, 1]
+    """The kernel's slot lookup (code_signed_key / code_unsigned_key), in NumPy: scale the quotient,
+    convert to binary16 (round to nearest even), mask the pattern into a byte address."""
+    xs = (x * KEY_SCALE).astype(np.float32)
+    with np.errstate(over="ignore", invalid="ignore"):
+        h = xs.astype(np.float16).view(np.uint16).astype(np.uint32)
+    addr = (h & 0xFFF0) if signed else (h & 0x7FF8)
+    base = offs[4] if signed else offs[5]
+    mid = np.empty(x.size, np.float32)
+    lo = np.empty(x.size, np.uint32)
+    words = img.view(np.uint32)
+    idx = (base + addr) // 4
+    mid = words[idx].copy().view(np.float32)
+    lo = words[idx + 1]
     with np.errstate(invalid="ignore"):
-        return (lo + (x > mid)).astype(np.int64)
+        return (lo + (xs > mid)).astype(np.int64)
 
 
 @pytest.mark.parametrize("signed", [True, False])
@@ -142,10 +141,11 @@ def test_slot_lookup_equals_search(signed):
     rng = np.random.default_rng(13)
     near = np.concatenate([np.nextafter(mid, np.float32(-2)), mid, np.nextafter(mid, np.float32(2)),
                            np.nextafter(table, np.float32(-2)), table, np.nextafter(table, np.float32(2))])
-    # every slot boundary of the key, both sides
-    mant = 6 if signed else 7
-    kb = (np.arange(100 << mant, (127 << mant) + 2, dtype=np.uint32) << (23 - mant))
-    edges = np.concatenate([kb, kb - 1, kb + 1]).view(np.float32)
+    # every boundary between binary16 values of the scaled quotient, and its float32 neighbours
+    halves = np.arange(0, 0x6C01, dtype=np.uint16).view(np.float16).astype(np.float32)  # 0 .. 4096
+    ties = ((halves[:-1].astype(np.float64) + halves[1:].astype(np.float64)) / 2).astype(np.float32)
+    edges = np.concatenate([halves, ties, np.nextafter(ties, np.float32(-1)), np.nextafter(ties, np.float32(1e9))])
+    edges = (edges / KEY_SCALE).astype(np.float32)
     rnd = rng.integers(0, 0x3F800001, 4_000_000, dtype=np.uint32).view(np.float32)
     logu = (10.0 ** rng.uniform(-12, 0, 1_000_000)).astype(np.float32)
     xs = np.concatenate([near, edges, rnd, logu, np.array([0.0, 1.0, 1e-45, 1e-30], np.float32)]).astype(np.float32)
