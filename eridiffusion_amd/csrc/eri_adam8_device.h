@@ -23,7 +23,7 @@ struct DevTensor {
     float *absmax_m;
     float *absmax_v;
     uint64_t numel;
-    uint32_t block_start; /* first block of this tensor within its dtype group */
+    uint32_t full_start;  /* number of full 2048-element blocks in the rows before this one (same dtype) */
     float grad_scale;
 };
 static_assert(sizeof(DevTensor) == 64, "DevTensor must stay 64 bytes");
@@ -66,7 +66,7 @@ static_assert(kLdsImageBytes % 16 == 0, "the image is staged in 16-byte words");
 
 /* Launchers implemented in eri_adam8_kernels.hip; `stream` is a hipStream_t.  All return a
  * hipError_t as int.  `lds_image` is the device copy of the kLdsImageBytes table image. */
-int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, int dtype_tag,
+int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_blocks, int dtype_tag,
                 const EriAdam8Hyper &h, const void *lds_image, uint32_t grid, uint32_t wg, void *stream);
 int launch_state_init(uint8_t *m, uint8_t *v, float *absmax_m, float *absmax_v, uint64_t numel, void *stream);
 int launch_dequantize(const uint8_t *codes, const float *absmax, int signed_map, uint64_t numel, float *out,

@@ -172,21 +172,25 @@ __device__ __forceinline__ void adam_elem(float p, float g, float m_old, float v
         if (BF16) us = bf16_round(us); // :197-198
         pn = p - us;                   // :205
     } else {
-        float r;
         if (EXACT) {
             float den = sqrtf(v) + h.eps; // adam8bit_enhanced.rs:263
-            r = m / den;                  // :264
+            float r = m / den;            // :264
+            float u = r;
+            if (WD) { // :267-271
+                float pw = p * h.weight_decay;
+                u = r + pw;
+            }
+            float us = u * h.step_size; // :274
+            pn = p - us;                // :275
         } else {
+            // bf16 parameters: hardware square root and reciprocal (1 ulp each) and two fused
+            // multiply-adds; the fp32 result is within a few ulp of the exact chain, which moves
+            // the bf16 rounding of p by at most one step, rarely
             float den = __builtin_amdgcn_sqrtf(v) + h.eps;
-            r = m * __builtin_amdgcn_rcpf(den);
+            float r = m * __builtin_amdgcn_rcpf(den);
+            float u = WD ? __builtin_fmaf(p, h.weight_decay, r) : r;
+            pn = __builtin_fmaf(-u, h.step_size, p);
         }
-        float u = r;
-        if (WD) { // :267-271
-            float pw = p * h.weight_decay;
-            u = r + pw;
-        }
-        float us = u * h.step_size; // :274
-        pn = p - us;                // :275
     }
 }
 
@@ -402,6 +406,17 @@ __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint
 
 extern __shared__ uint4 lds_raw[];
 
+/* Row owning full block `blk`: the last row whose full_start is <= blk (rows without full blocks
+ * share their successor's full_start and are skipped by taking the last).  All wave-uniform. */
+__device__ __forceinline__ uint32_t find_row(const DevTensor *rows, uint32_t n_rows, uint32_t from, uint32_t blk) {
+    uint32_t lo = from, hi = n_rows; // rows[lo].full_start <= blk
+    while (hi - lo > 1) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (rows[mid].full_start <= blk) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
 template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB>
 __global__ __launch_bounds__(1024) void adam8_step_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
                                                           uint32_t total_blocks, EriAdam8Hyper h,
@@ -423,22 +438,21 @@ __global__ __launch_bounds__(1024) void adam8_step_kernel(const DevTensor *__res
     const uint32_t stride = gridDim.x * waves_per_wg;
     const BlockDiv dbc1(h.bc1), dbc2(h.bc2);
 
-    uint32_t ti = 0; // rows[ti].block_start <= blk; blk only grows, so the search restarts from ti
-    for (uint32_t blk = wave; blk < total_blocks; blk += stride) {
-        uint32_t lo = ti, hi = n_rows; // answer in [lo, hi)
-        while (hi - lo > 1) {
-            const uint32_t mid = (lo + hi) >> 1;
-            if (rows[mid].block_start <= blk) lo = mid; else hi = mid;
+    // partial last blocks first: one per row at most, spread over the waves
+    for (uint32_t r = wave; r < n_rows; r += stride) {
+        const DevTensor t = rows[r];
+        const uint32_t n = (uint32_t)(t.numel % kBlock);
+        if (n != 0) {
+            const float gscale = GS ? h.grad_scale * t.grad_scale : 1.0f;
+            tail_block<BF16, MODE, EXACT, WD, GS, KEYTAB>(t, (uint32_t)(t.numel / kBlock), n, lane, h, gscale, dbc1, dbc2, L);
         }
-        ti = lo;
+    }
+    uint32_t ti = 0; // rows[ti].full_start <= blk; blk only grows, so the search restarts from ti
+    for (uint32_t blk = wave; blk < total_blocks; blk += stride) {
+        ti = find_row(rows, n_rows, ti, blk);
         const DevTensor t = rows[ti];
-        const uint32_t lb = blk - t.block_start;
-        const uint64_t left = t.numel - (uint64_t)lb * kBlock;
         const float gscale = GS ? h.grad_scale * t.grad_scale : 1.0f;
-        if (left >= kBlock)
-            full_block<BF16, MODE, EXACT, WD, GS, KEYTAB>(t, lb, lane, h, gscale, dbc1, dbc2, L);
-        else
-            tail_block<BF16, MODE, EXACT, WD, GS, KEYTAB>(t, lb, (uint32_t)left, lane, h, gscale, dbc1, dbc2, L);
+        full_block<BF16, MODE, EXACT, WD, GS, KEYTAB>(t, blk - t.full_start, lane, h, gscale, dbc1, dbc2, L);
     }
 }
 
@@ -474,27 +488,6 @@ struct RawBlock {
     }
 };
 
-/* Where a wave is in the global block list (all wave-uniform). */
-struct Cursor {
-    uint32_t blk, ti, lb, left;
-    DevTensor t;
-    bool valid;
-    __device__ __forceinline__ void locate(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks) {
-        valid = blk < total_blocks;
-        if (!valid) return;
-        uint32_t lo = ti, hi = n_rows; // rows[lo].block_start <= blk; blk only grows
-        while (hi - lo > 1) {
-            const uint32_t mid = (lo + hi) >> 1;
-            if (rows[mid].block_start <= blk) lo = mid; else hi = mid;
-        }
-        ti = lo;
-        t = rows[ti];
-        lb = blk - t.block_start;
-        const uint64_t l = t.numel - (uint64_t)lb * kBlock;
-        left = l >= kBlock ? kBlock : (uint32_t)l;
-    }
-};
-
 template <int MODE, bool EXACT, bool WD, bool GS>
 __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTensor *__restrict__ rows,
                                                                    uint32_t n_rows, uint32_t total_blocks,
@@ -516,81 +509,93 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
     const uint32_t stride = gridDim.x * waves_per_wg;
     const BlockDiv dbc1(h.bc1), dbc2(h.bc2);
 
-    Cursor cur;
-    cur.blk = __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
-    cur.ti = 0;
-    cur.locate(rows, n_rows, total_blocks);
-    RawBlock raw;
-    if (cur.valid && cur.left == kBlock) raw.issue(cur.t, cur.lb, lane);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
+    // partial last blocks first: one per row at most, spread over the waves
+    for (uint32_t r = wave; r < n_rows; r += stride) {
+        const DevTensor t = rows[r];
+        const uint32_t n = (uint32_t)(t.numel % kBlock);
+        if (n != 0) {
+            const float gscale = GS ? h.grad_scale * t.grad_scale : 1.0f;
+            tail_block<true, MODE, EXACT, WD, GS, true>(t, (uint32_t)(t.numel / kBlock), n, lane, h, gscale, dbc1, dbc2, L);
+        }
+    }
+    if (wave >= total_blocks) return;
 
-    while (cur.valid) {
-        Cursor nxt;
-        nxt.blk = cur.blk + stride;
-        nxt.ti = cur.ti;
-        nxt.locate(rows, n_rows, total_blocks);
-        const bool prefetch = nxt.valid && nxt.left == kBlock;
-        const float gscale = GS ? h.grad_scale * cur.t.grad_scale : 1.0f;
-        if (cur.left == kBlock) {
-            const size_t e0 = (size_t)cur.lb * kBlock;
-            char *p = static_cast<char *>(cur.t.p) + e0 * 2;
-            uint8_t *mc = cur.t.m + e0;
-            uint8_t *vc = cur.t.v + e0;
-            float mf[32], vf[32];
-            float lm = 0.0f, lv = 0.0f;
-            const float a_m = raw.a_m, a_v = raw.a_v;
+    uint32_t blk = wave;
+    uint32_t ti = find_row(rows, n_rows, 0, blk);
+    DevTensor t = rows[ti];
+    RawBlock raw;
+    raw.issue(t, blk - t.full_start, lane);
+    while (true) {
+        // the block after this one; past the end the wave re-reads its last block (the loads must
+        // stay unconditional so that the raw registers have a single definition in the loop)
+        const uint32_t nblk = blk + stride;
+        const bool more = nblk < total_blocks;
+        const uint32_t pblk = more ? nblk : blk;
+        const uint32_t nti = find_row(rows, n_rows, ti, pblk);
+        const DevTensor nt = rows[nti];
+
+        const uint32_t lb = blk - t.full_start;
+        const float gscale = GS ? h.grad_scale * t.grad_scale : 1.0f;
+        const size_t e0 = (size_t)lb * kBlock;
+        char *p = static_cast<char *>(t.p) + e0 * 2;
+        uint8_t *mc = t.m + e0;
+        uint8_t *vc = t.v + e0;
+        float mf[32], vf[32];
+        float lm = 0.0f, lv = 0.0f;
+        const float a_m = raw.a_m, a_v = raw.a_v;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t o = c * 512 + lane * 8;
+            Raw8<true> pr, gr;
+            pr.w = raw.p[c];
+            gr.w = raw.g[c];
+            float pv[8], gv[8], pn[8];
+            pr.unpack(pv);
+            gr.unpack(gv);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const float m_old = L.map_s[byte_of(raw.m[c], k)] * a_m;
+                const float v_old = L.map_u[byte_of(raw.v[c], k)] * a_v;
+                float m, v;
+                adam_elem<MODE, EXACT, true, WD, GS>(pv[k], gv[k], m_old, v_old, h, gscale, dbc1, dbc2, m, v, pn[k]);
+                mf[c * 8 + k] = m;
+                vf[c * 8 + k] = v;
+                lm = fmaxf(lm, __builtin_fabsf(m));
+                lv = fmaxf(lv, __builtin_fabsf(v));
+            }
+            store8<true>(p, o, pn);
+        }
+        const float nam = wave_max(lm);
+        const float nav = wave_max(lv);
+        if (lane == 0) {
+            as_global(t.absmax_m)[lb] = nam;
+            as_global(t.absmax_v)[lb] = nav;
+        }
+        raw.issue(nt, pblk - nt.full_start, lane); // prefetch: in flight during the requantisation
+        const BlockDiv dm(nam, kKeyScale, kKeyScaleInv), dv(nav, kKeyScale, kKeyScaleInv);
+        if (dm.fast && dv.fast) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const uint32_t o = c * 512 + lane * 8;
-                Raw8<true> pr, gr;
-                pr.w = raw.p[c];
-                gr.w = raw.g[c];
-                float pv[8], gv[8], pn[8];
-                pr.unpack(pv);
-                gr.unpack(gv);
-#pragma unroll
-                for (int k = 0; k < 8; ++k) {
-                    const float m_old = L.map_s[byte_of(raw.m[c], k)] * a_m;
-                    const float v_old = L.map_u[byte_of(raw.v[c], k)] * a_v;
-                    float m, v;
-                    adam_elem<MODE, EXACT, true, WD, GS>(pv[k], gv[k], m_old, v_old, h, gscale, dbc1, dbc2, m, v, pn[k]);
-                    mf[c * 8 + k] = m;
-                    vf[c * 8 + k] = v;
-                    lm = fmaxf(lm, __builtin_fabsf(m));
-                    lv = fmaxf(lv, __builtin_fabsf(v));
-                }
-                store8<true>(p, o, pn);
-            }
-            const float nam = wave_max(lm);
-            const float nav = wave_max(lv);
-            if (lane == 0) {
-                as_global(cur.t.absmax_m)[cur.lb] = nam;
-                as_global(cur.t.absmax_v)[cur.lb] = nav;
-            }
-            if (prefetch) raw.issue(nxt.t, nxt.lb, lane);
-            const BlockDiv dm(nam, kKeyScale, kKeyScaleInv), dv(nav, kKeyScale, kKeyScaleInv);
-            if (dm.fast && dv.fast) {
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    const uint32_t o = c * 512 + lane * 8;
-                    u32x2 mw, vw;
-                    requant8<true, true>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
-                    __builtin_nontemporal_store(mw, as_global(reinterpret_cast<u32x2 *>(mc + o)));
-                    __builtin_nontemporal_store(vw, as_global(reinterpret_cast<u32x2 *>(vc + o)));
-                }
-            } else {
-                for (int c = 0; c < 4; ++c) {
-                    const uint32_t o = c * 512 + lane * 8;
-                    u32x2 mw, vw;
-                    requant8<false, true>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
-                    __builtin_nontemporal_store(mw, as_global(reinterpret_cast<u32x2 *>(mc + o)));
-                    __builtin_nontemporal_store(vw, as_global(reinterpret_cast<u32x2 *>(vc + o)));
-                }
+                u32x2 mw, vw;
+                requant8<true, true>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
+                __builtin_nontemporal_store(mw, as_global(reinterpret_cast<u32x2 *>(mc + o)));
+                __builtin_nontemporal_store(vw, as_global(reinterpret_cast<u32x2 *>(vc + o)));
             }
         } else {
-            tail_block<true, MODE, EXACT, WD, GS, true>(cur.t, cur.lb, cur.left, lane, h, gscale, dbc1, dbc2, L);
-            if (prefetch) raw.issue(nxt.t, nxt.lb, lane);
+            for (int c = 0; c < 4; ++c) {
+                const uint32_t o = c * 512 + lane * 8;
+                u32x2 mw, vw;
+                requant8<false, true>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
+                __builtin_nontemporal_store(mw, as_global(reinterpret_cast<u32x2 *>(mc + o)));
+                __builtin_nontemporal_store(vw, as_global(reinterpret_cast<u32x2 *>(vc + o)));
+            }
         }
-        cur = nxt;
+        if (!more) break;
+        blk = nblk;
+        ti = nti;
+        t = nt;
     }
 }
 

@@ -249,7 +249,7 @@ struct EriAdam8Table {
     struct Group {
         int dtype = 0;
         uint32_t n = 0;
-        uint32_t total_blocks = 0;
+        uint32_t total_blocks = 0; // full blocks only; a row's partial last block is handled per row
         eri::DevTensor *dev = nullptr;
         eri::DevTensor *pinned = nullptr;
         std::vector<uint32_t> src; // index into the caller's rows
@@ -316,9 +316,9 @@ void fill_group(EriAdam8Table::Group &g, const EriAdam8Tensor *rows) {
         d.absmax_m = r.absmax_m;
         d.absmax_v = r.absmax_v;
         d.numel = r.numel;
-        d.block_start = start;
+        d.full_start = start;
         d.grad_scale = r.grad_scale;
-        start += (uint32_t)blocks_of(r.numel);
+        start += (uint32_t)(r.numel / eri::kBlock);
     }
     g.total_blocks = start;
 }
@@ -613,10 +613,11 @@ int eri_adam8_step_table(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream)
         // spread over every compute unit instead of filling a few of them.
         uint32_t waves_per_wg = ctx->wg / eri::kWave;
         const uint32_t slots = ctx->cus * ctx->wg_per_cu;
-        const uint32_t per_slot = (g.total_blocks + slots - 1) / slots;
+        const uint32_t work = g.total_blocks > g.n ? g.total_blocks : g.n; // full blocks, or one tail per row
+        const uint32_t per_slot = (work + slots - 1) / slots;
         if (per_slot < waves_per_wg) waves_per_wg = per_slot < 4 ? 4 : per_slot;
         uint32_t grid = slots;
-        const uint32_t need = (g.total_blocks + waves_per_wg - 1) / waves_per_wg;
+        const uint32_t need = (work + waves_per_wg - 1) / waves_per_wg;
         if (grid > need) grid = need;
         if (grid == 0) grid = 1;
         rc = eri::launch_step(g.dev, g.n, g.total_blocks, g.dtype, *h, ctx->image, grid, waves_per_wg * eri::kWave, stream);
