@@ -249,6 +249,33 @@ __device__ __forceinline__ uint32_t byte_of(const u32x2 w, int k) {
     return (d >> (8 * (k & 3))) & 0xffu;
 }
 
+/* 4 * (byte k of the eight packed codes): the LDS byte offset of a float table entry, in one
+ * sub-dword-addressed shift (v_lshlrev_b32 with an SDWA byte select) instead of an extract and a
+ * shift.  k must be a compile-time constant after unrolling. */
+__device__ __forceinline__ uint32_t code_offset(const u32x2 w, int k) {
+    const uint32_t d = k < 4 ? w.x : w.y;
+    const uint32_t two = 2u;
+    uint32_t r;
+    switch (k & 3) {
+    case 0:
+        asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_0" : "=v"(r) : "v"(two), "v"(d));
+        break;
+    case 1:
+        asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_1" : "=v"(r) : "v"(two), "v"(d));
+        break;
+    case 2:
+        asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_2" : "=v"(r) : "v"(two), "v"(d));
+        break;
+    default:
+        asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_3" : "=v"(r) : "v"(two), "v"(d));
+        break;
+    }
+    return r;
+}
+__device__ __forceinline__ float lds_float_at(const float *table, uint32_t byte_offset) {
+    return *reinterpret_cast<const float *>(reinterpret_cast<const char *>(table) + byte_offset);
+}
+
 // ------------------------------------------------------------------------------------------
 // a full 2048-element block, one wavefront
 // ------------------------------------------------------------------------------------------
@@ -404,7 +431,9 @@ __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint
 // the step kernel
 // ------------------------------------------------------------------------------------------
 
-extern __shared__ uint4 lds_raw[];
+/* The table image, staged once per workgroup.  A static array: its LDS address is a compile-time
+ * constant, so table offsets fold into the ds_read immediates. */
+#define ERI_LDS_IMAGE __shared__ uint4 lds_raw[kLdsImageBytes / 16]
 
 /* Row owning full block `blk`: the last row whose full_start is <= blk (rows without full blocks
  * share their successor's full_start and are skipped by taking the last).  All wave-uniform. */
@@ -421,6 +450,7 @@ template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB>
 __global__ __launch_bounds__(1024) void adam8_step_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
                                                           uint32_t total_blocks, EriAdam8Hyper h,
                                                           const uint4 *__restrict__ lds_image) {
+    ERI_LDS_IMAGE;
     for (uint32_t i = threadIdx.x; i < kLdsImageBytes / 16; i += blockDim.x) lds_raw[i] = lds_image[i];
     __syncthreads();
     const char *base = reinterpret_cast<const char *>(lds_raw);
@@ -493,6 +523,7 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
                                                                    uint32_t n_rows, uint32_t total_blocks,
                                                                    EriAdam8Hyper h,
                                                                    const uint4 *__restrict__ lds_image) {
+    ERI_LDS_IMAGE;
     for (uint32_t i = threadIdx.x; i < kLdsImageBytes / 16; i += blockDim.x) lds_raw[i] = lds_image[i];
     __syncthreads();
     const char *base = reinterpret_cast<const char *>(lds_raw);
@@ -555,8 +586,8 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
             gr.unpack(gv);
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
-                const float m_old = L.map_s[byte_of(raw.m[c], k)] * a_m;
-                const float v_old = L.map_u[byte_of(raw.v[c], k)] * a_v;
+                const float m_old = lds_float_at(L.map_s, code_offset(raw.m[c], k)) * a_m;
+                const float v_old = lds_float_at(L.map_u, code_offset(raw.v[c], k)) * a_v;
                 float m, v;
                 adam_elem<MODE, EXACT, true, WD, GS>(pv[k], gv[k], m_old, v_old, h, gscale, dbc1, dbc2, m, v, pn[k]);
                 mf[c * 8 + k] = m;
@@ -603,14 +634,8 @@ template <int MODE, bool EXACT, bool WD, bool GS>
 static int launch_pipelined(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
                             const void *lds_image, uint32_t grid, uint32_t wg, hipStream_t s) {
     auto k = adam8_step_pipelined_kernel<MODE, EXACT, WD, GS>;
-    static bool attr_set = false; // the table image is larger than the 64 KiB default limit
-    if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  (int)kLdsImageBytes);
-        attr_set = true;
-    }
     if (wg > 768) wg = 768;
-    hipLaunchKernelGGL(k, dim3(grid), dim3(wg), kLdsImageBytes, s, rows, n_rows, total_blocks, h,
+    hipLaunchKernelGGL(k, dim3(grid), dim3(wg), 0, s, rows, n_rows, total_blocks, h,
                        static_cast<const uint4 *>(lds_image));
     return (int)hipGetLastError();
 }
@@ -619,13 +644,7 @@ template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB>
 static int launch_one(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
                       const void *lds_image, uint32_t grid, uint32_t wg, hipStream_t s) {
     auto k = adam8_step_kernel<BF16, MODE, EXACT, WD, GS, KEYTAB>;
-    static bool attr_set = false; // the table image exceeds the 64 KiB default only if it ever grows
-    if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(k), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  (int)kLdsImageBytes);
-        attr_set = true;
-    }
-    hipLaunchKernelGGL(k, dim3(grid), dim3(wg), kLdsImageBytes, s, rows, n_rows, total_blocks, h,
+    hipLaunchKernelGGL(k, dim3(grid), dim3(wg), 0, s, rows, n_rows, total_blocks, h,
                        static_cast<const uint4 *>(lds_image));
     return (int)hipGetLastError();
 }
