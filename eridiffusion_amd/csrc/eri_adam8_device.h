@@ -59,9 +59,11 @@ constexpr uint32_t kOffMapS = 0;                              /* 256 floats: cod
 constexpr uint32_t kOffMapU = kOffMapS + 1024;                /* 256 floats */
 constexpr uint32_t kOffMidS = kOffMapU + 1024;                /* 255 midpoints + one +inf */
 constexpr uint32_t kOffMidU = kOffMidS + 1024;
-constexpr uint32_t kOffKeyS = kOffMidU + 1024;                /* kSKeyCount slots, kSKeyStride apart */
-constexpr uint32_t kOffKeyU = kOffKeyS + kSKeyCount * kSKeyStride; /* kUKeyCount slots */
-constexpr uint32_t kLdsImageBytes = kOffKeyU + kUKeyCount * kUKeyStride;
+/* Both slot tables start below 64 KiB so that their offsets fit the 16-bit immediate of ds_read. */
+constexpr uint32_t kOffKeyU = kOffMidU + 1024;                /* kUKeyCount slots, kUKeyStride apart */
+constexpr uint32_t kOffKeyS = kOffKeyU + kUKeyCount * kUKeyStride; /* kSKeyCount slots */
+constexpr uint32_t kLdsImageBytes = kOffKeyS + kSKeyCount * kSKeyStride;
+static_assert(kOffKeyS < 65536 && kOffKeyU < 65536, "slot table offsets must fit a ds_read immediate");
 static_assert(kLdsImageBytes % 16 == 0, "the image is staged in 16-byte words");
 
 /* Launchers implemented in eri_adam8_kernels.hip; `stream` is a hipStream_t.  All return a
