@@ -28,6 +28,12 @@ class TensorRow(C.Structure):
                 ("block_start", C.c_uint64), ("dtype_tag", C.c_int32), ("grad_scale", C.c_float)]
 
 
+class Adam8bitConfigC(C.Structure):
+    _fields_ = [("lr", C.c_double), ("beta1", C.c_double), ("beta2", C.c_double), ("eps", C.c_double),
+                ("weight_decay", C.c_double), ("amsgrad", C.c_int32), ("block_wise", C.c_int32),
+                ("percentile_clipping", C.c_uint64)]
+
+
 class EriError(RuntimeError):
     def __init__(self, what, code, message):
         super().__init__("%s failed with code %d: %s" % (what, code, message))
@@ -38,6 +44,8 @@ class EriError(RuntimeError):
 EXPORTS = {
     # name: (restype, argtypes)
     "eri_last_error": (C.c_char_p, []),
+    "eri_set_last_error": (None, [C.c_char_p]),
+    "eri_hip_get_device": (C.c_int, [C.POINTER(C.c_int)]),
     "eri_hip_device_count": (C.c_int, [C.POINTER(C.c_int)]),
     "eri_hip_set_device": (C.c_int, [C.c_int]),
     "eri_hip_malloc_zeroed": (C.c_int, [C.c_int, C.c_size_t, C.POINTER(C.c_void_p)]),
@@ -63,6 +71,38 @@ EXPORTS = {
     "eri_adam8_step_multi": (C.c_int, [C.POINTER(TensorRow), C.c_uint32, C.POINTER(Hyper), C.c_void_p]),
     "eri_adam8_dequantize": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_uint64, C.c_void_p, C.c_void_p]),
     "eri_adam8_quantize": (C.c_int, [C.c_void_p, C.c_int, C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p]),
+    # ---- include/eri_adam8bit.h
+    "eri_param_create": (C.c_int, [C.c_void_p, C.c_uint64, C.c_int, C.POINTER(C.c_void_p)]),
+    "eri_param_set_grad": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "eri_param_set_data": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "eri_param_retain": (C.c_int, [C.c_void_p]),
+    "eri_param_release": (C.c_int, [C.c_void_p]),
+    "eri_adam8bit_config_default": (None, [C.POINTER(Adam8bitConfigC)]),
+    "eri_adam8bit_new": (C.c_int, [C.POINTER(C.c_void_p), C.c_uint32, C.POINTER(Adam8bitConfigC), C.c_void_p,
+                                   C.POINTER(C.c_void_p)]),
+    "eri_adam8bit_destroy": (C.c_int, [C.c_void_p]),
+    "eri_adam8bit_step": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint32)]),
+    "eri_adam8bit_zero_grad": (C.c_int, [C.c_void_p]),
+    "eri_adam8bit_current_lr": (C.c_double, [C.c_void_p]),
+    "eri_adam8bit_set_learning_rate": (C.c_int, [C.c_void_p, C.c_double]),
+    "eri_adam8bit_quantized_memory_usage": (C.c_uint64, [C.c_void_p]),
+    "eri_adam8bit_get_step": (C.c_uint64, [C.c_void_p]),
+    "eri_adam8bit_set_grad_scale": (C.c_int, [C.c_void_p, C.c_float]),
+    "eri_adam8bit_set_param_grad_scale": (C.c_int, [C.c_void_p, C.c_uint32, C.c_float]),
+    "eri_adam8bit_set_flags": (C.c_int, [C.c_void_p, C.c_uint32]),
+    "eri_adam8bit_save_state": (C.c_int, [C.c_void_p, C.c_char_p]),
+    "eri_adam8bit_load_state": (C.c_int, [C.c_void_p, C.c_char_p]),
+    "eri_adam8bit_state_ptrs": (C.c_int, [C.c_void_p, C.c_uint32] + [C.POINTER(C.c_void_p)] * 4),
+    "eri_adam8bit_fn_with_params": (C.c_int, [C.c_double] * 5 + [C.c_void_p, C.POINTER(C.c_void_p)]),
+    "eri_adam8bit_fn_destroy": (C.c_int, [C.c_void_p]),
+    "eri_adam8bit_fn_update": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_uint64, C.c_int, C.c_void_p]),
+    "eri_adam8bit_fn_step": (C.c_int, [C.c_void_p]),
+    "eri_adam8bit_fn_set_lr": (C.c_int, [C.c_void_p, C.c_float]),
+    "eri_adam8bit_fn_get_step": (C.c_uint64, [C.c_void_p]),
+    "eri_adam8bit_fn_memory_stats": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
+    "eri_adam8bit_fn_state_numel": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_uint64)]),
+    "eri_adam8bit_fn_get_state_fp32": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p]),
+    "eri_adam8bit_fn_load_state_fp32": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_uint64]),
 }
 
 _lib = None

@@ -1,0 +1,665 @@
+/*
+ * Host layer of the 8-bit Adam objects (include/eri_adam8bit.h), written against the C ABI of
+ * include/eri_optim8.h only: no HIP headers, no torch.  It holds what the reference's Rust structs
+ * hold -- the parameter handles, hyper-parameters, step counter and per-parameter 8-bit state --
+ * plus the cached device launch table, and turns every step() into one eri_adam8_step_table call.
+ *
+ * Reference structures mirrored here:
+ *   Adam8bit / Adam8bitConfig / OptimizerState   src/trainers/adam8bit_enhanced.rs:10-27,372-404
+ *   Adam8bit (functional) / Adam8bitState        src/trainers/adam8bit.rs:15-47
+ */
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <map>
+#include <memory>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include "../../include/eri_adam8bit.h"
+
+namespace {
+
+constexpr uint64_t kBlock = ERI_ADAM8_BLOCK;
+
+uint64_t blocks_of(uint64_t numel) { return (numel + kBlock - 1) / kBlock; }
+uint64_t align256(uint64_t n) { return (n + 255) & ~(uint64_t)255; }
+
+int fail(int code, const std::string &msg) {
+    eri_set_last_error(msg.c_str());
+    return code;
+}
+
+/* uint8 codes and per-block absmax of both moments, in one device allocation. */
+struct State8 {
+    void *base = nullptr;
+    uint8_t *m = nullptr, *v = nullptr;
+    float *absmax_m = nullptr, *absmax_v = nullptr;
+    uint64_t numel = 0;
+
+    int allocate(uint64_t n, void *stream) {
+        release();
+        const uint64_t nb = blocks_of(n);
+        const uint64_t o_v = align256(n), o_am = o_v + align256(n), o_av = o_am + align256(nb * 4);
+        const uint64_t total = o_av + align256(nb * 4);
+        int dev = 0;
+        int rc = eri_hip_get_device(&dev);
+        if (rc) return rc;
+        rc = eri_hip_malloc_zeroed(dev, total, &base);
+        if (rc) return rc;
+        char *b = static_cast<char *>(base);
+        m = reinterpret_cast<uint8_t *>(b);
+        v = reinterpret_cast<uint8_t *>(b + o_v);
+        absmax_m = reinterpret_cast<float *>(b + o_am);
+        absmax_v = reinterpret_cast<float *>(b + o_av);
+        numel = n;
+        // the state of a zeros tensor (adam8bit_enhanced.rs:179-197)
+        return eri_adam8_state_init(m, v, absmax_m, absmax_v, n, stream);
+    }
+    void release() {
+        if (base) eri_hip_free(base);
+        base = nullptr;
+        m = v = nullptr;
+        absmax_m = absmax_v = nullptr;
+        numel = 0;
+    }
+    uint64_t nbytes() const { return numel ? 2 * numel + 8 * blocks_of(numel) : 0; }
+    ~State8() { release(); }
+    State8() = default;
+    State8(const State8 &) = delete;
+    State8 &operator=(const State8 &) = delete;
+};
+
+// ---- a very small safetensors reader / writer ------------------------------------------------
+
+struct StEntry {
+    std::string dtype;
+    std::vector<uint64_t> shape;
+    uint64_t begin = 0, end = 0;
+};
+
+struct StFile {
+    std::map<std::string, std::string> metadata;
+    std::map<std::string, StEntry> tensors;
+    std::vector<char> data;
+};
+
+struct JsonCursor {
+    const char *p, *e;
+    bool ok = true;
+    void ws() { while (p < e && (*p == ' ' || *p == '\n' || *p == '\t' || *p == '\r')) ++p; }
+    bool eat(char c) {
+        ws();
+        if (p < e && *p == c) { ++p; return true; }
+        ok = false;
+        return false;
+    }
+    bool peek(char c) { ws(); return p < e && *p == c; }
+    std::string str() {
+        std::string out;
+        if (!eat('"')) return out;
+        while (p < e && *p != '"') {
+            if (*p == '\\' && p + 1 < e) { ++p; }
+            out.push_back(*p++);
+        }
+        if (p >= e) { ok = false; return out; }
+        ++p;
+        return out;
+    }
+    uint64_t num() {
+        ws();
+        uint64_t v = 0;
+        bool any = false;
+        while (p < e && *p >= '0' && *p <= '9') { v = v * 10 + (uint64_t)(*p++ - '0'); any = true; }
+        if (!any) ok = false;
+        return v;
+    }
+};
+
+bool parse_safetensors(const std::vector<char> &raw, StFile &out, std::string &why) {
+    if (raw.size() < 8) { why = "file shorter than its header length"; return false; }
+    uint64_t hlen = 0;
+    std::memcpy(&hlen, raw.data(), 8);
+    if (hlen > raw.size() - 8) { why = "header length exceeds the file"; return false; }
+    JsonCursor c{raw.data() + 8, raw.data() + 8 + hlen};
+    if (!c.eat('{')) { why = "header is not a JSON object"; return false; }
+    bool first = true;
+    while (c.ok && !c.peek('}')) {
+        if (!first && !c.eat(',')) break;
+        first = false;
+        const std::string key = c.str();
+        if (!c.eat(':') || !c.eat('{')) break;
+        bool f2 = true;
+        StEntry ent;
+        while (c.ok && !c.peek('}')) {
+            if (!f2 && !c.eat(',')) break;
+            f2 = false;
+            const std::string k2 = c.str();
+            if (!c.eat(':')) break;
+            if (key == "__metadata__") {
+                out.metadata[k2] = c.str();
+            } else if (k2 == "dtype") {
+                ent.dtype = c.str();
+            } else if (k2 == "shape" || k2 == "data_offsets") {
+                std::vector<uint64_t> vals;
+                if (!c.eat('[')) break;
+                while (c.ok && !c.peek(']')) {
+                    if (!vals.empty() && !c.eat(',')) break;
+                    vals.push_back(c.num());
+                }
+                c.eat(']');
+                if (k2 == "shape") ent.shape = vals;
+                else if (vals.size() == 2) { ent.begin = vals[0]; ent.end = vals[1]; }
+                else c.ok = false;
+            } else {
+                c.ok = false;
+            }
+        }
+        c.eat('}');
+        if (key != "__metadata__") out.tensors[key] = ent;
+    }
+    if (!c.ok || !c.eat('}')) { why = "malformed header"; return false; }
+    out.data.assign(raw.begin() + 8 + (std::ptrdiff_t)hlen, raw.end());
+    for (auto &kv : out.tensors)
+        if (kv.second.end < kv.second.begin || kv.second.end > out.data.size()) {
+            why = "tensor '" + kv.first + "' points outside the file";
+            return false;
+        }
+    return true;
+}
+
+struct StWriter {
+    std::ostringstream header;
+    std::vector<std::pair<const void *, uint64_t>> chunks; // host pointers
+    uint64_t offset = 0;
+    bool first = true;
+    void begin(const std::map<std::string, std::string> &meta) {
+        header << "{\"__metadata__\":{";
+        bool f = true;
+        for (auto &kv : meta) {
+            header << (f ? "" : ",") << "\"" << kv.first << "\":\"" << kv.second << "\"";
+            f = false;
+        }
+        header << "}";
+    }
+    void add(const std::string &name, const char *dtype, uint64_t count, const void *host, uint64_t bytes) {
+        header << ",\"" << name << "\":{\"dtype\":\"" << dtype << "\",\"shape\":[" << count << "],\"data_offsets\":["
+               << offset << "," << offset + bytes << "]}";
+        chunks.emplace_back(host, bytes);
+        offset += bytes;
+    }
+    bool write(const std::string &path) {
+        header << "}";
+        std::string h = header.str();
+        while (h.size() % 8) h.push_back(' ');
+        std::ofstream f(path, std::ios::binary | std::ios::trunc);
+        if (!f) return false;
+        const uint64_t hl = h.size();
+        f.write(reinterpret_cast<const char *>(&hl), 8);
+        f.write(h.data(), (std::streamsize)h.size());
+        for (auto &c : chunks) f.write(static_cast<const char *>(c.first), (std::streamsize)c.second);
+        return (bool)f;
+    }
+};
+
+} // namespace
+
+// ---------------------------------------------------------------------------------------------
+// Parameter
+// ---------------------------------------------------------------------------------------------
+
+struct EriParameter {
+    void *data = nullptr;
+    const void *grad = nullptr;
+    uint64_t numel = 0;
+    int32_t dtype = 0;
+    int refs = 1;
+};
+
+// ---------------------------------------------------------------------------------------------
+// Adam8bit over a parameter list
+// ---------------------------------------------------------------------------------------------
+
+struct EriAdam8bit {
+    std::vector<EriParameter *> params;
+    double lr = 1e-3, beta1 = 0.9, beta2 = 0.999, eps = 1e-8, wd = 0.01;
+    uint64_t step = 0;
+    uint32_t flags = 0;
+    float grad_scale = 1.0f;
+    std::vector<float> param_scale;
+    std::vector<std::unique_ptr<State8>> states; // index = parameter index; null before the first step
+    void *stream = nullptr;
+    EriAdam8Table *table = nullptr;
+    std::vector<uint32_t> table_ids;         // parameter indices the table was built for
+    std::vector<EriAdam8Tensor> table_rows;  // rows as last uploaded
+};
+
+struct EriAdam8bitFn {
+    double lr = 1e-4, beta1 = 0.9, beta2 = 0.999, eps = 1e-8, wd = 0.01;
+    uint64_t step = 0;
+    void *stream = nullptr;
+    std::map<std::string, std::unique_ptr<State8>> states;
+};
+
+extern "C" {
+
+int eri_param_create(void *data, uint64_t numel, int dtype_tag, EriParameter **out) {
+    if (!out) return fail(ERI_ERR_NULL, "out is NULL");
+    *out = nullptr;
+    if (!data) return fail(ERI_ERR_NULL, "parameter data is NULL");
+    if (dtype_tag != ERI_DTYPE_F32 && dtype_tag != ERI_DTYPE_BF16)
+        return fail(ERI_ERR_DTYPE, "Unsupported: 8-bit Adam takes F32 or BF16 parameters");
+    EriParameter *p = new EriParameter();
+    p->data = data;
+    p->numel = numel;
+    p->dtype = dtype_tag;
+    *out = p;
+    return 0;
+}
+
+int eri_param_set_grad(EriParameter *param, const void *grad) {
+    if (!param) return fail(ERI_ERR_NULL, "param is NULL");
+    param->grad = grad;
+    return 0;
+}
+
+int eri_param_set_data(EriParameter *param, void *data) {
+    if (!param || !data) return fail(ERI_ERR_NULL, "param or data is NULL");
+    param->data = data;
+    return 0;
+}
+
+int eri_param_retain(EriParameter *param) {
+    if (!param) return fail(ERI_ERR_NULL, "param is NULL");
+    ++param->refs;
+    return 0;
+}
+
+int eri_param_release(EriParameter *param) {
+    if (!param) return 0;
+    if (--param->refs == 0) delete param;
+    return 0;
+}
+
+void eri_adam8bit_config_default(EriAdam8bitConfig *cfg) {
+    if (!cfg) return;
+    cfg->lr = 1e-3;
+    cfg->beta1 = 0.9;
+    cfg->beta2 = 0.999;
+    cfg->eps = 1e-8;
+    cfg->weight_decay = 0.01;
+    cfg->amsgrad = 0;
+    cfg->block_wise = 1;
+    cfg->percentile_clipping = 99;
+}
+
+int eri_adam8bit_new(EriParameter *const *params, uint32_t n, const EriAdam8bitConfig *cfg, void *stream,
+                     EriAdam8bit **out) {
+    if (!out) return fail(ERI_ERR_NULL, "out is NULL");
+    *out = nullptr;
+    if (n && !params) return fail(ERI_ERR_NULL, "params is NULL");
+    EriAdam8bitConfig c;
+    eri_adam8bit_config_default(&c);
+    if (cfg) c = *cfg;
+    for (uint32_t i = 0; i < n; ++i)
+        if (!params[i]) return fail(ERI_ERR_NULL, "a parameter handle is NULL");
+    EriAdam8bit *o = new EriAdam8bit();
+    o->lr = c.lr;
+    o->beta1 = c.beta1;
+    o->beta2 = c.beta2;
+    o->eps = c.eps;
+    o->wd = c.weight_decay;
+    o->stream = stream;
+    o->params.assign(params, params + n);
+    for (auto *p : o->params) ++p->refs; // the optimizer holds clones of the handles (:222-223)
+    o->states.resize(n);
+    o->param_scale.assign(n, 1.0f);
+    *out = o;
+    return 0;
+}
+
+int eri_adam8bit_destroy(EriAdam8bit *o) {
+    if (!o) return 0;
+    if (o->table) eri_adam8_table_destroy(o->table);
+    for (auto *p : o->params) eri_param_release(p);
+    delete o;
+    return 0;
+}
+
+int eri_adam8bit_step(EriAdam8bit *o, uint32_t *skipped) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    o->step += 1; // :203
+    uint32_t skip = 0;
+    std::vector<uint32_t> ids;
+    std::vector<EriAdam8Tensor> rows;
+    uint64_t start = 0;
+    bool scaled = o->grad_scale != 1.0f;
+    for (uint32_t i = 0; i < o->params.size(); ++i) {
+        EriParameter *p = o->params[i];
+        if (!p->grad) { // :237-240
+            std::fprintf(stderr, "Warning: No gradient for param_%u\n", i);
+            ++skip;
+            continue;
+        }
+        if (p->numel == 0) return fail(ERI_ERR_EMPTY, "InvalidOperation: Empty tensor for quantization");
+        if (!o->states[i]) { // init_state :179-199
+            std::unique_ptr<State8> s(new State8());
+            int rc = s->allocate(p->numel, o->stream);
+            if (rc) return rc;
+            o->states[i] = std::move(s);
+        }
+        State8 &s = *o->states[i];
+        EriAdam8Tensor r;
+        std::memset(&r, 0, sizeof r);
+        r.p = p->data;
+        r.g = p->grad;
+        r.m = s.m;
+        r.v = s.v;
+        r.absmax_m = s.absmax_m;
+        r.absmax_v = s.absmax_v;
+        r.numel = p->numel;
+        r.block_start = start;
+        r.dtype_tag = p->dtype;
+        r.grad_scale = o->param_scale[i];
+        scaled = scaled || o->param_scale[i] != 1.0f;
+        start += blocks_of(p->numel);
+        ids.push_back(i);
+        rows.push_back(r);
+    }
+    if (skipped) *skipped = skip;
+    if (rows.empty()) return 0;
+    int rc = 0;
+    if (!o->table || ids != o->table_ids) {
+        if (o->table) eri_adam8_table_destroy(o->table);
+        o->table = nullptr;
+        rc = eri_adam8_table_create(rows.data(), (uint32_t)rows.size(), o->stream, &o->table);
+        if (rc) return rc;
+        o->table_ids = ids;
+        o->table_rows = rows;
+    } else if (std::memcmp(rows.data(), o->table_rows.data(), rows.size() * sizeof(EriAdam8Tensor)) != 0) {
+        rc = eri_adam8_table_update(o->table, rows.data(), (uint32_t)rows.size(), o->stream);
+        if (rc) return rc;
+        o->table_rows = rows;
+    }
+    EriAdam8Hyper h;
+    uint32_t flags = o->flags | (scaled ? (uint32_t)ERI_ADAM8_FLAG_GRAD_SCALE : 0u);
+    rc = eri_adam8_hyper_pack(o->lr, o->beta1, o->beta2, o->eps, o->wd, o->step, ERI_ADAM8_MODE_ERI, flags, &h);
+    if (rc) return rc;
+    h.grad_scale = o->grad_scale;
+    return eri_adam8_step_table(o->table, &h, o->stream);
+}
+
+int eri_adam8bit_zero_grad(EriAdam8bit *o) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    for (auto *p : o->params) p->grad = nullptr;
+    return 0;
+}
+
+double eri_adam8bit_current_lr(const EriAdam8bit *o) { return o ? o->lr : 0.0; }
+
+int eri_adam8bit_set_learning_rate(EriAdam8bit *o, double lr) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    o->lr = lr;
+    return 0;
+}
+
+uint64_t eri_adam8bit_quantized_memory_usage(const EriAdam8bit *o) {
+    uint64_t total = 0;
+    if (o)
+        for (auto &s : o->states)
+            if (s) total += s->nbytes();
+    return total;
+}
+
+uint64_t eri_adam8bit_get_step(const EriAdam8bit *o) { return o ? o->step : 0; }
+
+int eri_adam8bit_set_grad_scale(EriAdam8bit *o, float scale) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    o->grad_scale = scale;
+    return 0;
+}
+
+int eri_adam8bit_set_param_grad_scale(EriAdam8bit *o, uint32_t index, float scale) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    if (index >= o->param_scale.size()) return fail(ERI_ERR_ARG, "parameter index out of range");
+    o->param_scale[index] = scale;
+    return 0;
+}
+
+int eri_adam8bit_set_flags(EriAdam8bit *o, uint32_t flags) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    o->flags = flags;
+    return 0;
+}
+
+int eri_adam8bit_state_ptrs(const EriAdam8bit *o, uint32_t index, uint8_t **m, uint8_t **v, float **absmax_m,
+                            float **absmax_v) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    if (index >= o->states.size()) return fail(ERI_ERR_ARG, "parameter index out of range");
+    const State8 *s = o->states[index].get();
+    if (m) *m = s ? s->m : nullptr;
+    if (v) *v = s ? s->v : nullptr;
+    if (absmax_m) *absmax_m = s ? s->absmax_m : nullptr;
+    if (absmax_v) *absmax_v = s ? s->absmax_v : nullptr;
+    return 0;
+}
+
+int eri_adam8bit_save_state(EriAdam8bit *o, const char *path) {
+    if (!o || !path) return fail(ERI_ERR_NULL, "optimizer or path is NULL");
+    // stage every state to host memory, then write one safetensors file
+    std::vector<std::vector<char>> host;
+    StWriter w;
+    char buf[64];
+    std::map<std::string, std::string> meta;
+    meta["format"] = "eri-adam8bit-blockwise-v1";
+    meta["block_size"] = "2048";
+    std::snprintf(buf, sizeof buf, "%llu", (unsigned long long)o->step);
+    meta["step"] = buf;
+    std::snprintf(buf, sizeof buf, "%.17g", o->lr);
+    meta["learning_rate"] = buf;
+    w.begin(meta);
+    for (uint32_t i = 0; i < o->states.size(); ++i) {
+        const State8 *s = o->states[i].get();
+        if (!s) continue;
+        const uint64_t nb = blocks_of(s->numel);
+        const uint64_t sizes[4] = {s->numel, s->numel, nb * 4, nb * 4};
+        const void *src[4] = {s->m, s->v, s->absmax_m, s->absmax_v};
+        for (int k = 0; k < 4; ++k) {
+            host.emplace_back(sizes[k]);
+            int rc = eri_hip_memcpy_async(host.back().data(), src[k], sizes[k], 2, o->stream);
+            if (rc) return rc;
+        }
+    }
+    int rc = eri_hip_stream_sync(o->stream);
+    if (rc) return rc;
+    size_t h = 0;
+    for (uint32_t i = 0; i < o->states.size(); ++i) {
+        const State8 *s = o->states[i].get();
+        if (!s) continue;
+        const uint64_t nb = blocks_of(s->numel);
+        const std::string base = "optimizer.param_" + std::to_string(i);
+        w.add(base + ".m", "U8", s->numel, host[h].data(), s->numel);
+        w.add(base + ".v", "U8", s->numel, host[h + 1].data(), s->numel);
+        w.add(base + ".absmax_m", "F32", nb, host[h + 2].data(), nb * 4);
+        w.add(base + ".absmax_v", "F32", nb, host[h + 3].data(), nb * 4);
+        h += 4;
+    }
+    if (!w.write(path)) return fail(ERI_ERR_ARG, std::string("InvalidOperation: Failed to save optimizer: cannot write ") + path);
+    return 0;
+}
+
+int eri_adam8bit_load_state(EriAdam8bit *o, const char *path) {
+    if (!o || !path) return fail(ERI_ERR_NULL, "optimizer or path is NULL");
+    std::ifstream f(path, std::ios::binary);
+    if (!f) return fail(ERI_ERR_ARG, std::string("InvalidOperation: Failed to read optimizer: cannot open ") + path);
+    std::vector<char> raw((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+    StFile st;
+    std::string why;
+    if (!parse_safetensors(raw, st, why))
+        return fail(ERI_ERR_ARG, "InvalidOperation: Failed to deserialize optimizer: " + why);
+    if (!st.metadata.count("step") || !st.metadata.count("learning_rate"))
+        return fail(ERI_ERR_ARG, "InvalidOperation: Failed to deserialize optimizer: step / learning_rate missing");
+    // validate everything before touching the optimizer
+    struct Item { uint32_t idx; const StEntry *e[4]; };
+    std::vector<Item> items;
+    for (uint32_t i = 0; i < o->params.size(); ++i) {
+        const std::string base = "optimizer.param_" + std::to_string(i);
+        auto m = st.tensors.find(base + ".m");
+        if (m == st.tensors.end()) continue;
+        auto v = st.tensors.find(base + ".v"), am = st.tensors.find(base + ".absmax_m"), av = st.tensors.find(base + ".absmax_v");
+        if (v == st.tensors.end() || am == st.tensors.end() || av == st.tensors.end())
+            return fail(ERI_ERR_ARG, "InvalidOperation: Failed to deserialize optimizer: incomplete state for " + base);
+        const uint64_t n = o->params[i]->numel, nb = blocks_of(n);
+        const StEntry *e[4] = {&m->second, &v->second, &am->second, &av->second};
+        const uint64_t want[4] = {n, n, nb * 4, nb * 4};
+        const char *dt[4] = {"U8", "U8", "F32", "F32"};
+        for (int k = 0; k < 4; ++k)
+            if (e[k]->end - e[k]->begin != want[k] || e[k]->dtype != dt[k])
+                return fail(ERI_ERR_ARG, "InvalidOperation: Failed to deserialize optimizer: size or dtype mismatch for " + base);
+        items.push_back({i, {e[0], e[1], e[2], e[3]}});
+    }
+    for (auto &it : items) {
+        EriParameter *p = o->params[it.idx];
+        std::unique_ptr<State8> s(new State8());
+        int rc = s->allocate(p->numel, o->stream);
+        if (rc) return rc;
+        void *dst[4] = {s->m, s->v, s->absmax_m, s->absmax_v};
+        for (int k = 0; k < 4; ++k) {
+            rc = eri_hip_memcpy_async(dst[k], st.data.data() + it.e[k]->begin, it.e[k]->end - it.e[k]->begin, 1, o->stream);
+            if (rc) return rc;
+        }
+        rc = eri_hip_stream_sync(o->stream); // st.data is pageable and goes out of scope with this call
+        if (rc) return rc;
+        o->states[it.idx] = std::move(s);
+    }
+    o->step = std::strtoull(st.metadata["step"].c_str(), nullptr, 10);
+    o->lr = std::strtod(st.metadata["learning_rate"].c_str(), nullptr);
+    if (o->table) { // state pointers changed
+        eri_adam8_table_destroy(o->table);
+        o->table = nullptr;
+        o->table_ids.clear();
+    }
+    return 0;
+}
+
+// ---- functional flavour ------------------------------------------------------------------------
+
+int eri_adam8bit_fn_with_params(double lr, double beta1, double beta2, double eps, double weight_decay, void *stream,
+                                EriAdam8bitFn **out) {
+    if (!out) return fail(ERI_ERR_NULL, "out is NULL");
+    EriAdam8bitFn *o = new EriAdam8bitFn();
+    o->lr = lr;
+    o->beta1 = beta1;
+    o->beta2 = beta2;
+    o->eps = eps;
+    o->wd = weight_decay;
+    o->stream = stream;
+    *out = o;
+    return 0;
+}
+
+int eri_adam8bit_fn_destroy(EriAdam8bitFn *o) {
+    delete o;
+    return 0;
+}
+
+int eri_adam8bit_fn_update(EriAdam8bitFn *o, const char *name, const void *param, const void *grad, uint64_t numel,
+                           int dtype_tag, void *out) {
+    if (!o || !name || !param || !grad || !out) return fail(ERI_ERR_NULL, "update with NULL argument");
+    if (numel == 0) return fail(ERI_ERR_EMPTY, "InvalidOperation: Empty tensor for quantization");
+    if (dtype_tag != ERI_DTYPE_F32 && dtype_tag != ERI_DTYPE_BF16)
+        return fail(ERI_ERR_DTYPE, "Unsupported: 8-bit Adam takes F32 or BF16 parameters");
+    auto it = o->states.find(name);
+    if (it == o->states.end()) { // adam8bit.rs:126-130
+        std::unique_ptr<State8> s(new State8());
+        int rc = s->allocate(numel, o->stream);
+        if (rc) return rc;
+        it = o->states.emplace(name, std::move(s)).first;
+    } else if (it->second->numel != numel) {
+        return fail(ERI_ERR_ARG, std::string("state of '") + name + "' has a different size");
+    }
+    int rc = 0;
+    if (out != param) {
+        rc = eri_hip_memcpy_async(out, param, numel * (dtype_tag == ERI_DTYPE_F32 ? 4 : 2), 3, o->stream);
+        if (rc) return rc;
+    }
+    State8 &s = *it->second;
+    EriAdam8Tensor r;
+    std::memset(&r, 0, sizeof r);
+    r.p = out;
+    r.g = grad;
+    r.m = s.m;
+    r.v = s.v;
+    r.absmax_m = s.absmax_m;
+    r.absmax_v = s.absmax_v;
+    r.numel = numel;
+    r.block_start = 0;
+    r.dtype_tag = dtype_tag;
+    r.grad_scale = 1.0f;
+    EriAdam8Hyper h;
+    // the bias correction uses the counter as it stands; step() bumps it later (:107,:164)
+    rc = eri_adam8_hyper_pack(o->lr, o->beta1, o->beta2, o->eps, o->wd, o->step, ERI_ADAM8_MODE_L2,
+                              ERI_ADAM8_FLAG_EXACT_PARAM, &h);
+    if (rc) return rc;
+    return eri_adam8_step_multi(&r, 1, &h, o->stream);
+}
+
+int eri_adam8bit_fn_step(EriAdam8bitFn *o) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    o->step += 1;
+    return 0;
+}
+
+int eri_adam8bit_fn_set_lr(EriAdam8bitFn *o, float lr) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    o->lr = (double)lr; // `lr as f64`, adam8bit.rs:96
+    return 0;
+}
+
+uint64_t eri_adam8bit_fn_get_step(const EriAdam8bitFn *o) { return o ? o->step : 0; }
+
+int eri_adam8bit_fn_memory_stats(const EriAdam8bitFn *o, uint64_t *num_params, uint64_t *bytes) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    uint64_t b = 0;
+    for (auto &kv : o->states) b += kv.second->nbytes();
+    if (num_params) *num_params = o->states.size();
+    if (bytes) *bytes = b;
+    return 0;
+}
+
+int eri_adam8bit_fn_state_numel(const EriAdam8bitFn *o, const char *name, uint64_t *numel) {
+    if (!o || !name || !numel) return fail(ERI_ERR_NULL, "NULL argument");
+    auto it = o->states.find(name);
+    *numel = it == o->states.end() ? 0 : it->second->numel;
+    return 0;
+}
+
+int eri_adam8bit_fn_get_state_fp32(EriAdam8bitFn *o, const char *name, float *m_out, float *v_out) {
+    if (!o || !name || !m_out || !v_out) return fail(ERI_ERR_NULL, "NULL argument");
+    auto it = o->states.find(name);
+    if (it == o->states.end()) return fail(ERI_ERR_ARG, std::string("no optimizer state named '") + name + "'");
+    State8 &s = *it->second;
+    int rc = eri_adam8_dequantize(s.m, s.absmax_m, 1, s.numel, m_out, o->stream);
+    if (rc) return rc;
+    return eri_adam8_dequantize(s.v, s.absmax_v, 0, s.numel, v_out, o->stream);
+}
+
+int eri_adam8bit_fn_load_state_fp32(EriAdam8bitFn *o, const char *name, const float *m, const float *v,
+                                    uint64_t numel) {
+    if (!o || !name || !m || !v) return fail(ERI_ERR_NULL, "NULL argument");
+    if (numel == 0) return fail(ERI_ERR_EMPTY, "InvalidOperation: Empty tensor for quantization");
+    std::unique_ptr<State8> s(new State8());
+    int rc = s->allocate(numel, o->stream);
+    if (rc) return rc;
+    rc = eri_adam8_quantize(m, 1, numel, s->m, s->absmax_m, o->stream);
+    if (rc) return rc;
+    rc = eri_adam8_quantize(v, 0, numel, s->v, s->absmax_v, o->stream);
+    if (rc) return rc;
+    o->states[name] = std::move(s);
+    return 0;
+}
+
+} // extern "C"

@@ -350,6 +350,8 @@ extern "C" {
 
 const char *eri_last_error(void) { return g_err.c_str(); }
 
+void eri_set_last_error(const char *message) { g_err = message ? message : ""; }
+
 // ---- storage --------------------------------------------------------------------------------
 
 int eri_hip_device_count(int *count) {
@@ -360,6 +362,12 @@ int eri_hip_device_count(int *count) {
 
 int eri_hip_set_device(int device) {
     ERI_HIP(hipSetDevice(device));
+    return 0;
+}
+
+int eri_hip_get_device(int *device) {
+    if (!device) return fail(ERI_ERR_NULL, "device is NULL");
+    ERI_HIP(hipGetDevice(device));
     return 0;
 }
 

@@ -1,0 +1,103 @@
+/*
+ * eri_adam8bit -- the optimizer objects of EriDiffusion's 8-bit Adam, as a flat C API over
+ * eri_optim8.h.  It is the host layer a Rust `impl Adam8bit` (or any other binding) forwards to:
+ * it owns the 8-bit states, the step counter and the cached device launch table, and it calls
+ * nothing but the functions declared in eri_optim8.h.
+ *
+ * Two flavours, as in the reference:
+ *   EriAdam8bit    step() over a list of parameters that carry their gradients
+ *                  (src/trainers/adam8bit_enhanced.rs:160-369)
+ *   EriAdam8bitFn  per-tensor update(name, param, grad) keyed by name
+ *                  (src/trainers/adam8bit.rs:49-345)
+ * Return values follow eri_optim8.h: 0, a positive hipError_t, or a negative EriStatus;
+ * eri_last_error() holds the message.  Optimizer-level failures use the reference's wording
+ * ("Empty tensor for quantization", "Failed to read optimizer: ...", "Failed to deserialize
+ * optimizer: ...", adam8bit_enhanced.rs:46-50,351-357).
+ */
+#ifndef ERI_ADAM8BIT_H
+#define ERI_ADAM8BIT_H
+
+#include "eri_optim8.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- Parameter: a shared handle to a device tensor and its current gradient ------------------
+ * Stands where flame_core::Parameter stands in the reference (tensor(), grad(), apply_update()):
+ * the trainer and the optimizer hold the same handle, the optimizer updates the tensor in place.
+ * The handle never owns the device memory it points to (crates/core/tests/wrap_external.rs:25-30). */
+typedef struct EriParameter EriParameter;
+int eri_param_create(void *data, uint64_t numel, int dtype_tag, EriParameter **out);
+int eri_param_set_grad(EriParameter *param, const void *grad); /* NULL = no gradient this step */
+int eri_param_set_data(EriParameter *param, void *data);       /* Parameter::set_data */
+int eri_param_retain(EriParameter *param);                     /* Parameter::clone */
+int eri_param_release(EriParameter *param);
+
+/* ---- Adam8bitConfig (adam8bit_enhanced.rs:372-395) ------------------------------------------- */
+typedef struct EriAdam8bitConfig {
+    double lr;                    /* 1e-3 */
+    double beta1, beta2;          /* 0.9, 0.999 */
+    double eps;                   /* 1e-8 */
+    double weight_decay;          /* 0.01 */
+    int32_t amsgrad;              /* false; carried, not used (the reference never reads it) */
+    int32_t block_wise;           /* true; the state format here is always block-wise */
+    uint64_t percentile_clipping; /* 99; carried, the block-wise format does not clip */
+} EriAdam8bitConfig;
+void eri_adam8bit_config_default(EriAdam8bitConfig *cfg);
+
+/* ---- Adam8bit: step() over a parameter list --------------------------------------------------- */
+typedef struct EriAdam8bit EriAdam8bit;
+/* Adam8bit::new(params, config) :161.  `stream` (NULL = default) is used by every later call. */
+int eri_adam8bit_new(EriParameter *const *params, uint32_t n, const EriAdam8bitConfig *cfg, void *stream,
+                     EriAdam8bit **out);
+int eri_adam8bit_destroy(EriAdam8bit *opt);
+/* step() :202-291.  Parameters without a gradient are skipped ("Warning: No gradient for
+ * param_N" on stderr, :237-240); `skipped`, if not NULL, receives how many. */
+int eri_adam8bit_step(EriAdam8bit *opt, uint32_t *skipped);
+int eri_adam8bit_zero_grad(EriAdam8bit *opt);                               /* :294 */
+double eri_adam8bit_current_lr(const EriAdam8bit *opt);                     /* :302 */
+int eri_adam8bit_set_learning_rate(EriAdam8bit *opt, double lr);            /* :307 */
+uint64_t eri_adam8bit_quantized_memory_usage(const EriAdam8bit *opt);       /* :312 */
+uint64_t eri_adam8bit_get_step(const EriAdam8bit *opt);
+/* Extras the trainers apply around the step, folded into it here:
+ * a global clip factor (pipeline_flux_lora_sequential.rs:1198-1213) and a per-parameter gradient
+ * multiplier (:759-766).  1.0 switches either off. */
+int eri_adam8bit_set_grad_scale(EriAdam8bit *opt, float scale);
+int eri_adam8bit_set_param_grad_scale(EriAdam8bit *opt, uint32_t index, float scale);
+int eri_adam8bit_set_flags(EriAdam8bit *opt, uint32_t flags); /* ERI_ADAM8_FLAG_EXACT_PARAM etc. */
+/* save_state / load_state :330-368.  The file is a safetensors container with, per parameter that
+ * has state, `optimizer.param_N.m` / `.v` (U8 codes) and `.absmax_m` / `.absmax_v` (F32), and the
+ * step counter and learning rate in its metadata. */
+int eri_adam8bit_save_state(EriAdam8bit *opt, const char *path);
+int eri_adam8bit_load_state(EriAdam8bit *opt, const char *path);
+/* Device pointers of one parameter's state (NULL before its first step). */
+int eri_adam8bit_state_ptrs(const EriAdam8bit *opt, uint32_t index, uint8_t **m, uint8_t **v, float **absmax_m,
+                            float **absmax_v);
+
+/* ---- functional flavour ------------------------------------------------------------------------ */
+typedef struct EriAdam8bitFn EriAdam8bitFn;
+/* Adam8bit::with_params(lr, beta1, beta2, eps, wd), adam8bit.rs:69-86 */
+int eri_adam8bit_fn_with_params(double lr, double beta1, double beta2, double eps, double weight_decay, void *stream,
+                                EriAdam8bitFn **out);
+int eri_adam8bit_fn_destroy(EriAdam8bitFn *opt);
+/* update(name, param, grad) -> new tensor, :101-208.  `param` is left untouched, the new values are
+ * written to `out` (numel elements of the same dtype; it may alias `param`). */
+int eri_adam8bit_fn_update(EriAdam8bitFn *opt, const char *name, const void *param, const void *grad, uint64_t numel,
+                           int dtype_tag, void *out);
+int eri_adam8bit_fn_step(EriAdam8bitFn *opt);                   /* :89-92, only bumps the counter */
+int eri_adam8bit_fn_set_lr(EriAdam8bitFn *opt, float lr);       /* :95-98 */
+uint64_t eri_adam8bit_fn_get_step(const EriAdam8bitFn *opt);    /* :311-313 */
+/* memory_stats() :253-266: number of named states and their bytes */
+int eri_adam8bit_fn_memory_stats(const EriAdam8bitFn *opt, uint64_t *num_params, uint64_t *bytes);
+/* get_state_as_tensors / load_state_from_tensors :296-329, one name at a time: fp32 moments.
+ * `numel` of an unknown name reads 0. */
+int eri_adam8bit_fn_state_numel(const EriAdam8bitFn *opt, const char *name, uint64_t *numel);
+int eri_adam8bit_fn_get_state_fp32(EriAdam8bitFn *opt, const char *name, float *m_out, float *v_out);
+int eri_adam8bit_fn_load_state_fp32(EriAdam8bitFn *opt, const char *name, const float *m, const float *v,
+                                    uint64_t numel);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ERI_ADAM8BIT_H */

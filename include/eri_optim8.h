@@ -46,6 +46,8 @@ typedef enum EriStatus {
 
 /* Message for the last failing call on this thread ("" if none).  Never NULL. */
 const char *eri_last_error(void);
+/* Lets a layer built on this ABI (include/eri_adam8bit.h, a language binding) leave its own message. */
+void eri_set_last_error(const char *message);
 
 /* ---------------------------------------------------------------------------------------------
  * Device storage.  Replaces the cudarc-backed seam of the reference:
@@ -58,6 +60,7 @@ const char *eri_last_error(void);
  * ------------------------------------------------------------------------------------------- */
 int eri_hip_device_count(int *count);
 int eri_hip_set_device(int device);
+int eri_hip_get_device(int *device);
 int eri_hip_malloc_zeroed(int device, size_t bytes, void **out); /* 256-byte aligned, zero-filled */
 int eri_hip_free(void *ptr);
 void *eri_hip_host_alloc(size_t bytes);                          /* pinned; NULL on failure */

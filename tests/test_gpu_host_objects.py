@@ -1,0 +1,203 @@
+"""GPU tests of the optimizer objects (include/eri_adam8bit.h) against the oracle: the list-of-
+parameters step with a skipped parameter and folded gradient scales, save/load of the 8-bit state
+(read back with the safetensors package), and the functional per-tensor flavour."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import harness as hs
+import oracle_c as oc
+
+pytestmark = pytest.mark.gpu
+LR, B1, B2, EPS, WD = 1e-3, 0.9, 0.999, 1e-8, 0.01
+
+
+def _L():
+    from eridiffusion_amd import _lib
+    return _lib
+
+
+def _sync():
+    import torch
+    torch.cuda.synchronize()
+
+
+def _make(sizes, bf16, seed):
+    ps, gs = hs.make_inputs(sizes, bf16, seed)
+    states = hs.oracle_states(sizes)
+    gt = hs.GpuTensors(ps, gs, states, bf16)
+    return ps, gs, states, gt
+
+
+def _new_optimizer(gt, stream=None, flags=2):
+    L = _L()
+    n = len(gt.p)
+    handles = (C.c_void_p * n)()
+    for i in range(n):
+        h = C.c_void_p()
+        L.check(L.lib().eri_param_create(gt.ptr(gt.p[i]), gt.p[i][2], 2 if gt.bf16 else 0, C.byref(h)), "param_create")
+        handles[i] = h
+    cfg = L.Adam8bitConfigC()
+    L.lib().eri_adam8bit_config_default(C.byref(cfg))
+    opt = C.c_void_p()
+    L.check(L.lib().eri_adam8bit_new(handles, n, C.byref(cfg), stream, C.byref(opt)), "adam8bit_new")
+    L.check(L.lib().eri_adam8bit_set_flags(opt, flags), "set_flags")
+    return opt, handles
+
+
+def _fetch_states(opt, gt):
+    import torch
+    L = _L()
+    out = []
+    for i in range(len(gt.p)):
+        ptrs = [C.c_void_p() for _ in range(4)]
+        L.check(L.lib().eri_adam8bit_state_ptrs(opt, i, *[C.byref(p) for p in ptrs]), "state_ptrs")
+        if not ptrs[0].value:
+            out.append(None)
+            continue
+        n = gt.p[i][2]
+        nb = (n + 2047) // 2048
+        arrs = []
+        for p, (cnt, dt) in zip(ptrs, ((n, np.uint8), (n, np.uint8), (nb, np.float32), (nb, np.float32))):
+            host = np.empty(cnt, dt)
+            L.check(L.lib().eri_hip_memcpy_async(host.ctypes.data, p.value, host.nbytes, 2, None), "d2h")
+            L.check(L.lib().eri_hip_stream_sync(None), "sync")
+            arrs.append(host)
+        out.append(arrs)
+    return out
+
+
+@pytest.mark.parametrize("bf16", [True, False])
+def test_step_over_parameter_list_with_a_missing_gradient(bf16, capfd):
+    L = _L()
+    sizes = [2048 * 3 + 11, 777, 2048 * 2, 5000]
+    ps, gs, states, gt = _make(sizes, bf16, 41 + bf16)
+    opt, handles = _new_optimizer(gt)
+    live = [0, 2, 3]  # parameter 1 never gets a gradient
+    for t in (1, 2, 3):
+        g_t = hs.fresh_grads(sizes, bf16, 900 + t)
+        gt.set_grads(g_t)
+        for i in range(4):
+            L.check(L.lib().eri_param_set_grad(handles[i], gt.ptr(gt.g[i]) if i in live else None), "set_grad")
+        skipped = C.c_uint32()
+        L.check(L.lib().eri_adam8bit_step(opt, C.byref(skipped)), "step")
+        assert skipped.value == 1
+        for i in live:
+            hs.oracle_step([ps[i]], [g_t[i]], [states[i]], (LR, B1, B2, EPS, WD, t), bf16)
+    _sync()
+    assert "No gradient for param_1" in capfd.readouterr().err
+    got_p = [gt.down(b) for b in gt.p]
+    got_st = _fetch_states(opt, gt)
+    assert got_st[1] is None  # no state was created for the parameter without gradients
+    assert np.array_equal(got_p[1], ps[1])
+    hs.compare([got_p[i] for i in live], [got_st[i] for i in live], [ps[i] for i in live],
+               [states[i] for i in live], bf16, True, "host-step")
+    want_bytes = sum(2 * sizes[i] + 8 * ((sizes[i] + 2047) // 2048) for i in live)
+    assert L.lib().eri_adam8bit_quantized_memory_usage(opt) == want_bytes
+    assert L.lib().eri_adam8bit_get_step(opt) == 3
+    L.lib().eri_adam8bit_destroy(opt)
+
+
+def test_clip_factor_and_per_parameter_multiplier_are_folded_in():
+    L = _L()
+    sizes = [2048 * 2 + 5, 4096]
+    ps, gs, states, gt = _make(sizes, True, 51)
+    opt, handles = _new_optimizer(gt)
+    L.check(L.lib().eri_adam8bit_set_grad_scale(opt, 0.5), "grad_scale")
+    L.check(L.lib().eri_adam8bit_set_param_grad_scale(opt, 1, 0.25), "param_scale")
+    for i in range(2):
+        L.check(L.lib().eri_param_set_grad(handles[i], gt.ptr(gt.g[i])), "set_grad")
+    L.check(L.lib().eri_adam8bit_step(opt, None), "step")
+    _sync()
+    # the kernel multiplies by hyper.grad_scale * tensor.grad_scale, one product, one multiply
+    for i, s in enumerate((np.float32(0.5) * np.float32(1.0), np.float32(0.5) * np.float32(0.25))):
+        hs.oracle_step([ps[i]], [gs[i]], [states[i]], (LR, B1, B2, EPS, WD, 1), True, grad_scale=float(s))
+    hs.compare([gt.down(b) for b in gt.p], _fetch_states(opt, gt), ps, states, True, True, "host-scales")
+    L.lib().eri_adam8bit_destroy(opt)
+
+
+def test_save_and_load_state_round_trip(tmp_path):
+    from safetensors import safe_open
+    L = _L()
+    sizes = [2048 * 2 + 100, 300, 4096]
+    ps, gs, states, gt = _make(sizes, True, 61)
+    opt, handles = _new_optimizer(gt)
+    for i in range(3):
+        L.check(L.lib().eri_param_set_grad(handles[i], gt.ptr(gt.g[i])), "set_grad")
+    for t in (1, 2):
+        L.check(L.lib().eri_adam8bit_step(opt, None), "step")
+        hs.oracle_step(ps, gs, states, (LR, B1, B2, EPS, WD, t), True)
+    L.check(L.lib().eri_adam8bit_set_learning_rate(opt, 7e-4), "set_lr")
+    path = str(tmp_path / "optimizer.safetensors")
+    L.check(L.lib().eri_adam8bit_save_state(opt, path.encode()), "save_state")
+    with safe_open(path, framework="np") as f:
+        meta = f.metadata()
+        assert meta["step"] == "2" and float(meta["learning_rate"]) == 7e-4 and meta["block_size"] == "2048"
+        for i in range(3):
+            base = "optimizer.param_%d" % i
+            assert np.array_equal(f.get_tensor(base + ".m"), states[i][0])
+            assert np.array_equal(f.get_tensor(base + ".v"), states[i][1])
+            assert np.array_equal(f.get_tensor(base + ".absmax_m").view(np.uint32), states[i][2].view(np.uint32))
+            assert np.array_equal(f.get_tensor(base + ".absmax_v").view(np.uint32), states[i][3].view(np.uint32))
+    # a fresh optimizer over the same parameters resumes from the file and takes the same third step
+    opt2, handles2 = _new_optimizer(gt)
+    L.check(L.lib().eri_adam8bit_load_state(opt2, path.encode()), "load_state")
+    assert L.lib().eri_adam8bit_get_step(opt2) == 2 and L.lib().eri_adam8bit_current_lr(opt2) == 7e-4
+    for i in range(3):
+        L.check(L.lib().eri_param_set_grad(handles2[i], gt.ptr(gt.g[i])), "set_grad")
+    L.check(L.lib().eri_adam8bit_step(opt2, None), "step")
+    _sync()
+    hs.oracle_step(ps, gs, states, (7e-4, B1, B2, EPS, WD, 3), True)
+    hs.compare([gt.down(b) for b in gt.p], _fetch_states(opt2, gt), ps, states, True, True, "resume")
+    L.lib().eri_adam8bit_destroy(opt)
+    L.lib().eri_adam8bit_destroy(opt2)
+
+
+@pytest.mark.parametrize("bf16", [True, False])
+def test_functional_update_returns_a_new_tensor(bf16):
+    import torch
+    L = _L()
+    n = 2048 * 3 + 77
+    ps, gs = hs.make_inputs([n], bf16, 71 + bf16)
+    states = hs.oracle_states([n])
+    dev = torch.device("cuda:0")
+    item = 2 if bf16 else 4
+    p_dev = torch.from_numpy(ps[0].view(np.uint8).copy()).to(dev)
+    out_dev = torch.zeros(n * item, dtype=torch.uint8, device=dev)
+    g_dev = torch.from_numpy(gs[0].view(np.uint8).copy()).to(dev)
+    opt = C.c_void_p()
+    L.check(L.lib().eri_adam8bit_fn_with_params(1e-4, B1, B2, EPS, WD, None, C.byref(opt)), "with_params")
+    p0 = ps[0].copy()
+    for call in range(3):  # update, update, step, update: calls 1 and 2 both see counter 0 -> s = 1
+        src = p_dev if call == 0 else out_dev
+        L.check(L.lib().eri_adam8bit_fn_update(opt, b"layer.lora_down", src.data_ptr(), g_dev.data_ptr(), n,
+                                               2 if bf16 else 0, out_dev.data_ptr()), "fn_update")
+        step = 0 if call < 2 else 1
+        hs.oracle_step(ps, gs, states, (1e-4, B1, B2, EPS, WD, step), bf16, mode=oc.MODE_L2)
+        if call == 1:
+            L.check(L.lib().eri_adam8bit_fn_step(opt), "fn_step")
+    _sync()
+    dt = np.uint16 if bf16 else np.float32
+    assert np.array_equal(p_dev.cpu().numpy().view(dt), p0)  # the input tensor is left alone
+    got = out_dev.cpu().numpy().view(dt)
+    assert np.array_equal(got.view(np.uint16 if bf16 else np.uint32), ps[0].view(np.uint16 if bf16 else np.uint32))
+    # fp32 export equals the oracle's dequantisation; re-import quantises to the same codes
+    m_out = torch.empty(n, dtype=torch.float32, device=dev)
+    v_out = torch.empty(n, dtype=torch.float32, device=dev)
+    L.check(L.lib().eri_adam8bit_fn_get_state_fp32(opt, b"layer.lora_down", m_out.data_ptr(), v_out.data_ptr()), "get")
+    _sync()
+    want_m = np.empty(n, np.float32)
+    want_v = np.empty(n, np.float32)
+    oc.lib().eri_oracle_dequantize(oc.ptr(states[0][0]), oc.ptr(states[0][2]), oc.ptr(hs.MAPS[0]), n, oc.ptr(want_m))
+    oc.lib().eri_oracle_dequantize(oc.ptr(states[0][1]), oc.ptr(states[0][3]), oc.ptr(hs.MAPS[1]), n, oc.ptr(want_v))
+    assert np.array_equal(m_out.cpu().numpy().view(np.uint32), want_m.view(np.uint32))
+    assert np.array_equal(v_out.cpu().numpy().view(np.uint32), want_v.view(np.uint32))
+    cnt, nbytes = C.c_uint64(), C.c_uint64()
+    L.check(L.lib().eri_adam8bit_fn_memory_stats(opt, C.byref(cnt), C.byref(nbytes)), "memory_stats")
+    assert (cnt.value, nbytes.value) == (1, 2 * n + 8 * ((n + 2047) // 2048))
+    L.check(L.lib().eri_adam8bit_fn_load_state_fp32(opt, b"other", m_out.data_ptr(), v_out.data_ptr(), n), "load")
+    numel = C.c_uint64()
+    L.check(L.lib().eri_adam8bit_fn_state_numel(opt, b"other", C.byref(numel)), "numel")
+    assert numel.value == n
+    L.lib().eri_adam8bit_fn_destroy(opt)

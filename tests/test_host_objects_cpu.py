@@ -1,0 +1,98 @@
+"""CPU-only checks of the optimizer objects' host logic (include/eri_adam8bit.h): handles, defaults,
+counters and the error answers that are given before any device is touched."""
+import ctypes as C
+import os
+import struct
+
+import pytest
+
+from eridiffusion_amd import _lib as L
+
+
+def test_config_default_matches_the_reference():
+    # adam8bit_enhanced.rs:383-395
+    c = L.Adam8bitConfigC()
+    L.lib().eri_adam8bit_config_default(C.byref(c))
+    assert (c.lr, c.beta1, c.beta2, c.eps, c.weight_decay) == (1e-3, 0.9, 0.999, 1e-8, 0.01)
+    assert (c.amsgrad, c.block_wise, c.percentile_clipping) == (0, 1, 99)
+
+
+def test_parameter_handle_errors():
+    out = C.c_void_p()
+    assert L.lib().eri_param_create(None, 10, L.DTYPE_BF16, C.byref(out)) == -1
+    assert L.lib().eri_param_create(0x1000, 10, L.DTYPE_F16, C.byref(out)) == -4
+    assert b"F32 or BF16" in L.lib().eri_last_error()
+    assert L.lib().eri_param_create(0x1000, 10, L.DTYPE_BF16, C.byref(out)) == 0
+    assert L.lib().eri_param_retain(out) == 0
+    assert L.lib().eri_param_release(out) == 0
+    assert L.lib().eri_param_release(out) == 0
+
+
+def _optimizer(n_params=2, numel=4096):
+    handles = (C.c_void_p * n_params)()
+    for i in range(n_params):
+        h = C.c_void_p()
+        assert L.lib().eri_param_create(0x10000 * (i + 1), numel, L.DTYPE_BF16, C.byref(h)) == 0
+        handles[i] = h
+    opt = C.c_void_p()
+    assert L.lib().eri_adam8bit_new(handles, n_params, None, None, C.byref(opt)) == 0
+    return opt, handles
+
+
+def test_step_without_gradients_only_counts_and_warns(capfd):
+    opt, handles = _optimizer()
+    skipped = C.c_uint32()
+    assert L.lib().eri_adam8bit_step(opt, C.byref(skipped)) == 0  # nothing to launch: no device needed
+    assert skipped.value == 2
+    assert L.lib().eri_adam8bit_get_step(opt) == 1
+    assert "Warning: No gradient for param_0" in capfd.readouterr().err
+    assert L.lib().eri_adam8bit_quantized_memory_usage(opt) == 0
+    assert L.lib().eri_adam8bit_current_lr(opt) == 1e-3
+    assert L.lib().eri_adam8bit_set_learning_rate(opt, 5e-5) == 0
+    assert L.lib().eri_adam8bit_current_lr(opt) == 5e-5
+    assert L.lib().eri_adam8bit_set_param_grad_scale(opt, 7, 1.0) == -6
+    assert L.lib().eri_adam8bit_zero_grad(opt) == 0
+    L.lib().eri_adam8bit_destroy(opt)
+    for h in handles:
+        L.lib().eri_param_release(h)
+
+
+def test_load_state_rejects_missing_and_corrupt_files(tmp_path):
+    opt, handles = _optimizer()
+    rc = L.lib().eri_adam8bit_load_state(opt, str(tmp_path / "nope.safetensors").encode())
+    assert rc == -6 and b"Failed to read optimizer" in L.lib().eri_last_error()
+    bad = tmp_path / "short.safetensors"
+    bad.write_bytes(b"\x05\x00")
+    rc = L.lib().eri_adam8bit_load_state(opt, str(bad).encode())
+    assert rc == -6 and b"Failed to deserialize optimizer" in L.lib().eri_last_error()
+    bad.write_bytes(struct.pack("<Q", 1 << 40) + b"{}")
+    assert L.lib().eri_adam8bit_load_state(opt, str(bad).encode()) == -6
+    hdr = b'{"__metadata__":{"step":"3"}}'
+    bad.write_bytes(struct.pack("<Q", len(hdr)) + hdr)
+    rc = L.lib().eri_adam8bit_load_state(opt, str(bad).encode())
+    assert rc == -6 and b"learning_rate missing" in L.lib().eri_last_error()
+    hdr = (b'{"__metadata__":{"step":"3","learning_rate":"0.1"},'
+           b'"optimizer.param_0.m":{"dtype":"U8","shape":[4096],"data_offsets":[0,4096]}}')
+    bad.write_bytes(struct.pack("<Q", len(hdr)) + hdr + bytes(4096))
+    rc = L.lib().eri_adam8bit_load_state(opt, str(bad).encode())
+    assert rc == -6 and b"incomplete state" in L.lib().eri_last_error()
+    assert L.lib().eri_adam8bit_get_step(opt) == 0  # a refused file leaves the optimizer untouched
+    L.lib().eri_adam8bit_destroy(opt)
+
+
+def test_functional_flavour_counters_and_errors():
+    opt = C.c_void_p()
+    assert L.lib().eri_adam8bit_fn_with_params(1e-4, 0.9, 0.999, 1e-8, 0.01, None, C.byref(opt)) == 0
+    assert L.lib().eri_adam8bit_fn_get_step(opt) == 0
+    assert L.lib().eri_adam8bit_fn_step(opt) == 0 and L.lib().eri_adam8bit_fn_get_step(opt) == 1
+    assert L.lib().eri_adam8bit_fn_set_lr(opt, 3e-4) == 0
+    n, b = C.c_uint64(5), C.c_uint64(5)
+    assert L.lib().eri_adam8bit_fn_memory_stats(opt, C.byref(n), C.byref(b)) == 0 and (n.value, b.value) == (0, 0)
+    assert L.lib().eri_adam8bit_fn_update(opt, b"w", 0x1000, 0x2000, 0, L.DTYPE_BF16, 0x1000) == -3
+    assert b"Empty tensor for quantization" in L.lib().eri_last_error()
+    assert L.lib().eri_adam8bit_fn_update(opt, b"w", 0x1000, 0x2000, 16, L.DTYPE_I32, 0x1000) == -4
+    assert L.lib().eri_adam8bit_fn_update(opt, None, 0x1000, 0x2000, 16, L.DTYPE_BF16, 0x1000) == -1
+    numel = C.c_uint64(9)
+    assert L.lib().eri_adam8bit_fn_state_numel(opt, b"w", C.byref(numel)) == 0 and numel.value == 0
+    assert L.lib().eri_adam8bit_fn_get_state_fp32(opt, b"w", 0x1000, 0x2000) == -6
+    L.lib().eri_adam8bit_fn_destroy(opt)
