@@ -1,12 +1,12 @@
-"""Python mirror of the reference's 8-bit Adam surface, on top of the C ABI.
+"""Python face of the optimizer objects declared in include/eri_adam8bit.h.
 
 `Adam8bit` keeps the method set of EriDiffusion's list-of-parameters optimizer
 (src/trainers/adam8bit_enhanced.rs:160-369: new / step / zero_grad / current_lr /
-set_learning_rate / quantized_memory_usage), `Adam8bitConfig` its configuration
-(:372-395), and `Adam8bitFunctional` the per-tensor flavour
-(src/trainers/adam8bit.rs:49-345: with_params / update / step / set_lr / get_step /
-get_state_as_tensors / load_state_from_tensors).  torch is used for device memory and the current
-stream only; every update runs in the library's HIP kernel.
+set_learning_rate / quantized_memory_usage / save_state / load_state), `Adam8bitConfig` its
+configuration (:372-395), and `Adam8bitFunctional` the per-tensor flavour
+(src/trainers/adam8bit.rs:49-345: with_params / update / step / set_lr / get_step / memory_stats /
+get_state_as_tensors / load_state_from_tensors).  Every method forwards to the C functions of the
+same name; torch supplies device memory and the current stream, nothing else.
 """
 import ctypes as C
 from dataclasses import dataclass
@@ -14,8 +14,7 @@ from typing import Dict, List, Optional, Tuple
 
 import torch
 
-from . import _lib
-from ._lib import BLOCK, DTYPE_BF16, DTYPE_F32, MODE_ERI, MODE_L2, TensorRow, check, hyper_pack, lib
+from ._lib import DTYPE_BF16, DTYPE_F32, Adam8bitConfigC, check, lib
 
 
 def _dtype_tag(t: torch.Tensor) -> int:
@@ -30,83 +29,9 @@ def _stream_ptr() -> int:
     return torch.cuda.current_stream().cuda_stream
 
 
-class State8:
-    """uint8 codes + per-block absmax of both moments for one tensor."""
-
-    def __init__(self, numel: int, device):
-        nb = (numel + BLOCK - 1) // BLOCK
-        self.m = torch.empty(numel, dtype=torch.uint8, device=device)
-        self.v = torch.empty(numel, dtype=torch.uint8, device=device)
-        self.absmax_m = torch.empty(nb, dtype=torch.float32, device=device)
-        self.absmax_v = torch.empty(nb, dtype=torch.float32, device=device)
-        check(lib().eri_adam8_state_init(self.m.data_ptr(), self.v.data_ptr(), self.absmax_m.data_ptr(),
-                                         self.absmax_v.data_ptr(), numel, _stream_ptr()), "eri_adam8_state_init")
-
-    def nbytes(self) -> int:
-        return self.m.numel() + self.v.numel() + 4 * (self.absmax_m.numel() + self.absmax_v.numel())
-
-
-def build_rows(params, grads, states, grad_scales=None):
-    """ctypes array of launch-table rows for parallel lists of tensors and states."""
-    n = len(params)
-    rows = (TensorRow * n)()
-    start = 0
-    for i, (p, g, s) in enumerate(zip(params, grads, states)):
-        if g.dtype != p.dtype or g.numel() != p.numel():
-            raise ValueError("gradient %d does not match its parameter in dtype or size" % i)
-        if not (p.is_contiguous() and g.is_contiguous()):
-            raise ValueError("parameter/gradient %d is not contiguous" % i)
-        r = rows[i]
-        r.p, r.g = p.data_ptr(), g.data_ptr()
-        r.m, r.v = s.m.data_ptr(), s.v.data_ptr()
-        r.absmax_m, r.absmax_v = s.absmax_m.data_ptr(), s.absmax_v.data_ptr()
-        r.numel = p.numel()
-        r.block_start = start
-        r.dtype_tag = _dtype_tag(p)
-        r.grad_scale = 1.0 if grad_scales is None else float(grad_scales[i])
-        start += (p.numel() + BLOCK - 1) // BLOCK
-    return rows
-
-
-class LaunchTable:
-    """Device-resident launch table (eri_adam8_table_*)."""
-
-    def __init__(self, rows):
-        self.n = len(rows)
-        self._h = C.c_void_p()
-        check(lib().eri_adam8_table_create(rows, self.n, _stream_ptr(), C.byref(self._h)), "eri_adam8_table_create")
-        self._key = bytes(rows)
-
-    def update(self, rows):
-        key = bytes(rows)
-        if key != self._key:
-            check(lib().eri_adam8_table_update(self._h, rows, len(rows), _stream_ptr()), "eri_adam8_table_update")
-            self._key = key
-
-    def step(self, hyper):
-        check(lib().eri_adam8_step_table(self._h, C.byref(hyper), _stream_ptr()), "eri_adam8_step_table")
-
-    def info(self) -> Tuple[int, int]:
-        a, b = C.c_uint64(), C.c_uint64()
-        check(lib().eri_adam8_table_info(self._h, C.byref(a), C.byref(b)), "eri_adam8_table_info")
-        return a.value, b.value
-
-    def close(self):
-        if self._h:
-            lib().eri_adam8_table_destroy(self._h)
-            self._h = C.c_void_p()
-
-    def __del__(self):
-        try:
-            self.close()
-        except Exception:
-            pass
-
-
 @dataclass
 class Adam8bitConfig:
-    """adam8bit_enhanced.rs:372-395.  amsgrad, block_wise and percentile_clipping are carried for
-    interface compatibility; the blockwise format has no clipping and is always block-wise."""
+    """adam8bit_enhanced.rs:372-395; amsgrad, block_wise and percentile_clipping are carried only."""
     lr: float = 1e-3
     betas: Tuple[float, float] = (0.9, 0.999)
     eps: float = 1e-8
@@ -117,141 +42,169 @@ class Adam8bitConfig:
 
 
 class Adam8bit:
-    """`step()` over a list of parameters that carry their gradients (`.grad`)."""
+    """`step()` over a list of tensors that carry their gradients in `.grad`."""
 
     def __init__(self, params: List[torch.Tensor], config: Optional[Adam8bitConfig] = None, flags: int = 0):
         config = config or Adam8bitConfig()
         self.params = list(params)
-        self.learning_rate = float(config.lr)
-        self.beta1, self.beta2 = map(float, config.betas)
-        self.epsilon = float(config.eps)
-        self.weight_decay = float(config.weight_decay)
-        self.step_count = 0
-        self.flags = flags
-        self.grad_scale = None  # set to a float to fold a clip factor into the step
-        self._states: Dict[int, State8] = {}
-        self._table: Optional[LaunchTable] = None
-        self._table_ids: Optional[Tuple[int, ...]] = None
-        lib()  # fail now, not at the first step, if the HIP library is missing
+        for p in self.params:
+            if not p.is_contiguous():
+                raise ValueError("parameters must be contiguous")
+        self._handles = (C.c_void_p * len(self.params))()
+        for i, p in enumerate(self.params):
+            h = C.c_void_p()
+            check(lib().eri_param_create(p.data_ptr(), p.numel(), _dtype_tag(p), C.byref(h)), "eri_param_create")
+            self._handles[i] = h
+        cfg = Adam8bitConfigC(config.lr, config.betas[0], config.betas[1], config.eps, config.weight_decay,
+                              int(config.amsgrad), int(config.block_wise), config.percentile_clipping)
+        self._opt = C.c_void_p()
+        check(lib().eri_adam8bit_new(self._handles, len(self.params), C.byref(cfg), _stream_ptr(),
+                                     C.byref(self._opt)), "eri_adam8bit_new")
+        if flags:
+            check(lib().eri_adam8bit_set_flags(self._opt, flags), "eri_adam8bit_set_flags")
+        self._live = []
 
-    def step(self) -> None:
-        """adam8bit_enhanced.rs:202-291; parameters without a gradient are skipped with a warning."""
-        self.step_count += 1
-        idx, ps, gs = [], [], []
+    def step(self) -> int:
+        """One optimizer step; returns how many parameters were skipped for lack of a gradient."""
+        live = []
         for i, p in enumerate(self.params):
             g = p.grad
-            if g is None:
-                print("Warning: No gradient for param_%d" % i)
-                continue
-            if p.numel() == 0:
-                raise RuntimeError("InvalidOperation: Empty tensor for quantization")
-            if i not in self._states:
-                self._states[i] = State8(p.numel(), p.device)
-            idx.append(i)
-            ps.append(p.data)
-            gs.append(g if g.dtype == p.dtype else g.to(p.dtype))
-        if not idx:
-            return
-        rows = build_rows(ps, gs, [self._states[i] for i in idx])
-        ids = tuple(idx)
-        if self._table is None or self._table_ids != ids:
-            if self._table is not None:
-                self._table.close()
-            self._table = LaunchTable(rows)
-            self._table_ids = ids
-        else:
-            self._table.update(rows)
-        self._live = gs  # keep cast gradients alive until the stream has consumed them
-        h = hyper_pack(self.learning_rate, self.beta1, self.beta2, self.epsilon, self.weight_decay,
-                       self.step_count, MODE_ERI, self.flags, self.grad_scale)
-        self._table.step(h)
+            if g is not None:
+                if g.dtype != p.dtype:
+                    g = g.to(p.dtype)
+                g = g.contiguous()
+                live.append(g)
+            check(lib().eri_param_set_data(self._handles[i], p.data_ptr()), "eri_param_set_data")
+            check(lib().eri_param_set_grad(self._handles[i], g.data_ptr() if g is not None else None),
+                  "eri_param_set_grad")
+        self._live = live  # cast gradients must outlive the launch
+        skipped = C.c_uint32()
+        check(lib().eri_adam8bit_step(self._opt, C.byref(skipped)), "eri_adam8bit_step")
+        return skipped.value
 
     def zero_grad(self) -> None:
+        check(lib().eri_adam8bit_zero_grad(self._opt), "eri_adam8bit_zero_grad")
         for p in self.params:
             p.grad = None
 
     def current_lr(self) -> float:
-        return self.learning_rate
+        return lib().eri_adam8bit_current_lr(self._opt)
 
     def set_learning_rate(self, lr: float) -> None:
-        self.learning_rate = float(lr)
+        check(lib().eri_adam8bit_set_learning_rate(self._opt, lr), "eri_adam8bit_set_learning_rate")
+
+    def set_grad_scale(self, scale: float) -> None:
+        check(lib().eri_adam8bit_set_grad_scale(self._opt, scale), "eri_adam8bit_set_grad_scale")
 
     def quantized_memory_usage(self) -> int:
-        return sum(s.nbytes() for s in self._states.values())
+        return lib().eri_adam8bit_quantized_memory_usage(self._opt)
 
-    def state(self, index: int) -> State8:
-        return self._states[index]
+    def get_step(self) -> int:
+        return lib().eri_adam8bit_get_step(self._opt)
+
+    def save_state(self, path: str) -> None:
+        check(lib().eri_adam8bit_save_state(self._opt, str(path).encode()), "eri_adam8bit_save_state")
+
+    def load_state(self, path: str) -> None:
+        check(lib().eri_adam8bit_load_state(self._opt, str(path).encode()), "eri_adam8bit_load_state")
+
+    def close(self) -> None:
+        if self._opt:
+            lib().eri_adam8bit_destroy(self._opt)
+            self._opt = C.c_void_p()
+            for h in self._handles:
+                lib().eri_param_release(h)
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 class Adam8bitFunctional:
-    """Per-tensor flavour keyed by name (adam8bit.rs): update() returns the new parameter tensor,
-    step() only bumps the counter."""
+    """Per-tensor flavour keyed by name: update() returns the new parameter tensor, step() only
+    bumps the counter (adam8bit.rs:89-92,101-208)."""
 
-    def __init__(self, learning_rate=1e-4, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.01, flags=0):
-        self.learning_rate, self.beta1, self.beta2 = float(learning_rate), float(beta1), float(beta2)
-        self.eps, self.weight_decay = float(eps), float(weight_decay)
-        self.step_count = 0
-        self.flags = flags
-        self._states: Dict[str, State8] = {}
-        lib()
+    def __init__(self, learning_rate=1e-4, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.01):
+        self._opt = C.c_void_p()
+        check(lib().eri_adam8bit_fn_with_params(learning_rate, beta1, beta2, eps, weight_decay, _stream_ptr(),
+                                                C.byref(self._opt)), "eri_adam8bit_fn_with_params")
+        self._names: List[str] = []
 
     @classmethod
     def with_params(cls, learning_rate, beta1, beta2, eps, weight_decay):
         return cls(learning_rate, beta1, beta2, eps, weight_decay)
 
     def step(self) -> None:
-        self.step_count += 1
+        check(lib().eri_adam8bit_fn_step(self._opt), "eri_adam8bit_fn_step")
 
     def set_lr(self, lr: float) -> None:
-        self.learning_rate = float(lr)
+        check(lib().eri_adam8bit_fn_set_lr(self._opt, lr), "eri_adam8bit_fn_set_lr")
 
     def get_step(self) -> int:
-        return self.step_count
+        return lib().eri_adam8bit_fn_get_step(self._opt)
 
     def update(self, name: str, param: torch.Tensor, grad: torch.Tensor) -> torch.Tensor:
-        if param.numel() == 0:
-            raise RuntimeError("InvalidOperation: Empty tensor for quantization")
-        new = param.detach().clone()
-        g = grad if grad.dtype == param.dtype else grad.to(param.dtype)
-        if name not in self._states:
-            self._states[name] = State8(param.numel(), param.device)
-        rows = build_rows([new], [g.contiguous()], [self._states[name]])
-        h = hyper_pack(self.learning_rate, self.beta1, self.beta2, self.eps, self.weight_decay,
-                       self.step_count, MODE_L2, self.flags)
-        check(lib().eri_adam8_step_multi(rows, 1, C.byref(h), _stream_ptr()), "eri_adam8_step_multi")
-        return new
+        p = param.detach().contiguous()
+        g = (grad if grad.dtype == p.dtype else grad.to(p.dtype)).contiguous()
+        out = torch.empty_like(p)
+        check(lib().eri_adam8bit_fn_update(self._opt, name.encode(), p.data_ptr(), g.data_ptr(), p.numel(),
+                                           _dtype_tag(p), out.data_ptr()), "eri_adam8bit_fn_update")
+        if name not in self._names:
+            self._names.append(name)
+        return out
 
     def memory_stats(self) -> Tuple[int, int]:
-        return len(self._states), sum(s.nbytes() for s in self._states.values())
+        n, b = C.c_uint64(), C.c_uint64()
+        check(lib().eri_adam8bit_fn_memory_stats(self._opt, C.byref(n), C.byref(b)), "eri_adam8bit_fn_memory_stats")
+        return n.value, b.value
 
     def get_state_as_tensors(self) -> Dict[str, Tuple[torch.Tensor, torch.Tensor]]:
         out = {}
-        for name, s in self._states.items():
-            m = torch.empty(s.m.numel(), dtype=torch.float32, device=s.m.device)
+        for name in self._names:
+            numel = C.c_uint64()
+            check(lib().eri_adam8bit_fn_state_numel(self._opt, name.encode(), C.byref(numel)), "state_numel")
+            m = torch.empty(numel.value, dtype=torch.float32, device="cuda")
             v = torch.empty_like(m)
-            check(lib().eri_adam8_dequantize(s.m.data_ptr(), s.absmax_m.data_ptr(), 1, m.numel(), m.data_ptr(),
-                                             _stream_ptr()), "eri_adam8_dequantize")
-            check(lib().eri_adam8_dequantize(s.v.data_ptr(), s.absmax_v.data_ptr(), 0, v.numel(), v.data_ptr(),
-                                             _stream_ptr()), "eri_adam8_dequantize")
+            check(lib().eri_adam8bit_fn_get_state_fp32(self._opt, name.encode(), m.data_ptr(), v.data_ptr()),
+                  "eri_adam8bit_fn_get_state_fp32")
             out[name] = (m, v)
         return out
 
     def load_state_from_tensors(self, state: Dict[str, Tuple[torch.Tensor, torch.Tensor]]) -> None:
-        self._states.clear()
         for name, (m, v) in state.items():
             m = m.detach().to(torch.float32).contiguous().view(-1)
             v = v.detach().to(torch.float32).contiguous().view(-1)
-            s = State8(m.numel(), m.device)
-            check(lib().eri_adam8_quantize(m.data_ptr(), 1, m.numel(), s.m.data_ptr(), s.absmax_m.data_ptr(),
-                                           _stream_ptr()), "eri_adam8_quantize")
-            check(lib().eri_adam8_quantize(v.data_ptr(), 0, v.numel(), s.v.data_ptr(), s.absmax_v.data_ptr(),
-                                           _stream_ptr()), "eri_adam8_quantize")
-            self._states[name] = s
+            check(lib().eri_adam8bit_fn_load_state_fp32(self._opt, name.encode(), m.data_ptr(), v.data_ptr(),
+                                                        m.numel()), "eri_adam8bit_fn_load_state_fp32")
+            if name not in self._names:
+                self._names.append(name)
+
+    def close(self) -> None:
+        if self._opt:
+            lib().eri_adam8bit_fn_destroy(self._opt)
+            self._opt = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 def update_params_8bit(optimizer: Adam8bitFunctional, params: Dict[str, torch.Tensor],
                        grads: Dict[str, torch.Tensor]) -> None:
-    """adam8bit.rs:333-345."""
+    """adam8bit.rs:333-345: every named parameter that has a gradient is replaced by its update."""
     for name in list(params.keys()):
         if name in grads:
             params[name] = optimizer.update(name, params[name], grads[name])
+
+
+def create_optimizer(optimizer_type: str, params: List[torch.Tensor], learning_rate=1e-4, weight_decay=0.01,
+                     betas=(0.9, 0.999), eps=1e-8):
+    """String-keyed factory (src/trainers/training/optimization.rs:30-58,
+    src/optimizers/memory_efficient_optimizers.rs:285-308)."""
+    if optimizer_type in ("adam8bit", "adamw8bit", "adamw_8bit"):
+        return Adam8bit(params, Adam8bitConfig(lr=learning_rate, betas=betas, eps=eps, weight_decay=weight_decay))
+    raise ValueError("InvalidOperation: Unknown optimizer: %s" % optimizer_type)

@@ -1,0 +1,76 @@
+"""The Python face over torch tensors: a LoRA-shaped training loop against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+import harness as hs
+import oracle_c as oc
+from oracle import adam8_numpy as onp
+
+pytestmark = pytest.mark.gpu
+
+
+def _bf16_tensor(bits):
+    return torch.from_numpy(bits.view(np.int16).copy()).view(torch.bfloat16).cuda()
+
+
+def _bits(t):
+    return t.detach().cpu().view(torch.int16).numpy().view(np.uint16)
+
+
+def test_adam8bit_over_torch_parameters_matches_the_oracle(tmp_path):
+    from eridiffusion_amd.adam8bit import Adam8bit, Adam8bitConfig, create_optimizer
+    sizes = [16 * 640, 1280 * 16, 300]
+    ps, _ = hs.make_inputs(sizes, True, 5, p_std=1e-2)
+    states = hs.oracle_states(sizes)
+    params = [_bf16_tensor(p) for p in ps]
+    opt = Adam8bit(params, Adam8bitConfig(lr=1e-3), flags=2)
+    for t in (1, 2, 3):
+        gs = hs.fresh_grads(sizes, True, 100 + t, 1e-3)
+        for p, g in zip(params, gs):
+            p.grad = _bf16_tensor(g)
+        assert opt.step() == 0
+        hs.oracle_step(ps, gs, states, (1e-3, 0.9, 0.999, 1e-8, 0.01, t), True)
+        opt.zero_grad()
+    torch.cuda.synchronize()
+    for p, want in zip(params, ps):
+        assert np.array_equal(_bits(p), want)
+    assert opt.get_step() == 3 and opt.current_lr() == 1e-3
+    assert opt.quantized_memory_usage() == sum(2 * n + 8 * ((n + 2047) // 2048) for n in sizes)
+    assert opt.step() == 3  # no gradients left: every parameter skipped, nothing launched
+    opt.save_state(tmp_path / "opt.safetensors")
+    again = create_optimizer("adamw8bit", params, learning_rate=1e-3)
+    again.load_state(tmp_path / "opt.safetensors")
+    assert again.get_step() == 4
+    with pytest.raises(ValueError, match="Unknown optimizer"):
+        create_optimizer("lion", params)
+
+
+def test_functional_flavour_over_torch_tensors():
+    from eridiffusion_amd.adam8bit import Adam8bitFunctional, update_params_8bit
+    n = 2048 * 2 + 9
+    ps, gs = hs.make_inputs([n], False, 9)
+    states = hs.oracle_states([n])
+    opt = Adam8bitFunctional.with_params(1e-4, 0.9, 0.999, 1e-8, 0.01)
+    params = {"blk.lora_up": torch.from_numpy(ps[0].copy()).cuda(), "frozen": torch.ones(8, device="cuda")}
+    grads = {"blk.lora_up": torch.from_numpy(gs[0].copy()).cuda()}
+    before = params["blk.lora_up"]
+    update_params_8bit(opt, params, grads)
+    opt.step()
+    hs.oracle_step(ps, gs, states, (1e-4, 0.9, 0.999, 1e-8, 0.01, 0), False, mode=oc.MODE_L2)
+    torch.cuda.synchronize()
+    assert params["blk.lora_up"] is not before and np.array_equal(before.cpu().numpy(), hs.make_inputs([n], False, 9)[0][0])
+    assert np.array_equal(params["blk.lora_up"].cpu().numpy().view(np.uint32), ps[0].view(np.uint32))
+    assert opt.get_step() == 1 and opt.memory_stats() == (1, 2 * n + 8 * 3)
+    st = opt.get_state_as_tensors()
+    m, v = st["blk.lora_up"]
+    want_m = hs.MAPS[0][states[0][0]] * np.repeat(states[0][2], 2048)[:n]
+    assert np.array_equal(m.cpu().numpy(), want_m.astype(np.float32))
+    fresh = Adam8bitFunctional()
+    fresh.load_state_from_tensors(st)
+    assert fresh.memory_stats() == (1, 2 * n + 8 * 3)
+    m2, _ = fresh.get_state_as_tensors()["blk.lora_up"]
+    # re-quantising exported moments loses at most half a map step of the (possibly smaller) new absmax
+    m_np, m2_np = m.cpu().numpy(), m2.cpu().numpy()
+    step = np.diff(hs.MAPS[0]).max() / 2 * np.repeat(states[0][2], 2048)[:n]
+    assert np.all(np.abs(m2_np - m_np) <= step * 1.0001)
