@@ -1,0 +1,127 @@
+"""Parity at the benchmark's full size: the FLUX-12B-shaped set (780 bf16 tensors, 11.9e9
+parameters, ~72 GB resident).  The oracle cannot sweep that in reasonable time, so the check is
+(a) the oracle on a sample of blocks -- first, last and partial blocks of tensors plus random ones --
+whose inputs are copied out before the step, and (b) properties that hold for every block and are
+cheap to evaluate on the device: each block's largest second moment carries code 255 and its largest
+first moment code 0 or 255 (value / absmax = +-1 exactly), absmax is positive and finite, and no
+code outside a tensor's extent was touched (guard values between tensors survive)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import harness as hs
+import oracle_c as oc
+
+pytestmark = pytest.mark.gpu
+BLOCK = 2048
+
+
+def test_flux12b_full_size_sampled_blocks_and_block_properties():
+    import torch
+    from eridiffusion_amd import _lib as L
+    from eridiffusion_amd import workloads as W
+
+    free, total = torch.cuda.mem_get_info()
+    if free < 80e9:
+        pytest.skip("needs ~75 GB of free device memory")
+    tensors = W.c5_flux_full()
+    sizes = [W.numel(s) for _, s in tensors]
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(0xE21D + 5)
+    GUARD = 256  # poisoned bytes after every tensor's codes
+
+    def arena(byte_sizes):
+        offs, tot = [], 0
+        for b in byte_sizes:
+            offs.append(tot)
+            tot += (b + GUARD + 255) // 256 * 256
+        return torch.empty(tot, dtype=torch.uint8, device=dev), offs
+
+    p_buf, p_off = arena([2 * n for n in sizes])
+    g_buf, g_off = arena([2 * n for n in sizes])
+    m_buf, m_off = arena(sizes)
+    v_buf, v_off = arena(sizes)
+    nbs = [(n + BLOCK - 1) // BLOCK for n in sizes]
+    am_buf, am_off = arena([4 * b for b in nbs])
+    av_buf, av_off = arena([4 * b for b in nbs])
+    m_buf.fill_(0xEE)
+    v_buf.fill_(0xEE)
+    stream = torch.cuda.current_stream().cuda_stream
+    rows = (L.TensorRow * len(sizes))()
+    start = 0
+    for i, n in enumerate(sizes):
+        p_buf[p_off[i]:p_off[i] + 2 * n].view(torch.bfloat16).copy_(torch.randn(n, device=dev, generator=gen).mul_(0.02))
+        g_buf[g_off[i]:g_off[i] + 2 * n].view(torch.bfloat16).copy_(torch.randn(n, device=dev, generator=gen).mul_(1e-3))
+        r = rows[i]
+        r.p, r.g = p_buf.data_ptr() + p_off[i], g_buf.data_ptr() + g_off[i]
+        r.m, r.v = m_buf.data_ptr() + m_off[i], v_buf.data_ptr() + v_off[i]
+        r.absmax_m, r.absmax_v = am_buf.data_ptr() + am_off[i], av_buf.data_ptr() + av_off[i]
+        r.numel, r.block_start, r.dtype_tag, r.grad_scale = n, start, L.DTYPE_BF16, 1.0
+        start += nbs[i]
+        L.check(L.lib().eri_adam8_state_init(r.m, r.v, r.absmax_m, r.absmax_v, n, stream), "state_init")
+    table = C.c_void_p()
+    L.check(L.lib().eri_adam8_table_create(rows, len(rows), stream, C.byref(table)), "table_create")
+    total_numel, total_blocks = C.c_uint64(), C.c_uint64()
+    L.check(L.lib().eri_adam8_table_info(table, C.byref(total_numel), C.byref(total_blocks)), "table_info")
+    assert total_numel.value == 11_901_408_320 and total_blocks.value == 5_811_496
+
+    rng = np.random.default_rng(3)
+    sample = set()
+    for i in range(len(sizes)):
+        sample.add((i, 0))
+        sample.add((i, nbs[i] - 1))
+    big = [i for i in range(len(sizes)) if nbs[i] > 4]
+    for _ in range(400):
+        i = int(rng.choice(big))
+        sample.add((i, int(rng.integers(0, nbs[i]))))
+    sample = sorted(sample)
+
+    def grab():
+        out = []
+        for i, b in sample:
+            lo = b * BLOCK
+            n = min(BLOCK, sizes[i] - lo)
+            out.append((p_buf[p_off[i] + 2 * lo:p_off[i] + 2 * (lo + n)].cpu().numpy().view(np.uint16).copy(),
+                        g_buf[g_off[i] + 2 * lo:g_off[i] + 2 * (lo + n)].cpu().numpy().view(np.uint16).copy(),
+                        m_buf[m_off[i] + lo:m_off[i] + lo + n].cpu().numpy().copy(),
+                        v_buf[v_off[i] + lo:v_off[i] + lo + n].cpu().numpy().copy(),
+                        am_buf[am_off[i] + 4 * b:am_off[i] + 4 * b + 4].cpu().numpy().view(np.float32).copy(),
+                        av_buf[av_off[i] + 4 * b:av_off[i] + 4 * b + 4].cpu().numpy().view(np.float32).copy()))
+        return out
+
+    hyper = (1e-4, 0.9, 0.999, 1e-8, 0.01)
+    flips = 0
+    for t in (1, 2):
+        before = grab()
+        h = L.hyper_pack(*hyper, t, L.MODE_ERI, 0)
+        L.check(L.lib().eri_adam8_step_table(table, C.byref(h), stream), "step_table")
+        torch.cuda.synchronize()
+        after = grab()
+        ho = oc.hyper_pack(*hyper, t)
+        for (p, g, m, v, am, av), got in zip(before, after):
+            rc = oc.step_tensor(p, g, m, v, am, av, ho, hs.MAPS, oc.DT_BF16, 1)
+            assert rc == 0
+            assert np.array_equal(got[2], m) and np.array_equal(got[3], v)
+            assert np.array_equal(got[4].view(np.uint32), am.view(np.uint32))
+            assert np.array_equal(got[5].view(np.uint32), av.view(np.uint32))
+            d = hs.bf16_ulp_distance(got[0], p)
+            assert d.max() <= 1
+            flips += int((d != 0).sum())
+    print("full-size sample: %d blocks x 2 steps, bf16 parameters one ulp off: %d" % (len(sample), flips), flush=True)
+
+    # properties of every block
+    for i, n in enumerate(sizes):
+        nf = n // BLOCK
+        if nf:
+            mv = m_buf[m_off[i]:m_off[i] + nf * BLOCK].view(nf, BLOCK)
+            vv = v_buf[v_off[i]:v_off[i] + nf * BLOCK].view(nf, BLOCK)
+            assert bool((vv.max(dim=1).values == 255).all())
+            assert bool(((mv.max(dim=1).values == 255) | (mv.min(dim=1).values == 0)).all())
+        am = am_buf[am_off[i]:am_off[i] + 4 * nbs[i]].view(torch.float32)
+        av = av_buf[av_off[i]:av_off[i] + 4 * nbs[i]].view(torch.float32)
+        assert bool(torch.isfinite(am).all()) and bool((am > 0).all()) and bool((av > 0).all())
+        assert bool((m_buf[m_off[i] + n:m_off[i] + n + GUARD] == 0xEE).all())
+        assert bool((v_buf[v_off[i] + n:v_off[i] + n + GUARD] == 0xEE).all())
+    L.lib().eri_adam8_table_destroy(table)
