@@ -1,0 +1,248 @@
+//! Drop-in for `src/trainers/adam8bit_enhanced.rs` and `src/trainers/adam8bit.rs`: the same public
+//! items and signatures, every method forwarding to the C ABI in `eri_optim8_sys`.
+//!
+//! Source text only (no Rust toolchain where this repository is built).  It assumes what the
+//! reference already uses from flame-core: `Parameter::{tensor, grad}`, `Tensor::{dtype, shape,
+//! device, cuda_ptr, cuda_ptr_mut}` and `device().cuda_stream_raw_ptr()`
+//! (crates/core/src/tensor_narrow.rs:197-201).
+use std::collections::HashMap;
+use std::ffi::{CStr, CString};
+use std::os::raw::c_void;
+use std::path::Path;
+
+use flame_core::device::CudaStreamRawPtrExt;
+use flame_core::{DType, Error, Parameter, Result, Tensor};
+
+use crate::eri_optim8_sys as sys;
+
+fn check(code: i32, what: &str) -> Result<()> {
+    if code == 0 {
+        return Ok(());
+    }
+    let msg = unsafe { CStr::from_ptr(sys::eri_last_error()) }.to_string_lossy().into_owned();
+    // same shape as tensor_narrow.rs:221-227: "... failed with code N"
+    Err(Error::InvalidOperation(format!("{what} failed with code {code}: {msg}")))
+}
+
+fn dtype_tag(dt: DType) -> Result<i32> {
+    match dt {
+        DType::F32 => Ok(sys::ERI_DTYPE_F32),
+        DType::BF16 => Ok(sys::ERI_DTYPE_BF16),
+        other => Err(Error::Unsupported(format!("8-bit Adam takes F32 or BF16 parameters, got {other:?}"))),
+    }
+}
+
+/// adam8bit_enhanced.rs:372-395
+#[derive(Debug, Clone)]
+pub struct Adam8bitConfig {
+    pub lr: f64,
+    pub betas: (f64, f64),
+    pub eps: f64,
+    pub weight_decay: f64,
+    pub amsgrad: bool,
+    pub block_wise: bool,
+    pub percentile_clipping: usize,
+}
+
+impl Default for Adam8bitConfig {
+    fn default() -> Self {
+        Self { lr: 1e-3, betas: (0.9, 0.999), eps: 1e-8, weight_decay: 0.01, amsgrad: false, block_wise: true, percentile_clipping: 99 }
+    }
+}
+
+/// adam8bit_enhanced.rs:10-27.  The quantised states live on the device, owned by the C side.
+pub struct Adam8bit {
+    pub params: Vec<Parameter>,
+    handles: Vec<*mut sys::EriParameter>,
+    opt: *mut sys::EriAdam8bit,
+    live_grads: Vec<Tensor>, // gradients cast to the parameter dtype must outlive the launch
+}
+
+unsafe impl Send for Adam8bit {}
+unsafe impl Sync for Adam8bit {}
+
+impl Adam8bit {
+    /// adam8bit_enhanced.rs:161
+    pub fn new(params: Vec<Parameter>, config: Adam8bitConfig) -> Result<Self> {
+        let mut handles = Vec::with_capacity(params.len());
+        let mut stream: *mut c_void = std::ptr::null_mut();
+        for p in &params {
+            let t = p.tensor()?;
+            stream = t.device().cuda_stream_raw_ptr();
+            let mut h = std::ptr::null_mut();
+            let numel: usize = t.shape().dims().iter().product();
+            check(unsafe { sys::eri_param_create(t.cuda_ptr_mut() as *mut c_void, numel as u64, dtype_tag(t.dtype())?, &mut h) }, "eri_param_create")?;
+            handles.push(h);
+        }
+        let cfg = sys::EriAdam8bitConfig {
+            lr: config.lr, beta1: config.betas.0, beta2: config.betas.1, eps: config.eps,
+            weight_decay: config.weight_decay, amsgrad: config.amsgrad as i32,
+            block_wise: config.block_wise as i32, percentile_clipping: config.percentile_clipping as u64,
+        };
+        let mut opt = std::ptr::null_mut();
+        check(unsafe { sys::eri_adam8bit_new(handles.as_ptr(), handles.len() as u32, &cfg, stream, &mut opt) }, "eri_adam8bit_new")?;
+        Ok(Self { params, handles, opt, live_grads: Vec::new() })
+    }
+
+    /// adam8bit_enhanced.rs:202-291.  One kernel launch for all parameters; parameters without a
+    /// gradient are skipped with the reference's warning.
+    pub fn step(&mut self) -> Result<()> {
+        self.live_grads.clear();
+        for (p, &h) in self.params.iter().zip(&self.handles) {
+            let t = p.tensor()?;
+            check(unsafe { sys::eri_param_set_data(h, t.cuda_ptr_mut() as *mut c_void) }, "eri_param_set_data")?;
+            let g = match p.grad() {
+                Some(g) if g.dtype() != t.dtype() => Some(g.to_dtype(t.dtype())?),
+                other => other,
+            };
+            let ptr = g.as_ref().map(|g| g.cuda_ptr() as *const c_void).unwrap_or(std::ptr::null());
+            check(unsafe { sys::eri_param_set_grad(h, ptr) }, "eri_param_set_grad")?;
+            if let Some(g) = g {
+                self.live_grads.push(g);
+            }
+        }
+        check(unsafe { sys::eri_adam8bit_step(self.opt, std::ptr::null_mut()) }, "eri_adam8bit_step")
+    }
+
+    /// adam8bit_enhanced.rs:294
+    pub fn zero_grad(&mut self) -> Result<()> {
+        check(unsafe { sys::eri_adam8bit_zero_grad(self.opt) }, "eri_adam8bit_zero_grad")
+    }
+    /// :302
+    pub fn current_lr(&self) -> f64 {
+        unsafe { sys::eri_adam8bit_current_lr(self.opt) }
+    }
+    /// :307
+    pub fn set_learning_rate(&mut self, lr: f64) {
+        unsafe { sys::eri_adam8bit_set_learning_rate(self.opt, lr) };
+    }
+    /// :312
+    pub fn quantized_memory_usage(&self) -> usize {
+        unsafe { sys::eri_adam8bit_quantized_memory_usage(self.opt) as usize }
+    }
+    /// Fold the global-norm clip factor into the next steps instead of rewriting every gradient
+    /// (pipeline_flux_lora_sequential.rs:1198-1213).
+    pub fn set_grad_scale(&mut self, scale: f32) -> Result<()> {
+        check(unsafe { sys::eri_adam8bit_set_grad_scale(self.opt, scale) }, "eri_adam8bit_set_grad_scale")
+    }
+    /// :330
+    pub fn save_state(&self, path: &Path) -> Result<()> {
+        let c = CString::new(path.to_string_lossy().as_bytes()).map_err(|e| Error::InvalidOperation(e.to_string()))?;
+        check(unsafe { sys::eri_adam8bit_save_state(self.opt, c.as_ptr()) }, "eri_adam8bit_save_state")
+    }
+    /// :350
+    pub fn load_state(&mut self, path: &Path) -> Result<()> {
+        let c = CString::new(path.to_string_lossy().as_bytes()).map_err(|e| Error::InvalidOperation(e.to_string()))?;
+        check(unsafe { sys::eri_adam8bit_load_state(self.opt, c.as_ptr()) }, "eri_adam8bit_load_state")
+    }
+}
+
+impl Drop for Adam8bit {
+    fn drop(&mut self) {
+        unsafe {
+            sys::eri_adam8bit_destroy(self.opt);
+            for &h in &self.handles {
+                sys::eri_param_release(h);
+            }
+        }
+    }
+}
+
+/// Functional flavour, `src/trainers/adam8bit.rs:15-28`: states keyed by the name given to update().
+pub struct Adam8bitFunctional {
+    opt: *mut sys::EriAdam8bitFn,
+    names: Vec<String>,
+}
+
+unsafe impl Send for Adam8bitFunctional {}
+unsafe impl Sync for Adam8bitFunctional {}
+
+impl Adam8bitFunctional {
+    /// adam8bit.rs:69-86
+    pub fn with_params(learning_rate: f64, beta1: f64, beta2: f64, eps: f64, weight_decay: f64) -> Self {
+        let mut opt = std::ptr::null_mut();
+        unsafe { sys::eri_adam8bit_fn_with_params(learning_rate, beta1, beta2, eps, weight_decay, std::ptr::null_mut(), &mut opt) };
+        Self { opt, names: Vec::new() }
+    }
+    /// :89-92
+    pub fn step(&mut self) -> Result<()> {
+        check(unsafe { sys::eri_adam8bit_fn_step(self.opt) }, "eri_adam8bit_fn_step")
+    }
+    /// :95-98
+    pub fn set_lr(&mut self, lr: f32) -> Result<()> {
+        check(unsafe { sys::eri_adam8bit_fn_set_lr(self.opt, lr) }, "eri_adam8bit_fn_set_lr")
+    }
+    /// :311-313
+    pub fn get_step(&self) -> usize {
+        unsafe { sys::eri_adam8bit_fn_get_step(self.opt) as usize }
+    }
+    /// :101-208: returns the updated tensor, the input is left alone
+    pub fn update(&mut self, name: &str, param: &Tensor, grad: &Tensor) -> Result<Tensor> {
+        let out = Tensor::zeros_dtype(param.shape().clone(), param.dtype(), param.device().clone())?;
+        let g = if grad.dtype() != param.dtype() { grad.to_dtype(param.dtype())? } else { grad.clone() };
+        let numel: usize = param.shape().dims().iter().product();
+        let c = CString::new(name).map_err(|e| Error::InvalidOperation(e.to_string()))?;
+        check(unsafe {
+            sys::eri_adam8bit_fn_update(self.opt, c.as_ptr(), param.cuda_ptr() as *const c_void, g.cuda_ptr() as *const c_void,
+                                        numel as u64, dtype_tag(param.dtype())?, out.cuda_ptr_mut() as *mut c_void)
+        }, "eri_adam8bit_fn_update")?;
+        if !self.names.iter().any(|n| n == name) {
+            self.names.push(name.to_string());
+        }
+        Ok(out)
+    }
+    /// :253-266
+    pub fn memory_stats(&self) -> (usize, usize) {
+        let (mut n, mut b) = (0u64, 0u64);
+        unsafe { sys::eri_adam8bit_fn_memory_stats(self.opt, &mut n, &mut b) };
+        (n as usize, b as usize)
+    }
+    /// :296-308: fp32 moments per name, the layout the trainers write as `optimizer.{name}.m|.v`
+    /// (pipeline_flux_lora_sequential.rs:1481-1487)
+    pub fn get_state_as_tensors(&self, device: &flame_core::device::Device) -> Result<HashMap<String, (Tensor, Tensor)>> {
+        let mut out = HashMap::new();
+        for name in &self.names {
+            let c = CString::new(name.as_str()).unwrap();
+            let mut numel = 0u64;
+            check(unsafe { sys::eri_adam8bit_fn_state_numel(self.opt, c.as_ptr(), &mut numel) }, "eri_adam8bit_fn_state_numel")?;
+            let shape = flame_core::Shape::from_dims(&[numel as usize]);
+            let m = Tensor::zeros(shape.clone(), device.cuda_device_arc())?;
+            let v = Tensor::zeros(shape, device.cuda_device_arc())?;
+            check(unsafe { sys::eri_adam8bit_fn_get_state_fp32(self.opt, c.as_ptr(), m.cuda_ptr_mut() as *mut f32, v.cuda_ptr_mut() as *mut f32) },
+                  "eri_adam8bit_fn_get_state_fp32")?;
+            out.insert(name.clone(), (m, v));
+        }
+        Ok(out)
+    }
+    /// :316-329
+    pub fn load_state_from_tensors(&mut self, state: HashMap<String, (Tensor, Tensor)>) -> Result<()> {
+        for (name, (m, v)) in state {
+            let m = m.to_dtype(DType::F32)?;
+            let v = v.to_dtype(DType::F32)?;
+            let numel: usize = m.shape().dims().iter().product();
+            let c = CString::new(name.as_str()).map_err(|e| Error::InvalidOperation(e.to_string()))?;
+            check(unsafe { sys::eri_adam8bit_fn_load_state_fp32(self.opt, c.as_ptr(), m.cuda_ptr() as *const f32, v.cuda_ptr() as *const f32, numel as u64) },
+                  "eri_adam8bit_fn_load_state_fp32")?;
+            if !self.names.contains(&name) {
+                self.names.push(name);
+            }
+        }
+        Ok(())
+    }
+}
+
+impl Drop for Adam8bitFunctional {
+    fn drop(&mut self) {
+        unsafe { sys::eri_adam8bit_fn_destroy(self.opt) };
+    }
+}
+
+/// adam8bit.rs:333-345
+pub fn update_params_8bit(optimizer: &mut Adam8bitFunctional, params: &mut HashMap<String, Tensor>, grads: &HashMap<String, Tensor>) -> Result<()> {
+    for (name, param) in params.iter_mut() {
+        if let Some(grad) = grads.get(name) {
+            *param = optimizer.update(name, param, grad)?;
+        }
+    }
+    Ok(())
+}

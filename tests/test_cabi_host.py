@@ -25,6 +25,16 @@ def test_library_exports_every_declared_symbol():
     assert declared == set(L.EXPORTS), "binding table and header disagree: %s" % (declared ^ set(L.EXPORTS))
 
 
+def test_rust_binding_source_declares_every_symbol():
+    """The Rust `extern "C"` block shipped as source must name exactly the header's functions."""
+    header = open(os.path.join(ROOT, "include", "eri_optim8.h")).read() + \
+        open(os.path.join(ROOT, "include", "eri_adam8bit.h")).read()
+    declared = set(re.findall(r"\b(eri_[a-z0-9_]+)\s*\(", header))
+    rust = open(os.path.join(ROOT, "eridiffusion_amd", "rust", "eri_optim8_sys.rs")).read()
+    bound = set(re.findall(r"pub fn (eri_[a-z0-9_]+)\s*\(", rust))
+    assert bound == declared, bound ^ declared
+
+
 def test_struct_layouts_match_the_header():
     assert C.sizeof(L.Hyper) == 48
     assert C.sizeof(L.TensorRow) == 72
