@@ -280,9 +280,59 @@ __device__ __forceinline__ float lds_float_at(const float *table, uint32_t byte_
 // a full 2048-element block, one wavefront
 // ------------------------------------------------------------------------------------------
 
+/*
+ * acc.byte[k] = lo + (xs > mid): the compare, the add and the insertion into the packed word of four
+ * codes in two instructions -- a carry-in add whose SDWA destination select writes one byte and
+ * preserves the others.  Every block opens with the compare, so two byte writes into the same
+ * register are never adjacent (the sub-dword write needs one instruction before its result is
+ * read); the last byte is followed by an s_nop before the store consumes the word.
+ * k must be a compile-time constant after unrolling.
+ */
+__device__ __forceinline__ void pack_code(uint32_t &acc, int k, float xs, float mid, uint32_t lo) {
+    const uint32_t zero = 0u;
+    switch (k & 3) {
+    case 0:
+        asm("v_cmp_gt_f32 vcc, %1, %2\n\t"
+            "v_addc_co_u32_sdwa %0, vcc, %3, %4, vcc dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:DWORD"
+            : "=v"(acc) : "v"(xs), "v"(mid), "v"(lo), "v"(zero) : "vcc");
+        break;
+    case 1:
+        asm("v_cmp_gt_f32 vcc, %1, %2\n\t"
+            "v_addc_co_u32_sdwa %0, vcc, %3, %4, vcc dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD"
+            : "+v"(acc) : "v"(xs), "v"(mid), "v"(lo), "v"(zero) : "vcc");
+        break;
+    case 2:
+        asm("v_cmp_gt_f32 vcc, %1, %2\n\t"
+            "v_addc_co_u32_sdwa %0, vcc, %3, %4, vcc dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD"
+            : "+v"(acc) : "v"(xs), "v"(mid), "v"(lo), "v"(zero) : "vcc");
+        break;
+    default:
+        asm("v_cmp_gt_f32 vcc, %1, %2\n\t"
+            "v_addc_co_u32_sdwa %0, vcc, %3, %4, vcc dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD\n\t"
+            "s_nop 0"
+            : "+v"(acc) : "v"(xs), "v"(mid), "v"(lo), "v"(zero) : "vcc");
+        break;
+    }
+}
+
 template <bool FAST_DIV, bool KEYTAB>
 __device__ __forceinline__ void requant8(const float *mf, const float *vf, const BlockDiv &dm, const BlockDiv &dv,
                                          const Lds &L, u32x2 &mw, u32x2 &vw) {
+    if (KEYTAB && FAST_DIV) { // the hot path: slot lookup, codes packed by byte-select writes
+        uint32_t am[2], av[2];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const float xm = dm.div_fast(mf[k]); // times kKeyScale
+            const float xv = dv.div_fast(vf[k]);
+            const KeySlot sm = *reinterpret_cast<const KeySlot *>(L.key_s + (half_key(xm) & 0xfff0u));
+            const KeySlot sv = *reinterpret_cast<const KeySlot *>(L.key_u + (half_key(xv) & 0x7ff8u));
+            pack_code(am[k >> 2], k, xm, sm.mid, sm.lo);
+            pack_code(av[k >> 2], k, xv, sv.mid, sv.lo);
+        }
+        mw.x = am[0]; mw.y = am[1];
+        vw.x = av[0]; vw.y = av[1];
+        return;
+    }
     uint32_t cm[8], cv[8];
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
