@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(_HERE, "liberi_optim8.so")
 BLOCK = 2048
 DTYPE_F32, DTYPE_F16, DTYPE_BF16, DTYPE_I32 = 0, 1, 2, 3
 MODE_ERI, MODE_L2 = 0, 1
-FLAG_GRAD_SCALE, FLAG_EXACT_PARAM, FLAG_BSEARCH, FLAG_NO_PIPELINE = 1, 2, 4, 8
+FLAG_GRAD_SCALE, FLAG_EXACT_PARAM, FLAG_BSEARCH, FLAG_NO_PIPELINE, FLAG_CLIP_FROM_TABLE = 1, 2, 4, 8, 16
 
 
 class Hyper(C.Structure):
@@ -68,6 +68,8 @@ EXPORTS = {
     "eri_adam8_table_destroy": (C.c_int, [C.c_void_p]),
     "eri_adam8_table_info": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "eri_adam8_step_table": (C.c_int, [C.c_void_p, C.POINTER(Hyper), C.c_void_p]),
+    "eri_adam8_grad_norm": (C.c_int, [C.c_void_p, C.c_float, C.c_float, C.c_void_p]),
+    "eri_adam8_grad_norm_read": (C.c_int, [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_void_p]),
     "eri_adam8_step_multi": (C.c_int, [C.POINTER(TensorRow), C.c_uint32, C.POINTER(Hyper), C.c_void_p]),
     "eri_adam8_dequantize": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_uint64, C.c_void_p, C.c_void_p]),
     "eri_adam8_quantize": (C.c_int, [C.c_void_p, C.c_int, C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p]),
@@ -89,6 +91,8 @@ EXPORTS = {
     "eri_adam8bit_get_step": (C.c_uint64, [C.c_void_p]),
     "eri_adam8bit_set_grad_scale": (C.c_int, [C.c_void_p, C.c_float]),
     "eri_adam8bit_set_param_grad_scale": (C.c_int, [C.c_void_p, C.c_uint32, C.c_float]),
+    "eri_adam8bit_set_max_grad_norm": (C.c_int, [C.c_void_p, C.c_float, C.c_float]),
+    "eri_adam8bit_last_grad_norm": (C.c_int, [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
     "eri_adam8bit_set_flags": (C.c_int, [C.c_void_p, C.c_uint32]),
     "eri_adam8bit_save_state": (C.c_int, [C.c_void_p, C.c_char_p]),
     "eri_adam8bit_load_state": (C.c_int, [C.c_void_p, C.c_char_p]),

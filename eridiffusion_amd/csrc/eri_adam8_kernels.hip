@@ -499,8 +499,11 @@ __device__ __forceinline__ uint32_t find_row(const DevTensor *rows, uint32_t n_r
 template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB>
 __global__ __launch_bounds__(1024) void adam8_step_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
                                                           uint32_t total_blocks, EriAdam8Hyper h,
-                                                          const uint4 *__restrict__ lds_image) {
+                                                          const uint4 *__restrict__ lds_image,
+        const float *__restrict__ dev_scale) {
     ERI_LDS_IMAGE;
+    // clip factor left on the device by the gradient-norm pass (1.0 when there is none)
+    const float tscale = (GS && dev_scale) ? *dev_scale : 1.0f;
     for (uint32_t i = threadIdx.x; i < kLdsImageBytes / 16; i += blockDim.x) lds_raw[i] = lds_image[i];
     __syncthreads();
     const char *base = reinterpret_cast<const char *>(lds_raw);
@@ -523,7 +526,7 @@ __global__ __launch_bounds__(1024) void adam8_step_kernel(const DevTensor *__res
         const DevTensor t = rows[r];
         const uint32_t n = (uint32_t)(t.numel % kBlock);
         if (n != 0) {
-            const float gscale = GS ? h.grad_scale * t.grad_scale : 1.0f;
+            const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
             tail_block<BF16, MODE, EXACT, WD, GS, KEYTAB>(t, (uint32_t)(t.numel / kBlock), n, lane, h, gscale, dbc1, dbc2, L);
         }
     }
@@ -531,7 +534,7 @@ __global__ __launch_bounds__(1024) void adam8_step_kernel(const DevTensor *__res
     for (uint32_t blk = wave; blk < total_blocks; blk += stride) {
         ti = find_row(rows, n_rows, ti, blk);
         const DevTensor t = rows[ti];
-        const float gscale = GS ? h.grad_scale * t.grad_scale : 1.0f;
+        const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
         full_block<BF16, MODE, EXACT, WD, GS, KEYTAB>(t, blk - t.full_start, lane, h, gscale, dbc1, dbc2, L);
     }
 }
@@ -572,8 +575,11 @@ template <int MODE, bool EXACT, bool WD, bool GS>
 __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTensor *__restrict__ rows,
                                                                    uint32_t n_rows, uint32_t total_blocks,
                                                                    EriAdam8Hyper h,
-                                                                   const uint4 *__restrict__ lds_image) {
+                                                                   const uint4 *__restrict__ lds_image,
+        const float *__restrict__ dev_scale) {
     ERI_LDS_IMAGE;
+    // clip factor left on the device by the gradient-norm pass (1.0 when there is none)
+    const float tscale = (GS && dev_scale) ? *dev_scale : 1.0f;
     for (uint32_t i = threadIdx.x; i < kLdsImageBytes / 16; i += blockDim.x) lds_raw[i] = lds_image[i];
     __syncthreads();
     const char *base = reinterpret_cast<const char *>(lds_raw);
@@ -596,7 +602,7 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
         const DevTensor t = rows[r];
         const uint32_t n = (uint32_t)(t.numel % kBlock);
         if (n != 0) {
-            const float gscale = GS ? h.grad_scale * t.grad_scale : 1.0f;
+            const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
             tail_block<true, MODE, EXACT, WD, GS, true>(t, (uint32_t)(t.numel / kBlock), n, lane, h, gscale, dbc1, dbc2, L);
         }
     }
@@ -617,7 +623,7 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
         const DevTensor nt = rows[nti];
 
         const uint32_t lb = blk - t.full_start;
-        const float gscale = GS ? h.grad_scale * t.grad_scale : 1.0f;
+        const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
         const size_t e0 = (size_t)lb * kBlock;
         char *p = static_cast<char *>(t.p) + e0 * 2;
         uint8_t *mc = t.m + e0;
@@ -682,30 +688,30 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
 
 template <int MODE, bool EXACT, bool WD, bool GS>
 static int launch_pipelined(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
-                            const void *lds_image, uint32_t grid, uint32_t wg, hipStream_t s) {
+                            const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg, hipStream_t s) {
     auto k = adam8_step_pipelined_kernel<MODE, EXACT, WD, GS>;
     if (wg > 768) wg = 768;
     hipLaunchKernelGGL(k, dim3(grid), dim3(wg), 0, s, rows, n_rows, total_blocks, h,
-                       static_cast<const uint4 *>(lds_image));
+                       static_cast<const uint4 *>(lds_image), dev_scale);
     return (int)hipGetLastError();
 }
 
 template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB>
 static int launch_one(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
-                      const void *lds_image, uint32_t grid, uint32_t wg, hipStream_t s) {
+                      const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg, hipStream_t s) {
     auto k = adam8_step_kernel<BF16, MODE, EXACT, WD, GS, KEYTAB>;
     hipLaunchKernelGGL(k, dim3(grid), dim3(wg), 0, s, rows, n_rows, total_blocks, h,
-                       static_cast<const uint4 *>(lds_image));
+                       static_cast<const uint4 *>(lds_image), dev_scale);
     return (int)hipGetLastError();
 }
 
 template <bool BF16, int MODE, bool EXACT>
 static int launch_flags(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
-                        const void *img, uint32_t grid, uint32_t wg, hipStream_t s) {
+                        const void *img, const float *dev_scale, uint32_t grid, uint32_t wg, hipStream_t s) {
     const bool wd = h.weight_decay > 0.0f;
     const bool gs = (h.flags & ERI_ADAM8_FLAG_GRAD_SCALE) != 0;
     const bool bs = (h.flags & ERI_ADAM8_FLAG_BSEARCH) != 0;
-#define ERI_GO(W, G, K) return launch_one<BF16, MODE, EXACT, W, G, K>(rows, n_rows, total_blocks, h, img, grid, wg, s)
+#define ERI_GO(W, G, K) return launch_one<BF16, MODE, EXACT, W, G, K>(rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s)
     if (bs) { // cross-check path: only the two decay variants are built for it
         if (wd) { if (gs) ERI_GO(true, true, false); ERI_GO(true, false, false); }
         if (gs) ERI_GO(false, true, false);
@@ -713,11 +719,11 @@ static int launch_flags(const DevTensor *rows, uint32_t n_rows, uint32_t total_b
     }
     if (BF16 && (h.flags & ERI_ADAM8_FLAG_NO_PIPELINE) == 0) {
         if (wd) {
-            if (gs) return launch_pipelined<MODE, EXACT, true, true>(rows, n_rows, total_blocks, h, img, grid, wg, s);
-            return launch_pipelined<MODE, EXACT, true, false>(rows, n_rows, total_blocks, h, img, grid, wg, s);
+            if (gs) return launch_pipelined<MODE, EXACT, true, true>(rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s);
+            return launch_pipelined<MODE, EXACT, true, false>(rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s);
         }
-        if (gs) return launch_pipelined<MODE, EXACT, false, true>(rows, n_rows, total_blocks, h, img, grid, wg, s);
-        return launch_pipelined<MODE, EXACT, false, false>(rows, n_rows, total_blocks, h, img, grid, wg, s);
+        if (gs) return launch_pipelined<MODE, EXACT, false, true>(rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s);
+        return launch_pipelined<MODE, EXACT, false, false>(rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s);
     }
     if (wd) { if (gs) ERI_GO(true, true, true); ERI_GO(true, false, true); }
     if (gs) ERI_GO(false, true, true);
@@ -726,20 +732,21 @@ static int launch_flags(const DevTensor *rows, uint32_t n_rows, uint32_t total_b
 }
 
 int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, int dtype_tag,
-                const EriAdam8Hyper &h, const void *lds_image, uint32_t grid, uint32_t wg, void *stream) {
+                const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg,
+                void *stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool exact = (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0;
     if (dtype_tag == ERI_DTYPE_F32) {
         if (h.mode == ERI_ADAM8_MODE_L2)
-            return launch_flags<false, ERI_ADAM8_MODE_L2, true>(rows, n_rows, total_blocks, h, lds_image, grid, wg, s);
-        return launch_flags<false, ERI_ADAM8_MODE_ERI, true>(rows, n_rows, total_blocks, h, lds_image, grid, wg, s);
+            return launch_flags<false, ERI_ADAM8_MODE_L2, true>(rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, s);
+        return launch_flags<false, ERI_ADAM8_MODE_ERI, true>(rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, s);
     }
     if (h.mode == ERI_ADAM8_MODE_L2) {
-        if (exact) return launch_flags<true, ERI_ADAM8_MODE_L2, true>(rows, n_rows, total_blocks, h, lds_image, grid, wg, s);
-        return launch_flags<true, ERI_ADAM8_MODE_L2, false>(rows, n_rows, total_blocks, h, lds_image, grid, wg, s);
+        if (exact) return launch_flags<true, ERI_ADAM8_MODE_L2, true>(rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, s);
+        return launch_flags<true, ERI_ADAM8_MODE_L2, false>(rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, s);
     }
-    if (exact) return launch_flags<true, ERI_ADAM8_MODE_ERI, true>(rows, n_rows, total_blocks, h, lds_image, grid, wg, s);
-    return launch_flags<true, ERI_ADAM8_MODE_ERI, false>(rows, n_rows, total_blocks, h, lds_image, grid, wg, s);
+    if (exact) return launch_flags<true, ERI_ADAM8_MODE_ERI, true>(rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, s);
+    return launch_flags<true, ERI_ADAM8_MODE_ERI, false>(rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, s);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -821,6 +828,104 @@ int launch_quantize(const float *x, int signed_map, uint64_t numel, uint8_t *cod
     if (grid > 8192) grid = 8192;
     hipLaunchKernelGGL(quantize_kernel, dim3((uint32_t)grid), dim3(256), 0, static_cast<hipStream_t>(stream), x,
                        numel, nblocks, codes, absmax, mid);
+    return (int)hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------------
+// global gradient norm over the launch table (the trainers' clip_gradients,
+// src/trainers/pipeline_flux_lora_sequential.rs:1198-1213,1939-1950), without a host round trip:
+// pass 1 leaves one fp32 sum of squares per block, pass 2 adds them in f64 and writes the norm and
+// the clip factor to device memory, where the step kernel reads it.
+// ------------------------------------------------------------------------------------------
+
+__device__ __forceinline__ float wave_sum(float x) {
+    // fixed reduction tree, so the result does not depend on scheduling
+    x += dpp_mov<0xB1, 0xf>(x);
+    x += dpp_mov<0x4E, 0xf>(x);
+    x += dpp_mov<0x141, 0xf>(x);
+    x += dpp_mov<0x140, 0xf>(x); // every lane: its row's sum
+    float r = u2f((uint32_t)__builtin_amdgcn_readlane((int)f2u(x), 15));
+    r += u2f((uint32_t)__builtin_amdgcn_readlane((int)f2u(x), 31));
+    r += u2f((uint32_t)__builtin_amdgcn_readlane((int)f2u(x), 47));
+    r += u2f((uint32_t)__builtin_amdgcn_readlane((int)f2u(x), 63));
+    return r;
+}
+
+template <bool BF16>
+__global__ __launch_bounds__(256) void grad_sumsq_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
+                                                         uint32_t total_blocks, float *__restrict__ partial) {
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t waves_per_wg = blockDim.x / kWave;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
+    const uint32_t stride = gridDim.x * waves_per_wg;
+    for (uint32_t r = wave; r < n_rows; r += stride) { // partial last blocks; rows without one leave 0
+        const DevTensor t = rows[r];
+        const uint32_t n = (uint32_t)(t.numel % kBlock);
+        const size_t e0 = (size_t)(t.numel / kBlock) * kBlock;
+        float acc = 0.0f;
+        for (uint32_t i = lane; i < n; i += kWave) {
+            const float g = load1<BF16>(t.g, e0 + i);
+            acc += g * g;
+        }
+        acc = wave_sum(acc);
+        if (lane == 0) partial[total_blocks + r] = acc;
+    }
+    uint32_t ti = 0;
+    for (uint32_t blk = wave; blk < total_blocks; blk += stride) {
+        ti = find_row(rows, n_rows, ti, blk);
+        const DevTensor t = rows[ti];
+        const size_t e0 = (size_t)(blk - t.full_start) * kBlock;
+        float acc = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            Raw8<BF16> raw;
+            raw.load(static_cast<const char *>(t.g) + e0 * (BF16 ? 2 : 4), c * 512 + lane * 8);
+            float g[8];
+            raw.unpack(g);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) acc += g[k] * g[k];
+        }
+        acc = wave_sum(acc);
+        if (lane == 0) partial[blk] = acc;
+    }
+}
+
+__global__ __launch_bounds__(1024) void grad_norm_finish_kernel(const float *__restrict__ partial, uint32_t n,
+                                                                float max_norm, float denom_eps,
+                                                                float *__restrict__ out /* norm, scale */) {
+    __shared__ double sh[1024];
+    double acc = 0.0;
+    for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) acc += (double)partial[i];
+    sh[threadIdx.x] = acc;
+    __syncthreads();
+    for (uint32_t s = blockDim.x / 2; s > 0; s >>= 1) {
+        if (threadIdx.x < s) sh[threadIdx.x] += sh[threadIdx.x + s];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        const float norm = (float)sqrt(sh[0]);
+        float scale = 1.0f;
+        // clip only a finite norm above the limit (crates/training/src/optimizer.rs:79-84)
+        if (max_norm > 0.0f && norm > max_norm && norm <= 3.4028234e38f) scale = max_norm / (norm + denom_eps);
+        out[0] = norm;
+        out[1] = scale;
+    }
+}
+
+int launch_grad_sumsq(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, int dtype_tag, float *partial,
+                      uint32_t grid, void *stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype_tag == ERI_DTYPE_F32)
+        hipLaunchKernelGGL(grad_sumsq_kernel<false>, dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, partial);
+    else
+        hipLaunchKernelGGL(grad_sumsq_kernel<true>, dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, partial);
+    return (int)hipGetLastError();
+}
+
+int launch_grad_norm_finish(const float *partial, uint32_t n, float max_norm, float denom_eps, float *out,
+                            void *stream) {
+    hipLaunchKernelGGL(grad_norm_finish_kernel, dim3(1), dim3(1024), 0, static_cast<hipStream_t>(stream), partial, n,
+                       max_norm, denom_eps, out);
     return (int)hipGetLastError();
 }
 

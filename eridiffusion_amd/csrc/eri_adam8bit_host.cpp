@@ -229,6 +229,7 @@ struct EriAdam8bit {
     uint64_t step = 0;
     uint32_t flags = 0;
     float grad_scale = 1.0f;
+    float max_grad_norm = 0.0f, clip_denom_eps = 0.0f;
     std::vector<float> param_scale;
     std::vector<std::unique_ptr<State8>> states; // index = parameter index; null before the first step
     void *stream = nullptr;
@@ -384,8 +385,14 @@ int eri_adam8bit_step(EriAdam8bit *o, uint32_t *skipped) {
         if (rc) return rc;
         o->table_rows = rows;
     }
+    const bool clip = o->max_grad_norm > 0.0f;
+    if (clip) {
+        rc = eri_adam8_grad_norm(o->table, o->max_grad_norm, o->clip_denom_eps, o->stream);
+        if (rc) return rc;
+    }
     EriAdam8Hyper h;
-    uint32_t flags = o->flags | (scaled ? (uint32_t)ERI_ADAM8_FLAG_GRAD_SCALE : 0u);
+    uint32_t flags = o->flags | ((scaled || clip) ? (uint32_t)ERI_ADAM8_FLAG_GRAD_SCALE : 0u) |
+                     (clip ? (uint32_t)ERI_ADAM8_FLAG_CLIP_FROM_TABLE : 0u);
     rc = eri_adam8_hyper_pack(o->lr, o->beta1, o->beta2, o->eps, o->wd, o->step, ERI_ADAM8_MODE_ERI, flags, &h);
     if (rc) return rc;
     h.grad_scale = o->grad_scale;
@@ -427,6 +434,19 @@ int eri_adam8bit_set_param_grad_scale(EriAdam8bit *o, uint32_t index, float scal
     if (index >= o->param_scale.size()) return fail(ERI_ERR_ARG, "parameter index out of range");
     o->param_scale[index] = scale;
     return 0;
+}
+
+int eri_adam8bit_set_max_grad_norm(EriAdam8bit *o, float max_norm, float denom_eps) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    o->max_grad_norm = max_norm;
+    o->clip_denom_eps = denom_eps;
+    return 0;
+}
+
+int eri_adam8bit_last_grad_norm(EriAdam8bit *o, float *norm, float *scale) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    if (!o->table) return fail(ERI_ERR_ARG, "no step has run yet");
+    return eri_adam8_grad_norm_read(o->table, norm, scale, o->stream);
 }
 
 int eri_adam8bit_set_flags(EriAdam8bit *o, uint32_t flags) {

@@ -253,6 +253,7 @@ struct EriAdam8Table {
         eri::DevTensor *dev = nullptr;
         eri::DevTensor *pinned = nullptr;
         std::vector<uint32_t> src; // index into the caller's rows
+        bool unit_scales = true;   // every row's grad_scale is exactly 1
     };
     int device = 0;
     uint32_t n = 0;
@@ -263,6 +264,9 @@ struct EriAdam8Table {
     std::vector<int32_t> dtype;
     hipEvent_t uploaded = nullptr;
     bool upload_pending = false;
+    float *partial = nullptr;  // one sum of squares per block (full blocks, then one slot per row) per group
+    float *norm_out = nullptr; // device: {norm, clip factor}
+    uint32_t n_partial = 0;
 };
 
 namespace {
@@ -306,7 +310,9 @@ int validate_rows(const EriAdam8Tensor *rows, uint32_t n) {
 
 void fill_group(EriAdam8Table::Group &g, const EriAdam8Tensor *rows) {
     uint32_t start = 0;
+    g.unit_scales = true;
     for (uint32_t j = 0; j < g.n; ++j) {
+        if (rows[g.src[j]].grad_scale != 1.0f) g.unit_scales = false;
         const EriAdam8Tensor &r = rows[g.src[j]];
         eri::DevTensor &d = g.pinned[j];
         d.p = r.p;
@@ -341,6 +347,8 @@ void destroy_table(EriAdam8Table *t) {
         if (g.pinned) (void)hipHostFree(g.pinned);
     }
     if (t->uploaded) (void)hipEventDestroy(t->uploaded);
+    if (t->partial) (void)hipFree(t->partial);
+    if (t->norm_out) (void)hipFree(t->norm_out);
     delete t;
 }
 
@@ -628,9 +636,60 @@ int eri_adam8_step_table(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream)
         const uint32_t need = (work + waves_per_wg - 1) / waves_per_wg;
         if (grid > need) grid = need;
         if (grid == 0) grid = 1;
-        rc = eri::launch_step(g.dev, g.n, g.total_blocks, g.dtype, *h, ctx->image, grid, waves_per_wg * eri::kWave, stream);
+        EriAdam8Hyper hh = *h;
+        const float *dev_scale = nullptr;
+        if (hh.flags & ERI_ADAM8_FLAG_CLIP_FROM_TABLE) {
+            if (!t->norm_out) return fail(ERI_ERR_ARG, "ERI_ADAM8_FLAG_CLIP_FROM_TABLE without a prior eri_adam8_grad_norm");
+            dev_scale = t->norm_out + 1;
+            if (!(hh.flags & ERI_ADAM8_FLAG_GRAD_SCALE)) { // the scale path is needed; neutral host-side factors
+                hh.flags |= ERI_ADAM8_FLAG_GRAD_SCALE;
+                hh.grad_scale = 1.0f;
+                if (!g.unit_scales) return fail(ERI_ERR_ARG, "ERI_ADAM8_FLAG_CLIP_FROM_TABLE needs per-tensor grad_scale = 1 unless ERI_ADAM8_FLAG_GRAD_SCALE is set");
+            }
+        }
+        rc = eri::launch_step(g.dev, g.n, g.total_blocks, g.dtype, hh, ctx->image, dev_scale, grid, waves_per_wg * eri::kWave, stream);
         if (rc) return hip_fail((hipError_t)rc, "adam8 step launch");
     }
+    return 0;
+}
+
+int eri_adam8_grad_norm(EriAdam8Table *t, float max_norm, float denom_eps, void *stream) {
+    if (!t) return fail(ERI_ERR_NULL, "table is NULL");
+    DeviceCtx *ctx = nullptr;
+    int rc = get_ctx(&ctx);
+    if (rc) return rc;
+    if (!t->partial) {
+        uint32_t n = 0;
+        for (auto &g : t->groups)
+            if (g.n) n += g.total_blocks + g.n;
+        ERI_HIP(hipMalloc((void **)&t->partial, sizeof(float) * (n ? n : 1)));
+        ERI_HIP(hipMalloc((void **)&t->norm_out, sizeof(float) * 2));
+        t->n_partial = n;
+    }
+    uint32_t off = 0;
+    for (auto &g : t->groups) {
+        if (g.n == 0) continue;
+        const uint32_t work = g.total_blocks > g.n ? g.total_blocks : g.n;
+        uint32_t grid = (work + 3) / 4;
+        const uint32_t cap = ctx->cus * 8;
+        if (grid > cap) grid = cap;
+        rc = eri::launch_grad_sumsq(g.dev, g.n, g.total_blocks, g.dtype, t->partial + off, grid, stream);
+        if (rc) return hip_fail((hipError_t)rc, "gradient sum-of-squares launch");
+        off += g.total_blocks + g.n;
+    }
+    rc = eri::launch_grad_norm_finish(t->partial, t->n_partial, max_norm, denom_eps, t->norm_out, stream);
+    if (rc) return hip_fail((hipError_t)rc, "gradient norm launch");
+    return 0;
+}
+
+int eri_adam8_grad_norm_read(EriAdam8Table *t, float *norm, float *scale, void *stream) {
+    if (!t) return fail(ERI_ERR_NULL, "table is NULL");
+    if (!t->norm_out) return fail(ERI_ERR_ARG, "no gradient norm has been computed for this table");
+    float host[2] = {0.0f, 1.0f};
+    ERI_HIP(hipMemcpyAsync(host, t->norm_out, sizeof host, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream)));
+    ERI_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    if (norm) *norm = host[0];
+    if (scale) *scale = host[1];
     return 0;
 }
 

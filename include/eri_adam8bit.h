@@ -66,6 +66,13 @@ uint64_t eri_adam8bit_get_step(const EriAdam8bit *opt);
 int eri_adam8bit_set_grad_scale(EriAdam8bit *opt, float scale);
 int eri_adam8bit_set_param_grad_scale(EriAdam8bit *opt, uint32_t index, float scale);
 int eri_adam8bit_set_flags(EriAdam8bit *opt, uint32_t flags); /* ERI_ADAM8_FLAG_EXACT_PARAM etc. */
+/* Global-norm clipping inside step(): max_norm > 0 makes every step first reduce the gradients' global
+ * L2 norm on the device (eri_adam8_grad_norm) and apply max_norm / (norm + denom_eps) when the norm is
+ * above max_norm -- the trainers' clip_gradients (pipeline_flux_lora_sequential.rs:737,1198-1213)
+ * without its per-tensor host reads and gradient rewrites.  max_norm <= 0 switches it off. */
+int eri_adam8bit_set_max_grad_norm(EriAdam8bit *opt, float max_norm, float denom_eps);
+/* Norm and clip factor of the last step that clipped (waits for the optimizer's stream). */
+int eri_adam8bit_last_grad_norm(EriAdam8bit *opt, float *norm, float *scale);
 /* save_state / load_state :330-368.  The file is a safetensors container with, per parameter that
  * has state, `optimizer.param_N.m` / `.v` (U8 codes) and `.absmax_m` / `.absmax_v` (F32), and the
  * step counter and learning rate in its metadata. */

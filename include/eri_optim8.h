@@ -90,8 +90,10 @@ enum {
                                              tensors too (F32 tensors always use them) */
     ERI_ADAM8_FLAG_BSEARCH = 1u << 2,     /* requantise by binary search of the LDS midpoint table
                                              instead of the float-keyed slot table (same codes) */
-    ERI_ADAM8_FLAG_NO_PIPELINE = 1u << 3  /* BF16: use the plain kernel, not the one that prefetches
+    ERI_ADAM8_FLAG_NO_PIPELINE = 1u << 3, /* BF16: use the plain kernel, not the one that prefetches
                                              the next block (same results; for A/B measurements) */
+    ERI_ADAM8_FLAG_CLIP_FROM_TABLE = 1u << 4 /* also multiply gradients by the clip factor the last
+                                             eri_adam8_grad_norm left in the table (device memory) */
 };
 
 /* Per-step scalars, already cast where the reference casts them.  Fill with eri_adam8_hyper_pack. */
@@ -149,6 +151,18 @@ int eri_adam8_table_info(const EriAdam8Table *table, uint64_t *total_numel, uint
 
 /* One optimizer step over every tensor of the table: one kernel launch per dtype present. */
 int eri_adam8_step_table(EriAdam8Table *table, const EriAdam8Hyper *hyper, void *stream);
+
+/* Global L2 norm of every gradient of the table and the clip factor it implies, both left in device
+ * memory owned by the table -- no host round trip (the reference reads one scalar back per tensor:
+ * compute_gradient_norm, src/trainers/pipeline_flux_lora_sequential.rs:1939-1950).
+ *   norm  = (float)sqrt(sum of g*g), squares and per-block sums in fp32, blocks added in f64
+ *   scale = max_norm / (norm + denom_eps) if max_norm > 0 and norm is finite and above max_norm, else 1
+ * denom_eps = 0 reproduces clip_gradients (pipeline_flux_lora_sequential.rs:1198-1213), 1e-6
+ * clip_grads_global_norm_fp32_tensors (crates/training/src/optimizer.rs:58-85).  A following step with
+ * ERI_ADAM8_FLAG_CLIP_FROM_TABLE applies the factor inside the kernel instead of rewriting gradients. */
+int eri_adam8_grad_norm(EriAdam8Table *table, float max_norm, float denom_eps, void *stream);
+/* Copies the last norm and clip factor to the host; waits for `stream`. */
+int eri_adam8_grad_norm_read(EriAdam8Table *table, float *norm, float *scale, void *stream);
 
 /* Convenience for callers that keep no handle: keeps one cached table per calling thread and
  * re-uploads it only when `rows` changed since that thread's last call. */

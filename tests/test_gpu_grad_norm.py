@@ -1,0 +1,110 @@
+"""Global gradient norm on the device and the clip factor folded into the step."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import harness as hs
+import oracle_c as oc
+from oracle import adam8_numpy as onp
+
+pytestmark = pytest.mark.gpu
+LR, B1, B2, EPS, WD = 1e-4, 0.9, 0.999, 1e-8, 0.01
+
+
+def _L():
+    from eridiffusion_amd import _lib
+    return _lib
+
+
+def _f32(gs, bf16):
+    return [onp.bf16_to_f32(g) if bf16 else g for g in gs]
+
+
+@pytest.mark.parametrize("bf16", [True, False])
+@pytest.mark.parametrize("max_norm,denom", [(0.05, 0.0), (0.05, 1e-6), (1e9, 0.0)])
+def test_norm_and_clip_factor_then_step(bf16, max_norm, denom):
+    import torch
+    L = _L()
+    sizes = [2048 * 5 + 333, 7, 2048, 4096 + 1, 320, 100000]
+    ps, gs = hs.make_inputs(sizes, bf16, 77 + bf16, g_std=1e-3)
+    states = hs.oracle_states(sizes)
+    gt = hs.GpuTensors(ps, gs, states, bf16)
+    rows = gt.rows()
+    stream = torch.cuda.current_stream().cuda_stream
+    table = C.c_void_p()
+    L.check(L.lib().eri_adam8_table_create(rows, len(rows), stream, C.byref(table)), "table_create")
+    L.check(L.lib().eri_adam8_grad_norm(table, max_norm, denom, stream), "grad_norm")
+    norm, scale = C.c_float(), C.c_float()
+    L.check(L.lib().eri_adam8_grad_norm_read(table, C.byref(norm), C.byref(scale), stream), "grad_norm_read")
+    # tolerance: squares are exact products rounded to fp32 and each lane adds 32 of them in fp32
+    # before the f64 total; 2e-6 relative on the norm covers that with margin
+    want = np.sqrt(sum(float(np.sum(g.astype(np.float32).astype(np.float64) ** 2)) for g in _f32(gs, bf16)))
+    assert abs(norm.value - want) <= 2e-6 * want
+    if norm.value > max_norm:
+        assert scale.value == np.float32(max_norm) / (np.float32(norm.value) + np.float32(denom))
+        assert scale.value < 1
+    else:
+        assert scale.value == 1.0
+    h = L.hyper_pack(LR, B1, B2, EPS, WD, 1, L.MODE_ERI, L.FLAG_EXACT_PARAM | L.FLAG_CLIP_FROM_TABLE)
+    L.check(L.lib().eri_adam8_step_table(table, C.byref(h), stream), "step_table")
+    torch.cuda.synchronize()
+    hs.oracle_step(ps, gs, states, (LR, B1, B2, EPS, WD, 1), bf16, grad_scale=float(scale.value))
+    got_p, got_st = gt.fetch()
+    stats = hs.compare(got_p, got_st, ps, states, bf16, True, "clip")
+    assert stats["code_mismatch"] == 0
+    L.lib().eri_adam8_table_destroy(table)
+
+
+def test_non_finite_gradients_do_not_clip():
+    import torch
+    L = _L()
+    sizes = [4096, 100]
+    ps, gs = hs.make_inputs(sizes, False, 5)
+    gs[0][17] = np.inf
+    gt = hs.GpuTensors(ps, gs, hs.oracle_states(sizes), False)
+    rows = gt.rows()
+    table = C.c_void_p()
+    L.check(L.lib().eri_adam8_table_create(rows, len(rows), None, C.byref(table)), "table_create")
+    L.check(L.lib().eri_adam8_grad_norm(table, 1.0, 0.0, None), "grad_norm")
+    norm, scale = C.c_float(), C.c_float()
+    L.check(L.lib().eri_adam8_grad_norm_read(table, C.byref(norm), C.byref(scale), None), "read")
+    assert np.isinf(norm.value) and scale.value == 1.0
+    h = L.hyper_pack(LR, B1, B2, EPS, WD, 1, L.MODE_ERI, L.FLAG_CLIP_FROM_TABLE)
+    fresh = C.c_void_p()
+    L.check(L.lib().eri_adam8_table_create(rows, len(rows), None, C.byref(fresh)), "table_create")
+    assert L.lib().eri_adam8_step_table(fresh, C.byref(h), None) == -6  # no norm was computed for that table
+    L.lib().eri_adam8_table_destroy(table)
+    L.lib().eri_adam8_table_destroy(fresh)
+
+
+def test_optimizer_object_clips_inside_step():
+    import torch
+    L = _L()
+    sizes = [2048 * 3 + 5, 640]
+    ps, gs = hs.make_inputs(sizes, True, 91, g_std=1e-2)
+    states = hs.oracle_states(sizes)
+    gt = hs.GpuTensors(ps, gs, states, True)
+    handles = (C.c_void_p * 2)()
+    for i in range(2):
+        hnd = C.c_void_p()
+        L.check(L.lib().eri_param_create(gt.ptr(gt.p[i]), sizes[i], 2, C.byref(hnd)), "param_create")
+        L.check(L.lib().eri_param_set_grad(hnd, gt.ptr(gt.g[i])), "set_grad")
+        handles[i] = hnd
+    opt = C.c_void_p()
+    L.check(L.lib().eri_adam8bit_new(handles, 2, None, None, C.byref(opt)), "new")
+    L.check(L.lib().eri_adam8bit_set_flags(opt, L.FLAG_EXACT_PARAM), "flags")
+    L.check(L.lib().eri_adam8bit_set_max_grad_norm(opt, 0.5, 0.0), "max_norm")
+    L.check(L.lib().eri_adam8bit_set_param_grad_scale(opt, 1, 0.5), "param_scale")
+    L.check(L.lib().eri_adam8bit_step(opt, None), "step")
+    norm, scale = C.c_float(), C.c_float()
+    L.check(L.lib().eri_adam8bit_last_grad_norm(opt, C.byref(norm), C.byref(scale)), "last_norm")
+    assert norm.value > 0.5 and scale.value == np.float32(0.5) / np.float32(norm.value)
+    torch.cuda.synchronize()
+    for i, ts in enumerate((1.0, 0.5)):
+        s = (np.float32(1.0) * np.float32(ts)) * np.float32(scale.value)
+        hs.oracle_step([ps[i]], [gs[i]], [states[i]], (1e-3, B1, B2, EPS, WD, 1), True, grad_scale=float(s))
+    got_p = [gt.down(b) for b in gt.p]
+    for g, w in zip(got_p, ps):
+        assert np.array_equal(g, w)
+    L.lib().eri_adam8bit_destroy(opt)
