@@ -34,6 +34,21 @@ class Adam8bitConfigC(C.Structure):
                 ("percentile_clipping", C.c_uint64)]
 
 
+class AdamW32Row(C.Structure):
+    _fields_ = [("p", C.c_void_p), ("g", C.c_void_p), ("m", C.c_void_p), ("v", C.c_void_p), ("numel", C.c_uint64),
+                ("dtype_tag", C.c_int32), ("reserved", C.c_int32)]
+
+
+class AdamW32Hyper(C.Structure):
+    _fields_ = [("lr", C.c_float), ("beta1", C.c_float), ("beta2", C.c_float), ("eps", C.c_float),
+                ("weight_decay", C.c_float)]
+
+
+class EmaRow(C.Structure):
+    _fields_ = [("shadow", C.c_void_p), ("p", C.c_void_p), ("numel", C.c_uint64), ("dtype_tag", C.c_int32),
+                ("reserved", C.c_int32)]
+
+
 class EriError(RuntimeError):
     def __init__(self, what, code, message):
         super().__init__("%s failed with code %d: %s" % (what, code, message))
@@ -73,6 +88,8 @@ EXPORTS = {
     "eri_adam8_step_multi": (C.c_int, [C.POINTER(TensorRow), C.c_uint32, C.POINTER(Hyper), C.c_void_p]),
     "eri_adam8_dequantize": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_uint64, C.c_void_p, C.c_void_p]),
     "eri_adam8_quantize": (C.c_int, [C.c_void_p, C.c_int, C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "eri_adamw32_step_multi": (C.c_int, [C.POINTER(AdamW32Row), C.c_uint32, C.POINTER(AdamW32Hyper), C.c_void_p]),
+    "eri_ema_update_multi": (C.c_int, [C.POINTER(EmaRow), C.c_uint32, C.c_float, C.c_void_p]),
     # ---- include/eri_adam8bit.h
     "eri_param_create": (C.c_int, [C.c_void_p, C.c_uint64, C.c_int, C.POINTER(C.c_void_p)]),
     "eri_param_set_grad": (C.c_int, [C.c_void_p, C.c_void_p]),

@@ -929,4 +929,168 @@ int launch_grad_norm_finish(const float *partial, uint32_t n, float max_norm, fl
     return (int)hipGetLastError();
 }
 
+// ------------------------------------------------------------------------------------------
+// plain element-wise sweeps over a row table: 32-bit AdamW and EMA.  One wave per 2048-element
+// block, 8 elements per lane and pass, partial last blocks element by element.  HBM-bound:
+// AdamW bf16 22 B/param (read 2+2+4+4, write 2+4+4), fp32 28 B/param; EMA 3 x element size.
+// ------------------------------------------------------------------------------------------
+
+__device__ __forceinline__ uint32_t find_elem_row(const ElemRow *rows, uint32_t n_rows, uint32_t from, uint32_t blk) {
+    uint32_t lo = from, hi = n_rows;
+    while (hi - lo > 1) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (rows[mid].full_start <= blk) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
+/* crates/common/optim/src/adamw.rs:34-54, one rounded operation per line */
+__device__ __forceinline__ void adamw32_elem(float p, float g, float &m, float &v, const EriAdamW32Hyper &h, float omb1,
+                                             float omb2, float neg_lr, float &pn) {
+    float ms = m * h.beta1;
+    float gs = g * omb1;
+    m = ms + gs;
+    float vs = v * h.beta2;
+    float g2 = g * g;
+    float g2s = g2 * omb2;
+    v = vs + g2s;
+    float denom = sqrtf(v) + h.eps;
+    float update = m / denom;
+    float wd = h.weight_decay != 0.0f ? p * h.weight_decay : 0.0f;
+    float total = update + wd;
+    float step = total * neg_lr;
+    pn = p + step;
+}
+
+template <bool BF16>
+__device__ __forceinline__ void store1(void *base, size_t i, float x) {
+    if (BF16) as_global(static_cast<uint16_t *>(base))[i] = (uint16_t)bf16_bits(x);
+    else as_global(static_cast<float *>(base))[i] = x;
+}
+
+template <bool BF16>
+__global__ __launch_bounds__(256) void adamw32_kernel(const ElemRow *__restrict__ rows, uint32_t n_rows,
+                                                      uint32_t total_blocks, EriAdamW32Hyper h) {
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t waves_per_wg = blockDim.x / kWave;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
+    const uint32_t stride = gridDim.x * waves_per_wg;
+    const float omb1 = 1.0f - h.beta1, omb2 = 1.0f - h.beta2, neg_lr = -h.lr; // adamw.rs:36,42,53
+    for (uint32_t r = wave; r < n_rows; r += stride) {
+        const ElemRow t = rows[r];
+        const uint32_t n = (uint32_t)(t.numel % kBlock);
+        const size_t e0 = (size_t)(t.numel / kBlock) * kBlock;
+        ERI_GLOBAL float *mp = as_global(static_cast<float *>(t.c));
+        ERI_GLOBAL float *vp = as_global(static_cast<float *>(t.d));
+        for (uint32_t i = lane; i < n; i += kWave) {
+            float m = mp[e0 + i], v = vp[e0 + i], pn;
+            adamw32_elem(load1<BF16>(t.a, e0 + i), load1<BF16>(t.b, e0 + i), m, v, h, omb1, omb2, neg_lr, pn);
+            mp[e0 + i] = m;
+            vp[e0 + i] = v;
+            store1<BF16>(t.a, e0 + i, pn);
+        }
+    }
+    uint32_t ti = 0;
+    for (uint32_t blk = wave; blk < total_blocks; blk += stride) {
+        ti = find_elem_row(rows, n_rows, ti, blk);
+        const ElemRow t = rows[ti];
+        const size_t e0 = (size_t)(blk - t.full_start) * kBlock;
+        char *p = static_cast<char *>(t.a) + e0 * (BF16 ? 2 : 4);
+        const char *g = static_cast<const char *>(t.b) + e0 * (BF16 ? 2 : 4);
+        float *m = static_cast<float *>(t.c) + e0;
+        float *v = static_cast<float *>(t.d) + e0;
+        Raw8<BF16> pr[4], gr[4];
+        Raw8<false> mr[4], vr[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t o = c * 512 + lane * 8;
+            pr[c].load(p, o);
+            gr[c].load(g, o);
+            mr[c].load(m, o);
+            vr[c].load(v, o);
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t o = c * 512 + lane * 8;
+            float pv[8], gv[8], mv[8], vv[8], pn[8];
+            pr[c].unpack(pv);
+            gr[c].unpack(gv);
+            mr[c].unpack(mv);
+            vr[c].unpack(vv);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) adamw32_elem(pv[k], gv[k], mv[k], vv[k], h, omb1, omb2, neg_lr, pn[k]);
+            store8<BF16>(p, o, pn);
+            store8<false>(m, o, mv);
+            store8<false>(v, o, vv);
+        }
+    }
+}
+
+/* src/trainers/ema_enhanced.rs:91-100 */
+__device__ __forceinline__ float ema_elem(float shadow, float p, float decay, float omd) {
+    float a = shadow * decay;
+    float b = p * omd;
+    return a + b;
+}
+
+template <bool BF16>
+__global__ __launch_bounds__(256) void ema_kernel(const ElemRow *__restrict__ rows, uint32_t n_rows,
+                                                  uint32_t total_blocks, float decay) {
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t waves_per_wg = blockDim.x / kWave;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
+    const uint32_t stride = gridDim.x * waves_per_wg;
+    const float omd = 1.0f - decay; // ema_enhanced.rs:96
+    for (uint32_t r = wave; r < n_rows; r += stride) {
+        const ElemRow t = rows[r];
+        const uint32_t n = (uint32_t)(t.numel % kBlock);
+        const size_t e0 = (size_t)(t.numel / kBlock) * kBlock;
+        for (uint32_t i = lane; i < n; i += kWave)
+            store1<BF16>(t.a, e0 + i, ema_elem(load1<BF16>(t.a, e0 + i), load1<BF16>(t.b, e0 + i), decay, omd));
+    }
+    uint32_t ti = 0;
+    for (uint32_t blk = wave; blk < total_blocks; blk += stride) {
+        ti = find_elem_row(rows, n_rows, ti, blk);
+        const ElemRow t = rows[ti];
+        const size_t e0 = (size_t)(blk - t.full_start) * kBlock;
+        char *s = static_cast<char *>(t.a) + e0 * (BF16 ? 2 : 4);
+        const char *p = static_cast<const char *>(t.b) + e0 * (BF16 ? 2 : 4);
+        Raw8<BF16> sr[4], pr[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            sr[c].load(s, c * 512 + lane * 8);
+            pr[c].load(p, c * 512 + lane * 8);
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            float sv[8], pv[8], out[8];
+            sr[c].unpack(sv);
+            pr[c].unpack(pv);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) out[k] = ema_elem(sv[k], pv[k], decay, omd);
+            store8<BF16>(s, c * 512 + lane * 8, out);
+        }
+    }
+}
+
+int launch_adamw32(const ElemRow *rows, uint32_t n_rows, uint32_t total_blocks, int dtype_tag,
+                   const EriAdamW32Hyper &h, uint32_t grid, void *stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype_tag == ERI_DTYPE_F32)
+        hipLaunchKernelGGL(adamw32_kernel<false>, dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, h);
+    else
+        hipLaunchKernelGGL(adamw32_kernel<true>, dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, h);
+    return (int)hipGetLastError();
+}
+
+int launch_ema(const ElemRow *rows, uint32_t n_rows, uint32_t total_blocks, int dtype_tag, float decay,
+               uint32_t grid, void *stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype_tag == ERI_DTYPE_F32)
+        hipLaunchKernelGGL(ema_kernel<false>, dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, decay);
+    else
+        hipLaunchKernelGGL(ema_kernel<true>, dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, decay);
+    return (int)hipGetLastError();
+}
+
 } // namespace eri

@@ -747,3 +747,140 @@ int eri_adam8_quantize(const float *x, int signed_map, uint64_t numel, uint8_t *
 }
 
 } // extern "C"
+
+// ---- plain sweeps: 32-bit AdamW, EMA ---------------------------------------------------------
+
+namespace {
+
+/* Device copy of a row table that changes rarely: re-uploaded only when the rows differ from the
+ * last call, through a pinned mirror whose previous copy is waited for before it is overwritten. */
+struct ElemCache {
+    struct Group {
+        std::vector<eri::ElemRow> rows;
+        eri::ElemRow *dev = nullptr, *pinned = nullptr;
+        uint32_t cap = 0, total_blocks = 0;
+    };
+    Group groups[2]; // F32, BF16
+    hipEvent_t ev = nullptr;
+    bool pending = false;
+    int device = -1;
+    ~ElemCache() {
+        for (auto &g : groups) {
+            if (g.dev) (void)hipFree(g.dev);
+            if (g.pinned) (void)hipHostFree(g.pinned);
+        }
+        if (ev) (void)hipEventDestroy(ev);
+    }
+    int sync(void *stream, uint32_t cus, int (*launch)(const eri::ElemRow *, uint32_t, uint32_t, int, uint32_t, void *, const void *),
+             const void *extra) {
+        int dev = 0;
+        ERI_HIP(hipGetDevice(&dev));
+        if (!ev) ERI_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+        for (int gi = 0; gi < 2; ++gi) {
+            Group &g = groups[gi];
+            const uint32_t n = (uint32_t)g.rows.size();
+            if (n == 0) continue;
+            bool same = dev == device && g.cap >= n && std::memcmp(g.pinned, g.rows.data(), n * sizeof(eri::ElemRow)) == 0;
+            if (!same) {
+                if (pending) {
+                    ERI_HIP(hipEventSynchronize(ev));
+                    pending = false;
+                }
+                if (g.cap < n || dev != device) {
+                    if (g.dev) (void)hipFree(g.dev);
+                    if (g.pinned) (void)hipHostFree(g.pinned);
+                    g.dev = g.pinned = nullptr;
+                    g.cap = n + n / 2 + 16;
+                    ERI_HIP(hipMalloc((void **)&g.dev, sizeof(eri::ElemRow) * g.cap));
+                    ERI_HIP(hipHostMalloc((void **)&g.pinned, sizeof(eri::ElemRow) * g.cap, hipHostMallocDefault));
+                }
+                std::memcpy(g.pinned, g.rows.data(), n * sizeof(eri::ElemRow));
+                ERI_HIP(hipMemcpyAsync(g.dev, g.pinned, n * sizeof(eri::ElemRow), hipMemcpyHostToDevice,
+                                       static_cast<hipStream_t>(stream)));
+                ERI_HIP(hipEventRecord(ev, static_cast<hipStream_t>(stream)));
+                pending = true;
+            }
+            const eri::ElemRow &last = g.rows.back();
+            const uint32_t total = last.full_start + (uint32_t)(last.numel / eri::kBlock);
+            const uint32_t work = total > n ? total : n;
+            uint32_t grid = (work + 3) / 4;
+            if (grid > cus * 16) grid = cus * 16;
+            int rc = launch(g.dev, n, total, gi == 0 ? ERI_DTYPE_F32 : ERI_DTYPE_BF16, grid, stream, extra);
+            if (rc) return hip_fail((hipError_t)rc, "element-wise sweep launch");
+        }
+        device = dev;
+        return 0;
+    }
+};
+
+int check_elem(const void *a, const void *b, uint64_t numel, int dtype, uint32_t i, uint64_t &blocks) {
+    char buf[128];
+    if (!a || !b) { std::snprintf(buf, sizeof buf, "row %u: NULL pointer", i); return fail(ERI_ERR_NULL, buf); }
+    if (numel == 0) { std::snprintf(buf, sizeof buf, "row %u: empty tensor", i); return fail(ERI_ERR_EMPTY, buf); }
+    if (dtype != ERI_DTYPE_F32 && dtype != ERI_DTYPE_BF16) { std::snprintf(buf, sizeof buf, "row %u: unsupported dtype tag %d", i, dtype); return fail(ERI_ERR_DTYPE, buf); }
+    if (((uintptr_t)a | (uintptr_t)b) & 15u) { std::snprintf(buf, sizeof buf, "row %u: pointers must be 16-byte aligned", i); return fail(ERI_ERR_ALIGN, buf); }
+    blocks += numel / eri::kBlock;
+    if (blocks > 0x7fffffffull) return fail(ERI_ERR_TOO_LARGE, "more than 2^31 - 1 blocks in one call");
+    return 0;
+}
+
+int adamw32_launch(const eri::ElemRow *rows, uint32_t n, uint32_t total, int dtype, uint32_t grid, void *stream, const void *extra) {
+    return eri::launch_adamw32(rows, n, total, dtype, *static_cast<const EriAdamW32Hyper *>(extra), grid, stream);
+}
+int ema_launch(const eri::ElemRow *rows, uint32_t n, uint32_t total, int dtype, uint32_t grid, void *stream, const void *extra) {
+    return eri::launch_ema(rows, n, total, dtype, *static_cast<const float *>(extra), grid, stream);
+}
+
+} // namespace
+
+extern "C" {
+
+int eri_adamw32_step_multi(const EriAdamW32Tensor *rows, uint32_t n, const EriAdamW32Hyper *hyper, void *stream) {
+    if (!rows || !hyper) return fail(ERI_ERR_NULL, "rows or hyper is NULL");
+    if (n == 0) return fail(ERI_ERR_ARG, "no rows");
+    thread_local ElemCache cache;
+    DeviceCtx *ctx = nullptr;
+    int rc = get_ctx(&ctx);
+    for (auto &g : cache.groups) g.rows.clear();
+    uint64_t blocks = 0;
+    uint32_t starts[2] = {0, 0};
+    for (uint32_t i = 0; i < n; ++i) {
+        const EriAdamW32Tensor &r = rows[i];
+        int e = check_elem(r.p, r.g, r.numel, r.dtype_tag, i, blocks);
+        if (e) return e;
+        if (!r.m || !r.v) return fail(ERI_ERR_NULL, "moment pointer is NULL");
+        if (((uintptr_t)r.m | (uintptr_t)r.v) & 15u) return fail(ERI_ERR_ALIGN, "moment pointers must be 16-byte aligned");
+        const int gi = r.dtype_tag == ERI_DTYPE_F32 ? 0 : 1;
+        eri::ElemRow d;
+        d.a = r.p; d.b = r.g; d.c = r.m; d.d = r.v; d.numel = r.numel; d.full_start = starts[gi]; d.pad = 0;
+        starts[gi] += (uint32_t)(r.numel / eri::kBlock);
+        cache.groups[gi].rows.push_back(d);
+    }
+    if (rc) return rc;
+    return cache.sync(stream, ctx->cus, adamw32_launch, hyper);
+}
+
+int eri_ema_update_multi(const EriEmaTensor *rows, uint32_t n, float decay, void *stream) {
+    if (!rows) return fail(ERI_ERR_NULL, "rows is NULL");
+    if (n == 0) return fail(ERI_ERR_ARG, "no rows");
+    thread_local ElemCache cache;
+    DeviceCtx *ctx = nullptr;
+    int rc = get_ctx(&ctx);
+    for (auto &g : cache.groups) g.rows.clear();
+    uint64_t blocks = 0;
+    uint32_t starts[2] = {0, 0};
+    for (uint32_t i = 0; i < n; ++i) {
+        const EriEmaTensor &r = rows[i];
+        int e = check_elem(r.shadow, r.p, r.numel, r.dtype_tag, i, blocks);
+        if (e) return e;
+        const int gi = r.dtype_tag == ERI_DTYPE_F32 ? 0 : 1;
+        eri::ElemRow d;
+        d.a = r.shadow; d.b = r.p; d.c = nullptr; d.d = nullptr; d.numel = r.numel; d.full_start = starts[gi]; d.pad = 0;
+        starts[gi] += (uint32_t)(r.numel / eri::kBlock);
+        cache.groups[gi].rows.push_back(d);
+    }
+    if (rc) return rc;
+    return cache.sync(stream, ctx->cus, ema_launch, &decay);
+}
+
+} // extern "C"

@@ -39,6 +39,16 @@ pub struct EriAdam8bitConfig {
     pub amsgrad: i32, pub block_wise: i32, pub percentile_clipping: u64,
 }
 
+#[repr(C)]
+#[derive(Clone, Copy)]
+pub struct EriAdamW32Tensor { pub p: *mut c_void, pub g: *const c_void, pub m: *mut f32, pub v: *mut f32, pub numel: u64, pub dtype_tag: i32, pub reserved: i32 }
+#[repr(C)]
+#[derive(Clone, Copy)]
+pub struct EriAdamW32Hyper { pub lr: f32, pub beta1: f32, pub beta2: f32, pub eps: f32, pub weight_decay: f32 }
+#[repr(C)]
+#[derive(Clone, Copy)]
+pub struct EriEmaTensor { pub shadow: *mut c_void, pub p: *const c_void, pub numel: u64, pub dtype_tag: i32, pub reserved: i32 }
+
 pub enum EriAdam8Table {}
 pub enum EriParameter {}
 pub enum EriAdam8bit {}
@@ -77,6 +87,9 @@ extern "C" {
     pub fn eri_adam8_step_multi(rows: *const EriAdam8Tensor, n: u32, hyper: *const EriAdam8Hyper, stream: *mut c_void) -> c_int;
     pub fn eri_adam8_dequantize(codes: *const u8, absmax: *const f32, signed_map: c_int, numel: u64, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn eri_adam8_quantize(x: *const f32, signed_map: c_int, numel: u64, codes: *mut u8, absmax: *mut f32, stream: *mut c_void) -> c_int;
+    // 32-bit sibling and EMA sweep
+    pub fn eri_adamw32_step_multi(rows: *const EriAdamW32Tensor, n: u32, hyper: *const EriAdamW32Hyper, stream: *mut c_void) -> c_int;
+    pub fn eri_ema_update_multi(rows: *const EriEmaTensor, n: u32, decay: f32, stream: *mut c_void) -> c_int;
     // optimizer objects
     pub fn eri_param_create(data: *mut c_void, numel: u64, dtype_tag: c_int, out: *mut *mut EriParameter) -> c_int;
     pub fn eri_param_set_grad(param: *mut EriParameter, grad: *const c_void) -> c_int;

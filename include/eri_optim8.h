@@ -182,6 +182,43 @@ int eri_adam8_dequantize(const uint8_t *codes, const float *absmax, int signed_m
 int eri_adam8_quantize(const float *x, int signed_map, uint64_t numel, uint8_t *codes, float *absmax,
                        void *stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * 32-bit sibling: fused multi-tensor AdamW with fp32 moments, for tensors kept out of the 8-bit
+ * path.  Arithmetic of AdamW::step_with_grads (crates/common/optim/src/adamw.rs:20-58), one rounded
+ * fp32 operation per line there: no bias correction, decoupled decay,
+ *   m = m*b1 + g*(1-b1);  v = v*b2 + (g*g)*(1-b2);  p = p + ((m/(sqrt(v)+eps)) + p*wd) * (-lr)
+ * with p cast back to its dtype.  It replaces one launch and one temporary per operation there, and
+ * the never-built fused kernels of src/kernels/fused_adam.cu:108-148.
+ * ------------------------------------------------------------------------------------------- */
+typedef struct EriAdamW32Tensor {
+    void *p;          /* F32 or BF16, updated in place */
+    const void *g;    /* same dtype as p */
+    float *m;         /* fp32 first moment, numel elements */
+    float *v;         /* fp32 second moment */
+    uint64_t numel;
+    int32_t dtype_tag;
+    int32_t reserved;
+} EriAdamW32Tensor;
+
+typedef struct EriAdamW32Hyper {
+    float lr, beta1, beta2, eps, weight_decay; /* AdamWCfg, adamw.rs:7-8; lr is the per-call argument */
+} EriAdamW32Hyper;
+
+/* One launch per dtype over all rows; keeps a cached device copy of the rows per calling thread. */
+int eri_adamw32_step_multi(const EriAdamW32Tensor *rows, uint32_t n, const EriAdamW32Hyper *hyper, void *stream);
+
+/* Exponential moving average of parameters, shadow = decay*shadow + (1-decay)*p in fp32
+ * (EMA update, src/trainers/ema_enhanced.rs:79-108), one launch over all rows.
+ * `shadow` has the dtype of p. */
+typedef struct EriEmaTensor {
+    void *shadow;
+    const void *p;
+    uint64_t numel;
+    int32_t dtype_tag;
+    int32_t reserved;
+} EriEmaTensor;
+int eri_ema_update_multi(const EriEmaTensor *rows, uint32_t n, float decay, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -23,6 +23,10 @@
  *                              quantiser bypassed, block-max brute force, and bit-for-bit
  *                              agreement with the independent NumPy restatement
  *                              (oracle/adam8_numpy.py)                              pinned
+ *   eri_oracle_adamw32_step    closed form at step 1, float64 recurrence, the reference's
+ *                              own 2x2 test case                                     pinned
+ *   eri_oracle_ema_update      float64 closed form; bf16 intermediate rounding of flame-core
+ *                              unknown                                               parity unpinned (bf16)
  *   bit-level equality with the reference's own legacy per-tensor linear format
  *   (adam8bit.rs:211-241, flame-core's to_dtype(U8)/round semantics are absent)     parity unpinned
  *
@@ -265,6 +269,51 @@ void eri_oracle_quantize(const float *x, const float *map, uint64_t numel, uint8
             codes[base + i] = (uint8_t)eri_oracle_nearest_index(mid, q);
         }
         absmax[b] = a;
+    }
+}
+
+/* ---- 32-bit sibling and EMA ------------------------------------------------------------------ */
+
+/* AdamW::step_with_grads, crates/common/optim/src/adamw.rs:20-58: fp32 math on fp32 moments, no bias
+ * correction, decoupled decay, parameter cast back to its dtype.  Pinned by closed forms at the
+ * first step, a float64 recurrence and the reference's own test case (2x2 bf16 ones, grad ones,
+ * src/tests/adamw_step.rs:6-30). */
+void eri_oracle_adamw32_step(void *p, const void *g, float *m, float *v, uint64_t numel, int dtype, float lr,
+                             float beta1, float beta2, float eps, float wd) {
+    const float omb1 = 1.0f - beta1, omb2 = 1.0f - beta2, neg_lr = -lr;
+    for (uint64_t i = 0; i < numel; ++i) {
+        float pf = load_elem(p, i, dtype), gr = load_elem(g, i, dtype);
+        float ms = m[i] * beta1;       /* :35 */
+        float gs = gr * omb1;          /* :36 */
+        float mn = ms + gs;            /* :37 */
+        float vs = v[i] * beta2;       /* :40 */
+        float g2 = gr * gr;            /* :41 */
+        float g2s = g2 * omb2;         /* :42 */
+        float vn = vs + g2s;           /* :43 */
+        float denom = sqrtf(vn) + eps; /* :46 */
+        float update = mn / denom;     /* :47 */
+        float w = wd != 0.0f ? pf * wd : 0.0f; /* :50 */
+        float total = update + w;      /* :51 */
+        float step = total * neg_lr;   /* :52 */
+        float pn = pf + step;
+        m[i] = mn;
+        v[i] = vn;
+        if (dtype == ERI_ORACLE_F32) ((float *)p)[i] = pn;
+        else ((uint16_t *)p)[i] = eri_oracle_f32_to_bf16(pn); /* :55 */
+    }
+}
+
+/* EMA update, src/trainers/ema_enhanced.rs:91-100: shadow = shadow*decay + p*(1 - decay) in fp32,
+ * cast to the tensors' dtype.  Whether flame-core rounds the two products to bf16 first for bf16
+ * tensors cannot be read from the tree: parity unpinned for that detail. */
+void eri_oracle_ema_update(void *shadow, const void *p, uint64_t numel, int dtype, float decay) {
+    const float omd = 1.0f - decay;
+    for (uint64_t i = 0; i < numel; ++i) {
+        float a = load_elem(shadow, i, dtype) * decay;
+        float b = load_elem(p, i, dtype) * omd;
+        float s = a + b;
+        if (dtype == ERI_ORACLE_F32) ((float *)shadow)[i] = s;
+        else ((uint16_t *)shadow)[i] = eri_oracle_f32_to_bf16(s);
     }
 }
 

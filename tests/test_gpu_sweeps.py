@@ -1,0 +1,96 @@
+"""GPU parity of the 32-bit AdamW sibling and the EMA sweep against the oracle (bit-exact: every
+operation is an individually rounded fp32 operation on both sides)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle_c as oc
+from oracle import adam8_numpy as onp
+
+pytestmark = pytest.mark.gpu
+SIZES = [2048 * 3 + 17, 5, 2048, 4100, 640 * 16]
+
+
+def _up(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.uint8).reshape(-1).copy()).cuda()
+
+
+def _down(t, dtype):
+    return t.cpu().numpy().view(dtype)
+
+
+@pytest.mark.parametrize("bf16", [True, False])
+@pytest.mark.parametrize("wd", [0.01, 0.0])
+def test_adamw32_multi_tensor(bf16, wd):
+    import torch
+    from eridiffusion_amd import _lib as L
+    rng = np.random.default_rng(3 + bf16)
+    dt = np.uint16 if bf16 else np.float32
+    tag = 2 if bf16 else 0
+    ps, ms, vs = [], [], []
+    for n in SIZES:
+        p = (rng.standard_normal(n) * 0.02).astype(np.float32)
+        ps.append(onp.f32_to_bf16(p) if bf16 else p)
+        ms.append(np.zeros(n, np.float32))
+        vs.append(np.zeros(n, np.float32))
+    dp, dm, dv = [_up(a) for a in ps], [_up(a) for a in ms], [_up(a) for a in vs]
+    rows = (L.AdamW32Row * len(SIZES))()
+    h = L.AdamW32Hyper(1e-3, 0.9, 0.999, 1e-8, wd)
+    for step in range(3):
+        gs = []
+        for n in SIZES:
+            g = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+            gs.append(onp.f32_to_bf16(g) if bf16 else g)
+        dg = [_up(a) for a in gs]
+        for i, n in enumerate(SIZES):
+            rows[i].p, rows[i].g, rows[i].m, rows[i].v = dp[i].data_ptr(), dg[i].data_ptr(), dm[i].data_ptr(), dv[i].data_ptr()
+            rows[i].numel, rows[i].dtype_tag = n, tag
+            oc.lib().eri_oracle_adamw32_step(oc.ptr(ps[i]), oc.ptr(gs[i]), oc.ptr(ms[i]), oc.ptr(vs[i]), n, tag,
+                                             1e-3, 0.9, 0.999, 1e-8, wd)
+        L.check(L.lib().eri_adamw32_step_multi(rows, len(SIZES), C.byref(h), torch.cuda.current_stream().cuda_stream), "adamw32")
+        torch.cuda.synchronize()
+    for i in range(len(SIZES)):
+        assert np.array_equal(_down(dp[i], dt).view(np.uint16 if bf16 else np.uint32), ps[i].view(np.uint16 if bf16 else np.uint32))
+        assert np.array_equal(_down(dm[i], np.uint32), ms[i].view(np.uint32))
+        assert np.array_equal(_down(dv[i], np.uint32), vs[i].view(np.uint32))
+
+
+@pytest.mark.parametrize("bf16", [True, False])
+def test_ema_multi_tensor(bf16):
+    import torch
+    from eridiffusion_amd import _lib as L
+    rng = np.random.default_rng(9)
+    dt = np.uint16 if bf16 else np.float32
+    tag = 2 if bf16 else 0
+    sh, ps = [], []
+    for n in SIZES:
+        a = rng.standard_normal(n).astype(np.float32)
+        b = rng.standard_normal(n).astype(np.float32)
+        sh.append(onp.f32_to_bf16(a) if bf16 else a)
+        ps.append(onp.f32_to_bf16(b) if bf16 else b)
+    ds, dp = [_up(a) for a in sh], [_up(a) for a in ps]
+    rows = (L.EmaRow * len(SIZES))()
+    for i, n in enumerate(SIZES):
+        rows[i].shadow, rows[i].p, rows[i].numel, rows[i].dtype_tag = ds[i].data_ptr(), dp[i].data_ptr(), n, tag
+    for decay in (0.999, 0.9):
+        L.check(L.lib().eri_ema_update_multi(rows, len(SIZES), decay, torch.cuda.current_stream().cuda_stream), "ema")
+        for i, n in enumerate(SIZES):
+            oc.lib().eri_oracle_ema_update(oc.ptr(sh[i]), oc.ptr(ps[i]), n, tag, decay)
+    torch.cuda.synchronize()
+    for i in range(len(SIZES)):
+        assert np.array_equal(_down(ds[i], dt).view(np.uint16 if bf16 else np.uint32), sh[i].view(np.uint16 if bf16 else np.uint32))
+        assert np.array_equal(_down(dp[i], dt), ps[i])
+
+
+def test_sweep_argument_errors():
+    from eridiffusion_amd import _lib as L
+    rows = (L.EmaRow * 1)()
+    rows[0].shadow, rows[0].p, rows[0].numel, rows[0].dtype_tag = 0x1000, 0x2000, 0, 2
+    assert L.lib().eri_ema_update_multi(rows, 1, 0.9, None) == -3
+    rows[0].numel, rows[0].dtype_tag = 8, 1
+    assert L.lib().eri_ema_update_multi(rows, 1, 0.9, None) == -4
+    rows[0].dtype_tag, rows[0].p = 2, 0x2004
+    assert L.lib().eri_ema_update_multi(rows, 1, 0.9, None) == -2
+    assert L.lib().eri_ema_update_multi(None, 1, 0.9, None) == -1

@@ -1,0 +1,73 @@
+"""Pins the oracle's 32-bit AdamW and EMA restatements."""
+import numpy as np
+import torch
+
+import oracle_c as oc
+from oracle import adam8_numpy as onp
+
+
+def adamw(p, g, m, v, dtype, lr=1e-3, b1=0.9, b2=0.999, eps=1e-8, wd=0.01):
+    oc.lib().eri_oracle_adamw32_step(oc.ptr(p), oc.ptr(g), oc.ptr(m), oc.ptr(v), m.size, dtype, lr, b1, b2, eps, wd)
+
+
+def test_reference_test_case_two_by_two_bf16_ones():
+    # crates/common/optim/src/tests/adamw_step.rs:6-30: param = 1.0 (bf16, 2x2), grad = 1.0, one step
+    # with lr 1e-3, betas (0.9, 0.999), eps 1e-8, wd 0.01; the reference asserts sum |delta| > 0
+    one = onp.f32_to_bf16(np.ones(4, np.float32))
+    p, g = one.copy(), one.copy()
+    m, v = np.zeros(4, np.float32), np.zeros(4, np.float32)
+    adamw(p, g, m, v, oc.DT_BF16)
+    delta = np.abs(onp.bf16_to_f32(p) - 1.0).sum()
+    assert delta > 0
+    # closed form: m = 0.1, v = 0.001, update = 0.1/sqrt(0.001) = 3.1623, p = 1 - 1e-3*(3.1623 + 0.01) = 0.99683
+    want = torch.tensor(1 - 1e-3 * (0.1 / np.sqrt(0.001) + 0.01)).to(torch.bfloat16).float().item()
+    assert np.all(onp.bf16_to_f32(p) == np.float32(want))
+    assert np.allclose(m, 0.1, rtol=1e-6) and np.allclose(v, 0.001, rtol=2e-5)
+
+
+def test_adamw32_tracks_a_float64_recurrence_without_bias_correction():
+    rng = np.random.default_rng(0)
+    n = 5000
+    p0 = rng.standard_normal(n).astype(np.float32)
+    p = p0.copy()
+    m, v = np.zeros(n, np.float32), np.zeros(n, np.float32)
+    P, M, V = p0.astype(np.float64), np.zeros(n), np.zeros(n)
+    b1, b2 = float(np.float32(0.9)), float(np.float32(0.999))
+    for t in range(30):
+        g = (rng.standard_normal(n) * 1e-2).astype(np.float32)
+        adamw(p, g, m, v, oc.DT_F32, lr=1e-3, wd=0.01)
+        G = g.astype(np.float64)
+        M = b1 * M + (1 - b1) * G
+        V = b2 * V + (1 - b2) * G * G
+        P = P - 1e-3 * (M / (np.sqrt(V) + 1e-8) + float(np.float32(0.01)) * P)
+    assert np.allclose(p, P, rtol=0, atol=5e-6) and np.abs(P - p0).mean() > 1e-2
+    assert np.allclose(m, M, rtol=1e-5, atol=1e-9) and np.allclose(v, V, rtol=1e-4, atol=1e-12)
+
+
+def test_adamw32_zero_decay_leaves_no_decay_term():
+    rng = np.random.default_rng(1)
+    p0 = rng.standard_normal(64).astype(np.float32)
+    g = np.zeros(64, np.float32)
+    p = p0.copy()
+    adamw(p, g, np.zeros(64, np.float32), np.zeros(64, np.float32), oc.DT_F32, wd=0.0)
+    assert np.array_equal(p, p0)  # zero grad, zero state, no decay: 0/(0+eps) = 0
+    p = p0.copy()
+    adamw(p, g, np.zeros(64, np.float32), np.zeros(64, np.float32), oc.DT_F32, wd=0.5, lr=0.1)
+    assert np.allclose(p, p0 * (1 - 0.05), rtol=1e-6)
+
+
+def test_ema_is_a_convex_combination():
+    rng = np.random.default_rng(2)
+    s0 = rng.standard_normal(1000).astype(np.float32)
+    p = rng.standard_normal(1000).astype(np.float32)
+    s = s0.copy()
+    oc.lib().eri_oracle_ema_update(oc.ptr(s), oc.ptr(p), 1000, oc.DT_F32, 0.999)
+    d = float(np.float32(0.999))
+    assert np.allclose(s, d * s0.astype(np.float64) + (1 - d) * p, rtol=0, atol=3e-7)
+    same = p.copy()
+    oc.lib().eri_oracle_ema_update(oc.ptr(same), oc.ptr(p), 1000, oc.DT_F32, 0.5)
+    assert np.array_equal(same, p)  # shadow == p is a fixed point when decay = 0.5 (exact halves)
+    sb, pb = onp.f32_to_bf16(s0), onp.f32_to_bf16(p)
+    oc.lib().eri_oracle_ema_update(oc.ptr(sb), oc.ptr(pb), 1000, oc.DT_BF16, 0.9)
+    want = 0.9 * onp.bf16_to_f32(onp.f32_to_bf16(s0)).astype(np.float64) + 0.1 * onp.bf16_to_f32(pb)
+    assert np.all(np.abs(onp.bf16_to_f32(sb) - want) <= np.abs(want) * 2 ** -8 + 1e-30)
