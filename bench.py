@@ -30,6 +30,9 @@ def parse():
     ap.add_argument("--config", default="c5_flux12b_full")
     ap.add_argument("--flags", type=int, default=0, help="ERI_ADAM8_FLAG_* bits for the step")
     ap.add_argument("--cpu-sample", type=int, default=512 << 20, help="parameters in the CPU baseline sample (0 = skip)")
+    ap.add_argument("--kernel", choices=["adam8", "adam8_clip", "grad_norm", "adamw32", "ema"], default="adam8",
+                    help="what one step is: the 8-bit AdamW step (headline), the same preceded by the device-side "
+                         "gradient norm, the norm alone, the 32-bit AdamW sibling, or the EMA sweep")
     ap.add_argument("--alloc", choices=["arena", "tensor"], default="arena",
                     help="one flat allocation per kind of buffer, or one allocation per tensor and buffer")
     ap.add_argument("--calibrate-copy", type=int, default=0,
@@ -188,9 +191,45 @@ def main():
     table = C.c_void_p()
     L.check(L.lib().eri_adam8_table_create(rows, len(rows), stream, C.byref(table)), "table_create")
     hyper_args = (1e-4, 0.9, 0.999, 1e-8, 0.01)
+    bytes_per_param = BYTES_PER_PARAM[dt_name]
+    extra = []
+    if args.kernel == "adamw32":
+        a_m32 = Alloc(torch, [4 * n for n in sizes])
+        a_v32 = Alloc(torch, [4 * n for n in sizes])
+        extra += [a_m32, a_v32]
+        rows32 = (L.AdamW32Row * len(sizes))()
+        for i, n in enumerate(sizes):
+            rows32[i].p, rows32[i].g, rows32[i].m, rows32[i].v = a_p.ptr(i), a_g.ptr(i), a_m32.ptr(i), a_v32.ptr(i)
+            rows32[i].numel, rows32[i].dtype_tag = n, (L.DTYPE_BF16 if bf16 else L.DTYPE_F32)
+        h32 = L.AdamW32Hyper(1e-4, 0.9, 0.999, 1e-8, 0.01)
+        bytes_per_param = 3 * esz + 16
+    elif args.kernel == "ema":
+        a_sh = Alloc(torch, [n * esz for n in sizes])
+        extra.append(a_sh)
+        rows_e = (L.EmaRow * len(sizes))()
+        for i, n in enumerate(sizes):
+            rows_e[i].shadow, rows_e[i].p, rows_e[i].numel = a_sh.ptr(i), a_p.ptr(i), n
+            rows_e[i].dtype_tag = L.DTYPE_BF16 if bf16 else L.DTYPE_F32
+        bytes_per_param = 3 * esz
+    elif args.kernel == "grad_norm":
+        bytes_per_param = esz + 4.0 / 2048
+    elif args.kernel == "adam8_clip":
+        bytes_per_param += esz + 4.0 / 2048
 
     def step(t):
-        h = L.hyper_pack(*hyper_args, t, L.MODE_ERI, args.flags)
+        if args.kernel == "adamw32":
+            L.check(L.lib().eri_adamw32_step_multi(rows32, len(sizes), C.byref(h32), stream), "adamw32")
+            return
+        if args.kernel == "ema":
+            L.check(L.lib().eri_ema_update_multi(rows_e, len(sizes), 0.999, stream), "ema")
+            return
+        flags = args.flags
+        if args.kernel in ("grad_norm", "adam8_clip"):
+            L.check(L.lib().eri_adam8_grad_norm(table, 1.0, 0.0, stream), "grad_norm")
+            if args.kernel == "grad_norm":
+                return
+            flags |= L.FLAG_CLIP_FROM_TABLE
+        h = L.hyper_pack(*hyper_args, t, L.MODE_ERI, flags)
         L.check(L.lib().eri_adam8_step_table(table, C.byref(h), stream), "step_table")
 
     t = 0
@@ -210,17 +249,17 @@ def main():
     launch_ms = [a.elapsed_time(b) for a, b in ev]
     avg_launch_s = sum(launch_ms) / len(launch_ms) / 1e3
 
-    algo_bytes = BYTES_PER_PARAM[dt_name] * n_params
+    algo_bytes = bytes_per_param * n_params
     achieved = algo_bytes / avg_launch_s / 1e9
     traffic = None
     if os.path.exists(args.traffic_json):
         try:
             with open(args.traffic_json) as f:
-                traffic = json.load(f).get(args.config)
+                traffic = json.load(f).get(args.config) if args.kernel == "adam8" else None
         except Exception:
             traffic = None
     out = {
-        "metric": "params/sec per 8-bit AdamW step",
+        "metric": "params/sec per 8-bit AdamW step" if args.kernel == "adam8" else "params/sec per %s step" % args.kernel,
         "value": n_params * args.steps / wall,
         "unit": "params/s",
         "n_gpus": 1,
@@ -233,7 +272,7 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": args.config, "tensors": len(sizes), "params": n_params, "blocks": n_blocks,
-                   "param_dtype": dt_name, "state": "uint8 m/v + fp32 absmax per 2048-block", "flags": args.flags,
+                   "kernel": args.kernel, "param_dtype": dt_name, "state": "uint8 m/v + fp32 absmax per 2048-block", "flags": args.flags,
                    "resident_gb": round((n_params * (2 * esz + 2) + n_blocks * 8) / 1e9, 2)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                      "frac": achieved / PEAK_HBM_GBPS, "traffic": traffic,
@@ -241,7 +280,7 @@ def main():
                      "algorithmic_bytes": algo_bytes},
     }
     L.lib().eri_adam8_table_destroy(table)
-    for a in (a_p, a_g, a_m, a_v, a_am, a_av):
+    for a in [a_p, a_g, a_m, a_v, a_am, a_av] + extra:
         a.free()
     if args.cpu_sample > 0:
         out["cpu_baseline"] = cpu_baseline(tensors, bf16, args.cpu_sample, hyper_args)

@@ -71,11 +71,11 @@ static_assert(kLdsImageBytes % 16 == 0, "the image is staged in 16-byte words");
 int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_blocks, int dtype_tag,
                 const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg,
                 void *stream);
-/* Gradient norm: per-block sums of squares into partial[0 .. total_full_blocks + n_rows), then norm and
- * clip factor into out[0], out[1]. */
+/* Gradient norm: one f64 partial per wave (grid * 4 of them), then norm and clip factor into out[0], out[1]. */
+constexpr uint32_t kNormWavesPerWg = 4;
 int launch_grad_sumsq(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_blocks, int dtype_tag,
-                      float *partial, uint32_t grid, void *stream);
-int launch_grad_norm_finish(const float *partial, uint32_t n, float max_norm, float denom_eps, float *out,
+                      double *partial, uint32_t grid, void *stream);
+int launch_grad_norm_finish(const double *partial, uint32_t n, float max_norm, float denom_eps, float *out,
                             void *stream);
 int launch_state_init(uint8_t *m, uint8_t *v, float *absmax_m, float *absmax_v, uint64_t numel, void *stream);
 int launch_dequantize(const uint8_t *codes, const float *absmax, int signed_map, uint64_t numel, float *out,

@@ -834,7 +834,8 @@ int launch_quantize(const float *x, int signed_map, uint64_t numel, uint8_t *cod
 // ------------------------------------------------------------------------------------------
 // global gradient norm over the launch table (the trainers' clip_gradients,
 // src/trainers/pipeline_flux_lora_sequential.rs:1198-1213,1939-1950), without a host round trip:
-// pass 1 leaves one fp32 sum of squares per block, pass 2 adds them in f64 and writes the norm and
+// pass 1 forms one fp32 sum of squares per block and adds a wave's blocks in f64, pass 2 adds the waves'
+// partials and writes the norm and
 // the clip factor to device memory, where the step kernel reads it.
 // ------------------------------------------------------------------------------------------
 
@@ -853,12 +854,14 @@ __device__ __forceinline__ float wave_sum(float x) {
 
 template <bool BF16>
 __global__ __launch_bounds__(256) void grad_sumsq_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
-                                                         uint32_t total_blocks, float *__restrict__ partial) {
+                                                         uint32_t total_blocks, double *__restrict__ partial) {
+    // persistent: every wave adds the fp32 sums of its blocks in f64 and leaves one partial
     const uint32_t lane = threadIdx.x & (kWave - 1);
     const uint32_t waves_per_wg = blockDim.x / kWave;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
     const uint32_t stride = gridDim.x * waves_per_wg;
-    for (uint32_t r = wave; r < n_rows; r += stride) { // partial last blocks; rows without one leave 0
+    double total = 0.0;
+    for (uint32_t r = wave; r < n_rows; r += stride) { // partial last blocks
         const DevTensor t = rows[r];
         const uint32_t n = (uint32_t)(t.numel % kBlock);
         const size_t e0 = (size_t)(t.numel / kBlock) * kBlock;
@@ -867,35 +870,35 @@ __global__ __launch_bounds__(256) void grad_sumsq_kernel(const DevTensor *__rest
             const float g = load1<BF16>(t.g, e0 + i);
             acc += g * g;
         }
-        acc = wave_sum(acc);
-        if (lane == 0) partial[total_blocks + r] = acc;
+        total += (double)wave_sum(acc);
     }
     uint32_t ti = 0;
     for (uint32_t blk = wave; blk < total_blocks; blk += stride) {
         ti = find_row(rows, n_rows, ti, blk);
         const DevTensor t = rows[ti];
         const size_t e0 = (size_t)(blk - t.full_start) * kBlock;
+        Raw8<BF16> raw[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) raw[c].load(static_cast<const char *>(t.g) + e0 * (BF16 ? 2 : 4), c * 512 + lane * 8);
         float acc = 0.0f;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            Raw8<BF16> raw;
-            raw.load(static_cast<const char *>(t.g) + e0 * (BF16 ? 2 : 4), c * 512 + lane * 8);
             float g[8];
-            raw.unpack(g);
+            raw[c].unpack(g);
 #pragma unroll
             for (int k = 0; k < 8; ++k) acc += g[k] * g[k];
         }
-        acc = wave_sum(acc);
-        if (lane == 0) partial[blk] = acc;
+        total += (double)wave_sum(acc);
     }
+    if (lane == 0) partial[wave] = total;
 }
 
-__global__ __launch_bounds__(1024) void grad_norm_finish_kernel(const float *__restrict__ partial, uint32_t n,
+__global__ __launch_bounds__(1024) void grad_norm_finish_kernel(const double *__restrict__ partial, uint32_t n,
                                                                 float max_norm, float denom_eps,
                                                                 float *__restrict__ out /* norm, scale */) {
     __shared__ double sh[1024];
     double acc = 0.0;
-    for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) acc += (double)partial[i];
+    for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) acc += partial[i];
     sh[threadIdx.x] = acc;
     __syncthreads();
     for (uint32_t s = blockDim.x / 2; s > 0; s >>= 1) {
@@ -912,7 +915,7 @@ __global__ __launch_bounds__(1024) void grad_norm_finish_kernel(const float *__r
     }
 }
 
-int launch_grad_sumsq(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, int dtype_tag, float *partial,
+int launch_grad_sumsq(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, int dtype_tag, double *partial,
                       uint32_t grid, void *stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype_tag == ERI_DTYPE_F32)
@@ -922,7 +925,7 @@ int launch_grad_sumsq(const DevTensor *rows, uint32_t n_rows, uint32_t total_blo
     return (int)hipGetLastError();
 }
 
-int launch_grad_norm_finish(const float *partial, uint32_t n, float max_norm, float denom_eps, float *out,
+int launch_grad_norm_finish(const double *partial, uint32_t n, float max_norm, float denom_eps, float *out,
                             void *stream) {
     hipLaunchKernelGGL(grad_norm_finish_kernel, dim3(1), dim3(1024), 0, static_cast<hipStream_t>(stream), partial, n,
                        max_norm, denom_eps, out);

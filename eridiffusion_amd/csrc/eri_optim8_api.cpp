@@ -264,7 +264,7 @@ struct EriAdam8Table {
     std::vector<int32_t> dtype;
     hipEvent_t uploaded = nullptr;
     bool upload_pending = false;
-    float *partial = nullptr;  // one sum of squares per block (full blocks, then one slot per row) per group
+    double *partial = nullptr; // one sum of squares per wave of the norm pass, per group
     float *norm_out = nullptr; // device: {norm, clip factor}
     uint32_t n_partial = 0;
 };
@@ -658,25 +658,22 @@ int eri_adam8_grad_norm(EriAdam8Table *t, float max_norm, float denom_eps, void 
     DeviceCtx *ctx = nullptr;
     int rc = get_ctx(&ctx);
     if (rc) return rc;
+    const uint32_t grid_cap = ctx->cus * 8; // persistent: 8 workgroups of 4 waves per compute unit
     if (!t->partial) {
-        uint32_t n = 0;
-        for (auto &g : t->groups)
-            if (g.n) n += g.total_blocks + g.n;
-        ERI_HIP(hipMalloc((void **)&t->partial, sizeof(float) * (n ? n : 1)));
+        ERI_HIP(hipMalloc((void **)&t->partial, sizeof(double) * 2 * grid_cap * eri::kNormWavesPerWg));
         ERI_HIP(hipMalloc((void **)&t->norm_out, sizeof(float) * 2));
-        t->n_partial = n;
     }
     uint32_t off = 0;
     for (auto &g : t->groups) {
         if (g.n == 0) continue;
         const uint32_t work = g.total_blocks > g.n ? g.total_blocks : g.n;
-        uint32_t grid = (work + 3) / 4;
-        const uint32_t cap = ctx->cus * 8;
-        if (grid > cap) grid = cap;
+        uint32_t grid = (work + eri::kNormWavesPerWg - 1) / eri::kNormWavesPerWg;
+        if (grid > grid_cap) grid = grid_cap;
         rc = eri::launch_grad_sumsq(g.dev, g.n, g.total_blocks, g.dtype, t->partial + off, grid, stream);
         if (rc) return hip_fail((hipError_t)rc, "gradient sum-of-squares launch");
-        off += g.total_blocks + g.n;
+        off += grid * eri::kNormWavesPerWg;
     }
+    t->n_partial = off;
     rc = eri::launch_grad_norm_finish(t->partial, t->n_partial, max_norm, denom_eps, t->norm_out, stream);
     if (rc) return hip_fail((hipError_t)rc, "gradient norm launch");
     return 0;
