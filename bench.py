@@ -33,6 +33,7 @@ def parse():
     ap.add_argument("--kernel", choices=["adam8", "adam8_clip", "grad_norm", "adamw32", "ema"], default="adam8",
                     help="what one step is: the 8-bit AdamW step (headline), the same preceded by the device-side "
                          "gradient norm, the norm alone, the 32-bit AdamW sibling, or the EMA sweep")
+    ap.add_argument("--variants", default="", help="comma-separated kernel variants to time interleaved (A/B tool)")
     ap.add_argument("--alloc", choices=["arena", "tensor"], default="arena",
                     help="one flat allocation per kind of buffer, or one allocation per tensor and buffer")
     ap.add_argument("--calibrate-copy", type=int, default=0,
@@ -232,6 +233,23 @@ def main():
         h = L.hyper_pack(*hyper_args, t, L.MODE_ERI, flags)
         L.check(L.lib().eri_adam8_step_table(table, C.byref(h), stream), "step_table")
 
+    if args.variants:
+        vs = [int(x) for x in args.variants.split(",")]
+        acc = {v: [] for v in vs}
+        t = 0
+        for rep in range(args.steps):
+            for v in vs:
+                L.check(L.lib().eri_adam8_set_tuning(0, v), "set_tuning")
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                t += 1
+                a.record()
+                step(t)
+                b.record()
+                torch.cuda.synchronize()
+                if rep >= args.warmup:
+                    acc[v].append(a.elapsed_time(b))
+        print(json.dumps({"variants_ms": {str(v): sum(x) / len(x) for v, x in acc.items()}}))
+        return
     t = 0
     for _ in range(args.warmup):
         t += 1

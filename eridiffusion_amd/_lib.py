@@ -74,6 +74,7 @@ EXPORTS = {
     "eri_hip_stream_destroy": (C.c_int, [C.c_void_p]),
     "eri_hip_mem_info": (C.c_int, [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
     "eri_adam8_init": (C.c_int, []),
+    "eri_adam8_set_tuning": (C.c_int, [C.c_int, C.c_int]),
     "eri_adam8_get_maps": (C.c_int, [C.c_void_p, C.c_void_p]),
     "eri_adam8_table_image": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_size_t), C.POINTER(C.c_uint32)]),
     "eri_adam8_hyper_pack": (C.c_int, [C.c_double] * 5 + [C.c_uint64, C.c_int, C.c_uint32, C.POINTER(Hyper)]),

@@ -71,6 +71,7 @@ static_assert(kLdsImageBytes % 16 == 0, "the image is staged in 16-byte words");
 int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_blocks, int dtype_tag,
                 const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg,
                 void *stream);
+extern int g_kernel_variant;
 /* Gradient norm: one f64 partial per wave (grid * 4 of them), then norm and clip factor into out[0], out[1]. */
 constexpr uint32_t kNormWavesPerWg = 4;
 int launch_grad_sumsq(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_blocks, int dtype_tag,

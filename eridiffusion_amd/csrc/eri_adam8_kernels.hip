@@ -571,7 +571,7 @@ struct RawBlock {
     }
 };
 
-template <int MODE, bool EXACT, bool WD, bool GS>
+template <int MODE, bool EXACT, bool WD, bool GS, int V = 0>
 __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTensor *__restrict__ rows,
                                                                    uint32_t n_rows, uint32_t total_blocks,
                                                                    EriAdam8Hyper h,
@@ -629,6 +629,7 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
         uint8_t *mc = t.m + e0;
         uint8_t *vc = t.v + e0;
         float mf[32], vf[32];
+        u32x4 pw[4]; // updated parameters, packed, stored after the next block's loads are out
         float lm = 0.0f, lv = 0.0f;
         const float a_m = raw.a_m, a_v = raw.a_v;
 #pragma unroll
@@ -651,7 +652,11 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
                 lm = fmaxf(lm, __builtin_fabsf(m));
                 lv = fmaxf(lv, __builtin_fabsf(v));
             }
-            store8<true>(p, o, pn);
+            pw[c].x = bf16_pair(pn[0], pn[1]);
+            pw[c].y = bf16_pair(pn[2], pn[3]);
+            pw[c].z = bf16_pair(pn[4], pn[5]);
+            pw[c].w = bf16_pair(pn[6], pn[7]);
+            if (V == 1) __builtin_nontemporal_store(pw[c], as_global(reinterpret_cast<u32x4 *>(p) + c * 64 + lane));
         }
         const float nam = wave_max(lm);
         const float nav = wave_max(lv);
@@ -660,17 +665,42 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
             as_global(t.absmax_v)[lb] = nav;
         }
         raw.issue(nt, pblk - nt.full_start, lane); // prefetch: in flight during the requantisation
+        if (V == 0 || V == 3) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                __builtin_nontemporal_store(pw[c], as_global(reinterpret_cast<u32x4 *>(p) + c * 64 + lane));
+        }
         const BlockDiv dm(nam, kKeyScale, kKeyScaleInv), dv(nav, kKeyScale, kKeyScaleInv);
         if (dm.fast && dv.fast) {
+            u32x2 mws[4], vws[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const uint32_t o = c * 512 + lane * 8;
-                u32x2 mw, vw;
-                requant8<true, true>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
-                __builtin_nontemporal_store(mw, as_global(reinterpret_cast<u32x2 *>(mc + o)));
-                __builtin_nontemporal_store(vw, as_global(reinterpret_cast<u32x2 *>(vc + o)));
+                requant8<true, true>(mf + c * 8, vf + c * 8, dm, dv, L, mws[c], vws[c]);
+                if (V != 3) {
+                    __builtin_nontemporal_store(mws[c], as_global(reinterpret_cast<u32x2 *>(mc + o)));
+                    __builtin_nontemporal_store(vws[c], as_global(reinterpret_cast<u32x2 *>(vc + o)));
+                }
+            }
+            if (V == 3) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const uint32_t o = c * 512 + lane * 8;
+                    __builtin_nontemporal_store(mws[c], as_global(reinterpret_cast<u32x2 *>(mc + o)));
+                    __builtin_nontemporal_store(vws[c], as_global(reinterpret_cast<u32x2 *>(vc + o)));
+                }
+            }
+            if (V == 2) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    __builtin_nontemporal_store(pw[c], as_global(reinterpret_cast<u32x4 *>(p) + c * 64 + lane));
             }
         } else {
+            if (V == 2) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    __builtin_nontemporal_store(pw[c], as_global(reinterpret_cast<u32x4 *>(p) + c * 64 + lane));
+            }
             for (int c = 0; c < 4; ++c) {
                 const uint32_t o = c * 512 + lane * 8;
                 u32x2 mw, vw;
@@ -686,10 +716,17 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
     }
 }
 
+int g_kernel_variant = 0; // A/B switch for measurements (eri_adam8_set_tuning); 0 is the shipped schedule
+
 template <int MODE, bool EXACT, bool WD, bool GS>
 static int launch_pipelined(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
                             const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg, hipStream_t s) {
     auto k = adam8_step_pipelined_kernel<MODE, EXACT, WD, GS>;
+    if (MODE == ERI_ADAM8_MODE_ERI && !EXACT && WD && !GS) { // the benchmark configuration carries the variants
+        if (g_kernel_variant == 1) k = adam8_step_pipelined_kernel<MODE, EXACT, WD, GS, 1>;
+        if (g_kernel_variant == 2) k = adam8_step_pipelined_kernel<MODE, EXACT, WD, GS, 2>;
+        if (g_kernel_variant == 3) k = adam8_step_pipelined_kernel<MODE, EXACT, WD, GS, 3>;
+    }
     if (wg > 768) wg = 768;
     hipLaunchKernelGGL(k, dim3(grid), dim3(wg), 0, s, rows, n_rows, total_blocks, h,
                        static_cast<const uint4 *>(lds_image), dev_scale);

@@ -477,6 +477,15 @@ int eri_hip_mem_info(size_t *free_bytes, size_t *total_bytes) {
 
 // ---- optimizer ------------------------------------------------------------------------------
 
+int eri_adam8_set_tuning(int key, int value) {
+    if (key == 0) {
+        if (value < 0 || value > 3) return fail(ERI_ERR_ARG, "kernel variant out of range");
+        eri::g_kernel_variant = value;
+        return 0;
+    }
+    return fail(ERI_ERR_ARG, "unknown tuning key");
+}
+
 int eri_adam8_init(void) {
     DeviceCtx *c = nullptr;
     return get_ctx(&c);

@@ -73,6 +73,7 @@ extern "C" {
     pub fn eri_hip_mem_info(free_bytes: *mut usize, total_bytes: *mut usize) -> c_int;
     // the step
     pub fn eri_adam8_init() -> c_int;
+    pub fn eri_adam8_set_tuning(key: c_int, value: c_int) -> c_int;
     pub fn eri_adam8_get_maps(signed256: *mut f32, unsigned256: *mut f32) -> c_int;
     pub fn eri_adam8_table_image(out: *mut c_void, cap: usize, bytes: *mut usize, offsets: *mut u32) -> c_int;
     pub fn eri_adam8_hyper_pack(lr: f64, beta1: f64, beta2: f64, eps: f64, weight_decay: f64, step: u64, mode: c_int, flags: u32, out: *mut EriAdam8Hyper) -> c_int;

@@ -135,6 +135,10 @@ typedef struct EriAdam8Table EriAdam8Table; /* device-resident copy of a launch 
 /* Loads the quantisation tables onto the current device.  Optional: the first table does it. */
 int eri_adam8_init(void);
 
+/* Measurement switch, not part of the optimizer's behaviour: key 0 selects one of the store
+ * schedules of the bf16 step kernel (0 = shipped; all give identical results). */
+int eri_adam8_set_tuning(int key, int value);
+
 /* The two 256-entry maps (code -> value in [-1, 1] / [0, 1]) the states are expressed in. */
 int eri_adam8_get_maps(float *signed256, float *unsigned256);
 
