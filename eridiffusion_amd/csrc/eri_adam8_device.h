@@ -72,6 +72,10 @@ int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_bloc
                 const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg,
                 void *stream);
 extern int g_kernel_variant;
+/* Sum of |moment - dequantised moment| of the coming step, per row: err[2r] first moment, err[2r+1] second. */
+int launch_quant_error(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_blocks, int dtype_tag,
+                       const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale, double *err,
+                       uint32_t grid, void *stream);
 /* Gradient norm: one f64 partial per wave (grid * 4 of them), then norm and clip factor into out[0], out[1]. */
 constexpr uint32_t kNormWavesPerWg = 4;
 int launch_grad_sumsq(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_blocks, int dtype_tag,

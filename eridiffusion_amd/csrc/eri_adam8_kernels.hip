@@ -970,6 +970,109 @@ int launch_grad_norm_finish(const double *partial, uint32_t n, float max_norm, f
 }
 
 // ------------------------------------------------------------------------------------------
+// quantisation error of the step that is about to run (quantization_stats,
+// src/trainers/adam8bit_enhanced.rs:93-100,318-327): a read-only pass that forms the new moments
+// exactly as the step will, quantises them, and adds |value - dequantised value| per row in f64.
+// Diagnostics, not tuned: element by element, binary search.
+// ------------------------------------------------------------------------------------------
+
+__device__ __forceinline__ double wave_sum_f64(double x) {
+    for (int off = 32; off >= 1; off >>= 1) x += __shfl_xor(x, off, 64);
+    return x;
+}
+
+template <bool BF16, int MODE, bool WD, bool GS>
+__global__ __launch_bounds__(256) void quant_error_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
+                                                          uint32_t total_blocks, EriAdam8Hyper h,
+                                                          const float *__restrict__ lds_image,
+                                                          const float *__restrict__ dev_scale,
+                                                          double *__restrict__ err /* [2 * n_rows] */) {
+    __shared__ float tab[1024]; // signed map, unsigned map, signed midpoints, unsigned midpoints
+    for (uint32_t i = threadIdx.x; i < 1024; i += blockDim.x) tab[i] = lds_image[i];
+    __syncthreads();
+    const float *map_s = tab, *map_u = tab + 256, *mid_s = tab + 512, *mid_u = tab + 768;
+    const float tscale = (GS && dev_scale) ? *dev_scale : 1.0f;
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t waves_per_wg = blockDim.x / kWave;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
+    const uint32_t stride = gridDim.x * waves_per_wg;
+    const BlockDiv dbc1(h.bc1), dbc2(h.bc2);
+    // every block of every row, partial ones included: rows are walked block by block
+    uint32_t ti = 0;
+    const uint32_t all_blocks = total_blocks + n_rows; // full blocks, then one (possibly empty) tail per row
+    for (uint32_t w = wave; w < all_blocks; w += stride) {
+        uint32_t lb, n;
+        if (w < total_blocks) {
+            ti = find_row(rows, n_rows, ti, w);
+            lb = w - rows[ti].full_start;
+            n = kBlock;
+        } else {
+            ti = w - total_blocks;
+            lb = (uint32_t)(rows[ti].numel / kBlock);
+            n = (uint32_t)(rows[ti].numel % kBlock);
+            if (n == 0) continue;
+        }
+        const DevTensor t = rows[ti];
+        const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
+        const size_t e0 = (size_t)lb * kBlock;
+        ERI_GLOBAL const uint8_t *mc = as_global(static_cast<const uint8_t *>(t.m));
+        ERI_GLOBAL const uint8_t *vc = as_global(static_cast<const uint8_t *>(t.v));
+        const float a_m = as_global(t.absmax_m)[lb];
+        const float a_v = as_global(t.absmax_v)[lb];
+        float lm = 0.0f, lv = 0.0f;
+        for (uint32_t i = lane; i < n; i += kWave) {
+            const size_t e = e0 + i;
+            float m, v, pn;
+            adam_elem<MODE, true, BF16, WD, GS>(load1<BF16>(t.p, e), load1<BF16>(t.g, e), map_s[mc[e]] * a_m,
+                                                map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn);
+            lm = fmaxf(lm, __builtin_fabsf(m));
+            lv = fmaxf(lv, __builtin_fabsf(v));
+        }
+        const float nam = wave_max(lm);
+        const float nav = wave_max(lv);
+        const BlockDiv dm(nam), dv(nav);
+        double em = 0.0, ev = 0.0;
+        for (uint32_t i = lane; i < n; i += kWave) {
+            const size_t e = e0 + i;
+            float m, v, pn;
+            adam_elem<MODE, true, BF16, WD, GS>(load1<BF16>(t.p, e), load1<BF16>(t.g, e), map_s[mc[e]] * a_m,
+                                                map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn);
+            const float qm = map_s[code_bsearch(dm.div_slow(m), mid_s)] * nam;
+            const float qv = map_u[code_bsearch(dv.div_slow(v), mid_u)] * nav;
+            em += (double)__builtin_fabsf(m - qm);
+            ev += (double)__builtin_fabsf(v - qv);
+        }
+        em = wave_sum_f64(em);
+        ev = wave_sum_f64(ev);
+        if (lane == 0) {
+            atomicAdd(&err[2 * ti], em);
+            atomicAdd(&err[2 * ti + 1], ev);
+        }
+    }
+}
+
+__global__ void zero_f64_kernel(double *x, uint32_t n) {
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) x[i] = 0.0;
+}
+
+int launch_quant_error(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, int dtype_tag,
+                       const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale, double *err,
+                       uint32_t grid, void *stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const float *img = static_cast<const float *>(lds_image);
+    hipLaunchKernelGGL(zero_f64_kernel, dim3(64), dim3(256), 0, s, err, 2 * n_rows);
+    const bool bf16 = dtype_tag != ERI_DTYPE_F32, l2 = h.mode == ERI_ADAM8_MODE_L2;
+    const bool wd = h.weight_decay > 0.0f, gs = (h.flags & ERI_ADAM8_FLAG_GRAD_SCALE) != 0;
+#define ERI_QE(B, M, W, G) hipLaunchKernelGGL((quant_error_kernel<B, M, W, G>), dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, h, img, dev_scale, err)
+#define ERI_QE2(B, M) do { if (wd) { if (gs) ERI_QE(B, M, true, true); else ERI_QE(B, M, true, false); } else { if (gs) ERI_QE(B, M, false, true); else ERI_QE(B, M, false, false); } } while (0)
+    if (bf16) { if (l2) ERI_QE2(true, ERI_ADAM8_MODE_L2); else ERI_QE2(true, ERI_ADAM8_MODE_ERI); }
+    else { if (l2) ERI_QE2(false, ERI_ADAM8_MODE_L2); else ERI_QE2(false, ERI_ADAM8_MODE_ERI); }
+#undef ERI_QE2
+#undef ERI_QE
+    return (int)hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------------
 // plain element-wise sweeps over a row table: 32-bit AdamW and EMA.  One wave per 2048-element
 // block, 8 elements per lane and pass, partial last blocks element by element.  HBM-bound:
 // AdamW bf16 22 B/param (read 2+2+4+4, write 2+4+4), fp32 28 B/param; EMA 3 x element size.

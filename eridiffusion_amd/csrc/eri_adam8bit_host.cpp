@@ -230,6 +230,7 @@ struct EriAdam8bit {
     uint32_t flags = 0;
     float grad_scale = 1.0f;
     float max_grad_norm = 0.0f, clip_denom_eps = 0.0f;
+    bool track_qerr = false, have_qerr = false;
     std::vector<float> param_scale;
     std::vector<std::unique_ptr<State8>> states; // index = parameter index; null before the first step
     void *stream = nullptr;
@@ -380,6 +381,7 @@ int eri_adam8bit_step(EriAdam8bit *o, uint32_t *skipped) {
         if (rc) return rc;
         o->table_ids = ids;
         o->table_rows = rows;
+        o->have_qerr = false;
     } else if (std::memcmp(rows.data(), o->table_rows.data(), rows.size() * sizeof(EriAdam8Tensor)) != 0) {
         rc = eri_adam8_table_update(o->table, rows.data(), (uint32_t)rows.size(), o->stream);
         if (rc) return rc;
@@ -396,6 +398,11 @@ int eri_adam8bit_step(EriAdam8bit *o, uint32_t *skipped) {
     rc = eri_adam8_hyper_pack(o->lr, o->beta1, o->beta2, o->eps, o->wd, o->step, ERI_ADAM8_MODE_ERI, flags, &h);
     if (rc) return rc;
     h.grad_scale = o->grad_scale;
+    if (o->track_qerr) {
+        rc = eri_adam8_quant_error(o->table, &h, o->stream);
+        if (rc) return rc;
+        o->have_qerr = true;
+    }
     return eri_adam8_step_table(o->table, &h, o->stream);
 }
 
@@ -447,6 +454,22 @@ int eri_adam8bit_last_grad_norm(EriAdam8bit *o, float *norm, float *scale) {
     if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
     if (!o->table) return fail(ERI_ERR_ARG, "no step has run yet");
     return eri_adam8_grad_norm_read(o->table, norm, scale, o->stream);
+}
+
+int eri_adam8bit_track_quantization_error(EriAdam8bit *o, int enabled) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    o->track_qerr = enabled != 0;
+    return 0;
+}
+
+int eri_adam8bit_quantization_stats(EriAdam8bit *o, float *m_error, float *v_error) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    if (!o->have_qerr || !o->table) { // nothing tracked yet: the reference reports 0 for an empty map (:320)
+        if (m_error) *m_error = 0.0f;
+        if (v_error) *v_error = 0.0f;
+        return 0;
+    }
+    return eri_adam8_quant_error_read(o->table, m_error, v_error, o->stream);
 }
 
 int eri_adam8bit_set_flags(EriAdam8bit *o, uint32_t flags) {

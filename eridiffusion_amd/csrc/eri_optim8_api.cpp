@@ -267,6 +267,8 @@ struct EriAdam8Table {
     double *partial = nullptr; // one sum of squares per wave of the norm pass, per group
     float *norm_out = nullptr; // device: {norm, clip factor}
     uint32_t n_partial = 0;
+    double *qerr = nullptr;    // device: per row {sum |m - deq m|, sum |v - deq v|}, groups back to back
+    bool qerr_valid = false;
 };
 
 namespace {
@@ -349,6 +351,7 @@ void destroy_table(EriAdam8Table *t) {
     if (t->uploaded) (void)hipEventDestroy(t->uploaded);
     if (t->partial) (void)hipFree(t->partial);
     if (t->norm_out) (void)hipFree(t->norm_out);
+    if (t->qerr) (void)hipFree(t->qerr);
     delete t;
 }
 
@@ -696,6 +699,57 @@ int eri_adam8_grad_norm_read(EriAdam8Table *t, float *norm, float *scale, void *
     ERI_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
     if (norm) *norm = host[0];
     if (scale) *scale = host[1];
+    return 0;
+}
+
+int eri_adam8_quant_error(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream) {
+    if (!t || !h) return fail(ERI_ERR_NULL, "table or hyper is NULL");
+    if (h->mode != ERI_ADAM8_MODE_ERI && h->mode != ERI_ADAM8_MODE_L2) return fail(ERI_ERR_ARG, "unknown mode");
+    DeviceCtx *ctx = nullptr;
+    int rc = get_ctx(&ctx);
+    if (rc) return rc;
+    if (!t->qerr) ERI_HIP(hipMalloc((void **)&t->qerr, sizeof(double) * 2 * t->n));
+    uint32_t off = 0;
+    for (auto &g : t->groups) {
+        if (g.n == 0) continue;
+        EriAdam8Hyper hh = *h;
+        const float *dev_scale = nullptr;
+        if (hh.flags & ERI_ADAM8_FLAG_CLIP_FROM_TABLE) {
+            if (!t->norm_out) return fail(ERI_ERR_ARG, "ERI_ADAM8_FLAG_CLIP_FROM_TABLE without a prior eri_adam8_grad_norm");
+            dev_scale = t->norm_out + 1;
+            if (!(hh.flags & ERI_ADAM8_FLAG_GRAD_SCALE)) {
+                hh.flags |= ERI_ADAM8_FLAG_GRAD_SCALE;
+                hh.grad_scale = 1.0f;
+            }
+        }
+        uint32_t grid = (g.total_blocks + g.n + 3) / 4;
+        if (grid > ctx->cus * 8) grid = ctx->cus * 8;
+        rc = eri::launch_quant_error(g.dev, g.n, g.total_blocks, g.dtype, hh, ctx->image, dev_scale, t->qerr + 2 * off,
+                                     grid, stream);
+        if (rc) return hip_fail((hipError_t)rc, "quantisation error launch");
+        off += g.n;
+    }
+    t->qerr_valid = true;
+    return 0;
+}
+
+int eri_adam8_quant_error_read(EriAdam8Table *t, float *m_error, float *v_error, void *stream) {
+    if (!t) return fail(ERI_ERR_NULL, "table is NULL");
+    if (!t->qerr_valid) return fail(ERI_ERR_ARG, "no quantisation error has been computed for this table");
+    std::vector<double> host(2 * (size_t)t->n);
+    ERI_HIP(hipMemcpyAsync(host.data(), t->qerr, host.size() * sizeof(double), hipMemcpyDeviceToHost,
+                           static_cast<hipStream_t>(stream)));
+    ERI_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    double sm = 0.0, sv = 0.0;
+    uint32_t off = 0;
+    for (auto &g : t->groups)
+        for (uint32_t j = 0; j < g.n; ++j, ++off) {
+            const double n = (double)t->numel[g.src[j]];
+            sm += host[2 * off] / n;     // per-tensor mean, adam8bit_enhanced.rs:100
+            sv += host[2 * off + 1] / n;
+        }
+    if (m_error) *m_error = (float)(sm / (double)t->n); // mean over tensors, :319-324
+    if (v_error) *v_error = (float)(sv / (double)t->n);
     return 0;
 }
 

@@ -120,6 +120,15 @@ impl Adam8bit {
     pub fn quantized_memory_usage(&self) -> usize {
         unsafe { sys::eri_adam8bit_quantized_memory_usage(self.opt) as usize }
     }
+    /// :318.  Tracking is opt-in here (`track_quantization_error(true)`): it costs one read pass per step.
+    pub fn quantization_stats(&self) -> (f32, f32) {
+        let (mut m, mut v) = (0f32, 0f32);
+        unsafe { sys::eri_adam8bit_quantization_stats(self.opt, &mut m, &mut v) };
+        (m, v)
+    }
+    pub fn track_quantization_error(&mut self, enabled: bool) {
+        unsafe { sys::eri_adam8bit_track_quantization_error(self.opt, enabled as i32) };
+    }
     /// Fold the global-norm clip factor into the next steps instead of rewriting every gradient
     /// (pipeline_flux_lora_sequential.rs:1198-1213).
     pub fn set_grad_scale(&mut self, scale: f32) -> Result<()> {

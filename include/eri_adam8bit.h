@@ -73,6 +73,11 @@ int eri_adam8bit_set_flags(EriAdam8bit *opt, uint32_t flags); /* ERI_ADAM8_FLAG_
 int eri_adam8bit_set_max_grad_norm(EriAdam8bit *opt, float max_norm, float denom_eps);
 /* Norm and clip factor of the last step that clipped (waits for the optimizer's stream). */
 int eri_adam8bit_last_grad_norm(EriAdam8bit *opt, float *norm, float *scale);
+/* quantization_stats() :318-327: mean over parameters of the mean absolute quantisation error of the
+ * first and second moments at the last step.  Tracking costs one extra read pass per step, so it is
+ * opt-in: eri_adam8bit_track_quantization_error(opt, 1) before the steps of interest. */
+int eri_adam8bit_track_quantization_error(EriAdam8bit *opt, int enabled);
+int eri_adam8bit_quantization_stats(EriAdam8bit *opt, float *m_error, float *v_error);
 /* save_state / load_state :330-368.  The file is a safetensors container with, per parameter that
  * has state, `optimizer.param_N.m` / `.v` (U8 codes) and `.absmax_m` / `.absmax_v` (F32), and the
  * step counter and learning rate in its metadata. */

@@ -168,6 +168,14 @@ int eri_adam8_grad_norm(EriAdam8Table *table, float max_norm, float denom_eps, v
 /* Copies the last norm and clip factor to the host; waits for `stream`. */
 int eri_adam8_grad_norm_read(EriAdam8Table *table, float *norm, float *scale, void *stream);
 
+/* Quantisation error the next step will incur: a read-only pass that forms the new moments exactly as
+ * eri_adam8_step_table(table, hyper) would, quantises them and accumulates |value - dequantised value|.
+ * eri_adam8_quant_error_read then returns the mean over tensors of the per-tensor mean absolute error
+ * of the first and of the second moment -- quantization_stats(), adam8bit_enhanced.rs:318-327, whose
+ * per-tensor `quantization_error` is the same mean (:93-100).  Diagnostics; costs one read pass. */
+int eri_adam8_quant_error(EriAdam8Table *table, const EriAdam8Hyper *hyper, void *stream);
+int eri_adam8_quant_error_read(EriAdam8Table *table, float *m_error, float *v_error, void *stream);
+
 /* Convenience for callers that keep no handle: keeps one cached table per calling thread and
  * re-uploads it only when `rows` changed since that thread's last call. */
 int eri_adam8_step_multi(const EriAdam8Tensor *rows, uint32_t n, const EriAdam8Hyper *hyper, void *stream);
