@@ -118,6 +118,7 @@ EXPORTS = {
     "eri_adam8bit_set_flags": (C.c_int, [C.c_void_p, C.c_uint32]),
     "eri_adam8bit_save_state": (C.c_int, [C.c_void_p, C.c_char_p]),
     "eri_adam8bit_load_state": (C.c_int, [C.c_void_p, C.c_char_p]),
+    "eri_adam8bit_load_legacy_state": (C.c_int, [C.c_void_p, C.c_char_p]),
     "eri_adam8bit_state_ptrs": (C.c_int, [C.c_void_p, C.c_uint32] + [C.POINTER(C.c_void_p)] * 4),
     "eri_adam8bit_fn_with_params": (C.c_int, [C.c_double] * 5 + [C.c_void_p, C.POINTER(C.c_void_p)]),
     "eri_adam8bit_fn_destroy": (C.c_int, [C.c_void_p]),

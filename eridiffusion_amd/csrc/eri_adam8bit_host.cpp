@@ -588,6 +588,131 @@ int eri_adam8bit_load_state(EriAdam8bit *o, const char *path) {
     return 0;
 }
 
+namespace {
+
+/* Cursor over a bincode 1.x (default options) byte stream. */
+struct Bincode {
+    const unsigned char *p, *e;
+    bool ok = true;
+    bool need(size_t n) {
+        if ((size_t)(e - p) < n) ok = false;
+        return ok;
+    }
+    uint64_t u64() {
+        uint64_t v = 0;
+        if (need(8)) { std::memcpy(&v, p, 8); p += 8; }
+        return v;
+    }
+    float f32() {
+        float v = 0;
+        if (need(4)) { std::memcpy(&v, p, 4); p += 4; }
+        return v;
+    }
+    double f64() {
+        double v = 0;
+        if (need(8)) { std::memcpy(&v, p, 8); p += 8; }
+        return v;
+    }
+    int8_t i8() {
+        int8_t v = 0;
+        if (need(1)) { v = (int8_t)*p; p += 1; }
+        return v;
+    }
+};
+
+struct LegacyTensor {
+    std::vector<float> values; // dequantised
+};
+
+bool read_legacy_map(Bincode &b, std::map<std::string, LegacyTensor> &out) {
+    const uint64_t count = b.u64();
+    if (!b.ok || count > (1u << 24)) return false;
+    for (uint64_t k = 0; k < count; ++k) {
+        const uint64_t klen = b.u64();
+        if (!b.ok || klen > 4096 || !b.need(klen)) return false;
+        std::string key(reinterpret_cast<const char *>(b.p), (size_t)klen);
+        b.p += klen;
+        const uint64_t n = b.u64();
+        if (!b.ok || !b.need(n)) return false;
+        const int8_t *q = reinterpret_cast<const int8_t *>(b.p);
+        b.p += n;
+        const float scale = b.f32();
+        const int8_t zp = b.i8();
+        const uint64_t rank = b.u64();
+        if (!b.ok || rank > 16) return false;
+        for (uint64_t d = 0; d < rank; ++d) b.u64();
+        b.f32(); // quantization_error
+        if (!b.ok) return false;
+        LegacyTensor t;
+        t.values.resize(n);
+        for (uint64_t i = 0; i < n; ++i) { // to_tensor, adam8bit_enhanced.rs:117-129
+            float x = ((float)q[i] - (float)zp) * scale;
+            t.values[i] = std::isfinite(x) ? x : 0.0f;
+        }
+        out[key] = std::move(t);
+    }
+    return true;
+}
+
+} // namespace
+
+extern "C" int eri_adam8bit_load_legacy_state(EriAdam8bit *o, const char *path) {
+    if (!o || !path) return fail(ERI_ERR_NULL, "optimizer or path is NULL");
+    std::ifstream f(path, std::ios::binary);
+    if (!f) return fail(ERI_ERR_ARG, std::string("InvalidOperation: Failed to read optimizer: cannot open ") + path);
+    std::vector<unsigned char> raw((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+    Bincode b{raw.data(), raw.data() + raw.size()};
+    const uint64_t step = b.u64();
+    std::map<std::string, LegacyTensor> first, second;
+    if (!read_legacy_map(b, first) || !read_legacy_map(b, second))
+        return fail(ERI_ERR_ARG, "InvalidOperation: Failed to deserialize optimizer: truncated or malformed bincode");
+    const double lr = b.f64();
+    if (!b.ok || b.p != b.e)
+        return fail(ERI_ERR_ARG, "InvalidOperation: Failed to deserialize optimizer: trailing or missing bytes");
+    struct Item { uint32_t idx; const LegacyTensor *m, *v; };
+    std::vector<Item> items;
+    for (uint32_t i = 0; i < o->params.size(); ++i) {
+        const std::string key = "param_" + std::to_string(i);
+        auto m = first.find(key), v = second.find(key);
+        if (m == first.end() && v == second.end()) continue;
+        if (m == first.end() || v == second.end() || m->second.values.size() != o->params[i]->numel ||
+            v->second.values.size() != o->params[i]->numel)
+            return fail(ERI_ERR_ARG, "InvalidOperation: Failed to deserialize optimizer: state of " + key + " does not fit its parameter");
+        items.push_back({i, &m->second, &v->second});
+    }
+    for (auto &it : items) {
+        const uint64_t n = o->params[it.idx]->numel;
+        std::unique_ptr<State8> s(new State8());
+        int rc = s->allocate(n, o->stream);
+        if (rc) return rc;
+        void *tmp = nullptr;
+        int dev = 0;
+        rc = eri_hip_get_device(&dev);
+        if (rc) return rc;
+        rc = eri_hip_malloc_zeroed(dev, n * 4, &tmp);
+        if (rc) return rc;
+        for (int k = 0; k < 2 && rc == 0; ++k) {
+            const LegacyTensor *src = k == 0 ? it.m : it.v;
+            rc = eri_hip_memcpy_async(tmp, src->values.data(), n * 4, 1, o->stream);
+            if (rc == 0)
+                rc = eri_adam8_quantize(static_cast<const float *>(tmp), k == 0 ? 1 : 0, n, k == 0 ? s->m : s->v,
+                                        k == 0 ? s->absmax_m : s->absmax_v, o->stream);
+            if (rc == 0) rc = eri_hip_stream_sync(o->stream);
+        }
+        eri_hip_free(tmp);
+        if (rc) return rc;
+        o->states[it.idx] = std::move(s);
+    }
+    o->step = step;
+    o->lr = lr;
+    if (o->table) {
+        eri_adam8_table_destroy(o->table);
+        o->table = nullptr;
+        o->table_ids.clear();
+    }
+    return 0;
+}
+
 // ---- functional flavour ------------------------------------------------------------------------
 
 int eri_adam8bit_fn_with_params(double lr, double beta1, double beta2, double eps, double weight_decay, void *stream,

@@ -117,6 +117,7 @@ extern "C" {
     pub fn eri_adam8bit_set_flags(opt: *mut EriAdam8bit, flags: u32) -> c_int;
     pub fn eri_adam8bit_save_state(opt: *mut EriAdam8bit, path: *const c_char) -> c_int;
     pub fn eri_adam8bit_load_state(opt: *mut EriAdam8bit, path: *const c_char) -> c_int;
+    pub fn eri_adam8bit_load_legacy_state(opt: *mut EriAdam8bit, path: *const c_char) -> c_int;
     pub fn eri_adam8bit_state_ptrs(opt: *const EriAdam8bit, index: u32, m: *mut *mut u8, v: *mut *mut u8, absmax_m: *mut *mut f32, absmax_v: *mut *mut f32) -> c_int;
     pub fn eri_adam8bit_fn_with_params(lr: f64, beta1: f64, beta2: f64, eps: f64, weight_decay: f64, stream: *mut c_void, out: *mut *mut EriAdam8bitFn) -> c_int;
     pub fn eri_adam8bit_fn_destroy(opt: *mut EriAdam8bitFn) -> c_int;

@@ -83,6 +83,14 @@ int eri_adam8bit_quantization_stats(EriAdam8bit *opt, float *m_error, float *v_e
  * step counter and learning rate in its metadata. */
 int eri_adam8bit_save_state(EriAdam8bit *opt, const char *path);
 int eri_adam8bit_load_state(EriAdam8bit *opt, const char *path);
+/* Imports a state file written by the reference's own save_state (:330-347): bincode 1.x, default
+ * options, of OptimizerState { step: usize, first_moments, second_moments: HashMap<String,
+ * QuantizedTensor { quantized_data: Vec<i8>, scale: f32, zero_point: i8, shape: Vec<usize>,
+ * quantization_error: f32 }>, learning_rate: f64 } (:30-38,398-404), keys "param_N" (:226).  Each
+ * tensor is dequantised as the reference does, (q - zero_point) * scale with non-finite values set
+ * to 0 (:117-129), and re-quantised into the blockwise format.  No file of that format ships with
+ * the reference, so the layout follows bincode's documented defaults (little-endian, u64 lengths). */
+int eri_adam8bit_load_legacy_state(EriAdam8bit *opt, const char *path);
 /* Device pointers of one parameter's state (NULL before its first step). */
 int eri_adam8bit_state_ptrs(const EriAdam8bit *opt, uint32_t index, uint8_t **m, uint8_t **v, float **absmax_m,
                             float **absmax_v);

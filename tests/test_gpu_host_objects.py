@@ -201,3 +201,29 @@ def test_functional_update_returns_a_new_tensor(bf16):
     L.check(L.lib().eri_adam8bit_fn_state_numel(opt, b"other", C.byref(numel)), "numel")
     assert numel.value == n
     L.lib().eri_adam8bit_fn_destroy(opt)
+
+
+def test_legacy_bincode_state_is_imported_and_requantised(tmp_path):
+    import torch
+    from test_host_objects_cpu import _bincode_state
+    L = _L()
+    n = 2048 + 500
+    ps, gs, states, gt = _make([n], False, 81)
+    rng = np.random.default_rng(4)
+    qm = rng.integers(-128, 128, n).tolist()
+    qv = rng.integers(-128, 128, n).tolist()
+    sm, zm, sv, zv = 3e-5, -7, 2e-9, -128
+    path = tmp_path / "optimizer.pt"
+    path.write_bytes(_bincode_state(41, 3e-4, {"param_0": (qm, sm, zm, [n], 0.1)}, {"param_0": (qv, sv, zv, [n], 0.1)}))
+    opt, handles = _new_optimizer(gt)
+    L.check(L.lib().eri_adam8bit_load_legacy_state(opt, str(path).encode()), "load_legacy")
+    assert L.lib().eri_adam8bit_get_step(opt) == 41 and L.lib().eri_adam8bit_current_lr(opt) == 3e-4
+    got = _fetch_states(opt, gt)[0]
+    for k, (q, scale, zp, table) in enumerate(((qm, sm, zm, hs.MAPS[0]), (qv, sv, zv, hs.MAPS[1]))):
+        x = ((np.array(q, np.float32) - np.float32(zp)) * np.float32(scale)).astype(np.float32)  # (q - zp) * scale, :121
+        codes = np.empty(n, np.uint8)
+        absmax = np.empty(2, np.float32)
+        oc.lib().eri_oracle_quantize(oc.ptr(x), oc.ptr(table), n, oc.ptr(codes), oc.ptr(absmax))
+        assert np.array_equal(got[k], codes)
+        assert np.array_equal(got[2 + k].view(np.uint32), absmax.view(np.uint32))
+    L.lib().eri_adam8bit_destroy(opt)

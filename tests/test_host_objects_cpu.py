@@ -96,3 +96,37 @@ def test_functional_flavour_counters_and_errors():
     assert L.lib().eri_adam8bit_fn_state_numel(opt, b"w", C.byref(numel)) == 0 and numel.value == 0
     assert L.lib().eri_adam8bit_fn_get_state_fp32(opt, b"w", 0x1000, 0x2000) == -6
     L.lib().eri_adam8bit_fn_destroy(opt)
+
+
+def _bincode_state(step, lr, first, second):
+    """bincode 1.3 default options of the reference's OptimizerState (adam8bit_enhanced.rs:398-404)."""
+    def qt(q, scale, zp, shape, err):
+        b = struct.pack("<Q", len(q)) + bytes((x & 0xFF) for x in q) + struct.pack("<f", scale) + struct.pack("<b", zp)
+        b += struct.pack("<Q", len(shape)) + b"".join(struct.pack("<Q", d) for d in shape) + struct.pack("<f", err)
+        return b
+
+    def hmap(d):
+        b = struct.pack("<Q", len(d))
+        for k, v in d.items():
+            kb = k.encode()
+            b += struct.pack("<Q", len(kb)) + kb + qt(*v)
+        return b
+    return struct.pack("<Q", step) + hmap(first) + hmap(second) + struct.pack("<d", lr)
+
+
+def test_legacy_state_file_errors(tmp_path):
+    opt, handles = _optimizer(n_params=1, numel=8)
+    path = tmp_path / "optimizer.pt"
+    good = _bincode_state(7, 2e-4, {"param_0": ([1] * 8, 0.5, 0, [8], 0.0)}, {"param_0": ([2] * 8, 0.25, -1, [2, 4], 0.0)})
+    path.write_bytes(good[:-3])
+    assert L.lib().eri_adam8bit_load_legacy_state(opt, str(path).encode()) == -6
+    assert b"Failed to deserialize optimizer" in L.lib().eri_last_error()
+    path.write_bytes(good + b"\x00")
+    assert L.lib().eri_adam8bit_load_legacy_state(opt, str(path).encode()) == -6
+    wrong = _bincode_state(7, 2e-4, {"param_0": ([1] * 9, 0.5, 0, [9], 0.0)}, {"param_0": ([2] * 9, 0.25, 0, [9], 0.0)})
+    path.write_bytes(wrong)
+    rc = L.lib().eri_adam8bit_load_legacy_state(opt, str(path).encode())
+    assert rc == -6 and b"does not fit its parameter" in L.lib().eri_last_error()
+    assert L.lib().eri_adam8bit_load_legacy_state(opt, str(tmp_path / "missing").encode()) == -6
+    assert L.lib().eri_adam8bit_get_step(opt) == 0
+    L.lib().eri_adam8bit_destroy(opt)
