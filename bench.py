@@ -34,7 +34,7 @@ def parse():
                     help="what one step is: the 8-bit AdamW step (headline), the same preceded by the device-side "
                          "gradient norm, the norm alone, the 32-bit AdamW sibling, or the EMA sweep")
     ap.add_argument("--variants", default="", help="comma-separated kernel variants to time interleaved (A/B tool)")
-    ap.add_argument("--alloc", choices=["arena", "tensor"], default="arena",
+    ap.add_argument("--alloc", choices=["arena", "pool", "tensor"], default="arena",
                     help="one flat allocation per kind of buffer, or one allocation per tensor and buffer")
     ap.add_argument("--calibrate-copy", type=int, default=0,
                     help="instead of the benchmark, run a plain device copy of this many bytes three times "
@@ -92,6 +92,42 @@ class Arena:
     def free(self):
         from eridiffusion_amd import _lib as L
         L.lib().eri_hip_free(self.base)
+
+
+class Pool:
+    """One device allocation for everything (how a pooling allocator would hold a model): the six
+    buffers are consecutive ranges of it, each starting on a 2 MiB boundary."""
+    base = None
+    used = 0
+    capacity = 0
+
+    @classmethod
+    def reserve(cls, nbytes):
+        from eridiffusion_amd import _lib as L
+        out = C.c_void_p()
+        L.check(L.lib().eri_hip_malloc_zeroed(0, nbytes, C.byref(out)), "eri_hip_malloc_zeroed")
+        cls.base, cls.used, cls.capacity = out.value, 0, nbytes
+
+    def __init__(self, torch, sizes_bytes):
+        self.offsets = []
+        total = 0
+        for b in sizes_bytes:
+            self.offsets.append(total)
+            total += align(b)
+        self.nbytes = align(max(total, 256), 2 << 20)
+        if Pool.used + self.nbytes > Pool.capacity:
+            raise RuntimeError("pool exhausted")
+        self.base = Pool.base + Pool.used
+        Pool.used += self.nbytes
+
+    ptr = Arena.ptr
+    fill = Arena.fill
+
+    def free(self):
+        from eridiffusion_amd import _lib as L
+        if Pool.base is not None:
+            L.lib().eri_hip_free(Pool.base)
+            Pool.base = None
 
 
 def cpu_baseline(tensors, bf16, sample_params, hyper_args):
@@ -167,7 +203,10 @@ def main():
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream().cuda_stream
 
-    Alloc = Arena if args.alloc == "arena" else PerTensor
+    Alloc = {"arena": Arena, "pool": Pool, "tensor": PerTensor}[args.alloc]
+    if args.alloc == "pool":
+        extra_b = {"adamw32": 8, "ema": esz}.get(args.kernel, 0)
+        Pool.reserve(align(n_params * (2 * esz + 2 + extra_b) + n_blocks * 8 + 300 * len(sizes) * 8, 2 << 20) + (20 << 20))
     a_p = Alloc(torch, [n * esz for n in sizes])
     a_g = Alloc(torch, [n * esz for n in sizes])
     a_m = Alloc(torch, sizes)

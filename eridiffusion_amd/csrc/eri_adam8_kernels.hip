@@ -50,15 +50,39 @@ __device__ __forceinline__ float dpp_mov(float x) {
     return u2f((uint32_t)__builtin_amdgcn_update_dpp((int)f2u(x), (int)f2u(x), CTRL, ROW_MASK, 0xf, false));
 }
 
-/* Maximum over the 64 lanes of non-negative, NaN-free values, returned wave-uniform. */
+/* Maximum over the 64 lanes of non-negative, NaN-free values, returned wave-uniform.  Such floats
+ * order like their bit patterns, so the steps are unsigned integer maxima with the lane permutation
+ * folded into the instruction (v_max_u32_dpp); lanes a step does not write keep their value.  A DPP
+ * read of a register needs two wait states after the vector instruction that wrote it, and the
+ * assembler text below is opaque to the compiler's hazard handling, hence the explicit s_nop. */
+#define ERI_DPP_MAX(reg, ctrl) "v_max_u32_dpp " reg ", " reg ", " reg " " ctrl " bank_mask:0xf\n"
 __device__ __forceinline__ float wave_max(float x) {
-    x = fmaxf(x, dpp_mov<0xB1, 0xf>(x));  // quad_perm [1,0,3,2]
-    x = fmaxf(x, dpp_mov<0x4E, 0xf>(x));  // quad_perm [2,3,0,1]
-    x = fmaxf(x, dpp_mov<0x141, 0xf>(x)); // row_half_mirror
-    x = fmaxf(x, dpp_mov<0x140, 0xf>(x)); // row_mirror: every lane now holds its row's maximum
-    x = fmaxf(x, dpp_mov<0x142, 0xa>(x)); // row_bcast:15 into rows 1 and 3
-    x = fmaxf(x, dpp_mov<0x143, 0xc>(x)); // row_bcast:31 into rows 2 and 3
-    return u2f((uint32_t)__builtin_amdgcn_readlane((int)f2u(x), 63));
+    uint32_t u = f2u(x);
+    asm volatile("s_nop 1\n"
+                 ERI_DPP_MAX("%0", "quad_perm:[1,0,3,2] row_mask:0xf") "s_nop 1\n"
+                 ERI_DPP_MAX("%0", "quad_perm:[2,3,0,1] row_mask:0xf") "s_nop 1\n"
+                 ERI_DPP_MAX("%0", "row_half_mirror row_mask:0xf") "s_nop 1\n"
+                 ERI_DPP_MAX("%0", "row_mirror row_mask:0xf") "s_nop 1\n" // every lane holds its row's maximum
+                 ERI_DPP_MAX("%0", "row_bcast:15 row_mask:0xa") "s_nop 1\n" // into rows 1 and 3
+                 ERI_DPP_MAX("%0", "row_bcast:31 row_mask:0xc") "s_nop 1\n" // into rows 2 and 3
+                 : "+v"(u));
+    return u2f((uint32_t)__builtin_amdgcn_readlane((int)u, 63));
+}
+/* Two reductions at once: each chain's instruction fills one of the other's wait states. */
+__device__ __forceinline__ void wave_max2(float &a, float &b) {
+    uint32_t u = f2u(a), w = f2u(b);
+#define ERI_DPP_MAX2(ctrl) ERI_DPP_MAX("%0", ctrl) ERI_DPP_MAX("%1", ctrl) "s_nop 0\n"
+    asm volatile("s_nop 1\n"
+                 ERI_DPP_MAX2("quad_perm:[1,0,3,2] row_mask:0xf")
+                 ERI_DPP_MAX2("quad_perm:[2,3,0,1] row_mask:0xf")
+                 ERI_DPP_MAX2("row_half_mirror row_mask:0xf")
+                 ERI_DPP_MAX2("row_mirror row_mask:0xf")
+                 ERI_DPP_MAX2("row_bcast:15 row_mask:0xa")
+                 ERI_DPP_MAX2("row_bcast:31 row_mask:0xc")
+                 : "+v"(u), "+v"(w));
+#undef ERI_DPP_MAX2
+    a = u2f((uint32_t)__builtin_amdgcn_readlane((int)u, 63));
+    b = u2f((uint32_t)__builtin_amdgcn_readlane((int)w, 63));
 }
 
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return u2f(w << 16); }
@@ -397,8 +421,8 @@ __device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint
             store8<BF16>(p, o, pn);
         }
     }
-    const float nam = wave_max(lm);
-    const float nav = wave_max(lv);
+    float nam = lm, nav = lv;
+    wave_max2(nam, nav);
     if (lane == 0) {
         as_global(t.absmax_m)[lb] = nam;
         as_global(t.absmax_v)[lb] = nav;
@@ -455,8 +479,8 @@ __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint
         lm = fmaxf(lm, __builtin_fabsf(m));
         lv = fmaxf(lv, __builtin_fabsf(v));
     }
-    const float nam = wave_max(lm);
-    const float nav = wave_max(lv);
+    float nam = lm, nav = lv;
+    wave_max2(nam, nav);
     constexpr float ks = KEYTAB ? kKeyScale : 1.0f, ksi = KEYTAB ? kKeyScaleInv : 1.0f;
     const BlockDiv dm(nam, ks, ksi), dv(nav, ks, ksi);
     for (uint32_t i = lane; i < n; i += kWave) {
@@ -496,11 +520,28 @@ __device__ __forceinline__ uint32_t find_row(const DevTensor *rows, uint32_t n_r
     return lo;
 }
 
+/* The full blocks one wave walks.  Workgroup i of a launch runs on accelerator die (XCD) i mod 8.  The
+ * block list is cut into `chunks` contiguous ranges and workgroup i walks range i mod chunks, so with
+ * chunks == 8 each die sweeps its own part of every buffer instead of all dies advancing through one
+ * common window; on MI355X that made the sweep both a little faster and much less dependent on where
+ * the buffers happen to lie physically.  chunks == 1 is the plain grid-stride walk. */
+struct BlockWalk {
+    uint32_t first, end, stride;
+    __device__ __forceinline__ BlockWalk(uint32_t total_blocks, uint32_t chunks) {
+        const uint32_t waves_per_wg = blockDim.x / kWave;
+        const uint32_t per_chunk = (total_blocks + chunks - 1) / chunks;
+        const uint32_t lo = (blockIdx.x % chunks) * per_chunk;
+        end = lo + per_chunk < total_blocks ? lo + per_chunk : total_blocks;
+        stride = (gridDim.x / chunks) * waves_per_wg;
+        first = __builtin_amdgcn_readfirstlane(lo + (blockIdx.x / chunks) * waves_per_wg + threadIdx.x / kWave);
+    }
+};
+
 template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB>
 __global__ __launch_bounds__(1024) void adam8_step_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
                                                           uint32_t total_blocks, EriAdam8Hyper h,
                                                           const uint4 *__restrict__ lds_image,
-        const float *__restrict__ dev_scale) {
+                                                          const float *__restrict__ dev_scale, uint32_t chunks) {
     ERI_LDS_IMAGE;
     // clip factor left on the device by the gradient-norm pass (1.0 when there is none)
     const float tscale = (GS && dev_scale) ? *dev_scale : 1.0f;
@@ -531,7 +572,8 @@ __global__ __launch_bounds__(1024) void adam8_step_kernel(const DevTensor *__res
         }
     }
     uint32_t ti = 0; // rows[ti].full_start <= blk; blk only grows, so the search restarts from ti
-    for (uint32_t blk = wave; blk < total_blocks; blk += stride) {
+    const BlockWalk walk(total_blocks, chunks);
+    for (uint32_t blk = walk.first; blk < walk.end; blk += walk.stride) {
         ti = find_row(rows, n_rows, ti, blk);
         const DevTensor t = rows[ti];
         const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
@@ -576,7 +618,8 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
                                                                    uint32_t n_rows, uint32_t total_blocks,
                                                                    EriAdam8Hyper h,
                                                                    const uint4 *__restrict__ lds_image,
-        const float *__restrict__ dev_scale) {
+                                                                   const float *__restrict__ dev_scale,
+                                                                   uint32_t chunks) {
     ERI_LDS_IMAGE;
     // clip factor left on the device by the gradient-norm pass (1.0 when there is none)
     const float tscale = (GS && dev_scale) ? *dev_scale : 1.0f;
@@ -606,9 +649,10 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
             tail_block<true, MODE, EXACT, WD, GS, true>(t, (uint32_t)(t.numel / kBlock), n, lane, h, gscale, dbc1, dbc2, L);
         }
     }
-    if (wave >= total_blocks) return;
+    const BlockWalk walk(total_blocks, chunks);
+    uint32_t blk = walk.first;
+    if (blk >= walk.end) return;
 
-    uint32_t blk = wave;
     uint32_t ti = find_row(rows, n_rows, 0, blk);
     DevTensor t = rows[ti];
     RawBlock raw;
@@ -616,8 +660,8 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
     while (true) {
         // the block after this one; past the end the wave re-reads its last block (the loads must
         // stay unconditional so that the raw registers have a single definition in the loop)
-        const uint32_t nblk = blk + stride;
-        const bool more = nblk < total_blocks;
+        const uint32_t nblk = blk + walk.stride;
+        const bool more = nblk < walk.end;
         const uint32_t pblk = more ? nblk : blk;
         const uint32_t nti = find_row(rows, n_rows, ti, pblk);
         const DevTensor nt = rows[nti];
@@ -658,8 +702,8 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
             pw[c].w = bf16_pair(pn[6], pn[7]);
             if (V == 1) __builtin_nontemporal_store(pw[c], as_global(reinterpret_cast<u32x4 *>(p) + c * 64 + lane));
         }
-        const float nam = wave_max(lm);
-        const float nav = wave_max(lv);
+        float nam = lm, nav = lv;
+        wave_max2(nam, nav);
         if (lane == 0) {
             as_global(t.absmax_m)[lb] = nam;
             as_global(t.absmax_v)[lb] = nav;
@@ -716,6 +760,11 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
     }
 }
 
+int g_chunks = 8; // contiguous ranges of the block list (BlockWalk); 8 = one per accelerator die
+/* The chunked walk needs the same number of workgroups in every chunk. */
+static uint32_t chunks_for(uint32_t grid) {
+    return (g_chunks > 1 && grid % (uint32_t)g_chunks == 0) ? (uint32_t)g_chunks : 1u;
+}
 int g_kernel_variant = 0; // A/B switch for measurements (eri_adam8_set_tuning); 0 is the shipped schedule
 
 template <int MODE, bool EXACT, bool WD, bool GS>
@@ -729,7 +778,7 @@ static int launch_pipelined(const DevTensor *rows, uint32_t n_rows, uint32_t tot
     }
     if (wg > 768) wg = 768;
     hipLaunchKernelGGL(k, dim3(grid), dim3(wg), 0, s, rows, n_rows, total_blocks, h,
-                       static_cast<const uint4 *>(lds_image), dev_scale);
+                       static_cast<const uint4 *>(lds_image), dev_scale, chunks_for(grid));
     return (int)hipGetLastError();
 }
 
@@ -738,7 +787,7 @@ static int launch_one(const DevTensor *rows, uint32_t n_rows, uint32_t total_blo
                       const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg, hipStream_t s) {
     auto k = adam8_step_kernel<BF16, MODE, EXACT, WD, GS, KEYTAB>;
     hipLaunchKernelGGL(k, dim3(grid), dim3(wg), 0, s, rows, n_rows, total_blocks, h,
-                       static_cast<const uint4 *>(lds_image), dev_scale);
+                       static_cast<const uint4 *>(lds_image), dev_scale, chunks_for(grid));
     return (int)hipGetLastError();
 }
 
@@ -891,7 +940,8 @@ __device__ __forceinline__ float wave_sum(float x) {
 
 template <bool BF16>
 __global__ __launch_bounds__(256) void grad_sumsq_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
-                                                         uint32_t total_blocks, double *__restrict__ partial) {
+                                                         uint32_t total_blocks, double *__restrict__ partial,
+                                                         uint32_t chunks) {
     // persistent: every wave adds the fp32 sums of its blocks in f64 and leaves one partial
     const uint32_t lane = threadIdx.x & (kWave - 1);
     const uint32_t waves_per_wg = blockDim.x / kWave;
@@ -910,7 +960,8 @@ __global__ __launch_bounds__(256) void grad_sumsq_kernel(const DevTensor *__rest
         total += (double)wave_sum(acc);
     }
     uint32_t ti = 0;
-    for (uint32_t blk = wave; blk < total_blocks; blk += stride) {
+    const BlockWalk walk(total_blocks, chunks);
+    for (uint32_t blk = walk.first; blk < walk.end; blk += walk.stride) {
         ti = find_row(rows, n_rows, ti, blk);
         const DevTensor t = rows[ti];
         const size_t e0 = (size_t)(blk - t.full_start) * kBlock;
@@ -956,9 +1007,9 @@ int launch_grad_sumsq(const DevTensor *rows, uint32_t n_rows, uint32_t total_blo
                       uint32_t grid, void *stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype_tag == ERI_DTYPE_F32)
-        hipLaunchKernelGGL(grad_sumsq_kernel<false>, dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, partial);
+        hipLaunchKernelGGL(grad_sumsq_kernel<false>, dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, partial, chunks_for(grid));
     else
-        hipLaunchKernelGGL(grad_sumsq_kernel<true>, dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, partial);
+        hipLaunchKernelGGL(grad_sumsq_kernel<true>, dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, partial, chunks_for(grid));
     return (int)hipGetLastError();
 }
 
@@ -1028,8 +1079,8 @@ __global__ __launch_bounds__(256) void quant_error_kernel(const DevTensor *__res
             lm = fmaxf(lm, __builtin_fabsf(m));
             lv = fmaxf(lv, __builtin_fabsf(v));
         }
-        const float nam = wave_max(lm);
-        const float nav = wave_max(lv);
+        float nam = lm, nav = lv;
+        wave_max2(nam, nav);
         const BlockDiv dm(nam), dv(nav);
         double em = 0.0, ev = 0.0;
         for (uint32_t i = lane; i < n; i += kWave) {
@@ -1113,7 +1164,7 @@ __device__ __forceinline__ void store1(void *base, size_t i, float x) {
 
 template <bool BF16>
 __global__ __launch_bounds__(256) void adamw32_kernel(const ElemRow *__restrict__ rows, uint32_t n_rows,
-                                                      uint32_t total_blocks, EriAdamW32Hyper h) {
+                                                      uint32_t total_blocks, EriAdamW32Hyper h, uint32_t chunks) {
     const uint32_t lane = threadIdx.x & (kWave - 1);
     const uint32_t waves_per_wg = blockDim.x / kWave;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
@@ -1134,7 +1185,8 @@ __global__ __launch_bounds__(256) void adamw32_kernel(const ElemRow *__restrict_
         }
     }
     uint32_t ti = 0;
-    for (uint32_t blk = wave; blk < total_blocks; blk += stride) {
+    const BlockWalk walk(total_blocks, chunks);
+    for (uint32_t blk = walk.first; blk < walk.end; blk += walk.stride) {
         ti = find_elem_row(rows, n_rows, ti, blk);
         const ElemRow t = rows[ti];
         const size_t e0 = (size_t)(blk - t.full_start) * kBlock;
@@ -1178,7 +1230,7 @@ __device__ __forceinline__ float ema_elem(float shadow, float p, float decay, fl
 
 template <bool BF16>
 __global__ __launch_bounds__(256) void ema_kernel(const ElemRow *__restrict__ rows, uint32_t n_rows,
-                                                  uint32_t total_blocks, float decay) {
+                                                  uint32_t total_blocks, float decay, uint32_t chunks) {
     const uint32_t lane = threadIdx.x & (kWave - 1);
     const uint32_t waves_per_wg = blockDim.x / kWave;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
@@ -1192,7 +1244,8 @@ __global__ __launch_bounds__(256) void ema_kernel(const ElemRow *__restrict__ ro
             store1<BF16>(t.a, e0 + i, ema_elem(load1<BF16>(t.a, e0 + i), load1<BF16>(t.b, e0 + i), decay, omd));
     }
     uint32_t ti = 0;
-    for (uint32_t blk = wave; blk < total_blocks; blk += stride) {
+    const BlockWalk walk(total_blocks, chunks);
+    for (uint32_t blk = walk.first; blk < walk.end; blk += walk.stride) {
         ti = find_elem_row(rows, n_rows, ti, blk);
         const ElemRow t = rows[ti];
         const size_t e0 = (size_t)(blk - t.full_start) * kBlock;
@@ -1220,9 +1273,9 @@ int launch_adamw32(const ElemRow *rows, uint32_t n_rows, uint32_t total_blocks, 
                    const EriAdamW32Hyper &h, uint32_t grid, void *stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype_tag == ERI_DTYPE_F32)
-        hipLaunchKernelGGL(adamw32_kernel<false>, dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, h);
+        hipLaunchKernelGGL(adamw32_kernel<false>, dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, h, chunks_for(grid));
     else
-        hipLaunchKernelGGL(adamw32_kernel<true>, dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, h);
+        hipLaunchKernelGGL(adamw32_kernel<true>, dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, h, chunks_for(grid));
     return (int)hipGetLastError();
 }
 
@@ -1230,9 +1283,9 @@ int launch_ema(const ElemRow *rows, uint32_t n_rows, uint32_t total_blocks, int 
                uint32_t grid, void *stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype_tag == ERI_DTYPE_F32)
-        hipLaunchKernelGGL(ema_kernel<false>, dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, decay);
+        hipLaunchKernelGGL(ema_kernel<false>, dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, decay, chunks_for(grid));
     else
-        hipLaunchKernelGGL(ema_kernel<true>, dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, decay);
+        hipLaunchKernelGGL(ema_kernel<true>, dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, decay, chunks_for(grid));
     return (int)hipGetLastError();
 }
 

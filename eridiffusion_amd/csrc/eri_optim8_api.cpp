@@ -219,6 +219,7 @@ int get_ctx(DeviceCtx **out) {
         c.cus = (uint32_t)prop.multiProcessorCount;
         c.wg = (uint32_t)env_u32("ERI_ADAM8_WG", 64, 1024, 1024) & ~63u;
         c.wg_per_cu = (uint32_t)env_u32("ERI_ADAM8_WG_PER_CU", 1, 16, 1);
+        eri::g_chunks = env_u32("ERI_ADAM8_CHUNKS", 1, 4096, 8);
         ERI_HIP(hipMalloc(&c.image, eri::kLdsImageBytes));
         ERI_HIP(hipMemcpy(c.image, t.image.data(), eri::kLdsImageBytes, hipMemcpyHostToDevice));
         c.ready = true;
@@ -390,7 +391,16 @@ int eri_hip_malloc_zeroed(int device, size_t bytes, void **out) {
     ERI_HIP(hipGetDevice(&prev));
     if (prev != device) ERI_HIP(hipSetDevice(device));
     void *p = nullptr;
-    hipError_t e = hipMalloc(&p, bytes);
+    static const bool contiguous = std::getenv("ERI_HIP_MALLOC_CONTIGUOUS") && std::atoi(std::getenv("ERI_HIP_MALLOC_CONTIGUOUS")) != 0;
+    auto device_alloc = [&](void **q) -> hipError_t {
+        if (contiguous && bytes >= kRecycleThreshold) {
+            hipError_t ce = hipExtMallocWithFlags(q, bytes, hipDeviceMallocContiguous);
+            if (ce == hipSuccess) return ce;
+            (void)hipGetLastError();
+        }
+        return hipMalloc(q, bytes);
+    };
+    hipError_t e = device_alloc(&p);
     // Placement conditioning.  On MI355X the first physical placement a large allocation receives
     // sustains visibly less write bandwidth than the placement the same request receives once the
     // range has been handed back to the driver (measured with a plain streaming kernel: 4.6 vs
@@ -399,7 +409,7 @@ int eri_hip_malloc_zeroed(int device, size_t bytes, void **out) {
     if (e == hipSuccess && bytes >= kRecycleThreshold && recycle_enabled()) {
         e = hipFree(p);
         p = nullptr;
-        if (e == hipSuccess) e = hipMalloc(&p, bytes);
+        if (e == hipSuccess) e = device_alloc(&p);
     }
     if (e == hipSuccess) e = hipMemset(p, 0, bytes);
     if (prev != device) (void)hipSetDevice(prev);
@@ -480,7 +490,19 @@ int eri_hip_mem_info(size_t *free_bytes, size_t *total_bytes) {
 
 // ---- optimizer ------------------------------------------------------------------------------
 
+static int g_grid_override = 0; // measurement switch: persistent workgroups of the step (0 = one per slot)
+
 int eri_adam8_set_tuning(int key, int value) {
+    if (key == 2) {
+        if (value < 1 || value > 4096) return fail(ERI_ERR_ARG, "chunk count out of range");
+        eri::g_chunks = value;
+        return 0;
+    }
+    if (key == 1) {
+        if (value < 0 || value > 65536) return fail(ERI_ERR_ARG, "grid override out of range");
+        g_grid_override = value;
+        return 0;
+    }
     if (key == 0) {
         if (value < 0 || value > 3) return fail(ERI_ERR_ARG, "kernel variant out of range");
         eri::g_kernel_variant = value;
@@ -640,7 +662,7 @@ int eri_adam8_step_table(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream)
         // One wavefront per block.  A small table gets smaller workgroups so that its blocks still
         // spread over every compute unit instead of filling a few of them.
         uint32_t waves_per_wg = ctx->wg / eri::kWave;
-        const uint32_t slots = ctx->cus * ctx->wg_per_cu;
+        const uint32_t slots = g_grid_override ? (uint32_t)g_grid_override : ctx->cus * ctx->wg_per_cu;
         const uint32_t work = g.total_blocks > g.n ? g.total_blocks : g.n; // full blocks, or one tail per row
         const uint32_t per_slot = (work + slots - 1) / slots;
         if (per_slot < waves_per_wg) waves_per_wg = per_slot < 4 ? 4 : per_slot;
