@@ -142,6 +142,10 @@ def lib():
         if not os.path.exists(LIB_PATH):
             raise RuntimeError("%s is missing: build it with `make -C eridiffusion_amd/csrc` "
                                "(there is no CPU or PyTorch fallback)" % LIB_PATH)
+        try:  # PyTorch ships its own copy of the HIP runtime: when both live in one process the library
+            import torch  # noqa: F401  must bind to that copy, so torch is loaded first (two runtimes crash)
+        except ImportError:
+            pass
         L = C.CDLL(LIB_PATH)
         for name, (res, args) in EXPORTS.items():
             fn = getattr(L, name)
