@@ -86,6 +86,7 @@ EXPORTS = {
     "eri_adam8_step_table": (C.c_int, [C.c_void_p, C.POINTER(Hyper), C.c_void_p]),
     "eri_adam8_grad_norm": (C.c_int, [C.c_void_p, C.c_float, C.c_float, C.c_void_p]),
     "eri_adam8_grad_norm_read": (C.c_int, [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_void_p]),
+    "eri_adam8_grad_nonfinite_read": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint64), C.c_void_p]),
     "eri_adam8_quant_error": (C.c_int, [C.c_void_p, C.POINTER(Hyper), C.c_void_p]),
     "eri_adam8_quant_error_read": (C.c_int, [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_void_p]),
     "eri_adam8_step_multi": (C.c_int, [C.POINTER(TensorRow), C.c_uint32, C.POINTER(Hyper), C.c_void_p]),
@@ -113,6 +114,7 @@ EXPORTS = {
     "eri_adam8bit_set_param_grad_scale": (C.c_int, [C.c_void_p, C.c_uint32, C.c_float]),
     "eri_adam8bit_set_max_grad_norm": (C.c_int, [C.c_void_p, C.c_float, C.c_float]),
     "eri_adam8bit_last_grad_norm": (C.c_int, [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
+    "eri_adam8bit_last_nonfinite_grads": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint64)]),
     "eri_adam8bit_track_quantization_error": (C.c_int, [C.c_void_p, C.c_int]),
     "eri_adam8bit_quantization_stats": (C.c_int, [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
     "eri_adam8bit_set_flags": (C.c_int, [C.c_void_p, C.c_uint32]),

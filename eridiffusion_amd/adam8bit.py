@@ -96,6 +96,34 @@ class Adam8bit:
     def set_grad_scale(self, scale: float) -> None:
         check(lib().eri_adam8bit_set_grad_scale(self._opt, scale), "eri_adam8bit_set_grad_scale")
 
+    def set_max_grad_norm(self, max_norm: float, denom_eps: float = 0.0) -> None:
+        """Global-norm clipping inside step(): norm on the device, factor applied by the step kernel
+        (clip_gradients, src/trainers/pipeline_flux_lora_sequential.rs:1198-1213).  <= 0 switches it off."""
+        check(lib().eri_adam8bit_set_max_grad_norm(self._opt, max_norm, denom_eps), "eri_adam8bit_set_max_grad_norm")
+
+    def last_grad_norm(self) -> Tuple[float, float]:
+        """(norm, clip factor) of the last step that clipped; waits for the stream."""
+        n, s = C.c_float(), C.c_float()
+        check(lib().eri_adam8bit_last_grad_norm(self._opt, C.byref(n), C.byref(s)), "eri_adam8bit_last_grad_norm")
+        return n.value, s.value
+
+    def last_nonfinite_grads(self) -> int:
+        """NaN / infinite gradient elements seen by the norm pass of the last step that clipped."""
+        c = C.c_uint64()
+        check(lib().eri_adam8bit_last_nonfinite_grads(self._opt, C.byref(c)), "eri_adam8bit_last_nonfinite_grads")
+        return c.value
+
+    def track_quantization_error(self, enabled: bool = True) -> None:
+        check(lib().eri_adam8bit_track_quantization_error(self._opt, int(enabled)),
+              "eri_adam8bit_track_quantization_error")
+
+    def quantization_stats(self) -> Tuple[float, float]:
+        """adam8bit_enhanced.rs:318-327: mean absolute quantisation error of (first, second) moments."""
+        m, v = C.c_float(), C.c_float()
+        check(lib().eri_adam8bit_quantization_stats(self._opt, C.byref(m), C.byref(v)),
+              "eri_adam8bit_quantization_stats")
+        return m.value, v.value
+
     def quantized_memory_usage(self) -> int:
         return lib().eri_adam8bit_quantized_memory_usage(self._opt)
 

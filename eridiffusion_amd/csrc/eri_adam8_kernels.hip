@@ -925,6 +925,9 @@ int launch_quantize(const float *x, int signed_map, uint64_t numel, uint8_t *cod
 // the clip factor to device memory, where the step kernel reads it.
 // ------------------------------------------------------------------------------------------
 
+/* 1.0 for NaN and +-infinity, else 0.0 */
+__device__ __forceinline__ float not_finite(float x) { return (__builtin_fabsf(x) <= 3.4028234e38f) ? 0.0f : 1.0f; }
+
 __device__ __forceinline__ float wave_sum(float x) {
     // fixed reduction tree, so the result does not depend on scheduling
     x += dpp_mov<0xB1, 0xf>(x);
@@ -947,17 +950,19 @@ __global__ __launch_bounds__(256) void grad_sumsq_kernel(const DevTensor *__rest
     const uint32_t waves_per_wg = blockDim.x / kWave;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
     const uint32_t stride = gridDim.x * waves_per_wg;
-    double total = 0.0;
+    double total = 0.0, bad = 0.0;
     for (uint32_t r = wave; r < n_rows; r += stride) { // partial last blocks
         const DevTensor t = rows[r];
         const uint32_t n = (uint32_t)(t.numel % kBlock);
         const size_t e0 = (size_t)(t.numel / kBlock) * kBlock;
-        float acc = 0.0f;
+        float acc = 0.0f, nf = 0.0f;
         for (uint32_t i = lane; i < n; i += kWave) {
             const float g = load1<BF16>(t.g, e0 + i);
             acc += g * g;
+            nf += not_finite(g);
         }
         total += (double)wave_sum(acc);
+        bad += (double)wave_sum(nf);
     }
     uint32_t ti = 0;
     const BlockWalk walk(total_blocks, chunks);
@@ -976,21 +981,44 @@ __global__ __launch_bounds__(256) void grad_sumsq_kernel(const DevTensor *__rest
 #pragma unroll
             for (int k = 0; k < 8; ++k) acc += g[k] * g[k];
         }
-        total += (double)wave_sum(acc);
+        const float block_sum = wave_sum(acc);
+        total += (double)block_sum;
+        if (not_finite(block_sum) != 0.0f) { // rare: count the NaN / infinite elements of this block
+            float nf = 0.0f;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                float g[8];
+                raw[c].unpack(g);
+#pragma unroll
+                for (int k = 0; k < 8; ++k) nf += not_finite(g[k]);
+            }
+            bad += (double)wave_sum(nf);
+        }
     }
-    if (lane == 0) partial[wave] = total;
+    if (lane == 0) {
+        partial[2 * wave] = total;
+        partial[2 * wave + 1] = bad;
+    }
 }
 
 __global__ __launch_bounds__(1024) void grad_norm_finish_kernel(const double *__restrict__ partial, uint32_t n,
                                                                 float max_norm, float denom_eps,
-                                                                float *__restrict__ out /* norm, scale */) {
-    __shared__ double sh[1024];
-    double acc = 0.0;
-    for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) acc += partial[i];
+                                                                float *__restrict__ out /* norm, scale, u64 count */) {
+    // partial holds, per wave of the first pass, the sum of squares and the count of non-finite elements
+    __shared__ double sh[1024], shb[1024];
+    double acc = 0.0, bad = 0.0;
+    for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) {
+        acc += partial[2 * i];
+        bad += partial[2 * i + 1];
+    }
     sh[threadIdx.x] = acc;
+    shb[threadIdx.x] = bad;
     __syncthreads();
     for (uint32_t s = blockDim.x / 2; s > 0; s >>= 1) {
-        if (threadIdx.x < s) sh[threadIdx.x] += sh[threadIdx.x + s];
+        if (threadIdx.x < s) {
+            sh[threadIdx.x] += sh[threadIdx.x + s];
+            shb[threadIdx.x] += shb[threadIdx.x + s];
+        }
         __syncthreads();
     }
     if (threadIdx.x == 0) {
@@ -1000,6 +1028,7 @@ __global__ __launch_bounds__(1024) void grad_norm_finish_kernel(const double *__
         if (max_norm > 0.0f && norm > max_norm && norm <= 3.4028234e38f) scale = max_norm / (norm + denom_eps);
         out[0] = norm;
         out[1] = scale;
+        *reinterpret_cast<unsigned long long *>(out + 2) = (unsigned long long)shb[0];
     }
 }
 

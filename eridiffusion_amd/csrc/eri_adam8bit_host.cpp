@@ -456,6 +456,12 @@ int eri_adam8bit_last_grad_norm(EriAdam8bit *o, float *norm, float *scale) {
     return eri_adam8_grad_norm_read(o->table, norm, scale, o->stream);
 }
 
+int eri_adam8bit_last_nonfinite_grads(EriAdam8bit *o, uint64_t *count) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    if (!o->table) return fail(ERI_ERR_ARG, "no step has run yet");
+    return eri_adam8_grad_nonfinite_read(o->table, count, o->stream);
+}
+
 int eri_adam8bit_track_quantization_error(EriAdam8bit *o, int enabled) {
     if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
     o->track_qerr = enabled != 0;

@@ -694,8 +694,9 @@ int eri_adam8_grad_norm(EriAdam8Table *t, float max_norm, float denom_eps, void 
     if (rc) return rc;
     const uint32_t grid_cap = ctx->cus * 8; // persistent: 8 workgroups of 4 waves per compute unit
     if (!t->partial) {
-        ERI_HIP(hipMalloc((void **)&t->partial, sizeof(double) * 2 * grid_cap * eri::kNormWavesPerWg));
-        ERI_HIP(hipMalloc((void **)&t->norm_out, sizeof(float) * 2));
+        // two groups at most, and per wave a sum of squares and a count
+        ERI_HIP(hipMalloc((void **)&t->partial, sizeof(double) * 2 * 2 * grid_cap * eri::kNormWavesPerWg));
+        ERI_HIP(hipMalloc((void **)&t->norm_out, sizeof(float) * 4)); // norm, scale, 64-bit count
     }
     uint32_t off = 0;
     for (auto &g : t->groups) {
@@ -703,7 +704,7 @@ int eri_adam8_grad_norm(EriAdam8Table *t, float max_norm, float denom_eps, void 
         const uint32_t work = g.total_blocks > g.n ? g.total_blocks : g.n;
         uint32_t grid = (work + eri::kNormWavesPerWg - 1) / eri::kNormWavesPerWg;
         if (grid > grid_cap) grid = grid_cap;
-        rc = eri::launch_grad_sumsq(g.dev, g.n, g.total_blocks, g.dtype, t->partial + off, grid, stream);
+        rc = eri::launch_grad_sumsq(g.dev, g.n, g.total_blocks, g.dtype, t->partial + 2 * off, grid, stream);
         if (rc) return hip_fail((hipError_t)rc, "gradient sum-of-squares launch");
         off += grid * eri::kNormWavesPerWg;
     }
@@ -721,6 +722,16 @@ int eri_adam8_grad_norm_read(EriAdam8Table *t, float *norm, float *scale, void *
     ERI_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
     if (norm) *norm = host[0];
     if (scale) *scale = host[1];
+    return 0;
+}
+
+int eri_adam8_grad_nonfinite_read(EriAdam8Table *t, uint64_t *count, void *stream) {
+    if (!t || !count) return fail(ERI_ERR_NULL, "table or count is NULL");
+    if (!t->norm_out) return fail(ERI_ERR_ARG, "no gradient norm has been computed for this table");
+    unsigned long long host = 0;
+    ERI_HIP(hipMemcpyAsync(&host, t->norm_out + 2, sizeof host, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream)));
+    ERI_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    *count = host;
     return 0;
 }
 

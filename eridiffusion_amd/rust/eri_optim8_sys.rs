@@ -85,6 +85,7 @@ extern "C" {
     pub fn eri_adam8_step_table(table: *mut EriAdam8Table, hyper: *const EriAdam8Hyper, stream: *mut c_void) -> c_int;
     pub fn eri_adam8_grad_norm(table: *mut EriAdam8Table, max_norm: f32, denom_eps: f32, stream: *mut c_void) -> c_int;
     pub fn eri_adam8_grad_norm_read(table: *mut EriAdam8Table, norm: *mut f32, scale: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn eri_adam8_grad_nonfinite_read(table: *mut EriAdam8Table, count: *mut u64, stream: *mut c_void) -> c_int;
     pub fn eri_adam8_quant_error(table: *mut EriAdam8Table, hyper: *const EriAdam8Hyper, stream: *mut c_void) -> c_int;
     pub fn eri_adam8_quant_error_read(table: *mut EriAdam8Table, m_error: *mut f32, v_error: *mut f32, stream: *mut c_void) -> c_int;
     pub fn eri_adam8_step_multi(rows: *const EriAdam8Tensor, n: u32, hyper: *const EriAdam8Hyper, stream: *mut c_void) -> c_int;
@@ -112,6 +113,7 @@ extern "C" {
     pub fn eri_adam8bit_set_param_grad_scale(opt: *mut EriAdam8bit, index: u32, scale: f32) -> c_int;
     pub fn eri_adam8bit_set_max_grad_norm(opt: *mut EriAdam8bit, max_norm: f32, denom_eps: f32) -> c_int;
     pub fn eri_adam8bit_last_grad_norm(opt: *mut EriAdam8bit, norm: *mut f32, scale: *mut f32) -> c_int;
+    pub fn eri_adam8bit_last_nonfinite_grads(opt: *mut EriAdam8bit, count: *mut u64) -> c_int;
     pub fn eri_adam8bit_track_quantization_error(opt: *mut EriAdam8bit, enabled: c_int) -> c_int;
     pub fn eri_adam8bit_quantization_stats(opt: *mut EriAdam8bit, m_error: *mut f32, v_error: *mut f32) -> c_int;
     pub fn eri_adam8bit_set_flags(opt: *mut EriAdam8bit, flags: u32) -> c_int;

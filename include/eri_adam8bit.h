@@ -73,6 +73,8 @@ int eri_adam8bit_set_flags(EriAdam8bit *opt, uint32_t flags); /* ERI_ADAM8_FLAG_
 int eri_adam8bit_set_max_grad_norm(EriAdam8bit *opt, float max_norm, float denom_eps);
 /* Norm and clip factor of the last step that clipped (waits for the optimizer's stream). */
 int eri_adam8bit_last_grad_norm(EriAdam8bit *opt, float *norm, float *scale);
+/* NaN / infinite gradient elements seen by the norm pass of the last step that clipped (same wait). */
+int eri_adam8bit_last_nonfinite_grads(EriAdam8bit *opt, uint64_t *count);
 /* quantization_stats() :318-327: mean over parameters of the mean absolute quantisation error of the
  * first and second moments at the last step.  Tracking costs one extra read pass per step, so it is
  * opt-in: eri_adam8bit_track_quantization_error(opt, 1) before the steps of interest. */

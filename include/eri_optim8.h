@@ -167,6 +167,13 @@ int eri_adam8_step_table(EriAdam8Table *table, const EriAdam8Hyper *hyper, void 
 int eri_adam8_grad_norm(EriAdam8Table *table, float max_norm, float denom_eps, void *stream);
 /* Copies the last norm and clip factor to the host; waits for `stream`. */
 int eri_adam8_grad_norm_read(EriAdam8Table *table, float *norm, float *scale, void *stream);
+/* How many gradient elements of the table were NaN or +-infinity in the last eri_adam8_grad_norm; waits
+ * for `stream`.  Such values propagate through the step (a NaN gradient gives a NaN parameter, as with
+ * the reference's tensor ops), so a trainer can check this, or the norm, before it steps (the
+ * reference's trainers test the loss instead: pipeline_flux_lora_sequential.rs:1137).
+ * The count costs nothing on clean gradients: elements are examined only in blocks whose sum of
+ * squares is not finite. */
+int eri_adam8_grad_nonfinite_read(EriAdam8Table *table, uint64_t *count, void *stream);
 
 /* Quantisation error the next step will incur: a read-only pass that forms the new moments exactly as
  * eri_adam8_step_table(table, hyper) would, quantises them and accumulates |value - dequantised value|.

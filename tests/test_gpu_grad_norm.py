@@ -70,6 +70,9 @@ def test_non_finite_gradients_do_not_clip():
     norm, scale = C.c_float(), C.c_float()
     L.check(L.lib().eri_adam8_grad_norm_read(table, C.byref(norm), C.byref(scale), None), "read")
     assert np.isinf(norm.value) and scale.value == 1.0
+    bad = C.c_uint64(99)
+    L.check(L.lib().eri_adam8_grad_nonfinite_read(table, C.byref(bad), None), "nonfinite_read")
+    assert bad.value == 1
     h = L.hyper_pack(LR, B1, B2, EPS, WD, 1, L.MODE_ERI, L.FLAG_CLIP_FROM_TABLE)
     fresh = C.c_void_p()
     L.check(L.lib().eri_adam8_table_create(rows, len(rows), None, C.byref(fresh)), "table_create")
@@ -108,3 +111,41 @@ def test_optimizer_object_clips_inside_step():
     for g, w in zip(got_p, ps):
         assert np.array_equal(g, w)
     L.lib().eri_adam8bit_destroy(opt)
+
+
+@pytest.mark.parametrize("bf16", [True, False])
+def test_non_finite_gradient_count(bf16):
+    """NaN and +-inf elements are counted exactly, in full blocks and in partial last blocks; huge
+    finite values whose squares overflow make the norm infinite but are not counted."""
+    L = _L()
+    sizes = [2048 * 4 + 100, 50, 2048 * 2, 2048 * 3 + 1]
+    ps, gs = hs.make_inputs(sizes, bf16, 13)
+
+    def put(i, j, value):
+        gs[i][j] = onp.f32_to_bf16(np.array([value], np.float32))[0] if bf16 else value
+
+    put(0, 5, np.nan); put(0, 2048 * 2 + 77, -np.inf); put(0, 2048 * 4 + 99, np.inf)   # full blocks and the tail
+    put(1, 49, np.nan)                                                               # a tensor that is only a tail
+    put(2, 2048 + 3, np.nan); put(2, 2048 + 4, np.nan); put(2, 4095, np.inf)          # three in one block
+    put(3, 10, 3.0e38)                                                               # finite, square overflows
+    want = sum(int(np.count_nonzero(~np.isfinite(g))) for g in _f32(gs, bf16))
+    assert want == 7
+    gt = hs.GpuTensors(ps, gs, hs.oracle_states(sizes), bf16)
+    rows = gt.rows()
+    table = C.c_void_p()
+    L.check(L.lib().eri_adam8_table_create(rows, len(rows), None, C.byref(table)), "table_create")
+    for _ in range(2):  # the count does not accumulate over calls
+        L.check(L.lib().eri_adam8_grad_norm(table, 1.0, 0.0, None), "grad_norm")
+        bad = C.c_uint64()
+        L.check(L.lib().eri_adam8_grad_nonfinite_read(table, C.byref(bad), None), "nonfinite_read")
+        assert bad.value == want
+    L.lib().eri_adam8_table_destroy(table)
+    # clean gradients: zero
+    ps, gs = hs.make_inputs(sizes, bf16, 14)
+    gt = hs.GpuTensors(ps, gs, hs.oracle_states(sizes), bf16)
+    rows = gt.rows()
+    L.check(L.lib().eri_adam8_table_create(rows, len(rows), None, C.byref(table)), "table_create")
+    L.check(L.lib().eri_adam8_grad_norm(table, 1.0, 0.0, None), "grad_norm")
+    L.check(L.lib().eri_adam8_grad_nonfinite_read(table, C.byref(bad), None), "nonfinite_read")
+    assert bad.value == 0
+    L.lib().eri_adam8_table_destroy(table)
