@@ -134,6 +134,22 @@ impl Adam8bit {
     pub fn set_grad_scale(&mut self, scale: f32) -> Result<()> {
         check(unsafe { sys::eri_adam8bit_set_grad_scale(self.opt, scale) }, "eri_adam8bit_set_grad_scale")
     }
+    /// Global-norm clipping inside step(): norm on the device, factor applied by the step kernel.
+    pub fn set_max_grad_norm(&mut self, max_norm: f32, denom_eps: f32) -> Result<()> {
+        check(unsafe { sys::eri_adam8bit_set_max_grad_norm(self.opt, max_norm, denom_eps) }, "eri_adam8bit_set_max_grad_norm")
+    }
+    /// (norm, clip factor, NaN/inf gradient elements) of the last step that clipped.
+    pub fn last_grad_norm(&mut self) -> Result<(f32, f32, u64)> {
+        let (mut n, mut s, mut bad) = (0f32, 1f32, 0u64);
+        check(unsafe { sys::eri_adam8bit_last_grad_norm(self.opt, &mut n, &mut s) }, "eri_adam8bit_last_grad_norm")?;
+        check(unsafe { sys::eri_adam8bit_last_nonfinite_grads(self.opt, &mut bad) }, "eri_adam8bit_last_nonfinite_grads")?;
+        Ok((n, s, bad))
+    }
+    /// Imports a file written by the reference's own save_state (bincode of OptimizerState, :330-347).
+    pub fn load_legacy_state(&mut self, path: &Path) -> Result<()> {
+        let c = CString::new(path.to_string_lossy().as_bytes()).map_err(|e| Error::InvalidOperation(e.to_string()))?;
+        check(unsafe { sys::eri_adam8bit_load_legacy_state(self.opt, c.as_ptr()) }, "eri_adam8bit_load_legacy_state")
+    }
     /// :330
     pub fn save_state(&self, path: &Path) -> Result<()> {
         let c = CString::new(path.to_string_lossy().as_bytes()).map_err(|e| Error::InvalidOperation(e.to_string()))?;
@@ -254,4 +270,73 @@ pub fn update_params_8bit(optimizer: &mut Adam8bitFunctional, params: &mut HashM
         }
     }
     Ok(())
+}
+
+// ---- the reference's optimizer traits ---------------------------------------------------------
+// Paths as in the reference tree; each impl only forwards to the methods above.
+
+/// `OptimizerWrapper { step, zero_grad, vars }`, crates/training/src/optimizers/wrapper.rs:40-44.
+impl crate::optimizers::wrapper::OptimizerWrapper for Adam8bit {
+    fn step(&mut self) -> Result<()> {
+        Adam8bit::step(self)
+    }
+    fn zero_grad(&mut self) {
+        let _ = Adam8bit::zero_grad(self);
+    }
+    fn vars(&mut self) -> &mut [Parameter] {
+        self.params.as_mut_slice()
+    }
+}
+
+/// `training::OptimizerTrait`, src/trainers/training/optimization.rs:61-73.  The reference's impl for
+/// Adam8bit is a set of placeholders (:75-103: step does nothing, get_lr returns 1e-4); here the
+/// per-parameter step() hands the gradient to the matching handle and the launch happens in
+/// `flush()`, which the trainer calls once per accumulation boundary where it called nothing before.
+impl crate::trainers::training::optimization::OptimizerTrait for Adam8bit {
+    fn step(&mut self, param: &Parameter, grad: &Tensor) -> Result<()> {
+        let t = param.tensor()?;
+        let at = self.params.iter().position(|p| p.tensor().map(|q| q.cuda_ptr() == t.cuda_ptr()).unwrap_or(false))
+            .ok_or_else(|| Error::InvalidOperation("parameter is not owned by this optimizer".into()))?;
+        let g = if grad.dtype() != t.dtype() { grad.to_dtype(t.dtype())? } else { grad.clone() };
+        check(unsafe { sys::eri_param_set_grad(self.handles[at], g.cuda_ptr() as *const c_void) }, "eri_param_set_grad")?;
+        self.live_grads.push(g);
+        Ok(())
+    }
+    fn zero_grad(&mut self) -> Result<()> {
+        Adam8bit::zero_grad(self)
+    }
+    fn get_lr(&self) -> f32 {
+        self.current_lr() as f32
+    }
+    fn set_lr(&mut self, lr: f32) {
+        self.set_learning_rate(lr as f64)
+    }
+    fn state_dict(&self) -> Result<HashMap<String, Tensor>> {
+        Err(Error::Unsupported("the 8-bit state is saved with save_state(path), not as tensors".into()))
+    }
+    fn load_state_dict(&mut self, _state: HashMap<String, Tensor>) -> Result<()> {
+        Err(Error::Unsupported("the 8-bit state is loaded with load_state(path)".into()))
+    }
+}
+
+impl Adam8bit {
+    /// Launches the step for the gradients handed over through `OptimizerTrait::step`.
+    pub fn flush(&mut self) -> Result<()> {
+        let rc = check(unsafe { sys::eri_adam8bit_step(self.opt, std::ptr::null_mut()) }, "eri_adam8bit_step");
+        self.live_grads.clear();
+        rc
+    }
+}
+
+/// String-keyed factory, src/trainers/training/optimization.rs:30-58 and
+/// src/optimizers/memory_efficient_optimizers.rs:285-308.
+pub fn create_optimizer(optimizer_type: &str, parameters: Vec<Parameter>, learning_rate: f64, betas: Option<(f64, f64)>,
+                        eps: Option<f64>, weight_decay: Option<f64>) -> Result<Adam8bit> {
+    match optimizer_type {
+        "adam8bit" | "adamw8bit" | "adamw_8bit" => Adam8bit::new(parameters, Adam8bitConfig {
+            lr: learning_rate, betas: betas.unwrap_or((0.9, 0.999)), eps: eps.unwrap_or(1e-8),
+            weight_decay: weight_decay.unwrap_or(0.0), ..Adam8bitConfig::default()
+        }),
+        other => Err(Error::InvalidOperation(format!("Unknown optimizer: {other}"))),
+    }
 }
