@@ -11,7 +11,7 @@ LIB_PATH = os.path.join(_HERE, "liberi_optim8.so")
 
 BLOCK = 2048
 DTYPE_F32, DTYPE_F16, DTYPE_BF16, DTYPE_I32 = 0, 1, 2, 3
-MODE_ERI, MODE_L2 = 0, 1
+MODE_ERI, MODE_L2, MODE_BNB = 0, 1, 2
 FLAG_GRAD_SCALE, FLAG_EXACT_PARAM, FLAG_BSEARCH, FLAG_NO_PIPELINE, FLAG_CLIP_FROM_TABLE = 1, 2, 4, 8, 16
 
 
@@ -113,6 +113,7 @@ EXPORTS = {
     "eri_adam8bit_set_grad_scale": (C.c_int, [C.c_void_p, C.c_float]),
     "eri_adam8bit_set_param_grad_scale": (C.c_int, [C.c_void_p, C.c_uint32, C.c_float]),
     "eri_adam8bit_set_max_grad_norm": (C.c_int, [C.c_void_p, C.c_float, C.c_float]),
+    "eri_adam8bit_set_mode": (C.c_int, [C.c_void_p, C.c_int]),
     "eri_adam8bit_last_grad_norm": (C.c_int, [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
     "eri_adam8bit_last_nonfinite_grads": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint64)]),
     "eri_adam8bit_track_quantization_error": (C.c_int, [C.c_void_p, C.c_int]),

@@ -96,6 +96,10 @@ class Adam8bit:
     def set_grad_scale(self, scale: float) -> None:
         check(lib().eri_adam8bit_set_grad_scale(self._opt, scale), "eri_adam8bit_set_grad_scale")
 
+    def set_mode(self, mode: int) -> None:
+        """MODE_ERI (the reference's update, default) or MODE_BNB."""
+        check(lib().eri_adam8bit_set_mode(self._opt, mode), "eri_adam8bit_set_mode")
+
     def set_max_grad_norm(self, max_norm: float, denom_eps: float = 0.0) -> None:
         """Global-norm clipping inside step(): norm on the device, factor applied by the step kernel
         (clip_gradients, src/trainers/pipeline_flux_lora_sequential.rs:1198-1213).  <= 0 switches it off."""

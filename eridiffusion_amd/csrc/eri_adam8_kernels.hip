@@ -195,6 +195,12 @@ __device__ __forceinline__ void adam_elem(float p, float g, float m_old, float v
         float us = upd * h.step_size; // :196
         if (BF16) us = bf16_round(us); // :197-198
         pn = p - us;                   // :205
+    } else if (MODE == ERI_ADAM8_MODE_BNB) { // h.eps carries sqrt(bc2), h.weight_decay is the factor 1 - lr*wd
+        float den = sqrtf(v) + h.eps;
+        float r = m / den;
+        float us = r * h.step_size;
+        pn = p - us;
+        if (WD) pn = pn * h.weight_decay;
     } else {
         if (EXACT) {
             float den = sqrtf(v) + h.eps; // adam8bit_enhanced.rs:263
@@ -339,10 +345,18 @@ __device__ __forceinline__ void pack_code(uint32_t &acc, int k, float xs, float 
     }
 }
 
-template <bool FAST_DIV, bool KEYTAB>
+/* Mode BNB: a first-moment code whose map value has the other sign than the moment moves one entry
+ * toward the moment's sign.  The signed map is negative below entry 127, zero at 127 and positive
+ * above, and the quotient has the moment's sign, so the only case is a negative moment that
+ * rounds to the zero entry: it takes entry 126, the negative value nearest zero. */
+__device__ __forceinline__ uint32_t keep_sign(uint32_t code, float m, float absmax) {
+    return (code == 127u && (f2u(m) >> 31) != 0u && absmax != 0.0f) ? 126u : code;
+}
+
+template <bool FAST_DIV, bool KEYTAB, bool KEEP_SIGN = false>
 __device__ __forceinline__ void requant8(const float *mf, const float *vf, const BlockDiv &dm, const BlockDiv &dv,
                                          const Lds &L, u32x2 &mw, u32x2 &vw) {
-    if (KEYTAB && FAST_DIV) { // the hot path: slot lookup, codes packed by byte-select writes
+    if (KEYTAB && FAST_DIV && !KEEP_SIGN) { // the hot path: slot lookup, codes packed by byte-select writes
         uint32_t am[2], av[2];
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
@@ -363,6 +377,7 @@ __device__ __forceinline__ void requant8(const float *mf, const float *vf, const
         const float xm = FAST_DIV ? dm.div_fast(mf[k]) : dm.div_slow(mf[k]); // times dm.scale
         const float xv = FAST_DIV ? dv.div_fast(vf[k]) : dv.div_slow(vf[k]);
         cm[k] = KEYTAB ? code_signed_key(xm, L.key_s) : code_bsearch(xm, L.mid_s);
+        if (KEEP_SIGN) cm[k] = keep_sign(cm[k], mf[k], dm.a);
         cv[k] = KEYTAB ? code_unsigned_key(xv, L.key_u) : code_bsearch(xv, L.mid_u);
     }
     mw.x = cm[0] | (cm[1] << 8) | (cm[2] << 16) | (cm[3] << 24);
@@ -434,7 +449,7 @@ __device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint
         for (int c = 0; c < 4; ++c) {
             const uint32_t o = c * 512 + lane * 8;
             u32x2 mw, vw;
-            requant8<true, KEYTAB>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
+            requant8<true, KEYTAB, MODE == ERI_ADAM8_MODE_BNB>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
             *as_global(reinterpret_cast<u32x2 *>(mc + o)) = mw;
             *as_global(reinterpret_cast<u32x2 *>(vc + o)) = vw;
         }
@@ -443,7 +458,7 @@ __device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint
         for (int c = 0; c < 4; ++c) {
             const uint32_t o = c * 512 + lane * 8;
             u32x2 mw, vw;
-            requant8<false, KEYTAB>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
+            requant8<false, KEYTAB, MODE == ERI_ADAM8_MODE_BNB>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
             *as_global(reinterpret_cast<u32x2 *>(mc + o)) = mw;
             *as_global(reinterpret_cast<u32x2 *>(vc + o)) = vw;
         }
@@ -490,7 +505,9 @@ __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint
                                              L.map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn);
         const float xm = dm.div_slow(m);
         const float xv = dv.div_slow(v);
-        mc[e] = (uint8_t)(KEYTAB ? code_signed_key(xm, L.key_s) : code_bsearch(xm, L.mid_s));
+        uint32_t cm = KEYTAB ? code_signed_key(xm, L.key_s) : code_bsearch(xm, L.mid_s);
+        if (MODE == ERI_ADAM8_MODE_BNB) cm = keep_sign(cm, m, nam);
+        mc[e] = (uint8_t)cm;
         vc[e] = (uint8_t)(KEYTAB ? code_unsigned_key(xv, L.key_u) : code_bsearch(xv, L.mid_u));
         if (BF16) as_global(static_cast<uint16_t *>(t.p))[e] = (uint16_t)bf16_bits(pn);
         else as_global(static_cast<float *>(t.p))[e] = pn;
@@ -822,6 +839,20 @@ int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, i
                 void *stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool exact = (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0;
+    if (h.mode == ERI_ADAM8_MODE_BNB) { // plain kernel, slot table, IEEE arithmetic; the decay is a factor
+        const bool wd = h.weight_decay != 1.0f;
+        const bool gs = (h.flags & ERI_ADAM8_FLAG_GRAD_SCALE) != 0;
+#define ERI_BNB(B, W, G) return launch_one<B, ERI_ADAM8_MODE_BNB, true, W, G, true>(rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, s)
+        if (dtype_tag == ERI_DTYPE_F32) {
+            if (wd) { if (gs) ERI_BNB(false, true, true); ERI_BNB(false, true, false); }
+            if (gs) ERI_BNB(false, false, true);
+            ERI_BNB(false, false, false);
+        }
+        if (wd) { if (gs) ERI_BNB(true, true, true); ERI_BNB(true, true, false); }
+        if (gs) ERI_BNB(true, false, true);
+        ERI_BNB(true, false, false);
+#undef ERI_BNB
+    }
     if (dtype_tag == ERI_DTYPE_F32) {
         if (h.mode == ERI_ADAM8_MODE_L2)
             return launch_flags<false, ERI_ADAM8_MODE_L2, true>(rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, s);

@@ -228,6 +228,7 @@ struct EriAdam8bit {
     double lr = 1e-3, beta1 = 0.9, beta2 = 0.999, eps = 1e-8, wd = 0.01;
     uint64_t step = 0;
     uint32_t flags = 0;
+    int mode = ERI_ADAM8_MODE_ERI;
     float grad_scale = 1.0f;
     float max_grad_norm = 0.0f, clip_denom_eps = 0.0f;
     bool track_qerr = false, have_qerr = false;
@@ -395,11 +396,17 @@ int eri_adam8bit_step(EriAdam8bit *o, uint32_t *skipped) {
     EriAdam8Hyper h;
     uint32_t flags = o->flags | ((scaled || clip) ? (uint32_t)ERI_ADAM8_FLAG_GRAD_SCALE : 0u) |
                      (clip ? (uint32_t)ERI_ADAM8_FLAG_CLIP_FROM_TABLE : 0u);
-    rc = eri_adam8_hyper_pack(o->lr, o->beta1, o->beta2, o->eps, o->wd, o->step, ERI_ADAM8_MODE_ERI, flags, &h);
+    rc = eri_adam8_hyper_pack(o->lr, o->beta1, o->beta2, o->eps, o->wd, o->step, o->mode, flags, &h);
     if (rc) return rc;
     h.grad_scale = o->grad_scale;
     if (o->track_qerr) {
-        rc = eri_adam8_quant_error(o->table, &h, o->stream);
+        EriAdam8Hyper hq = h; // the moments of mode BNB are those of mode ERI; the statistics pass knows ERI
+        if (o->mode == ERI_ADAM8_MODE_BNB) {
+            rc = eri_adam8_hyper_pack(o->lr, o->beta1, o->beta2, o->eps, o->wd, o->step, ERI_ADAM8_MODE_ERI, flags, &hq);
+            if (rc) return rc;
+            hq.grad_scale = o->grad_scale;
+        }
+        rc = eri_adam8_quant_error(o->table, &hq, o->stream);
         if (rc) return rc;
         o->have_qerr = true;
     }
@@ -476,6 +483,14 @@ int eri_adam8bit_quantization_stats(EriAdam8bit *o, float *m_error, float *v_err
         return 0;
     }
     return eri_adam8_quant_error_read(o->table, m_error, v_error, o->stream);
+}
+
+int eri_adam8bit_set_mode(EriAdam8bit *o, int mode) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    if (mode != ERI_ADAM8_MODE_ERI && mode != ERI_ADAM8_MODE_BNB)
+        return fail(ERI_ERR_ARG, "the list-of-parameters optimizer steps in mode ERI or BNB");
+    o->mode = mode;
+    return 0;
 }
 
 int eri_adam8bit_set_flags(EriAdam8bit *o, uint32_t flags) {

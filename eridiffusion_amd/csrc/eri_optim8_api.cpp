@@ -542,7 +542,8 @@ int eri_adam8_table_image(void *out, size_t cap, size_t *bytes, uint32_t offsets
 int eri_adam8_hyper_pack(double lr, double beta1, double beta2, double eps, double weight_decay, uint64_t step,
                          int mode, uint32_t flags, EriAdam8Hyper *out) {
     if (!out) return fail(ERI_ERR_NULL, "out is NULL");
-    if (mode != ERI_ADAM8_MODE_ERI && mode != ERI_ADAM8_MODE_L2) return fail(ERI_ERR_ARG, "unknown mode");
+    if (mode != ERI_ADAM8_MODE_ERI && mode != ERI_ADAM8_MODE_L2 && mode != ERI_ADAM8_MODE_BNB)
+        return fail(ERI_ERR_ARG, "unknown mode");
     std::memset(out, 0, sizeof(*out));
     out->mode = mode;
     out->flags = flags;
@@ -567,6 +568,10 @@ int eri_adam8_hyper_pack(double lr, double beta1, double beta2, double eps, doub
         out->bc1 = (float)bc1;
         out->bc2 = (float)bc2;
         out->step_size = (float)(lr * (std::sqrt(bc2) / bc1)); // :215, cast at :274
+        if (mode == ERI_ADAM8_MODE_BNB) {
+            out->eps = (float)(eps * std::sqrt(bc2));
+            out->weight_decay = (float)(1.0 - lr * weight_decay); // decay factor
+        }
     }
     return 0;
 }
@@ -653,7 +658,8 @@ int eri_adam8_table_info(const EriAdam8Table *t, uint64_t *total_numel, uint64_t
 
 int eri_adam8_step_table(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream) {
     if (!t || !h) return fail(ERI_ERR_NULL, "table or hyper is NULL");
-    if (h->mode != ERI_ADAM8_MODE_ERI && h->mode != ERI_ADAM8_MODE_L2) return fail(ERI_ERR_ARG, "unknown mode");
+    if (h->mode != ERI_ADAM8_MODE_ERI && h->mode != ERI_ADAM8_MODE_L2 && h->mode != ERI_ADAM8_MODE_BNB)
+        return fail(ERI_ERR_ARG, "unknown mode");
     DeviceCtx *ctx = nullptr;
     int rc = get_ctx(&ctx);
     if (rc) return rc;
@@ -737,7 +743,8 @@ int eri_adam8_grad_nonfinite_read(EriAdam8Table *t, uint64_t *count, void *strea
 
 int eri_adam8_quant_error(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream) {
     if (!t || !h) return fail(ERI_ERR_NULL, "table or hyper is NULL");
-    if (h->mode != ERI_ADAM8_MODE_ERI && h->mode != ERI_ADAM8_MODE_L2) return fail(ERI_ERR_ARG, "unknown mode");
+    if (h->mode != ERI_ADAM8_MODE_ERI && h->mode != ERI_ADAM8_MODE_L2)
+        return fail(ERI_ERR_ARG, "the quantisation error pass knows the modes ERI and L2");
     DeviceCtx *ctx = nullptr;
     int rc = get_ctx(&ctx);
     if (rc) return rc;

@@ -11,6 +11,7 @@ pub const ERI_DTYPE_BF16: i32 = 2;
 pub const ERI_DTYPE_I32: i32 = 3;
 pub const ERI_ADAM8_MODE_ERI: i32 = 0;
 pub const ERI_ADAM8_MODE_L2: i32 = 1;
+pub const ERI_ADAM8_MODE_BNB: i32 = 2;
 pub const ERI_ADAM8_FLAG_GRAD_SCALE: u32 = 1;
 pub const ERI_ADAM8_FLAG_EXACT_PARAM: u32 = 2;
 pub const ERI_ADAM8_FLAG_BSEARCH: u32 = 4;
@@ -112,6 +113,7 @@ extern "C" {
     pub fn eri_adam8bit_set_grad_scale(opt: *mut EriAdam8bit, scale: f32) -> c_int;
     pub fn eri_adam8bit_set_param_grad_scale(opt: *mut EriAdam8bit, index: u32, scale: f32) -> c_int;
     pub fn eri_adam8bit_set_max_grad_norm(opt: *mut EriAdam8bit, max_norm: f32, denom_eps: f32) -> c_int;
+    pub fn eri_adam8bit_set_mode(opt: *mut EriAdam8bit, mode: c_int) -> c_int;
     pub fn eri_adam8bit_last_grad_norm(opt: *mut EriAdam8bit, norm: *mut f32, scale: *mut f32) -> c_int;
     pub fn eri_adam8bit_last_nonfinite_grads(opt: *mut EriAdam8bit, count: *mut u64) -> c_int;
     pub fn eri_adam8bit_track_quantization_error(opt: *mut EriAdam8bit, enabled: c_int) -> c_int;

@@ -66,6 +66,8 @@ uint64_t eri_adam8bit_get_step(const EriAdam8bit *opt);
 int eri_adam8bit_set_grad_scale(EriAdam8bit *opt, float scale);
 int eri_adam8bit_set_param_grad_scale(EriAdam8bit *opt, uint32_t index, float scale);
 int eri_adam8bit_set_flags(EriAdam8bit *opt, uint32_t flags); /* ERI_ADAM8_FLAG_EXACT_PARAM etc. */
+/* ERI_ADAM8_MODE_ERI (default: the reference's update) or ERI_ADAM8_MODE_BNB for later steps. */
+int eri_adam8bit_set_mode(EriAdam8bit *opt, int mode);
 /* Global-norm clipping inside step(): max_norm > 0 makes every step first reduce the gradients' global
  * L2 norm on the device (eri_adam8_grad_norm) and apply max_norm / (norm + denom_eps) when the norm is
  * above max_norm -- the trainers' clip_gradients (pipeline_flux_lora_sequential.rs:737,1198-1213)

@@ -80,8 +80,14 @@ int eri_hip_mem_info(size_t *free_bytes, size_t *total_bytes);
 typedef enum EriAdam8Mode {
     ERI_ADAM8_MODE_ERI = 0, /* Adam8bit::step,   src/trainers/adam8bit_enhanced.rs:202-291:
                                p -= step_size * (m / (sqrt(v) + eps) + wd * p) */
-    ERI_ADAM8_MODE_L2 = 1   /* Adam8bit::update, src/trainers/adam8bit.rs:101-208:
+    ERI_ADAM8_MODE_L2 = 1,  /* Adam8bit::update, src/trainers/adam8bit.rs:101-208:
                                g += wd * p; p -= cast(lr * (m/bc1) / (sqrt(max(v/bc2, 0)) + eps)) */
+    ERI_ADAM8_MODE_BNB = 2  /* not in the reference; the update of the library the state format comes from
+                               (bitsandbytes 8-bit blockwise Adam): p = (p - step_size * m / (sqrt(v) +
+                               eps*sqrt(bc2))) * (1 - lr*wd), and a first-moment code whose map value has the
+                               other sign than the moment moves one entry toward the moment's sign.  With
+                               wd = 0 this is the textbook Adam formula.  Moments as in ERI.  Always IEEE
+                               sqrt and divide; not available to eri_adam8_quant_error. */
 } EriAdam8Mode;
 
 enum {
@@ -98,6 +104,7 @@ enum {
 
 /* Per-step scalars, already cast where the reference casts them.  Fill with eri_adam8_hyper_pack. */
 typedef struct EriAdam8Hyper {
+    /* BNB: eps holds (float)(eps * sqrt(bc2)) and weight_decay the factor (float)(1 - lr*wd). */
     float beta1, beta2; /* (float)beta                               adam8bit_enhanced.rs:256,260 */
     float omb1, omb2;   /* ERI: 1.0f - (float)beta; L2: (float)(1.0 - beta)    :256,260 / adam8bit.rs:142,151 */
     float eps;          /* (float)eps                                :263 */

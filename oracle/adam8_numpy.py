@@ -7,6 +7,8 @@ bit; the shipped library and the Python package never import it.
 It follows the same two reference functions as the C oracle:
   * mode "eri": Adam8bit::step, src/trainers/adam8bit_enhanced.rs:202-291
   * mode "l2" : Adam8bit::update, src/trainers/adam8bit.rs:101-208
+  * mode "bnb": parameter update and sign rule of bitsandbytes' 8-bit blockwise Adam (the library the
+    state format comes from; not installed here, not used by the reference)
 with the state kept as uint8 codes into the bitsandbytes dynamic maps plus one fp32 absmax per
 2048-element block.  Every NumPy float32 operation below rounds once, which is the rounding
 behaviour of the reference's chain of separate tensor operations.
@@ -70,6 +72,9 @@ def hyper_pack(lr, beta1, beta2, eps, wd, step, mode="eri"):
         h["bc1"] = F32(bc1)
         h["bc2"] = F32(bc2)
         h["step_size"] = F32(lr * (math.sqrt(bc2) / bc1))
+        if mode == "bnb":  # eps rides on sqrt(bc2); the decay becomes a factor applied after the Adam term
+            h["eps"] = F32(eps * math.sqrt(bc2))
+            h["wd"] = F32(1.0 - lr * wd)
     return h
 
 
@@ -114,6 +119,10 @@ def step_tensor(p, g, m_code, v_code, absmax_m, absmax_v, h, map_s, map_u, bf16=
             if bf16:
                 us = bf16_to_f32(f32_to_bf16(us))
             pn = pf - us
+        elif h["mode"] == "bnb":
+            pn = pf - (m / (np.sqrt(v) + h["eps"])) * h["step_size"]
+            if h["wd"] != F32(1.0):
+                pn = pn * h["wd"]
         else:
             r = m / (np.sqrt(v) + h["eps"])
             u = r + pf * h["wd"] if h["wd"] > 0 else r
@@ -128,5 +137,8 @@ def step_tensor(p, g, m_code, v_code, absmax_m, absmax_v, h, map_s, map_u, bf16=
         xv = np.where(av_e == 0, F32(0), v / np.where(av_e == 0, F32(1), av_e)).astype(F32)
     mc = nearest_index(midpoints(map_s), xm)
     vc = nearest_index(midpoints(map_u), xv)
+    if h["mode"] == "bnb":  # a code whose map value has the other sign than the moment moves toward the moment
+        flip = (np.signbit(map_s[mc]) != np.signbit(m)) & (am_e != 0) & np.isfinite(m)
+        mc = np.where(flip, np.where(m > 0, mc.astype(np.int32) + 1, mc.astype(np.int32) - 1), mc).astype(np.uint8)
     p_out = f32_to_bf16(pn) if bf16 else pn.astype(F32)
     return p_out, mc, vc, am, av

@@ -7,6 +7,11 @@
  * It is a scalar restatement, one individually rounded fp32 operation per line, of
  *   - EriDiffusion's Adam8bit::step          src/trainers/adam8bit_enhanced.rs:202-291  (mode ERI)
  *   - EriDiffusion's functional Adam8bit::update  src/trainers/adam8bit.rs:101-208      (mode L2)
+ *   - mode BNB: the parameter update and the sign rule of the library the state format comes from
+ *     (bitsandbytes 8-bit blockwise Adam, csrc/kernels.cu kOptimizerStatic8bit2StateBlockwise; not
+ *     installed here, not used by the reference): eps scaled by sqrt(bc2), decay applied as a
+ *     factor (1 - lr*wd) after the Adam term, and a first-moment code whose map value has the
+ *     other sign than the moment moved one entry toward the moment's sign
  * with the state held in the blockwise format the optimizer is specified to use: uint8 codes
  * into the signed (first moment) and unsigned (second moment) 256-entry dynamic maps of
  * bitsandbytes (functional.py: create_dynamic_map), one fp32 absmax per 2048-element block.
@@ -23,6 +28,11 @@
  *                              quantiser bypassed, block-max brute force, and bit-for-bit
  *                              agreement with the independent NumPy restatement
  *                              (oracle/adam8_numpy.py)                              pinned
+ *   mode BNB of the step       with wd = 0 it IS torch.optim.Adam's formula (denominator
+ *                              sqrt(v)/sqrt(bc2) + eps): 60 steps against torch.optim.Adam;
+ *                              decay factor and sign rule by closed form.  Bit-level equality
+ *                              with bitsandbytes itself (its fast division, its
+ *                              quantisation search)                                  parity unpinned
  *   eri_oracle_adamw32_step    closed form at step 1, float64 recurrence, the reference's
  *                              own 2x2 test case                                     pinned
  *   eri_oracle_ema_update      float64 closed form; bf16 intermediate rounding of flame-core
@@ -43,7 +53,7 @@
 
 #define ERI_ORACLE_BLOCK 2048
 
-enum { ERI_ORACLE_MODE_ERI = 0, ERI_ORACLE_MODE_L2 = 1 };
+enum { ERI_ORACLE_MODE_ERI = 0, ERI_ORACLE_MODE_L2 = 1, ERI_ORACLE_MODE_BNB = 2 };
 enum { ERI_ORACLE_F32 = 0, ERI_ORACLE_BF16 = 2 };
 
 typedef struct EriOracleHyper {
@@ -52,8 +62,10 @@ typedef struct EriOracleHyper {
     float omb1;         /* ERI: 1.0f - (float)beta1 (fp32 subtraction)    :256
                            L2 : (float)(1.0 - beta1)  (f64 subtraction)   adam8bit.rs:142 */
     float omb2;         /* same for beta2                                 :260 / adam8bit.rs:151 */
-    float eps;          /* (float)eps                                     :263 / adam8bit.rs:186 */
-    float weight_decay; /* (float)wd                                      :268 / adam8bit.rs:117 */
+    float eps;          /* (float)eps                                     :263 / adam8bit.rs:186
+                           BNB: (float)(eps * sqrt(bc2)) */
+    float weight_decay; /* (float)wd                                      :268 / adam8bit.rs:117
+                           BNB: the decay factor (float)(1 - lr*wd) */
     float step_size;    /* ERI: (float)(lr*sqrt(bc2)/bc1)                 :213-215,:274
                            L2 : (float)lr                                 adam8bit.rs:193 */
     float bc1;          /* L2 : (float)(1 - beta1^s), s = max(step,1)     adam8bit.rs:164-168 */
@@ -133,6 +145,10 @@ void eri_oracle_hyper_pack(double lr, double beta1, double beta2, double eps, do
         h->bc1 = (float)bc1;
         h->bc2 = (float)bc2;
         h->step_size = (float)(lr * (sqrt(bc2) / bc1));
+        if (mode == ERI_ORACLE_MODE_BNB) {
+            h->eps = (float)(eps * sqrt(bc2));
+            h->weight_decay = (float)(1.0 - lr * wd);
+        }
     }
 }
 
@@ -184,6 +200,12 @@ static void step_block(void *p, const void *g, uint8_t *mc, uint8_t *vc, float *
             if (dtype == ERI_ORACLE_BF16)               /* :197-198 update cast to the param dtype */
                 us = eri_oracle_bf16_to_f32(eri_oracle_f32_to_bf16(us));
             pn = pf - us;                               /* :205 */
+        } else if (h->mode == ERI_ORACLE_MODE_BNB) {
+            float den = sqrtf(v) + h->eps;              /* eps already times sqrt(bc2) */
+            float r = m / den;
+            float us = r * h->step_size;
+            pn = pf - us;
+            if (h->weight_decay != 1.0f) pn = pn * h->weight_decay; /* decay factor, after the Adam term */
         } else {
             float den = sqrtf(v) + h->eps;              /* adam8bit_enhanced.rs:263 */
             float r = m / den;                          /* :264 */
@@ -202,7 +224,12 @@ static void step_block(void *p, const void *g, uint8_t *mc, uint8_t *vc, float *
         const uint64_t e = base + (uint64_t)i;
         float xm = (new_am == 0.0f) ? 0.0f : mbuf[i] / new_am;
         float xv = (new_av == 0.0f) ? 0.0f : vbuf[i] / new_av;
-        mc[e] = (uint8_t)eri_oracle_nearest_index(mid_s, xm);
+        int cm = eri_oracle_nearest_index(mid_s, xm);
+        if (h->mode == ERI_ORACLE_MODE_BNB && new_am != 0.0f && isfinite(mbuf[i]) &&
+            (signbit(map_s[cm]) != 0) != (signbit(mbuf[i]) != 0)) {
+            if (mbuf[i] > 0.0f) cm += 1; else cm -= 1; /* keep the sign of the first moment */
+        }
+        mc[e] = (uint8_t)cm;
         vc[e] = (uint8_t)eri_oracle_nearest_index(mid_u, xv);
     }
     *am = new_am;

@@ -9,7 +9,7 @@ import numpy as np
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 ORACLE_DIR = os.path.join(ROOT, "oracle")
 BLOCK = 2048
-MODE_ERI, MODE_L2 = 0, 1
+MODE_ERI, MODE_L2, MODE_BNB = 0, 1, 2
 DT_F32, DT_BF16 = 0, 2
 
 

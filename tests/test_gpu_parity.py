@@ -12,6 +12,7 @@ import pytest
 
 import harness as hs
 import oracle_c as oc
+from oracle import adam8_numpy as onp
 
 pytestmark = pytest.mark.gpu
 
@@ -45,7 +46,7 @@ def gpu_steps(gt, steps_grads, first_step, mode=0, flags=0, wd=WD, lr=LR, grad_s
         if gs is not None:
             gt.set_grads(gs)
         step = first_step + k
-        h = L.hyper_pack(lr, B1, B2, EPS, wd, step if mode == 0 else step - 1, mode, flags, grad_scale)
+        h = L.hyper_pack(lr, B1, B2, EPS, wd, step - 1 if mode == 1 else step, mode, flags, grad_scale)
         if use_multi:
             L.check(L.lib().eri_adam8_step_multi(rows, len(rows), C.byref(h), _stream()), "step_multi")
         else:
@@ -59,18 +60,18 @@ def run_case(sizes, bf16, seed, steps=3, mode=0, flags=0, wd=WD, p_std=0.02, g_s
              grad_scale=None, use_multi=False, label=""):
     ps, gs = hs.make_inputs(sizes, bf16, seed, p_std, g_std)
     states = hs.oracle_states(sizes)
-    omode = oc.MODE_ERI if mode == 0 else oc.MODE_L2
+    omode = {0: oc.MODE_ERI, 1: oc.MODE_L2, 2: oc.MODE_BNB}[mode]
     for t in range(1, prior + 1):  # seed the states with a few oracle steps
         g_t = hs.fresh_grads(sizes, bf16, seed * 1000 + t, g_std)
-        hs.oracle_step(ps, g_t, states, (LR, B1, B2, EPS, wd, t if mode == 0 else t - 1), bf16, omode, grad_scale)
+        hs.oracle_step(ps, g_t, states, (LR, B1, B2, EPS, wd, t - 1 if mode == 1 else t), bf16, omode, grad_scale)
     gt = hs.GpuTensors(ps, gs, states, bf16)
     all_g = [gs] + [hs.fresh_grads(sizes, bf16, seed * 7777 + k, g_std) for k in range(1, steps)]
     for k, g_k in enumerate(all_g):
         t = prior + 1 + k
-        hs.oracle_step(ps, g_k, states, (LR, B1, B2, EPS, wd, t if mode == 0 else t - 1), bf16, omode, grad_scale)
+        hs.oracle_step(ps, g_k, states, (LR, B1, B2, EPS, wd, t - 1 if mode == 1 else t), bf16, omode, grad_scale)
     gpu_steps(gt, [None] + all_g[1:], prior + 1, mode, flags, wd, grad_scale=grad_scale, use_multi=use_multi)
     got_p, got_st = gt.fetch()
-    exact = (not bf16) or bool(flags & 2)
+    exact = (not bf16) or bool(flags & 2) or mode == 2
     stats = hs.compare(got_p, got_st, ps, states, bf16, exact, label)
     print("%s: params=%d code_mismatch=%d param_1ulp=%d" % (label, stats["params"], stats["code_mismatch"],
                                                               stats["param_1ulp"]), flush=True)
@@ -105,6 +106,42 @@ def test_fp32_ragged_multi_tensor(flags):
 def test_l2_mode_follows_the_functional_update(bf16, wd):
     sizes = [2048 * 5 + 77, 320, 2048, 9]
     run_case(sizes, bf16, 300 + bf16, steps=3, mode=1, flags=2, wd=wd, label="l2-bf16%d-wd%g" % (bf16, wd))
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("wd,gscale", [(0.0, None), (0.01, None), (0.01, 0.37)])
+def test_bnb_mode(bf16, wd, gscale):
+    sizes = [2048 * 5 + 77, 320, 2048, 9, 2047, 40000]
+    run_case(sizes, bf16, 350 + bf16, steps=3, mode=2, wd=wd, grad_scale=gscale, prior=2,
+             label="bnb-bf16%d-wd%g-gs%s" % (bf16, wd, gscale))
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_bnb_mode_keeps_the_sign_of_tiny_first_moments(bf16):
+    # moments 1e-9 of the block's largest round to the zero entry: BNB stores 126 for the negative
+    # ones (full blocks and a partial last block), ERI 127; the oracle must agree element for element
+    sizes = [2048 * 2 + 300]
+    ps, gs = hs.make_inputs(sizes, bf16, 360)
+    g = np.zeros(sizes[0], np.float32)
+    for base in (0, 2048, 4096):
+        g[base] = 1.0
+        g[base + 1:base + 40:2] = 1e-9
+        g[base + 2:base + 40:2] = -1e-9
+        g[base + 100:base + 200] = np.linspace(-1e-3, 1e-3, 100, dtype=np.float32)
+    gs = [onp.f32_to_bf16(g) if bf16 else g]
+    for mode, zero_code in ((0, 127), (2, 126)):
+        p_m = [ps[0].copy()]
+        states = hs.oracle_states(sizes)
+        gt = hs.GpuTensors(p_m, gs, states, bf16)
+        omode = oc.MODE_ERI if mode == 0 else oc.MODE_BNB
+        hs.oracle_step(p_m, gs, states, (LR, B1, B2, EPS, WD, 1), bf16, omode)
+        gpu_steps(gt, [None], 1, mode, flags=2)
+        got_p, got_st = gt.fetch()
+        stats = hs.compare(got_p, got_st, p_m, states, bf16, True, "sign-%d" % mode)
+        assert stats["code_mismatch"] == 0
+        for base in (0, 2048, 4096):
+            assert np.all(got_st[0][0][base + 2:base + 40:2] == zero_code)
+            assert np.all(got_st[0][0][base + 1:base + 40:2] == 127)
 
 
 def test_no_weight_decay_variant():

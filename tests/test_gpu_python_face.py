@@ -74,3 +74,34 @@ def test_functional_flavour_over_torch_tensors():
     m_np, m2_np = m.cpu().numpy(), m2.cpu().numpy()
     step = np.diff(hs.MAPS[0]).max() / 2 * np.repeat(states[0][2], 2048)[:n]
     assert np.all(np.abs(m2_np - m_np) <= step * 1.0001)
+
+
+def test_mode_bnb_with_clipping_and_statistics_through_the_python_face():
+    """set_mode(MODE_BNB), clipping inside step() and the error statistics, against the oracle."""
+    from eridiffusion_amd import _lib as L
+    from eridiffusion_amd.adam8bit import Adam8bit, Adam8bitConfig
+    sizes = [2048 * 3 + 17, 640]
+    ps, _ = hs.make_inputs(sizes, True, 15, p_std=1e-2)
+    states = hs.oracle_states(sizes)
+    params = [_bf16_tensor(p) for p in ps]
+    opt = Adam8bit(params, Adam8bitConfig(lr=1e-3))
+    opt.set_mode(L.MODE_BNB)
+    opt.set_max_grad_norm(0.05)
+    opt.track_quantization_error(True)
+    with pytest.raises(L.EriError):
+        opt.set_mode(L.MODE_L2)
+    for t in (1, 2):
+        gs = hs.fresh_grads(sizes, True, 200 + t, 1e-3)
+        for p, g in zip(params, gs):
+            p.grad = _bf16_tensor(g)
+        assert opt.step() == 0
+        norm, scale = opt.last_grad_norm()
+        assert norm > 0.05 and scale == np.float32(0.05) / np.float32(norm)
+        assert opt.last_nonfinite_grads() == 0
+        hs.oracle_step(ps, gs, states, (1e-3, 0.9, 0.999, 1e-8, 0.01, t), True, mode=oc.MODE_BNB,
+                       grad_scale=float(np.float32(1.0) * np.float32(scale)))
+    torch.cuda.synchronize()
+    for p, want in zip(params, ps):
+        assert np.array_equal(_bits(p), want)
+    m_err, v_err = opt.quantization_stats()
+    assert 0 < m_err < 1e-4 and 0 < v_err < 1e-6

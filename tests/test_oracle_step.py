@@ -179,9 +179,9 @@ def _agree(n, bf16, mode, steps, seed, p_std, g_std, wd=WD, threads=1):
     for t in range(1, steps + 1):
         g32 = (rng.standard_normal(n) * g_std).astype(np.float32)
         g = onp.f32_to_bf16(g32) if bf16 else g32
-        step = t if mode == oc.MODE_ERI else t - 1
+        step = t - 1 if mode == oc.MODE_L2 else t
         run_c(p_c, g, st_c, step, oc.DT_BF16 if bf16 else oc.DT_F32, mode, wd=wd, threads=threads)
-        hn = onp.hyper_pack(LR, B1, B2, EPS, wd, step, "eri" if mode == oc.MODE_ERI else "l2")
+        hn = onp.hyper_pack(LR, B1, B2, EPS, wd, step, {oc.MODE_ERI: "eri", oc.MODE_L2: "l2", oc.MODE_BNB: "bnb"}[mode])
         p_n, *st_n = onp.step_tensor(p_n, g, *st_n, hn, *MAPS, bf16=bf16)
         assert np.array_equal(p_c.view(np.uint16 if bf16 else np.uint32), p_n.view(np.uint16 if bf16 else np.uint32)), t
         for a, b in zip(st_c, st_n):
@@ -195,7 +195,7 @@ def test_two_restatements_agree_config1_fp32_eleven_steps():
     assert st[2].min() > 0 and len(np.unique(st[0])) > 100 and len(np.unique(st[1])) > 100
 
 
-@pytest.mark.parametrize("mode", [oc.MODE_ERI, oc.MODE_L2])
+@pytest.mark.parametrize("mode", [oc.MODE_ERI, oc.MODE_L2, oc.MODE_BNB])
 @pytest.mark.parametrize("bf16", [False, True])
 def test_two_restatements_agree_ragged(mode, bf16):
     _agree(7 * 2048 + 1234, bf16, mode, 6, 17 + mode + 2 * bf16, 0.02, 1e-3)
@@ -250,3 +250,79 @@ def test_l2_mode_first_call_follows_the_functional_update():
     g2 = g.astype(np.float64) + WD * p0.astype(np.float64)
     want = p0 - LR * g2 / (np.abs(g2) + EPS)
     assert np.allclose(p, want, rtol=0, atol=6e-7)  # two fp32 roundings near |p| ~ 3
+
+
+# ---- mode BNB: eps under the bias correction, decay as a factor, sign of the first moment kept ----
+
+def test_bnb_scalars():
+    t = 7
+    h = oc.hyper_pack(LR, B1, B2, EPS, WD, t, oc.MODE_BNB)
+    e = oc.hyper_pack(LR, B1, B2, EPS, WD, t, oc.MODE_ERI)
+    assert h.step_size == e.step_size and h.omb1 == e.omb1 and h.omb2 == e.omb2
+    assert h.eps == np.float32(EPS * math.sqrt(1 - B2 ** t))
+    assert h.weight_decay == np.float32(1.0 - LR * WD) and h.weight_decay < 1
+    assert oc.hyper_pack(LR, B1, B2, EPS, 0.0, t, oc.MODE_BNB).weight_decay == 1.0
+
+
+def test_bnb_is_torch_adam_without_decay():
+    # with eps riding on sqrt(bc2) the update is lr/bc1 * m / (sqrt(v/bc2) + eps): Adam itself.  Same
+    # exactly-quantisable gradients as the ERI test above, and no eps adjustment this time.
+    n = 3 * 2048
+    rng = np.random.default_rng(2)
+    p0 = rng.standard_normal(n).astype(np.float32)
+    p = p0.copy()
+    st = oc.state_init(n)
+    tp = torch.tensor(p0.astype(np.float64), requires_grad=True)
+    opt = torch.optim.Adam([tp], lr=1e-2, betas=(B1, B2), eps=1e-8)
+    for t in range(1, 61):
+        per_block = 10.0 ** rng.uniform(-4, -2, 3)
+        g = np.repeat(per_block, 2048).astype(np.float32)
+        run_c(p, g, st, t, mode=oc.MODE_BNB, lr=1e-2, wd=0.0, eps=1e-8)
+        tp.grad = torch.tensor(g.astype(np.float64))
+        opt.step()
+    assert np.abs(tp.detach().numpy() - p0).min() > 0.3
+    assert np.allclose(p, tp.detach().numpy(), rtol=0, atol=8e-6)  # fp32-rounded betas, as in the ERI test
+
+
+def test_bnb_decay_is_a_factor_applied_after_the_adam_term():
+    n = 2048
+    rng = np.random.default_rng(61)
+    p0 = rng.standard_normal(n).astype(np.float32)
+    # zero gradient, zero state: the Adam term is 0 / (0 + eps) = 0 and only the factor remains
+    p = p0.copy()
+    run_c(p, np.zeros(n, np.float32), oc.state_init(n), 1, mode=oc.MODE_BNB, lr=1e-2, wd=0.5)
+    assert np.array_equal(p, p0 * np.float32(1.0 - 1e-2 * 0.5))
+    # with a gradient: (p - adam) * factor, where "p - adam" is what wd = 0 gives
+    g = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    pa, pb = p0.copy(), p0.copy()
+    run_c(pa, g, oc.state_init(n), 3, mode=oc.MODE_BNB, lr=1e-2, wd=0.0)
+    run_c(pb, g, oc.state_init(n), 3, mode=oc.MODE_BNB, lr=1e-2, wd=0.5)
+    assert np.array_equal(pb, pa * np.float32(1.0 - 1e-2 * 0.5))
+    assert not np.array_equal(pa, pb)
+
+
+def test_bnb_first_moment_keeps_its_sign():
+    # one element sets the block's scale; moments 1e-9 of it round to the zero entry (the smallest
+    # non-zero map value is 5.5e-7).  ERI stores 127 for both signs; BNB stores 126 for the negative one.
+    n = 2048
+    g = np.zeros(n, np.float32)
+    g[0] = 1.0
+    g[1], g[2] = 1e-9, -1e-9
+    g[3], g[4] = 1e-3, -1e-3
+    codes = {}
+    for mode in (oc.MODE_ERI, oc.MODE_BNB):
+        st = oc.state_init(n)
+        run_c(np.zeros(n, np.float32), g, st, 1, mode=mode, wd=0.0)
+        codes[mode] = st[0].copy()
+        assert st[0][0] == 255 and st[1][0] == 255
+    assert codes[oc.MODE_ERI][1] == 127 and codes[oc.MODE_ERI][2] == 127
+    assert codes[oc.MODE_BNB][1] == 127 and codes[oc.MODE_BNB][2] == 126
+    # everything else is untouched by the rule, zeros included
+    rest = np.ones(n, bool)
+    rest[2] = False
+    assert np.array_equal(codes[oc.MODE_ERI][rest], codes[oc.MODE_BNB][rest])
+    assert MAPS[0][126] < 0 and MAPS[0][127] == 0 and MAPS[0][codes[oc.MODE_BNB][4]] < 0 < MAPS[0][codes[oc.MODE_BNB][3]]
+    # a block of zeros keeps the codes of zero
+    st = oc.state_init(n)
+    run_c(np.ones(n, np.float32), np.zeros(n, np.float32), st, 1, mode=oc.MODE_BNB)
+    assert np.all(st[0] == 127) and np.all(st[1] == 0) and st[2][0] == 0
