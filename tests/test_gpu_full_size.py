@@ -125,3 +125,81 @@ def test_flux12b_full_size_sampled_blocks_and_block_properties():
         assert bool((m_buf[m_off[i] + n:m_off[i] + n + GUARD] == 0xEE).all())
         assert bool((v_buf[v_off[i] + n:v_off[i] + n + GUARD] == 0xEE).all())
     L.lib().eri_adam8_table_destroy(table)
+
+
+def test_one_tensor_past_two_to_the_32_elements():
+    """64-bit element offsets: a single bf16 tensor of 2**32 + 3*2048 + 5 elements (26 GB with its
+    gradient and states).  Blocks on both sides of element 2**32, the first, the last full and the
+    partial last block are checked against the oracle; every block must satisfy the code-255 property."""
+    import torch
+    from eridiffusion_amd import _lib as L
+
+    free, _ = torch.cuda.mem_get_info()
+    if free < 40e9:
+        pytest.skip("needs ~30 GB of free device memory")
+    n = (1 << 32) + 3 * BLOCK + 5
+    nb = (n + BLOCK - 1) // BLOCK
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(99)
+    p = torch.empty(n, dtype=torch.bfloat16, device=dev)
+    g = torch.empty(n, dtype=torch.bfloat16, device=dev)
+    step = 1 << 28
+    for lo in range(0, n, step):  # fill in pieces: randn over 2**32 elements at once would need 17 GB of fp32
+        hi = min(n, lo + step)
+        p[lo:hi] = torch.randn(hi - lo, device=dev, generator=gen).mul_(0.02)
+        g[lo:hi] = torch.randn(hi - lo, device=dev, generator=gen).mul_(1e-3)
+    GUARD = 256
+    m = torch.full((n + GUARD,), 0xEE, dtype=torch.uint8, device=dev)
+    v = torch.full((n + GUARD,), 0xEE, dtype=torch.uint8, device=dev)
+    am = torch.empty(nb, dtype=torch.float32, device=dev)
+    av = torch.empty(nb, dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    L.check(L.lib().eri_adam8_state_init(m.data_ptr(), v.data_ptr(), am.data_ptr(), av.data_ptr(), n, stream), "state_init")
+    row = (L.TensorRow * 1)()
+    r = row[0]
+    r.p, r.g, r.m, r.v, r.absmax_m, r.absmax_v = p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), am.data_ptr(), av.data_ptr()
+    r.numel, r.block_start, r.dtype_tag, r.grad_scale = n, 0, L.DTYPE_BF16, 1.0
+    table = C.c_void_p()
+    L.check(L.lib().eri_adam8_table_create(row, 1, stream, C.byref(table)), "table_create")
+    edge = (1 << 32) // BLOCK
+    sample = [0, 1, edge - 2, edge - 1, edge, edge + 1, edge + 2, nb - 2, nb - 1, 12345, edge // 2, edge + 1 - 7]
+
+    def grab():
+        out = []
+        for b in sample:
+            lo = b * BLOCK
+            k = min(BLOCK, n - lo)
+            out.append((p[lo:lo + k].view(torch.int16).cpu().numpy().view(np.uint16).copy(),
+                        g[lo:lo + k].view(torch.int16).cpu().numpy().view(np.uint16).copy(),
+                        m[lo:lo + k].cpu().numpy().copy(), v[lo:lo + k].cpu().numpy().copy(),
+                        am[b:b + 1].cpu().numpy().copy(), av[b:b + 1].cpu().numpy().copy()))
+        return out
+
+    hyper = (1e-4, 0.9, 0.999, 1e-8, 0.01)
+    for t in (1, 2):
+        before = grab()
+        h = L.hyper_pack(*hyper, t, L.MODE_ERI, L.FLAG_EXACT_PARAM)
+        L.check(L.lib().eri_adam8_step_table(table, C.byref(h), stream), "step_table")
+        torch.cuda.synchronize()
+        after = grab()
+        ho = oc.hyper_pack(*hyper, t)
+        for b, (pp, gg, mm, vv, a1, a2), got in zip(sample, before, after):
+            assert oc.step_tensor(pp, gg, mm, vv, a1, a2, ho, hs.MAPS, oc.DT_BF16, 1) == 0
+            assert np.array_equal(got[0], pp), b
+            assert np.array_equal(got[2], mm) and np.array_equal(got[3], vv), b
+            assert np.array_equal(got[4].view(np.uint32), a1.view(np.uint32)), b
+            assert np.array_equal(got[5].view(np.uint32), a2.view(np.uint32)), b
+    nf = n // BLOCK
+    assert bool((v[:nf * BLOCK].view(nf, BLOCK).max(dim=1).values == 255).all())
+    assert bool(torch.isfinite(am).all()) and bool((am > 0).all()) and bool((av > 0).all())
+    assert bool((m[n:] == 0xEE).all()) and bool((v[n:] == 0xEE).all())
+    # the gradient norm pass walks the same offsets
+    L.check(L.lib().eri_adam8_grad_norm(table, 1.0, 0.0, stream), "grad_norm")
+    norm, scale = C.c_float(), C.c_float()
+    L.check(L.lib().eri_adam8_grad_norm_read(table, C.byref(norm), C.byref(scale), stream), "norm_read")
+    want = 0.0
+    for lo in range(0, n, step):
+        want += float(g[lo:min(n, lo + step)].float().double().pow(2).sum())
+    assert abs(norm.value - want ** 0.5) <= 2e-6 * want ** 0.5
+    L.lib().eri_adam8_table_destroy(table)
