@@ -35,8 +35,8 @@ class Adam8bitConfigC(C.Structure):
 
 
 class AdamW32Row(C.Structure):
-    _fields_ = [("p", C.c_void_p), ("g", C.c_void_p), ("m", C.c_void_p), ("v", C.c_void_p), ("numel", C.c_uint64),
-                ("dtype_tag", C.c_int32), ("reserved", C.c_int32)]
+    _fields_ = [("p", C.c_void_p), ("g", C.c_void_p), ("m", C.c_void_p), ("v", C.c_void_p), ("master", C.c_void_p),
+                ("numel", C.c_uint64), ("dtype_tag", C.c_int32), ("reserved", C.c_int32)]
 
 
 class AdamW32Hyper(C.Structure):

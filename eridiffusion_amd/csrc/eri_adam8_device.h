@@ -89,17 +89,18 @@ int launch_dequantize(const uint8_t *codes, const float *absmax, int signed_map,
 int launch_quantize(const float *x, int signed_map, uint64_t numel, uint8_t *codes, float *absmax,
                     const void *lds_image, void *stream);
 
-/* Row of the plain element-wise sweeps (32-bit AdamW, EMA): up to four streams of one tensor. */
+/* Row of the plain element-wise sweeps (32-bit AdamW, EMA): up to five streams of one tensor. */
 struct ElemRow {
     void *a;        /* AdamW: p      EMA: shadow */
     const void *b;  /* AdamW: g      EMA: p */
     void *c;        /* AdamW: m (fp32) */
     void *d;        /* AdamW: v (fp32) */
+    void *e;        /* AdamW: fp32 master copy of p, or null */
     uint64_t numel;
     uint32_t full_start; /* full 2048-element blocks in the rows before this one */
     uint32_t pad;
 };
-static_assert(sizeof(ElemRow) == 48, "ElemRow must stay 48 bytes");
+static_assert(sizeof(ElemRow) == 56, "ElemRow must stay 56 bytes");
 
 int launch_adamw32(const ElemRow *rows, uint32_t n_rows, uint32_t total_full_blocks, int dtype_tag,
                    const EriAdamW32Hyper &h, uint32_t grid, void *stream);

@@ -1222,6 +1222,46 @@ __device__ __forceinline__ void store1(void *base, size_t i, float x) {
     else as_global(static_cast<float *>(base))[i] = x;
 }
 
+/* One full block of the 32-bit step.  MASTER: the parameter value comes from, and goes back to, an fp32
+ * master copy; the tensor itself only receives the rounded result (mixed precision,
+ * src/kernels/fused_adam.cu:151-193, with the arithmetic of adamw.rs). */
+template <bool BF16, bool MASTER>
+__device__ __forceinline__ void adamw32_block(const ElemRow &t, size_t e0, uint32_t lane, const EriAdamW32Hyper &h,
+                                              float omb1, float omb2, float neg_lr) {
+    char *p = static_cast<char *>(t.a) + e0 * (BF16 ? 2 : 4);
+    const char *g = static_cast<const char *>(t.b) + e0 * (BF16 ? 2 : 4);
+    float *m = static_cast<float *>(t.c) + e0;
+    float *v = static_cast<float *>(t.d) + e0;
+    float *w = MASTER ? static_cast<float *>(t.e) + e0 : nullptr;
+    Raw8<BF16> pr[4], gr[4];
+    Raw8<false> mr[4], vr[4], wr[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const uint32_t o = c * 512 + lane * 8;
+        if (MASTER) wr[c].load(w, o);
+        else pr[c].load(p, o);
+        gr[c].load(g, o);
+        mr[c].load(m, o);
+        vr[c].load(v, o);
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const uint32_t o = c * 512 + lane * 8;
+        float pv[8], gv[8], mv[8], vv[8], pn[8];
+        if (MASTER) wr[c].unpack(pv);
+        else pr[c].unpack(pv);
+        gr[c].unpack(gv);
+        mr[c].unpack(mv);
+        vr[c].unpack(vv);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) adamw32_elem(pv[k], gv[k], mv[k], vv[k], h, omb1, omb2, neg_lr, pn[k]);
+        store8<BF16>(p, o, pn);
+        if (MASTER) store8<false>(w, o, pn);
+        store8<false>(m, o, mv);
+        store8<false>(v, o, vv);
+    }
+}
+
 template <bool BF16>
 __global__ __launch_bounds__(256) void adamw32_kernel(const ElemRow *__restrict__ rows, uint32_t n_rows,
                                                       uint32_t total_blocks, EriAdamW32Hyper h, uint32_t chunks) {
@@ -1236,11 +1276,14 @@ __global__ __launch_bounds__(256) void adamw32_kernel(const ElemRow *__restrict_
         const size_t e0 = (size_t)(t.numel / kBlock) * kBlock;
         ERI_GLOBAL float *mp = as_global(static_cast<float *>(t.c));
         ERI_GLOBAL float *vp = as_global(static_cast<float *>(t.d));
+        ERI_GLOBAL float *wp = as_global(static_cast<float *>(t.e)); // fp32 master copy, or null
         for (uint32_t i = lane; i < n; i += kWave) {
             float m = mp[e0 + i], v = vp[e0 + i], pn;
-            adamw32_elem(load1<BF16>(t.a, e0 + i), load1<BF16>(t.b, e0 + i), m, v, h, omb1, omb2, neg_lr, pn);
+            const float pf = wp ? wp[e0 + i] : load1<BF16>(t.a, e0 + i);
+            adamw32_elem(pf, load1<BF16>(t.b, e0 + i), m, v, h, omb1, omb2, neg_lr, pn);
             mp[e0 + i] = m;
             vp[e0 + i] = v;
+            if (wp) wp[e0 + i] = pn;
             store1<BF16>(t.a, e0 + i, pn);
         }
     }
@@ -1250,34 +1293,8 @@ __global__ __launch_bounds__(256) void adamw32_kernel(const ElemRow *__restrict_
         ti = find_elem_row(rows, n_rows, ti, blk);
         const ElemRow t = rows[ti];
         const size_t e0 = (size_t)(blk - t.full_start) * kBlock;
-        char *p = static_cast<char *>(t.a) + e0 * (BF16 ? 2 : 4);
-        const char *g = static_cast<const char *>(t.b) + e0 * (BF16 ? 2 : 4);
-        float *m = static_cast<float *>(t.c) + e0;
-        float *v = static_cast<float *>(t.d) + e0;
-        Raw8<BF16> pr[4], gr[4];
-        Raw8<false> mr[4], vr[4];
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const uint32_t o = c * 512 + lane * 8;
-            pr[c].load(p, o);
-            gr[c].load(g, o);
-            mr[c].load(m, o);
-            vr[c].load(v, o);
-        }
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const uint32_t o = c * 512 + lane * 8;
-            float pv[8], gv[8], mv[8], vv[8], pn[8];
-            pr[c].unpack(pv);
-            gr[c].unpack(gv);
-            mr[c].unpack(mv);
-            vr[c].unpack(vv);
-#pragma unroll
-            for (int k = 0; k < 8; ++k) adamw32_elem(pv[k], gv[k], mv[k], vv[k], h, omb1, omb2, neg_lr, pn[k]);
-            store8<BF16>(p, o, pn);
-            store8<false>(m, o, mv);
-            store8<false>(v, o, vv);
-        }
+        if (t.e) adamw32_block<BF16, true>(t, e0, lane, h, omb1, omb2, neg_lr);
+        else adamw32_block<BF16, false>(t, e0, lane, h, omb1, omb2, neg_lr);
     }
 }
 

@@ -952,7 +952,8 @@ int eri_adamw32_step_multi(const EriAdamW32Tensor *rows, uint32_t n, const EriAd
         if (((uintptr_t)r.m | (uintptr_t)r.v) & 15u) return fail(ERI_ERR_ALIGN, "moment pointers must be 16-byte aligned");
         const int gi = r.dtype_tag == ERI_DTYPE_F32 ? 0 : 1;
         eri::ElemRow d;
-        d.a = r.p; d.b = r.g; d.c = r.m; d.d = r.v; d.numel = r.numel; d.full_start = starts[gi]; d.pad = 0;
+        if ((uintptr_t)r.master & 15u) return fail(ERI_ERR_ALIGN, "master pointer must be 16-byte aligned");
+        d.a = r.p; d.b = r.g; d.c = r.m; d.d = r.v; d.e = r.master; d.numel = r.numel; d.full_start = starts[gi]; d.pad = 0;
         starts[gi] += (uint32_t)(r.numel / eri::kBlock);
         cache.groups[gi].rows.push_back(d);
     }
@@ -975,7 +976,7 @@ int eri_ema_update_multi(const EriEmaTensor *rows, uint32_t n, float decay, void
         if (e) return e;
         const int gi = r.dtype_tag == ERI_DTYPE_F32 ? 0 : 1;
         eri::ElemRow d;
-        d.a = r.shadow; d.b = r.p; d.c = nullptr; d.d = nullptr; d.numel = r.numel; d.full_start = starts[gi]; d.pad = 0;
+        d.a = r.shadow; d.b = r.p; d.c = nullptr; d.d = nullptr; d.e = nullptr; d.numel = r.numel; d.full_start = starts[gi]; d.pad = 0;
         starts[gi] += (uint32_t)(r.numel / eri::kBlock);
         cache.groups[gi].rows.push_back(d);
     }

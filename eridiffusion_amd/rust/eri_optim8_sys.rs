@@ -42,7 +42,7 @@ pub struct EriAdam8bitConfig {
 
 #[repr(C)]
 #[derive(Clone, Copy)]
-pub struct EriAdamW32Tensor { pub p: *mut c_void, pub g: *const c_void, pub m: *mut f32, pub v: *mut f32, pub numel: u64, pub dtype_tag: i32, pub reserved: i32 }
+pub struct EriAdamW32Tensor { pub p: *mut c_void, pub g: *const c_void, pub m: *mut f32, pub v: *mut f32, pub master: *mut f32, pub numel: u64, pub dtype_tag: i32, pub reserved: i32 }
 #[repr(C)]
 #[derive(Clone, Copy)]
 pub struct EriAdamW32Hyper { pub lr: f32, pub beta1: f32, pub beta2: f32, pub eps: f32, pub weight_decay: f32 }

@@ -221,6 +221,9 @@ typedef struct EriAdamW32Tensor {
     const void *g;    /* same dtype as p */
     float *m;         /* fp32 first moment, numel elements */
     float *v;         /* fp32 second moment */
+    float *master;    /* NULL, or an fp32 master copy of p (numel elements): the step then reads and writes
+                         the master and stores its rounded value in p -- mixed precision as in
+                         src/kernels/fused_adam.cu:151-193, with the arithmetic above */
     uint64_t numel;
     int32_t dtype_tag;
     int32_t reserved;

@@ -305,11 +305,14 @@ void eri_oracle_quantize(const float *x, const float *map, uint64_t numel, uint8
  * correction, decoupled decay, parameter cast back to its dtype.  Pinned by closed forms at the
  * first step, a float64 recurrence and the reference's own test case (2x2 bf16 ones, grad ones,
  * src/tests/adamw_step.rs:6-30). */
+/* master != NULL: mixed precision (src/kernels/fused_adam.cu:151-193): the fp32 master copy is the value
+ * that is read and updated, and p receives its rounded value.  Pinned by: the master after any number
+ * of steps equals what the fp32 path gives on the same gradients, and p equals the rounded master. */
 void eri_oracle_adamw32_step(void *p, const void *g, float *m, float *v, uint64_t numel, int dtype, float lr,
-                             float beta1, float beta2, float eps, float wd) {
+                             float beta1, float beta2, float eps, float wd, float *master) {
     const float omb1 = 1.0f - beta1, omb2 = 1.0f - beta2, neg_lr = -lr;
     for (uint64_t i = 0; i < numel; ++i) {
-        float pf = load_elem(p, i, dtype), gr = load_elem(g, i, dtype);
+        float pf = master ? master[i] : load_elem(p, i, dtype), gr = load_elem(g, i, dtype);
         float ms = m[i] * beta1;       /* :35 */
         float gs = gr * omb1;          /* :36 */
         float mn = ms + gs;            /* :37 */
@@ -325,6 +328,7 @@ void eri_oracle_adamw32_step(void *p, const void *g, float *m, float *v, uint64_
         float pn = pf + step;
         m[i] = mn;
         v[i] = vn;
+        if (master) master[i] = pn;
         if (dtype == ERI_ORACLE_F32) ((float *)p)[i] = pn;
         else ((uint16_t *)p)[i] = eri_oracle_f32_to_bf16(pn); /* :55 */
     }

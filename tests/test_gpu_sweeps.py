@@ -48,13 +48,49 @@ def test_adamw32_multi_tensor(bf16, wd):
             rows[i].p, rows[i].g, rows[i].m, rows[i].v = dp[i].data_ptr(), dg[i].data_ptr(), dm[i].data_ptr(), dv[i].data_ptr()
             rows[i].numel, rows[i].dtype_tag = n, tag
             oc.lib().eri_oracle_adamw32_step(oc.ptr(ps[i]), oc.ptr(gs[i]), oc.ptr(ms[i]), oc.ptr(vs[i]), n, tag,
-                                             1e-3, 0.9, 0.999, 1e-8, wd)
+                                             1e-3, 0.9, 0.999, 1e-8, wd, None)
         L.check(L.lib().eri_adamw32_step_multi(rows, len(SIZES), C.byref(h), torch.cuda.current_stream().cuda_stream), "adamw32")
         torch.cuda.synchronize()
     for i in range(len(SIZES)):
         assert np.array_equal(_down(dp[i], dt).view(np.uint16 if bf16 else np.uint32), ps[i].view(np.uint16 if bf16 else np.uint32))
         assert np.array_equal(_down(dm[i], np.uint32), ms[i].view(np.uint32))
         assert np.array_equal(_down(dv[i], np.uint32), vs[i].view(np.uint32))
+
+
+def test_adamw32_with_fp32_master_copies():
+    """Rows with and without a master copy in one launch; bf16 parameters, bit-exact against the oracle."""
+    import torch
+    from eridiffusion_amd import _lib as L
+    rng = np.random.default_rng(21)
+    ps, ws, ms, vs = [], [], [], []
+    for i, n in enumerate(SIZES):
+        p = (rng.standard_normal(n) * 0.02).astype(np.float32)
+        ps.append(onp.f32_to_bf16(p))
+        ws.append(p.copy() if i % 2 == 0 else None)  # every other tensor keeps a master
+        ms.append(np.zeros(n, np.float32))
+        vs.append(np.zeros(n, np.float32))
+    dp, dm, dv = [_up(a) for a in ps], [_up(a) for a in ms], [_up(a) for a in vs]
+    dw = [_up(a) if a is not None else None for a in ws]
+    rows = (L.AdamW32Row * len(SIZES))()
+    h = L.AdamW32Hyper(1e-3, 0.9, 0.999, 1e-8, 0.01)
+    for step in range(3):
+        gs = [onp.f32_to_bf16((rng.standard_normal(n) * 1e-3).astype(np.float32)) for n in SIZES]
+        dg = [_up(a) for a in gs]
+        for i, n in enumerate(SIZES):
+            rows[i].p, rows[i].g, rows[i].m, rows[i].v = dp[i].data_ptr(), dg[i].data_ptr(), dm[i].data_ptr(), dv[i].data_ptr()
+            rows[i].master = dw[i].data_ptr() if dw[i] is not None else None
+            rows[i].numel, rows[i].dtype_tag = n, 2
+            oc.lib().eri_oracle_adamw32_step(oc.ptr(ps[i]), oc.ptr(gs[i]), oc.ptr(ms[i]), oc.ptr(vs[i]), n, 2,
+                                             1e-3, 0.9, 0.999, 1e-8, 0.01, oc.ptr(ws[i]) if ws[i] is not None else None)
+        L.check(L.lib().eri_adamw32_step_multi(rows, len(SIZES), C.byref(h), torch.cuda.current_stream().cuda_stream), "adamw32")
+        torch.cuda.synchronize()
+    for i in range(len(SIZES)):
+        assert np.array_equal(_down(dp[i], np.uint16), ps[i])
+        assert np.array_equal(_down(dm[i], np.uint32), ms[i].view(np.uint32))
+        assert np.array_equal(_down(dv[i], np.uint32), vs[i].view(np.uint32))
+        if ws[i] is not None:
+            assert np.array_equal(_down(dw[i], np.uint32), ws[i].view(np.uint32))
+            assert np.array_equal(ps[i], onp.f32_to_bf16(ws[i]))
 
 
 @pytest.mark.parametrize("bf16", [True, False])

@@ -6,8 +6,9 @@ import oracle_c as oc
 from oracle import adam8_numpy as onp
 
 
-def adamw(p, g, m, v, dtype, lr=1e-3, b1=0.9, b2=0.999, eps=1e-8, wd=0.01):
-    oc.lib().eri_oracle_adamw32_step(oc.ptr(p), oc.ptr(g), oc.ptr(m), oc.ptr(v), m.size, dtype, lr, b1, b2, eps, wd)
+def adamw(p, g, m, v, dtype, lr=1e-3, b1=0.9, b2=0.999, eps=1e-8, wd=0.01, master=None):
+    oc.lib().eri_oracle_adamw32_step(oc.ptr(p), oc.ptr(g), oc.ptr(m), oc.ptr(v), m.size, dtype, lr, b1, b2, eps, wd,
+                                     oc.ptr(master) if master is not None else None)
 
 
 def test_reference_test_case_two_by_two_bf16_ones():
@@ -54,6 +55,30 @@ def test_adamw32_zero_decay_leaves_no_decay_term():
     p = p0.copy()
     adamw(p, g, np.zeros(64, np.float32), np.zeros(64, np.float32), oc.DT_F32, wd=0.5, lr=0.1)
     assert np.allclose(p, p0 * (1 - 0.05), rtol=1e-6)
+
+
+def test_adamw32_master_copy_is_the_fp32_run_and_the_parameter_its_rounding():
+    # mixed precision: bf16 parameter and gradient, fp32 master.  The master must follow, bit for bit, an
+    # fp32 run fed the same (bf16-valued) gradients, and the bf16 parameter is the rounded master each step;
+    # without the master the bf16 parameter drifts away from that run (updates below half an ulp are lost).
+    rng = np.random.default_rng(5)
+    n = 3000
+    p32 = rng.standard_normal(n).astype(np.float32)
+    master = p32.copy()
+    p_mixed = onp.f32_to_bf16(p32)
+    p_plain = p_mixed.copy()
+    st = [[np.zeros(n, np.float32), np.zeros(n, np.float32)] for _ in range(3)]
+    for t in range(40):
+        g16 = onp.f32_to_bf16((rng.standard_normal(n) * 1e-2).astype(np.float32))
+        adamw(p32, onp.bf16_to_f32(g16), *st[0], oc.DT_F32, lr=1e-4)
+        adamw(p_mixed, g16, *st[1], oc.DT_BF16, lr=1e-4, master=master)
+        adamw(p_plain, g16, *st[2], oc.DT_BF16, lr=1e-4)
+        assert np.array_equal(master.view(np.uint32), p32.view(np.uint32))
+        assert np.array_equal(p_mixed, onp.f32_to_bf16(master))
+    assert np.array_equal(st[0][0], st[1][0]) and np.array_equal(st[0][1], st[1][1])
+    drift_plain = np.abs(onp.bf16_to_f32(p_plain) - p32).mean()
+    drift_mixed = np.abs(onp.bf16_to_f32(p_mixed) - p32).mean()
+    assert drift_plain > 1.5 * drift_mixed
 
 
 def test_ema_is_a_convex_combination():
