@@ -38,7 +38,7 @@ def test_rust_binding_source_declares_every_symbol():
 def test_struct_layouts_match_the_header():
     assert C.sizeof(L.Hyper) == 48
     assert C.sizeof(L.TensorRow) == 72
-    assert C.sizeof(L.AdamW32Row) == 56 and C.sizeof(L.EmaRow) == 24
+    assert C.sizeof(L.AdamW32Row) == 56 and C.sizeof(L.EmaRow) == 32
     assert L.TensorRow.numel.offset == 48 and L.TensorRow.dtype_tag.offset == 64
 
 
