@@ -247,3 +247,30 @@ def test_state_init_and_quantize_round_trip():
         assert np.array_equal(codes.cpu().numpy(), wc)
         assert np.array_equal(absmax.cpu().numpy().view(np.uint32), wa.view(np.uint32))
         assert np.array_equal(back.cpu().numpy().view(np.uint32), wb.view(np.uint32))
+
+
+def test_randomized_cases_against_the_oracle():
+    """Forty seeded random combinations of tensor lists (ragged, tiny, multi-block), dtype, mode, flags,
+    decay, gradient scale and prior history; every one must match the oracle to the bar above."""
+    rng = np.random.default_rng(20240607)
+    pool = [1, 3, 8, 63, 64, 65, 320, 511, 512, 1000, 2047, 2048, 2049, 4095, 4096, 5120, 10240, 12289, 20480, 65536 + 17]
+    flips = 0
+    for case in range(40):
+        k = int(rng.integers(1, 9))
+        sizes = [int(rng.choice(pool)) for _ in range(k)]
+        if rng.random() < 0.3:
+            sizes.append(int(rng.integers(1, 40000)))
+        bf16 = bool(rng.integers(0, 2))
+        mode = int(rng.choice([0, 0, 1, 2]))
+        flags = int(rng.choice([0, 2, 4, 8, 2 | 4, 2 | 8])) if mode != 2 else 0
+        if mode == 1:
+            flags |= 2  # the functional update is compared bit for bit
+        wd = float(rng.choice([0.0, 0.01, 0.1]))
+        gscale = None if rng.random() < 0.6 else float(rng.uniform(0.1, 2.0))
+        g_std = float(10.0 ** rng.uniform(-5, -1))
+        p_std = float(10.0 ** rng.uniform(-4, 0))
+        st = run_case(sizes, bf16, 9000 + case, steps=int(rng.integers(1, 4)), mode=mode, flags=flags, wd=wd,
+                      p_std=p_std, g_std=g_std, prior=int(rng.integers(0, 3)), grad_scale=gscale,
+                      use_multi=bool(rng.random() < 0.25), label="rand%d" % case)
+        flips += st["param_1ulp"]
+    print("randomized cases: bf16 parameters one ulp off on the approximate path: %d" % flips, flush=True)
