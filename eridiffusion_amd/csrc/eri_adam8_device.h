@@ -73,6 +73,7 @@ int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_bloc
                 void *stream);
 extern int g_kernel_variant;
 extern int g_chunks;
+extern int g_pipelined_waves;
 /* Sum of |moment - dequantised moment| of the coming step, per row: err[2r] first moment, err[2r+1] second. */
 int launch_quant_error(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_blocks, int dtype_tag,
                        const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale, double *err,

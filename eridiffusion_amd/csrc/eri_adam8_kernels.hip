@@ -777,6 +777,7 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
     }
 }
 
+int g_pipelined_waves = 0; // measurement switch: waves per workgroup of the pipelined kernel (0 = 12)
 int g_chunks = 8; // contiguous ranges of the block list (BlockWalk); 8 = one per accelerator die
 /* The chunked walk needs the same number of workgroups in every chunk. */
 static uint32_t chunks_for(uint32_t grid) {
@@ -794,6 +795,7 @@ static int launch_pipelined(const DevTensor *rows, uint32_t n_rows, uint32_t tot
         if (g_kernel_variant == 3) k = adam8_step_pipelined_kernel<MODE, EXACT, WD, GS, 3>;
     }
     if (wg > 768) wg = 768;
+    if (g_pipelined_waves >= 1 && g_pipelined_waves <= 12) wg = (uint32_t)g_pipelined_waves * kWave;
     hipLaunchKernelGGL(k, dim3(grid), dim3(wg), 0, s, rows, n_rows, total_blocks, h,
                        static_cast<const uint4 *>(lds_image), dev_scale, chunks_for(grid));
     return (int)hipGetLastError();

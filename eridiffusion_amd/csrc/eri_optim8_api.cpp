@@ -493,6 +493,11 @@ int eri_hip_mem_info(size_t *free_bytes, size_t *total_bytes) {
 static int g_grid_override = 0; // measurement switch: persistent workgroups of the step (0 = one per slot)
 
 int eri_adam8_set_tuning(int key, int value) {
+    if (key == 3) {
+        if (value < 0 || value > 12) return fail(ERI_ERR_ARG, "waves per workgroup out of range");
+        eri::g_pipelined_waves = value;
+        return 0;
+    }
     if (key == 2) {
         if (value < 1 || value > 4096) return fail(ERI_ERR_ARG, "chunk count out of range");
         eri::g_chunks = value;

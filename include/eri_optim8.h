@@ -142,8 +142,10 @@ typedef struct EriAdam8Table EriAdam8Table; /* device-resident copy of a launch 
 /* Loads the quantisation tables onto the current device.  Optional: the first table does it. */
 int eri_adam8_init(void);
 
-/* Measurement switch, not part of the optimizer's behaviour: key 0 selects one of the store
- * schedules of the bf16 step kernel (0 = shipped; all give identical results). */
+/* Measurement switches, not part of the optimizer's behaviour (all settings give identical results):
+ * key 0 = store schedule of the bf16 step kernel (0 = shipped), key 1 = number of persistent workgroups
+ * (0 = one per compute unit), key 2 = contiguous ranges the block list is cut into (8 = shipped, one per
+ * accelerator die; 1 = plain grid stride), key 3 = waves per workgroup of the bf16 step kernel (0 = 12). */
 int eri_adam8_set_tuning(int key, int value);
 
 /* The two 256-entry maps (code -> value in [-1, 1] / [0, 1]) the states are expressed in. */
