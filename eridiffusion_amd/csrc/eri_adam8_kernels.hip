@@ -579,8 +579,10 @@ __global__ __launch_bounds__(1024) void adam8_step_kernel(const DevTensor *__res
     const uint32_t stride = gridDim.x * waves_per_wg;
     const BlockDiv dbc1(h.bc1), dbc2(h.bc2);
 
-    // partial last blocks first: one per row at most, spread over the waves
-    for (uint32_t r = wave; r < n_rows; r += stride) {
+    // partial last blocks first: one per row at most, handed out from the last wave backwards -- the
+    // waves at the end of each range are the ones that get one full block fewer when the blocks do not
+    // divide evenly, so the slower element-wise tail lands where there is slack
+    for (uint32_t r = stride - 1 - wave; r < n_rows; r += stride) {
         const DevTensor t = rows[r];
         const uint32_t n = (uint32_t)(t.numel % kBlock);
         if (n != 0) {
@@ -657,8 +659,10 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
     const BlockDiv dbc1(h.bc1), dbc2(h.bc2);
 
     const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
-    // partial last blocks first: one per row at most, spread over the waves
-    for (uint32_t r = wave; r < n_rows; r += stride) {
+    // partial last blocks first: one per row at most, handed out from the last wave backwards -- the
+    // waves at the end of each range are the ones that get one full block fewer when the blocks do not
+    // divide evenly, so the slower element-wise tail lands where there is slack
+    for (uint32_t r = stride - 1 - wave; r < n_rows; r += stride) {
         const DevTensor t = rows[r];
         const uint32_t n = (uint32_t)(t.numel % kBlock);
         if (n != 0) {
