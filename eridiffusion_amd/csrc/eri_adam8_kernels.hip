@@ -562,7 +562,9 @@ __global__ __launch_bounds__(1024) void adam8_step_kernel(const DevTensor *__res
     ERI_LDS_IMAGE;
     // clip factor left on the device by the gradient-norm pass (1.0 when there is none)
     const float tscale = (GS && dev_scale) ? *dev_scale : 1.0f;
-    for (uint32_t i = threadIdx.x; i < kLdsImageBytes / 16; i += blockDim.x) lds_raw[i] = lds_image[i];
+    // the binary search needs the maps and midpoints only (4 KB); the slot tables are the other 96 KB
+    constexpr uint32_t staged = KEYTAB ? kLdsImageBytes : kOffKeyU;
+    for (uint32_t i = threadIdx.x; i < staged / 16; i += blockDim.x) lds_raw[i] = lds_image[i];
     __syncthreads();
     const char *base = reinterpret_cast<const char *>(lds_raw);
     Lds L;
