@@ -10,7 +10,8 @@
  * p, g, m, v crosses HBM once in each direction.
  *
  * The grid is persistent: workgroups stage the lookup tables into LDS once, then their waves walk
- * the global block list with a grid-sized stride, so consecutive waves touch consecutive blocks.
+ * the global block list -- cut into one contiguous range per accelerator die, see BlockWalk -- with
+ * the stride of their die's waves, so consecutive waves touch consecutive blocks.
  * The tensor that owns a block is found by a scalar binary search over the launch table.
  *
  * Arithmetic: every fp32 operation of the update is written as its own statement and the file is
