@@ -326,3 +326,50 @@ def test_bnb_first_moment_keeps_its_sign():
     st = oc.state_init(n)
     run_c(np.ones(n, np.float32), np.zeros(n, np.float32), st, 1, mode=oc.MODE_BNB)
     assert np.all(st[0] == 127) and np.all(st[1] == 0) and st[2][0] == 0
+
+
+def test_two_restatements_agree_on_randomized_cases_with_extreme_values():
+    """Thirty seeded random cases: sizes, dtype, mode, decay, gradient scale, magnitudes from 1e-30 to
+    1e30, exact zeros, and (in some cases) NaN and infinite gradients.  The scalar C and the vectorised
+    NumPy restatements must produce the same bits; NaN parameters are compared as NaN."""
+    rng = np.random.default_rng(424242)
+    modes = [(oc.MODE_ERI, "eri"), (oc.MODE_L2, "l2"), (oc.MODE_BNB, "bnb")]
+    for case in range(30):
+        n = int(rng.choice([1, 5, 2047, 2048, 2049, 5000, 3 * 2048 + 17]))
+        bf16 = bool(rng.integers(0, 2))
+        cmode, nmode = modes[int(rng.integers(0, 3))]
+        wd = float(rng.choice([0.0, 0.01, 0.3]))
+        gs = None if rng.random() < 0.5 else float(rng.uniform(0.05, 3.0))
+        mag_p = 10.0 ** rng.uniform(-6, 3)
+        mag_g = 10.0 ** rng.uniform(-30, 30) if rng.random() < 0.3 else 10.0 ** rng.uniform(-6, 0)
+        p32 = (rng.standard_normal(n) * mag_p).astype(np.float32)
+        p_c = onp.f32_to_bf16(p32) if bf16 else p32.copy()
+        p_n = p_c.copy()
+        st_c, st_n = oc.state_init(n), onp.state_init(n)
+        for t in range(1, 4):
+            with np.errstate(over="ignore"):
+                g32 = (rng.standard_normal(n) * mag_g).astype(np.float32)
+            g32[rng.random(n) < 0.05] = 0.0
+            if case % 5 == 4 and n > 4:
+                g32[int(rng.integers(0, n))] = np.nan
+                g32[int(rng.integers(0, n))] = np.inf
+                g32[int(rng.integers(0, n))] = -np.inf
+            g = onp.f32_to_bf16(g32) if bf16 else g32
+            step = t - 1 if cmode == oc.MODE_L2 else t
+            run_c(p_c, g, st_c, step, oc.DT_BF16 if bf16 else oc.DT_F32, cmode, wd=wd, gs=gs)
+            hn = onp.hyper_pack(LR, B1, B2, EPS, wd, step, nmode)
+            if gs is not None:
+                hn["grad_scale"] = gs
+            p_n, *st_n = onp.step_tensor(p_n, g, *st_n, hn, *MAPS, bf16=bf16)
+            fc = onp.bf16_to_f32(p_c) if bf16 else p_c
+            fn = onp.bf16_to_f32(p_n) if bf16 else p_n
+            both_nan = np.isnan(fc) & np.isnan(fn)
+            raw_c = p_c.view(np.uint16 if bf16 else np.uint32)
+            raw_n = p_n.view(np.uint16 if bf16 else np.uint32)
+            assert np.array_equal(raw_c[~both_nan], raw_n[~both_nan]), (case, t)
+            for k, (a, b) in enumerate(zip(st_c, st_n)):
+                a, b = np.asarray(a), np.asarray(b)
+                if k >= 2:  # absmax: NaN never enters (fmaxf ignores it), inf may
+                    assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), (case, t, k)
+                else:
+                    assert np.array_equal(a, b), (case, t, k)
