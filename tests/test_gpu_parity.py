@@ -144,6 +144,32 @@ def test_bnb_mode_keeps_the_sign_of_tiny_first_moments(bf16):
             assert np.all(got_st[0][0][base + 1:base + 40:2] == 127)
 
 
+@pytest.mark.parametrize("bf16", [False, True])
+def test_l2_mode_bias_correction_with_tiny_huge_and_infinite_moments(bf16):
+    """The functional update divides the moments by 1 - beta^s.  Gradients from the denormal range up to
+    values whose squares overflow, and infinities, must give the oracle's bits: the kernel's exactly
+    rounded fast division has to hand every out-of-range case to the IEEE division."""
+    n = 2048 * 2 + 700
+    rng = np.random.default_rng(31 + bf16)
+    mags = 10.0 ** rng.uniform(-45, 38, n)
+    with np.errstate(over="ignore"):
+        g = (rng.standard_normal(n) * mags).astype(np.float32)
+    g[::97] = 0.0
+    g[5], g[2048 + 9], g[4096 + 11] = np.inf, -np.inf, np.inf
+    ps, _ = hs.make_inputs([n], bf16, 33)
+    gs = [onp.f32_to_bf16(g) if bf16 else g]
+    g2 = [onp.f32_to_bf16((g * np.float32(0.5)).astype(np.float32)) if bf16 else (g * np.float32(0.5)).astype(np.float32)]
+    states = hs.oracle_states([n])
+    gt = hs.GpuTensors(ps, gs, states, bf16)
+    with np.errstate(all="ignore"):
+        hs.oracle_step(ps, gs, states, (LR, B1, B2, EPS, WD, 0), bf16, oc.MODE_L2)
+        hs.oracle_step(ps, g2, states, (LR, B1, B2, EPS, WD, 1), bf16, oc.MODE_L2)
+    gpu_steps(gt, [None, g2], 1, mode=1, flags=2)
+    got_p, got_st = gt.fetch()
+    stats = hs.compare(got_p, got_st, ps, states, bf16, True, "l2-range")
+    assert stats["code_mismatch"] == 0
+
+
 def test_no_weight_decay_variant():
     run_case([2048 * 9 + 3, 640], True, 400, steps=3, wd=0.0, flags=2, label="wd0")
     run_case([2048 * 9 + 3, 640], False, 401, steps=3, wd=0.0, label="wd0-fp32")
@@ -274,3 +300,47 @@ def test_randomized_cases_against_the_oracle():
                       use_multi=bool(rng.random() < 0.25), label="rand%d" % case)
         flips += st["param_1ulp"]
     print("randomized cases: bf16 parameters one ulp off on the approximate path: %d" % flips, flush=True)
+
+
+def test_randomized_extreme_values_against_the_oracle():
+    """Gradient magnitudes from 1e-30 to 1e30, exact zeros, NaN and infinities, both dtypes, all modes,
+    default (approximate bf16 update) and exact flags: states bit-exact, parameters to the bar, NaN in the
+    same places."""
+    rng = np.random.default_rng(777)
+    for case in range(24):
+        sizes = [int(rng.choice([5, 2047, 2048, 2049, 6 * 2048 + 100])) for _ in range(int(rng.integers(1, 4)))]
+        bf16 = bool(rng.integers(0, 2))
+        mode = int(rng.choice([0, 0, 1, 2]))
+        flags = 2 if mode == 1 else (0 if mode == 2 else int(rng.choice([0, 2, 4, 8])))
+        wd = float(rng.choice([0.0, 0.01]))
+        mag_g = 10.0 ** rng.uniform(-30, 30) if case % 2 else 10.0 ** rng.uniform(-8, 2)
+        ps, _ = hs.make_inputs(sizes, bf16, 3000 + case, p_std=float(10.0 ** rng.uniform(-4, 2)))
+        omode = {0: oc.MODE_ERI, 1: oc.MODE_L2, 2: oc.MODE_BNB}[mode]
+        states = hs.oracle_states(sizes)
+
+        def grads():
+            out = []
+            for n in sizes:
+                with np.errstate(over="ignore"):
+                    g = (rng.standard_normal(n) * mag_g).astype(np.float32)
+                g[rng.random(n) < 0.05] = 0.0
+                if case % 3 == 2 and n > 8:
+                    g[int(rng.integers(0, n))] = np.nan
+                    g[int(rng.integers(0, n))] = np.inf
+                    g[int(rng.integers(0, n))] = -np.inf
+                out.append(onp.f32_to_bf16(g) if bf16 else g)
+            return out
+
+        all_g = [grads() for _ in range(3)]
+        gt = hs.GpuTensors(ps, all_g[0], states, bf16)
+        with np.errstate(all="ignore"):
+            for k, g_k in enumerate(all_g):
+                hs.oracle_step(ps, g_k, states, (LR, B1, B2, EPS, wd, k if mode == 1 else k + 1), bf16, omode)
+        gpu_steps(gt, [None] + all_g[1:], 1, mode, flags, wd)
+        got_p, got_st = gt.fetch()
+        for i in range(len(sizes)):
+            for k in (2, 3):  # absmax may be infinite, never NaN
+                assert np.array_equal(got_st[i][k].view(np.uint32), states[i][k].view(np.uint32)), (case, i, k)
+        exact = (not bf16) or bool(flags & 2) or mode == 2
+        stats = hs.compare(got_p, got_st, ps, states, bf16, exact, "extreme%d" % case)
+        assert stats["code_mismatch"] == 0, case
