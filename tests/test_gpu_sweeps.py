@@ -130,3 +130,99 @@ def test_sweep_argument_errors():
     rows[0].dtype_tag, rows[0].p = 2, 0x2004
     assert L.lib().eri_ema_update_multi(rows, 1, 0.9, None) == -2
     assert L.lib().eri_ema_update_multi(None, 1, 0.9, None) == -1
+
+
+def _same_bits_nan_aware(got, want, bf16):
+    g32 = onp.bf16_to_f32(got) if bf16 else got
+    w32 = onp.bf16_to_f32(want) if bf16 else want
+    both_nan = np.isnan(g32) & np.isnan(w32)
+    raw = np.uint16 if bf16 else np.uint32
+    return np.array_equal(got.view(raw)[~both_nan], want.view(raw)[~both_nan])
+
+
+@pytest.mark.parametrize("bf16", [True, False])
+def test_sweeps_with_extreme_and_non_finite_values(bf16):
+    """Magnitudes from the denormal range to overflow, zeros, NaN and infinities through the 32-bit step
+    (with and without a master copy) and the EMA sweep: same bits as the oracle, NaN in the same places."""
+    import torch
+    from eridiffusion_amd import _lib as L
+    rng = np.random.default_rng(77 + bf16)
+    tag = 2 if bf16 else 0
+    n = 2048 * 2 + 333
+
+    def wild():
+        with np.errstate(over="ignore"):
+            x = (rng.standard_normal(n) * 10.0 ** rng.uniform(-44, 38, n)).astype(np.float32)
+        x[::53] = 0.0
+        x[7], x[2048 + 3], x[4096 + 100] = np.nan, np.inf, -np.inf
+        return x
+
+    for use_master in (False, True):
+        p32, g32 = wild(), wild()
+        p = onp.f32_to_bf16(p32) if bf16 else p32.copy()
+        g = onp.f32_to_bf16(g32) if bf16 else g32.copy()
+        w = (onp.bf16_to_f32(p) if bf16 else p).astype(np.float32).copy() if use_master else None
+        m, v = np.abs(wild()), np.abs(wild())
+        m[7] = 0.0
+        dp, dg, dm, dv = _up(p), _up(g), _up(m), _up(v)
+        dw = _up(w) if use_master else None
+        rows = (L.AdamW32Row * 1)()
+        rows[0].p, rows[0].g, rows[0].m, rows[0].v = dp.data_ptr(), dg.data_ptr(), dm.data_ptr(), dv.data_ptr()
+        rows[0].master = dw.data_ptr() if use_master else None
+        rows[0].numel, rows[0].dtype_tag = n, tag
+        h = L.AdamW32Hyper(1e-3, 0.9, 0.999, 1e-8, 0.01)
+        for _ in range(2):
+            L.check(L.lib().eri_adamw32_step_multi(rows, 1, C.byref(h), torch.cuda.current_stream().cuda_stream), "adamw32")
+            with np.errstate(all="ignore"):
+                oc.lib().eri_oracle_adamw32_step(oc.ptr(p), oc.ptr(g), oc.ptr(m), oc.ptr(v), n, tag, 1e-3, 0.9, 0.999, 1e-8, 0.01,
+                                                 oc.ptr(w) if use_master else None)
+        torch.cuda.synchronize()
+        assert _same_bits_nan_aware(_down(dp, np.uint16 if bf16 else np.float32), p, bf16)
+        assert _same_bits_nan_aware(_down(dm, np.float32), m, False)
+        assert _same_bits_nan_aware(_down(dv, np.float32), v, False)
+        if use_master:
+            assert _same_bits_nan_aware(_down(dw, np.float32), w, False)
+    sh32, p32 = wild(), wild()
+    sh = onp.f32_to_bf16(sh32) if bf16 else sh32
+    pp = onp.f32_to_bf16(p32) if bf16 else p32
+    ds, dp = _up(sh), _up(pp)
+    rows = (L.EmaRow * 1)()
+    rows[0].shadow, rows[0].p, rows[0].numel, rows[0].dtype_tag = ds.data_ptr(), dp.data_ptr(), n, tag
+    L.check(L.lib().eri_ema_update_multi(rows, 1, 0.999, torch.cuda.current_stream().cuda_stream), "ema")
+    with np.errstate(all="ignore"):
+        oc.lib().eri_oracle_ema_update(oc.ptr(sh), oc.ptr(pp), n, tag, 0.999)
+    torch.cuda.synchronize()
+    assert _same_bits_nan_aware(_down(ds, np.uint16 if bf16 else np.float32), sh, bf16)
+
+
+def test_quantize_dequantize_with_extreme_values():
+    """Checkpoint traffic: blocks whose maximum is denormal, huge or infinite, all-zero blocks, NaN."""
+    import torch
+    from eridiffusion_amd import _lib as L
+    import harness as hs
+    rng = np.random.default_rng(5150)
+    n = 2048 * 6 + 77
+    scale = np.repeat(10.0 ** np.array([-43.0, -30.0, 0.0, 30.0, 38.0, -5.0, 3.0]), 2048)[:n]
+    with np.errstate(over="ignore"):
+        x = (rng.standard_normal(n) * scale).astype(np.float32)
+    x[2048 * 2:2048 * 3] = 0.0
+    x[2048 * 5 + 9] = np.inf
+    x[2048 * 6 + 5] = np.nan
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+    for signed, table in ((1, hs.MAPS[0]), (0, hs.MAPS[1])):
+        xs = x if signed else np.abs(x)
+        xd = torch.from_numpy(xs).to(dev)
+        codes = torch.empty(n, dtype=torch.uint8, device=dev)
+        absmax = torch.empty(7, dtype=torch.float32, device=dev)
+        back = torch.empty(n, dtype=torch.float32, device=dev)
+        L.check(L.lib().eri_adam8_quantize(xd.data_ptr(), signed, n, codes.data_ptr(), absmax.data_ptr(), stream), "q")
+        L.check(L.lib().eri_adam8_dequantize(codes.data_ptr(), absmax.data_ptr(), signed, n, back.data_ptr(), stream), "dq")
+        torch.cuda.synchronize()
+        wc, wa, wb = np.empty(n, np.uint8), np.empty(7, np.float32), np.empty(n, np.float32)
+        with np.errstate(all="ignore"):
+            oc.lib().eri_oracle_quantize(oc.ptr(xs), oc.ptr(table), n, oc.ptr(wc), oc.ptr(wa))
+            oc.lib().eri_oracle_dequantize(oc.ptr(wc), oc.ptr(wa), oc.ptr(table), n, oc.ptr(wb))
+        assert np.array_equal(codes.cpu().numpy(), wc), signed
+        assert np.array_equal(absmax.cpu().numpy().view(np.uint32), wa.view(np.uint32)), signed
+        assert _same_bits_nan_aware(back.cpu().numpy(), wb, False), signed
