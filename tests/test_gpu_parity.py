@@ -344,3 +344,12 @@ def test_randomized_extreme_values_against_the_oracle():
         exact = (not bf16) or bool(flags & 2) or mode == 2
         stats = hs.compare(got_p, got_st, ps, states, bf16, exact, "extreme%d" % case)
         assert stats["code_mismatch"] == 0, case
+
+
+def test_five_thousand_small_tensors_in_one_launch():
+    """A long launch table: 5,000 tensors of 1 to 6,000 elements (most of them nothing but a partial
+    block), both through the table handle and through step_multi."""
+    rng = np.random.default_rng(5000)
+    sizes = [int(x) for x in rng.integers(1, 6000, 5000)]
+    run_case(sizes, True, 5001, steps=2, flags=2, label="5000-tensors")
+    run_case(sizes[:1500], False, 5002, steps=2, use_multi=True, label="1500-tensors-multi")
