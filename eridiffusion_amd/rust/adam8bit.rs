@@ -328,6 +328,55 @@ impl Adam8bit {
     }
 }
 
+/// crates/training/src/optimizers/adam8bit.rs:4-28.  The quantile fields steer the reference's per-tensor
+/// clipping (adam8bit_enhanced.rs:53-69); the blockwise format has no such step, so they are carried only.
+#[derive(Debug, Clone)]
+pub struct AdamW8bitConfig {
+    pub lr: f64,
+    pub beta1: f64,
+    pub beta2: f64,
+    pub epsilon: f64,
+    pub weight_decay: f64,
+    pub quantile_alpha: f32,
+    pub adaptive_quantization: bool,
+    pub quantization_warmup_steps: usize,
+}
+
+impl Default for AdamW8bitConfig {
+    fn default() -> Self {
+        Self { lr: 1e-3, beta1: 0.9, beta2: 0.999, epsilon: 1e-8, weight_decay: 0.01, quantile_alpha: 0.99,
+               adaptive_quantization: true, quantization_warmup_steps: 100 }
+    }
+}
+
+impl From<AdamW8bitConfig> for Adam8bitConfig {
+    fn from(c: AdamW8bitConfig) -> Self {
+        Self { lr: c.lr, betas: (c.beta1, c.beta2), eps: c.epsilon, weight_decay: c.weight_decay, ..Self::default() }
+    }
+}
+
+/// src/trainers/training/optimization.rs:9-27
+#[derive(Debug, Clone)]
+pub struct OptimizerConfig {
+    pub optimizer_type: String,
+    pub learning_rate: f64,
+    pub weight_decay: Option<f64>,
+    pub betas: Option<(f64, f64)>,
+    pub eps: Option<f64>,
+}
+
+impl Default for OptimizerConfig {
+    fn default() -> Self {
+        Self { optimizer_type: "adam8bit".to_string(), learning_rate: 1e-4, weight_decay: Some(0.01),
+               betas: Some((0.9, 0.999)), eps: Some(1e-8) }
+    }
+}
+
+/// optimization.rs:30-58 with its own argument list
+pub fn create_optimizer_from_config(config: &OptimizerConfig, parameters: Vec<Parameter>) -> Result<Adam8bit> {
+    create_optimizer(&config.optimizer_type, parameters, config.learning_rate, config.betas, config.eps, config.weight_decay)
+}
+
 /// String-keyed factory, src/trainers/training/optimization.rs:30-58 and
 /// src/optimizers/memory_efficient_optimizers.rs:285-308.
 pub fn create_optimizer(optimizer_type: &str, parameters: Vec<Parameter>, learning_rate: f64, betas: Option<(f64, f64)>,
