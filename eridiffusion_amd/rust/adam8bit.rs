@@ -356,25 +356,27 @@ impl From<AdamW8bitConfig> for Adam8bitConfig {
 }
 
 /// src/trainers/training/optimization.rs:9-27
-#[derive(Debug, Clone)]
+#[derive(Debug, Clone, serde::Serialize, serde::Deserialize)]
 pub struct OptimizerConfig {
     pub optimizer_type: String,
-    pub learning_rate: f64,
-    pub weight_decay: Option<f64>,
-    pub betas: Option<(f64, f64)>,
-    pub eps: Option<f64>,
+    pub learning_rate: f32,
+    pub weight_decay: Option<f32>,
+    pub betas: Option<(f32, f32)>,
+    pub eps: Option<f32>,
 }
 
 impl Default for OptimizerConfig {
     fn default() -> Self {
-        Self { optimizer_type: "adam8bit".to_string(), learning_rate: 1e-4, weight_decay: Some(0.01),
+        Self { optimizer_type: "adamw8bit".to_string(), learning_rate: 1e-4, weight_decay: Some(0.01),
                betas: Some((0.9, 0.999)), eps: Some(1e-8) }
     }
 }
 
-/// optimization.rs:30-58 with its own argument list
+/// optimization.rs:30-58 with its own argument list (f32 fields widened as the reference does, :38-41)
 pub fn create_optimizer_from_config(config: &OptimizerConfig, parameters: Vec<Parameter>) -> Result<Adam8bit> {
-    create_optimizer(&config.optimizer_type, parameters, config.learning_rate, config.betas, config.eps, config.weight_decay)
+    create_optimizer(&config.optimizer_type, parameters, config.learning_rate as f64,
+                     config.betas.map(|(a, b)| (a as f64, b as f64)), config.eps.map(|e| e as f64),
+                     config.weight_decay.map(|w| w as f64))
 }
 
 /// String-keyed factory, src/trainers/training/optimization.rs:30-58 and
