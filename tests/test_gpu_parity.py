@@ -80,7 +80,7 @@ def run_case(sizes, bf16, seed, steps=3, mode=0, flags=0, wd=WD, p_std=0.02, g_s
 
 
 def test_config1_flat_fp32_after_ten_prior_steps():
-    # BASELINE configuration 1: 2**20 fp32 params ~N(0, 0.02), grads ~N(0, 1e-3), states from ten
+    # benchmark configuration 1: 2**20 fp32 params ~N(0, 0.02), grads ~N(0, 1e-3), states from ten
     # prior steps, block 2048, lr 1e-4, betas (0.9, 0.999), eps 1e-8, wd 0.01; one step
     run_case([1 << 20], False, 0xE21D + 1, steps=1, prior=10, label="c1")
 
