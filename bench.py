@@ -29,7 +29,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--config", default="c5_flux12b_full")
     ap.add_argument("--flags", type=int, default=0, help="ERI_ADAM8_FLAG_* bits for the step")
-    ap.add_argument("--cpu-sample", type=int, default=512 << 20, help="parameters in the CPU baseline sample (0 = skip)")
+    ap.add_argument("--cpu-sample", type=int, default=2 << 30, help="parameters in the CPU baseline sample (0 = skip)")
     ap.add_argument("--kernel", choices=["adam8", "adam8_clip", "grad_norm", "adamw32", "ema"], default="adam8",
                     help="what one step is: the 8-bit AdamW step (headline), the same preceded by the device-side "
                          "gradient norm, the norm alone, the 32-bit AdamW sibling, or the EMA sweep")
