@@ -49,6 +49,12 @@ class EmaRow(C.Structure):
                 ("reserved", C.c_int32)]
 
 
+class MemoryReportC(C.Structure):
+    _fields_ = [("num_params", C.c_uint64), ("param_memory_gb", C.c_double), ("state_memory_gb", C.c_double),
+                ("total_memory_gb", C.c_double), ("memory_reduction_percent", C.c_double), ("has_reduction", C.c_int32),
+                ("description", C.c_char * 44)]
+
+
 class EriError(RuntimeError):
     def __init__(self, what, code, message):
         super().__init__("%s failed with code %d: %s" % (what, code, message))
@@ -113,6 +119,10 @@ EXPORTS = {
     "eri_adam8bit_set_grad_scale": (C.c_int, [C.c_void_p, C.c_float]),
     "eri_adam8bit_set_param_grad_scale": (C.c_int, [C.c_void_p, C.c_uint32, C.c_float]),
     "eri_adam8bit_set_max_grad_norm": (C.c_int, [C.c_void_p, C.c_float, C.c_float]),
+    "eri_analyze_optimizer_memory": (C.c_int, [C.c_uint64, C.c_char_p, C.POINTER(MemoryReportC)]),
+    "eri_ema_decay_from_half_life": (C.c_float, [C.c_uint64]),
+    "eri_ema_decay_from_window": (C.c_float, [C.c_uint64]),
+    "eri_ema_effective_decay": (C.c_float, [C.c_float, C.c_uint64, C.c_float, C.c_int]),
     "eri_adam8bit_set_mode": (C.c_int, [C.c_void_p, C.c_int]),
     "eri_adam8bit_last_grad_norm": (C.c_int, [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
     "eri_adam8bit_last_nonfinite_grads": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint64)]),

@@ -851,4 +851,51 @@ int eri_adam8bit_fn_load_state_fp32(EriAdam8bitFn *o, const char *name, const fl
     return 0;
 }
 
+// ---- helpers beside the optimizers ------------------------------------------------------------
+
+int eri_analyze_optimizer_memory(uint64_t num_params, const char *precision, EriOptimizerMemoryReport *out) {
+    if (!precision || !out) return fail(ERI_ERR_NULL, "precision or out is NULL");
+    const uint64_t param_bytes = num_params * 4; // adam8bit_enhanced.rs:407
+    const std::string p(precision);
+    uint64_t state_bytes = param_bytes * 2;
+    const char *desc = "Unknown precision";
+    if (p == "fp32") { state_bytes = param_bytes * 2; desc = "FP32 momentum states"; }
+    else if (p == "fp16") { state_bytes = param_bytes; desc = "FP16 momentum states"; }
+    else if (p == "8bit") { state_bytes = param_bytes / 2; desc = "8-bit quantized momentum states"; }
+    else if (p == "4bit") { state_bytes = param_bytes / 4; desc = "4-bit quantized momentum states"; }
+    const uint64_t total = param_bytes + state_bytes;
+    std::memset(out, 0, sizeof(*out));
+    out->num_params = num_params;
+    out->param_memory_gb = (double)param_bytes / 1e9;
+    out->state_memory_gb = (double)state_bytes / 1e9;
+    out->total_memory_gb = (double)total / 1e9;
+    out->has_reduction = p != "fp32";
+    out->memory_reduction_percent =
+        out->has_reduction ? (1.0 - (double)total / (double)(param_bytes * 3)) * 100.0 : 0.0; // :419-423
+    std::snprintf(out->description, sizeof(out->description), "%s", desc);
+    return 0;
+}
+
+float eri_ema_decay_from_half_life(uint64_t half_life_steps) { // ema_enhanced.rs:268-272
+    return std::pow(0.5f, 1.0f / (float)half_life_steps);
+}
+
+float eri_ema_decay_from_window(uint64_t window_size) { // :275-278
+    return 1.0f - 2.0f / ((float)window_size + 1.0f);
+}
+
+float eri_ema_effective_decay(float decay, uint64_t step, float power, int use_bias_correction) { // :106-127
+    float d = decay;
+    if (power != 1.0f) {
+        const float progress = std::fmin((float)step / 1000.0f, 1.0f);
+        d = std::pow(d, power * (1.0f - progress) + progress);
+    }
+    if (use_bias_correction && step < 1000) {
+        const float numerator = 1.0f - std::pow(d, (float)(int32_t)(step - 1));
+        const float denominator = 1.0f - std::pow(d, (float)(int32_t)step);
+        d = d * numerator / std::fmax(denominator, 1e-8f);
+    }
+    return d;
+}
+
 } // extern "C"

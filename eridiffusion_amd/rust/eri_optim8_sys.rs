@@ -50,6 +50,11 @@ pub struct EriAdamW32Hyper { pub lr: f32, pub beta1: f32, pub beta2: f32, pub ep
 #[derive(Clone, Copy)]
 pub struct EriEmaTensor { pub shadow: *mut c_void, pub p: *const c_void, pub numel: u64, pub dtype_tag: i32, pub reserved: i32 }
 
+#[repr(C)]
+#[derive(Clone, Copy)]
+pub struct EriOptimizerMemoryReport { pub num_params: u64, pub param_memory_gb: f64, pub state_memory_gb: f64, pub total_memory_gb: f64,
+    pub memory_reduction_percent: f64, pub has_reduction: i32, pub description: [c_char; 44] }
+
 pub enum EriAdam8Table {}
 pub enum EriParameter {}
 pub enum EriAdam8bit {}
@@ -113,6 +118,10 @@ extern "C" {
     pub fn eri_adam8bit_set_grad_scale(opt: *mut EriAdam8bit, scale: f32) -> c_int;
     pub fn eri_adam8bit_set_param_grad_scale(opt: *mut EriAdam8bit, index: u32, scale: f32) -> c_int;
     pub fn eri_adam8bit_set_max_grad_norm(opt: *mut EriAdam8bit, max_norm: f32, denom_eps: f32) -> c_int;
+    pub fn eri_analyze_optimizer_memory(num_params: u64, precision: *const c_char, out: *mut EriOptimizerMemoryReport) -> c_int;
+    pub fn eri_ema_decay_from_half_life(half_life_steps: u64) -> f32;
+    pub fn eri_ema_decay_from_window(window_size: u64) -> f32;
+    pub fn eri_ema_effective_decay(decay: f32, step: u64, power: f32, use_bias_correction: c_int) -> f32;
     pub fn eri_adam8bit_set_mode(opt: *mut EriAdam8bit, mode: c_int) -> c_int;
     pub fn eri_adam8bit_last_grad_norm(opt: *mut EriAdam8bit, norm: *mut f32, scale: *mut f32) -> c_int;
     pub fn eri_adam8bit_last_nonfinite_grads(opt: *mut EriAdam8bit, count: *mut u64) -> c_int;

@@ -121,6 +121,28 @@ int eri_adam8bit_fn_get_state_fp32(EriAdam8bitFn *opt, const char *name, float *
 int eri_adam8bit_fn_load_state_fp32(EriAdam8bitFn *opt, const char *name, const float *m, const float *v,
                                     uint64_t numel);
 
+/* ---- small host-side helpers that live beside the optimizers in the reference -------------------- */
+
+/* analyze_optimizer_memory(num_params, precision), adam8bit_enhanced.rs:406-431: the reference's coarse
+ * accounting (fp32 parameters; states of 8, 4, 2 or 1 bytes per parameter for "fp32", "fp16", "8bit",
+ * "4bit"; anything else counts as fp32 with the description "Unknown precision").
+ * memory_reduction_percent is against fp32 states and is absent (has_reduction = 0) for "fp32". */
+typedef struct EriOptimizerMemoryReport {
+    uint64_t num_params;
+    double param_memory_gb, state_memory_gb, total_memory_gb;
+    double memory_reduction_percent;
+    int32_t has_reduction;
+    char description[44];
+} EriOptimizerMemoryReport;
+int eri_analyze_optimizer_memory(uint64_t num_params, const char *precision, EriOptimizerMemoryReport *out);
+
+/* EMA decay helpers, src/trainers/ema_enhanced.rs:268-279 and compute_effective_decay :106-127
+ * (power schedule over the first 1000 steps, optional bias correction below step 1000).  The value
+ * they give is what a trainer passes to eri_ema_update_multi. */
+float eri_ema_decay_from_half_life(uint64_t half_life_steps);
+float eri_ema_decay_from_window(uint64_t window_size);
+float eri_ema_effective_decay(float decay, uint64_t step, float power, int use_bias_correction);
+
 #ifdef __cplusplus
 }
 #endif

@@ -189,3 +189,55 @@ def test_state_file_parsers_survive_random_corruption(tmp_path):
             assert rc > 0 or rc in (-1, -2, -3, -4, -5, -6, -7, -8)
     assert refused > 300
     L.lib().eri_adam8bit_destroy(opt)
+
+
+# ---- the reference's own unit tests for this path, restated ----------------------------------------
+
+def test_adam8bit_creation_as_in_the_reference():
+    # adam8bit_enhanced.rs:469-484: two parameters of 100 and 50 fp32 elements, default config
+    handles = (C.c_void_p * 2)()
+    for i, n in enumerate((100, 50)):
+        h = C.c_void_p()
+        L.check(L.lib().eri_param_create(0x10000 * (i + 1), n, L.DTYPE_F32, C.byref(h)), "eri_param_create")
+        handles[i] = h
+    opt = C.c_void_p()
+    L.check(L.lib().eri_adam8bit_new(handles, 2, None, None, C.byref(opt)), "eri_adam8bit_new")
+    assert L.lib().eri_adam8bit_current_lr(opt) == 1e-3
+    assert L.lib().eri_adam8bit_quantized_memory_usage(opt) == 0  # no state before the first step
+    L.lib().eri_adam8bit_destroy(opt)
+    for h in handles:
+        L.lib().eri_param_release(h)
+
+
+def test_memory_report_as_in_the_reference():
+    # adam8bit_enhanced.rs:500-508: 1e9 parameters, "8bit": states smaller than parameters.  That test also
+    # asserts a reduction above 60 %, which its own function (:406-431) cannot give: (4 + 2) GB against
+    # 3 * 4 GB is exactly 50 %.  The function is what is restated here.
+    rep = L.MemoryReportC()
+    L.check(L.lib().eri_analyze_optimizer_memory(1_000_000_000, b"8bit", C.byref(rep)), "analyze")
+    assert rep.has_reduction and rep.memory_reduction_percent == 50.0
+    assert rep.state_memory_gb < rep.param_memory_gb
+    assert rep.param_memory_gb == 4.0 and rep.state_memory_gb == 2.0 and rep.total_memory_gb == 6.0
+    assert rep.description == b"8-bit quantized momentum states"
+    L.check(L.lib().eri_analyze_optimizer_memory(1000, b"fp32", C.byref(rep)), "analyze")
+    assert not rep.has_reduction and rep.state_memory_gb == 2 * rep.param_memory_gb
+    L.check(L.lib().eri_analyze_optimizer_memory(1000, b"int3", C.byref(rep)), "analyze")
+    assert rep.description == b"Unknown precision" and rep.state_memory_gb == 2 * rep.param_memory_gb
+    assert L.lib().eri_analyze_optimizer_memory(1, None, C.byref(rep)) == -1
+
+
+def test_ema_decay_helpers_as_in_the_reference():
+    # ema_enhanced.rs:285-294
+    d = L.lib().eri_ema_decay_from_half_life(1000)
+    assert abs(d ** 1000 - 0.5) < 0.001
+    assert abs(L.lib().eri_ema_decay_from_window(99) - 0.98) < 0.001
+    # compute_effective_decay :106-127: plain decay without schedule or correction; bias correction gives
+    # decay * (1 - decay^(s-1)) / (1 - decay^s) below step 1000, which is 0 at the first step
+    assert L.lib().eri_ema_effective_decay(0.999, 5, 1.0, 0) == np.float32(0.999)
+    assert L.lib().eri_ema_effective_decay(0.999, 1, 1.0, 1) == 0.0
+    want = 0.999 * (1 - 0.999 ** 9) / (1 - 0.999 ** 10)
+    assert abs(L.lib().eri_ema_effective_decay(0.999, 10, 1.0, 1) - want) < 1e-4
+    assert L.lib().eri_ema_effective_decay(0.999, 2000, 1.0, 1) == np.float32(0.999)
+    # power schedule: exponent goes from `power` at step 0 to 1 at step 1000
+    assert abs(L.lib().eri_ema_effective_decay(0.9, 0, 2.0, 0) - 0.81) < 1e-6
+    assert abs(L.lib().eri_ema_effective_decay(0.9, 1000, 2.0, 0) - 0.9) < 1e-6
