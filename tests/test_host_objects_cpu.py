@@ -4,6 +4,7 @@ import ctypes as C
 import os
 import struct
 
+import numpy as np
 import pytest
 
 from eridiffusion_amd import _lib as L
