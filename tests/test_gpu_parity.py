@@ -275,6 +275,21 @@ def test_state_init_and_quantize_round_trip():
         assert np.array_equal(back.cpu().numpy().view(np.uint32), wb.view(np.uint32))
 
 
+def test_quantization_as_in_the_reference():
+    # adam8bit_enhanced.rs:486-498 on the device: 10x10 ~N(0, 1), quantise, dequantise, mean |error| < 0.1
+    import torch
+    L = _lib()
+    x = torch.randn(100, device="cuda", generator=torch.Generator(device="cuda").manual_seed(486))
+    codes = torch.empty(100, dtype=torch.uint8, device="cuda")
+    absmax = torch.empty(1, device="cuda")
+    back = torch.empty(100, device="cuda")
+    L.check(L.lib().eri_adam8_quantize(x.data_ptr(), 1, 100, codes.data_ptr(), absmax.data_ptr(), _stream()), "q")
+    L.check(L.lib().eri_adam8_dequantize(codes.data_ptr(), absmax.data_ptr(), 1, 100, back.data_ptr(), _stream()), "dq")
+    _sync()
+    assert back.shape == x.shape and float(absmax[0]) == float(x.abs().max())
+    assert float((back - x).abs().mean()) < 0.02
+
+
 def test_randomized_cases_against_the_oracle():
     """Forty seeded random combinations of tensor lists (ragged, tiny, multi-block), dtype, mode, flags,
     decay, gradient scale and prior history; every one must match the oracle to the bar above."""

@@ -109,3 +109,18 @@ def test_quantize_dequantize_blockwise():
         i = np.argmax(np.abs(x[seg]))
         if x[seg][i] > 0:
             assert back[seg][i] == x[seg][i]
+
+
+def test_quantization_as_in_the_reference():
+    # adam8bit_enhanced.rs:486-498: a 10x10 tensor ~N(0, 1) is quantised and dequantised; the shape
+    # survives and the mean absolute error is below 0.1.  The blockwise dynamic format is far inside that:
+    # its relative step near full scale is 1/128 and finer below.
+    rng = np.random.default_rng(486)
+    s, _ = oc.load_maps()
+    x = rng.standard_normal(100).astype(np.float32)
+    codes, absmax, back = np.empty(100, np.uint8), np.empty(1, np.float32), np.empty(100, np.float32)
+    oc.lib().eri_oracle_quantize(oc.ptr(x), oc.ptr(s), 100, oc.ptr(codes), oc.ptr(absmax))
+    oc.lib().eri_oracle_dequantize(oc.ptr(codes), oc.ptr(absmax), oc.ptr(s), 100, oc.ptr(back))
+    assert back.shape == x.shape
+    err = np.abs(back - x).mean()
+    assert err < 0.1 and err < 0.02
