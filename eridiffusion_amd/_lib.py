@@ -119,6 +119,16 @@ EXPORTS = {
     "eri_adam8bit_set_grad_scale": (C.c_int, [C.c_void_p, C.c_float]),
     "eri_adam8bit_set_param_grad_scale": (C.c_int, [C.c_void_p, C.c_uint32, C.c_float]),
     "eri_adam8bit_set_max_grad_norm": (C.c_int, [C.c_void_p, C.c_float, C.c_float]),
+    "eri_ema_new": (C.c_int, [C.c_float, C.c_int, C.c_float, C.c_void_p, C.POINTER(C.c_void_p)]),
+    "eri_ema_destroy": (C.c_int, [C.c_void_p]),
+    "eri_ema_init_from_params": (C.c_int, [C.c_void_p, C.POINTER(C.c_char_p), C.POINTER(C.c_void_p), C.c_uint32]),
+    "eri_ema_update": (C.c_int, [C.c_void_p, C.POINTER(C.c_char_p), C.POINTER(C.c_void_p), C.c_uint32]),
+    "eri_ema_copy_to": (C.c_int, [C.c_void_p, C.POINTER(C.c_char_p), C.POINTER(C.c_void_p), C.c_uint32]),
+    "eri_ema_step": (C.c_uint64, [C.c_void_p]),
+    "eri_ema_set_step": (C.c_int, [C.c_void_p, C.c_uint64]),
+    "eri_ema_current_decay": (C.c_float, [C.c_void_p]),
+    "eri_ema_num_shadows": (C.c_uint32, [C.c_void_p]),
+    "eri_ema_shadow": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p), C.POINTER(C.c_uint64), C.POINTER(C.c_int)]),
     "eri_analyze_optimizer_memory": (C.c_int, [C.c_uint64, C.c_char_p, C.POINTER(MemoryReportC)]),
     "eri_ema_decay_from_half_life": (C.c_float, [C.c_uint64]),
     "eri_ema_decay_from_window": (C.c_float, [C.c_uint64]),

@@ -225,6 +225,81 @@ class Adam8bitFunctional:
             pass
 
 
+class EMAModel:
+    """src/trainers/ema_enhanced.rs:12-204 over torch tensors: named shadow copies updated by one launch.
+    `params` is a dict name -> tensor (float32 or bfloat16, contiguous)."""
+
+    def __init__(self, decay: float, use_bias_correction: bool = True, power: float = 1.0):
+        self._ema = C.c_void_p()
+        check(lib().eri_ema_new(decay, int(use_bias_correction), power, _stream_ptr(), C.byref(self._ema)), "eri_ema_new")
+        self._handles: Dict[str, Tuple[C.c_void_p, int, int]] = {}
+
+    def _pack(self, params: Dict[str, torch.Tensor]):
+        names = (C.c_char_p * len(params))()
+        hs = (C.c_void_p * len(params))()
+        for i, (name, t) in enumerate(params.items()):
+            if not t.is_contiguous():
+                raise ValueError("parameters must be contiguous")
+            key = (t.data_ptr(), t.numel())
+            h = self._handles.get(name)
+            if h is None or (h[1], h[2]) != key:
+                if h is not None:
+                    lib().eri_param_release(h[0])
+                hnd = C.c_void_p()
+                check(lib().eri_param_create(t.data_ptr(), t.numel(), _dtype_tag(t), C.byref(hnd)), "eri_param_create")
+                h = (hnd, *key)
+                self._handles[name] = h
+            names[i] = name.encode()
+            hs[i] = h[0]
+        return names, hs, len(params)
+
+    def init_from_params(self, params: Dict[str, torch.Tensor]) -> None:
+        check(lib().eri_ema_init_from_params(self._ema, *self._pack(params)), "eri_ema_init_from_params")
+
+    def update(self, params: Dict[str, torch.Tensor]) -> None:
+        check(lib().eri_ema_update(self._ema, *self._pack(params)), "eri_ema_update")
+
+    def copy_to(self, params: Dict[str, torch.Tensor]) -> None:
+        check(lib().eri_ema_copy_to(self._ema, *self._pack(params)), "eri_ema_copy_to")
+
+    def step(self) -> int:
+        return lib().eri_ema_step(self._ema)
+
+    def set_step(self, step: int) -> None:
+        check(lib().eri_ema_set_step(self._ema, step), "eri_ema_set_step")
+
+    def current_decay(self) -> float:
+        return lib().eri_ema_current_decay(self._ema)
+
+    def shadow_params(self, like: Dict[str, torch.Tensor]) -> Dict[str, torch.Tensor]:
+        """Copies of the shadows of the names in `like` (torch cannot wrap foreign device memory)."""
+        out = {}
+        for name, t in like.items():
+            ptr, numel, tag = C.c_void_p(), C.c_uint64(), C.c_int()
+            check(lib().eri_ema_shadow(self._ema, name.encode(), C.byref(ptr), C.byref(numel), C.byref(tag)), "eri_ema_shadow")
+            dst = torch.empty(numel.value, dtype=torch.float32 if tag.value == DTYPE_F32 else torch.bfloat16, device=t.device)
+            check(lib().eri_hip_memcpy_async(dst.data_ptr(), ptr.value, dst.numel() * dst.element_size(), 3, _stream_ptr()), "memcpy")
+            out[name] = dst
+        return out
+
+    def __contains__(self, name: str) -> bool:
+        return lib().eri_ema_shadow(self._ema, name.encode(), None, None, None) == 0
+
+    def close(self) -> None:
+        if self._ema:
+            lib().eri_ema_destroy(self._ema)
+            self._ema = C.c_void_p()
+            for h in self._handles.values():
+                lib().eri_param_release(h[0])
+            self._handles = {}
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 def update_params_8bit(optimizer: Adam8bitFunctional, params: Dict[str, torch.Tensor],
                        grads: Dict[str, torch.Tensor]) -> None:
     """adam8bit.rs:333-345: every named parameter that has a gradient is replaced by its update."""

@@ -714,7 +714,6 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
         const float a_m = raw.a_m, a_v = raw.a_v;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            const uint32_t o = c * 512 + lane * 8;
             Raw8<true> pr, gr;
             pr.w = raw.p[c];
             gr.w = raw.g[c];

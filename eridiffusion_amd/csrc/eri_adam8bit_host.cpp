@@ -899,3 +899,157 @@ float eri_ema_effective_decay(float decay, uint64_t step, float power, int use_b
 }
 
 } // extern "C"
+
+// ---- EMAModel ------------------------------------------------------------------------------------
+
+struct EriEmaModel {
+    struct Shadow {
+        void *data = nullptr;
+        uint64_t numel = 0;
+        int32_t dtype = 0;
+    };
+    float decay = 0.999f, power = 1.0f;
+    bool bias_correction = true;
+    uint64_t step = 0;
+    void *stream = nullptr;
+    std::map<std::string, Shadow> shadows;
+    std::vector<EriEmaTensor> rows; // reused between updates
+    ~EriEmaModel() {
+        for (auto &kv : shadows)
+            if (kv.second.data) eri_hip_free(kv.second.data);
+    }
+};
+
+namespace {
+
+uint64_t elem_bytes(int32_t dtype) { return dtype == ERI_DTYPE_F32 ? 4 : 2; }
+
+// a fresh shadow holding a copy of the parameter (ema_enhanced.rs:72-73,100-103)
+int ema_adopt(EriEmaModel *e, const std::string &name, const EriParameter *p) {
+    if (!p || !p->data) return fail(ERI_ERR_NULL, "parameter without data: " + name);
+    if (p->numel == 0) return fail(ERI_ERR_EMPTY, "empty parameter: " + name);
+    if (p->dtype != ERI_DTYPE_F32 && p->dtype != ERI_DTYPE_BF16) return fail(ERI_ERR_DTYPE, "Unsupported: EMA takes F32 or BF16 parameters");
+    EriEmaModel::Shadow &s = e->shadows[name];
+    const uint64_t bytes = p->numel * elem_bytes(p->dtype);
+    if (!s.data || s.numel != p->numel || s.dtype != p->dtype) {
+        if (s.data) eri_hip_free(s.data);
+        s = EriEmaModel::Shadow();
+        int dev = 0;
+        int rc = eri_hip_get_device(&dev);
+        if (!rc) rc = eri_hip_malloc_zeroed(dev, bytes, &s.data);
+        if (rc) {
+            e->shadows.erase(name);
+            return rc;
+        }
+        s.numel = p->numel;
+        s.dtype = p->dtype;
+    }
+    return eri_hip_memcpy_async(s.data, p->data, bytes, 3, e->stream);
+}
+
+} // namespace
+
+extern "C" {
+
+int eri_ema_new(float decay, int use_bias_correction, float power, void *stream, EriEmaModel **out) {
+    if (!out) return fail(ERI_ERR_NULL, "out is NULL");
+    *out = nullptr;
+    if (!(0.0f < decay && decay <= 1.0f)) { // ema_enhanced.rs:36-41
+        char buf[96];
+        std::snprintf(buf, sizeof buf, "InvalidOperation: EMA decay must be in (0, 1], got %g", (double)decay);
+        return fail(ERI_ERR_ARG, buf);
+    }
+    EriEmaModel *e = new EriEmaModel();
+    e->decay = decay;
+    e->bias_correction = use_bias_correction != 0;
+    e->power = power;
+    e->stream = stream;
+    *out = e;
+    return 0;
+}
+
+int eri_ema_destroy(EriEmaModel *e) {
+    delete e;
+    return 0;
+}
+
+int eri_ema_init_from_params(EriEmaModel *e, const char *const *names, EriParameter *const *params, uint32_t n) {
+    if (!e || (n && (!names || !params))) return fail(ERI_ERR_NULL, "NULL argument");
+    for (uint32_t i = 0; i < n; ++i) {
+        if (!names[i]) return fail(ERI_ERR_NULL, "NULL name");
+        int rc = ema_adopt(e, names[i], params[i]);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+uint64_t eri_ema_step(const EriEmaModel *e) { return e ? e->step : 0; }
+
+int eri_ema_set_step(EriEmaModel *e, uint64_t step) {
+    if (!e) return fail(ERI_ERR_NULL, "ema is NULL");
+    e->step = step;
+    return 0;
+}
+
+float eri_ema_current_decay(const EriEmaModel *e) {
+    return e ? eri_ema_effective_decay(e->decay, e->step, e->power, e->bias_correction) : 0.0f;
+}
+
+uint32_t eri_ema_num_shadows(const EriEmaModel *e) { return e ? (uint32_t)e->shadows.size() : 0; }
+
+int eri_ema_shadow(const EriEmaModel *e, const char *name, void **data, uint64_t *numel, int *dtype_tag) {
+    if (!e || !name) return fail(ERI_ERR_NULL, "NULL argument");
+    auto it = e->shadows.find(name);
+    if (it == e->shadows.end()) return fail(ERI_ERR_ARG, std::string("InvalidOperation: No EMA weights found for parameter: ") + name);
+    if (data) *data = it->second.data;
+    if (numel) *numel = it->second.numel;
+    if (dtype_tag) *dtype_tag = it->second.dtype;
+    return 0;
+}
+
+int eri_ema_update(EriEmaModel *e, const char *const *names, EriParameter *const *params, uint32_t n) {
+    if (!e || (n && (!names || !params))) return fail(ERI_ERR_NULL, "NULL argument");
+    for (uint32_t i = 0; i < n; ++i)
+        if (!names[i] || !params[i] || !params[i]->data) return fail(ERI_ERR_NULL, "NULL name or parameter");
+    e->step += 1;                                      // ema_enhanced.rs:80
+    const float d = eri_ema_current_decay(e);           // :83
+    e->rows.clear();
+    for (uint32_t i = 0; i < n; ++i) {
+        auto it = e->shadows.find(names[i]);
+        const EriParameter *p = params[i];
+        if (it == e->shadows.end() || it->second.numel != p->numel || it->second.dtype != p->dtype) {
+            int rc = ema_adopt(e, names[i], p);          // :100-103 first time seeing this parameter
+            if (rc) return rc;
+            continue;
+        }
+        EriEmaTensor r;
+        r.shadow = it->second.data;
+        r.p = p->data;
+        r.numel = p->numel;
+        r.dtype_tag = p->dtype;
+        r.reserved = 0;
+        e->rows.push_back(r);
+    }
+    if (e->rows.empty()) return 0;
+    return eri_ema_update_multi(e->rows.data(), (uint32_t)e->rows.size(), d, e->stream); // :88-98
+}
+
+int eri_ema_copy_to(EriEmaModel *e, const char *const *names, EriParameter *const *params, uint32_t n) {
+    if (!e || (n && (!names || !params))) return fail(ERI_ERR_NULL, "NULL argument");
+    for (uint32_t i = 0; i < n; ++i) { // refuse before anything is copied
+        if (!names[i] || !params[i] || !params[i]->data) return fail(ERI_ERR_NULL, "NULL name or parameter");
+        auto it = e->shadows.find(names[i]);
+        if (it == e->shadows.end())
+            return fail(ERI_ERR_ARG, std::string("InvalidOperation: No EMA weights found for parameter: ") + names[i]);
+        if (it->second.numel != params[i]->numel || it->second.dtype != params[i]->dtype)
+            return fail(ERI_ERR_ARG, std::string("EMA weights do not fit parameter: ") + names[i]);
+    }
+    for (uint32_t i = 0; i < n; ++i) {
+        const EriEmaModel::Shadow &s = e->shadows[names[i]];
+        int rc = eri_hip_memcpy_async(params[i]->data, s.data, s.numel * elem_bytes(s.dtype), 3, e->stream);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+} // extern "C"

@@ -391,3 +391,79 @@ pub fn create_optimizer(optimizer_type: &str, parameters: Vec<Parameter>, learni
         other => Err(Error::InvalidOperation(format!("Unknown optimizer: {other}"))),
     }
 }
+
+// ---- EMAModel, src/trainers/ema_enhanced.rs:12-204 ---------------------------------------------
+
+pub struct EMAModel {
+    ema: *mut sys::EriEmaModel,
+}
+
+unsafe impl Send for EMAModel {}
+
+impl EMAModel {
+    /// :35-52 (bias correction on, power 1)
+    pub fn new(decay: f32, stream: *mut c_void) -> Result<Self> {
+        Self::with_config(decay, stream, true, 1.0)
+    }
+    /// :55-64
+    pub fn with_config(decay: f32, stream: *mut c_void, use_bias_correction: bool, power: f32) -> Result<Self> {
+        let mut ema = std::ptr::null_mut();
+        check(unsafe { sys::eri_ema_new(decay, use_bias_correction as i32, power, stream, &mut ema) }, "eri_ema_new")?;
+        Ok(Self { ema })
+    }
+    fn with_handles<R>(params: &HashMap<String, &Parameter>, f: impl FnOnce(*const *const std::os::raw::c_char, *const *mut sys::EriParameter, u32) -> i32, what: &str) -> Result<()> {
+        let names: Vec<CString> = params.keys().map(|k| CString::new(k.as_str()).unwrap()).collect();
+        let name_ptrs: Vec<*const std::os::raw::c_char> = names.iter().map(|c| c.as_ptr()).collect();
+        let mut handles = Vec::with_capacity(params.len());
+        for p in params.values() {
+            let t = p.tensor()?;
+            let numel: usize = t.shape().dims().iter().product();
+            let mut h = std::ptr::null_mut();
+            check(unsafe { sys::eri_param_create(t.cuda_ptr_mut() as *mut c_void, numel as u64, dtype_tag(t.dtype())?, &mut h) }, "eri_param_create")?;
+            handles.push(h);
+        }
+        let rc = f(name_ptrs.as_ptr(), handles.as_ptr(), handles.len() as u32);
+        for h in handles {
+            unsafe { sys::eri_param_release(h) };
+        }
+        check(rc, what)
+    }
+    /// :67-76
+    pub fn init_from_params(&mut self, params: &HashMap<String, &Parameter>) -> Result<()> {
+        let ema = self.ema;
+        Self::with_handles::<()>(params, |n, h, k| unsafe { sys::eri_ema_init_from_params(ema, n, h, k) }, "eri_ema_init_from_params")
+    }
+    /// :79-104, one launch over every known parameter
+    pub fn update(&mut self, params: &HashMap<String, &Parameter>) -> Result<()> {
+        let ema = self.ema;
+        Self::with_handles::<()>(params, |n, h, k| unsafe { sys::eri_ema_update(ema, n, h, k) }, "eri_ema_update")
+    }
+    /// :130-142 (the shadow's values are copied into the parameter's memory)
+    pub fn copy_to(&self, params: &HashMap<String, &Parameter>) -> Result<()> {
+        let ema = self.ema;
+        Self::with_handles::<()>(params, |n, h, k| unsafe { sys::eri_ema_copy_to(ema, n, h, k) }, "eri_ema_copy_to")
+    }
+    pub fn step(&self) -> usize {
+        unsafe { sys::eri_ema_step(self.ema) as usize }
+    }
+    pub fn set_step(&mut self, step: usize) {
+        unsafe { sys::eri_ema_set_step(self.ema, step as u64) };
+    }
+    pub fn current_decay(&self) -> f32 {
+        unsafe { sys::eri_ema_current_decay(self.ema) }
+    }
+}
+
+impl Drop for EMAModel {
+    fn drop(&mut self) {
+        unsafe { sys::eri_ema_destroy(self.ema) };
+    }
+}
+
+/// :268-279
+pub fn decay_from_half_life(half_life_steps: usize) -> f32 {
+    unsafe { sys::eri_ema_decay_from_half_life(half_life_steps as u64) }
+}
+pub fn decay_from_window(window_size: usize) -> f32 {
+    unsafe { sys::eri_ema_decay_from_window(window_size as u64) }
+}

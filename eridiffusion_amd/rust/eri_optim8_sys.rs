@@ -55,6 +55,7 @@ pub struct EriEmaTensor { pub shadow: *mut c_void, pub p: *const c_void, pub num
 pub struct EriOptimizerMemoryReport { pub num_params: u64, pub param_memory_gb: f64, pub state_memory_gb: f64, pub total_memory_gb: f64,
     pub memory_reduction_percent: f64, pub has_reduction: i32, pub description: [c_char; 44] }
 
+pub enum EriEmaModel {}
 pub enum EriAdam8Table {}
 pub enum EriParameter {}
 pub enum EriAdam8bit {}
@@ -118,6 +119,16 @@ extern "C" {
     pub fn eri_adam8bit_set_grad_scale(opt: *mut EriAdam8bit, scale: f32) -> c_int;
     pub fn eri_adam8bit_set_param_grad_scale(opt: *mut EriAdam8bit, index: u32, scale: f32) -> c_int;
     pub fn eri_adam8bit_set_max_grad_norm(opt: *mut EriAdam8bit, max_norm: f32, denom_eps: f32) -> c_int;
+    pub fn eri_ema_new(decay: f32, use_bias_correction: c_int, power: f32, stream: *mut c_void, out: *mut *mut EriEmaModel) -> c_int;
+    pub fn eri_ema_destroy(ema: *mut EriEmaModel) -> c_int;
+    pub fn eri_ema_init_from_params(ema: *mut EriEmaModel, names: *const *const c_char, params: *const *mut EriParameter, n: u32) -> c_int;
+    pub fn eri_ema_update(ema: *mut EriEmaModel, names: *const *const c_char, params: *const *mut EriParameter, n: u32) -> c_int;
+    pub fn eri_ema_copy_to(ema: *mut EriEmaModel, names: *const *const c_char, params: *const *mut EriParameter, n: u32) -> c_int;
+    pub fn eri_ema_step(ema: *const EriEmaModel) -> u64;
+    pub fn eri_ema_set_step(ema: *mut EriEmaModel, step: u64) -> c_int;
+    pub fn eri_ema_current_decay(ema: *const EriEmaModel) -> f32;
+    pub fn eri_ema_num_shadows(ema: *const EriEmaModel) -> u32;
+    pub fn eri_ema_shadow(ema: *const EriEmaModel, name: *const c_char, data: *mut *mut c_void, numel: *mut u64, dtype_tag: *mut c_int) -> c_int;
     pub fn eri_analyze_optimizer_memory(num_params: u64, precision: *const c_char, out: *mut EriOptimizerMemoryReport) -> c_int;
     pub fn eri_ema_decay_from_half_life(half_life_steps: u64) -> f32;
     pub fn eri_ema_decay_from_window(window_size: u64) -> f32;

@@ -136,6 +136,28 @@ typedef struct EriOptimizerMemoryReport {
 } EriOptimizerMemoryReport;
 int eri_analyze_optimizer_memory(uint64_t num_params, const char *precision, EriOptimizerMemoryReport *out);
 
+/* ---- EMAModel (src/trainers/ema_enhanced.rs:12-204): shadow copies of named parameters ----------------
+ * The shadows live in device memory owned by the object; update() is one eri_ema_update_multi launch
+ * over every parameter already known, plus a device copy for names seen for the first time (:100-103).
+ * eri_ema_new: decay outside (0, 1] is refused with "EMA decay must be in (0, 1], got ..." (:36-41);
+ * the reference's defaults are use_bias_correction = 1, power = 1 (:48-50; with_config :55-64). */
+typedef struct EriEmaModel EriEmaModel;
+int eri_ema_new(float decay, int use_bias_correction, float power, void *stream, EriEmaModel **out);
+int eri_ema_destroy(EriEmaModel *ema);
+/* init_from_params :67-76: every shadow becomes a copy of its parameter. */
+int eri_ema_init_from_params(EriEmaModel *ema, const char *const *names, EriParameter *const *params, uint32_t n);
+/* update :79-104: step += 1, then shadow = d*shadow + (1-d)*param with d = current_decay(). */
+int eri_ema_update(EriEmaModel *ema, const char *const *names, EriParameter *const *params, uint32_t n);
+/* copy_to :130-142: parameter memory <- shadow; an unknown name answers
+ * "No EMA weights found for parameter: ..." and nothing is copied. */
+int eri_ema_copy_to(EriEmaModel *ema, const char *const *names, EriParameter *const *params, uint32_t n);
+uint64_t eri_ema_step(const EriEmaModel *ema);             /* :175 */
+int eri_ema_set_step(EriEmaModel *ema, uint64_t step);     /* :180 */
+float eri_ema_current_decay(const EriEmaModel *ema);       /* :185 */
+uint32_t eri_ema_num_shadows(const EriEmaModel *ema);
+/* shadow_params() :170, one name at a time: device pointer, element count and dtype of a shadow. */
+int eri_ema_shadow(const EriEmaModel *ema, const char *name, void **data, uint64_t *numel, int *dtype_tag);
+
 /* EMA decay helpers, src/trainers/ema_enhanced.rs:268-279 and compute_effective_decay :106-127
  * (power schedule over the first 1000 steps, optional bias correction below step 1000).  The value
  * they give is what a trainer passes to eri_ema_update_multi. */

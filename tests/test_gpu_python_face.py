@@ -105,3 +105,51 @@ def test_mode_bnb_with_clipping_and_statistics_through_the_python_face():
         assert np.array_equal(_bits(p), want)
     m_err, v_err = opt.quantization_stats()
     assert 0 < m_err < 1e-4 and 0 < v_err < 1e-6
+
+
+def test_ema_model_as_in_the_reference_and_against_the_oracle():
+    """ema_enhanced.rs:296-318 restated (decay 0.999, one parameter of 10 fp32 values: init, one update,
+    step() == 1, the shadow is there), then the numbers: three updates of two parameters with the
+    effective decay of each step, a late-comer adopted by copy, and copy_to."""
+    from eridiffusion_amd import _lib as L
+    from eridiffusion_amd.adam8bit import EMAModel
+    ema = EMAModel(0.999)
+    param1 = torch.randn(10, device="cuda")
+    ema.init_from_params({"param1": param1})
+    ema.update({"param1": param1})
+    assert ema.step() == 1 and "param1" in ema and "other" not in ema
+
+    rng = np.random.default_rng(3)
+    ema = EMAModel(0.99, use_bias_correction=True, power=1.0)
+    w32 = rng.standard_normal(2048 * 2 + 77).astype(np.float32)
+    b16 = onp.f32_to_bf16(rng.standard_normal(640).astype(np.float32))
+    tw, tb = torch.from_numpy(w32.copy()).cuda(), _bf16_tensor(b16)
+    params = {"w": tw, "b": tb}
+    ema.init_from_params(params)
+    sh_w, sh_b = w32.copy(), b16.copy()
+    for step in (1, 2, 3):
+        w32 = (w32 + rng.standard_normal(w32.size).astype(np.float32) * np.float32(0.1)).astype(np.float32)
+        b16 = onp.f32_to_bf16(onp.bf16_to_f32(b16) + rng.standard_normal(b16.size).astype(np.float32) * np.float32(0.1))
+        tw.copy_(torch.from_numpy(w32))
+        tb.copy_(_bf16_tensor(b16))
+        if step == 3:
+            late = torch.full((33,), 2.5, device="cuda")
+            params["late"] = late
+        ema.update(params)
+        d = L.lib().eri_ema_effective_decay(0.99, step, 1.0, 1)
+        assert ema.current_decay() == d and ema.step() == step
+        oc.lib().eri_oracle_ema_update(oc.ptr(sh_w), oc.ptr(w32), w32.size, oc.DT_F32, d)
+        oc.lib().eri_oracle_ema_update(oc.ptr(sh_b), oc.ptr(b16), b16.size, oc.DT_BF16, d)
+    got = ema.shadow_params(params)
+    torch.cuda.synchronize()
+    assert np.array_equal(got["w"].cpu().numpy().view(np.uint32), sh_w.view(np.uint32))
+    assert np.array_equal(_bits(got["b"]), sh_b)
+    assert bool((got["late"] == 2.5).all())  # first seen at step 3: adopted as a copy
+    # the first step's effective decay is 0 (bias correction), so the shadow jumps to the parameter there
+    assert L.lib().eri_ema_effective_decay(0.99, 1, 1.0, 1) == 0.0
+    target = {"w": torch.zeros_like(tw), "b": torch.zeros_like(tb)}
+    ema.copy_to(target)
+    torch.cuda.synchronize()
+    assert torch.equal(target["w"], got["w"]) and torch.equal(target["b"], got["b"])
+    with pytest.raises(L.EriError, match="No EMA weights found for parameter: nope"):
+        ema.copy_to({"nope": torch.zeros(4, device="cuda")})

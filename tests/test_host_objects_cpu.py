@@ -242,3 +242,27 @@ def test_ema_decay_helpers_as_in_the_reference():
     # power schedule: exponent goes from `power` at step 0 to 1 at step 1000
     assert abs(L.lib().eri_ema_effective_decay(0.9, 0, 2.0, 0) - 0.81) < 1e-6
     assert abs(L.lib().eri_ema_effective_decay(0.9, 1000, 2.0, 0) - 0.9) < 1e-6
+
+
+def test_ema_model_host_logic():
+    ema = C.c_void_p()
+    for bad in (0.0, -0.1, 1.5, float("nan")):
+        assert L.lib().eri_ema_new(bad, 1, 1.0, None, C.byref(ema)) == -6
+        assert b"EMA decay must be in (0, 1], got" in L.lib().eri_last_error()  # ema_enhanced.rs:36-41
+    L.check(L.lib().eri_ema_new(0.999, 1, 1.0, None, C.byref(ema)), "eri_ema_new")
+    assert L.lib().eri_ema_step(ema) == 0 and L.lib().eri_ema_num_shadows(ema) == 0
+    L.check(L.lib().eri_ema_set_step(ema, 2000), "set_step")
+    assert L.lib().eri_ema_current_decay(ema) == np.float32(0.999)  # no correction from step 1000 on
+    L.check(L.lib().eri_ema_set_step(ema, 1), "set_step")
+    assert L.lib().eri_ema_current_decay(ema) == 0.0                # :121-125 at the first step
+    assert L.lib().eri_ema_shadow(ema, b"missing", None, None, None) == -6
+    assert b"No EMA weights found for parameter: missing" in L.lib().eri_last_error()  # :134-138
+    h = C.c_void_p()
+    L.check(L.lib().eri_param_create(0x4000, 16, L.DTYPE_BF16, C.byref(h)), "param")
+    names = (C.c_char_p * 1)(b"w")
+    hs = (C.c_void_p * 1)(h)
+    assert L.lib().eri_ema_copy_to(ema, names, hs, 1) == -6
+    assert L.lib().eri_ema_update(ema, None, hs, 1) == -1
+    assert L.lib().eri_ema_step(ema) == 1  # a refused call does not count a step
+    L.lib().eri_param_release(h)
+    L.lib().eri_ema_destroy(ema)
