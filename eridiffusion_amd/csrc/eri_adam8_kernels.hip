@@ -250,7 +250,8 @@ template <>
 struct Raw8<true> {
     u32x4 w;
     __device__ __forceinline__ void load(const void *base, uint32_t elem) {
-        w = *as_global(reinterpret_cast<const u32x4 *>(static_cast<const uint16_t *>(base) + elem));
+        // every byte these kernels stream is touched once per launch: non-temporal throughout
+        w = __builtin_nontemporal_load(as_global(reinterpret_cast<const u32x4 *>(static_cast<const uint16_t *>(base) + elem)));
     }
     __device__ __forceinline__ void unpack(float (&out)[8]) const {
         out[0] = bf16_lo(w.x); out[1] = bf16_hi(w.x); out[2] = bf16_lo(w.y); out[3] = bf16_hi(w.y);
@@ -262,6 +263,8 @@ struct Raw8<false> {
     f32x4 a, b;
     __device__ __forceinline__ void load(const void *base, uint32_t elem) {
         ERI_GLOBAL const f32x4 *q = as_global(reinterpret_cast<const f32x4 *>(static_cast<const float *>(base) + elem));
+        // a lane's two words share cache lines with its neighbours' across the two instructions, so these
+        // stay ordinary loads: streamed, the second instruction would fetch every line again
         a = q[0];
         b = q[1];
     }
@@ -282,7 +285,7 @@ __device__ __forceinline__ void store8(void *base, uint32_t elem, const float (&
         __builtin_nontemporal_store(w, as_global(reinterpret_cast<u32x4 *>(static_cast<uint16_t *>(base) + elem)));
     } else {
         ERI_GLOBAL f32x4 *q = as_global(reinterpret_cast<f32x4 *>(static_cast<float *>(base) + elem));
-        q[0] = f32x4{v[0], v[1], v[2], v[3]};
+        q[0] = f32x4{v[0], v[1], v[2], v[3]}; // half a line per instruction: left to the cache to merge
         q[1] = f32x4{v[4], v[5], v[6], v[7]};
     }
 }
@@ -425,8 +428,8 @@ __device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint
             const uint32_t o = (c0 + d) * 512 + lane * 8;
             pr[d].load(p, o);
             gr[d].load(g, o);
-            mr[d] = *as_global(reinterpret_cast<const u32x2 *>(mc + o));
-            vr[d] = *as_global(reinterpret_cast<const u32x2 *>(vc + o));
+            mr[d] = __builtin_nontemporal_load(as_global(reinterpret_cast<const u32x2 *>(mc + o)));
+            vr[d] = __builtin_nontemporal_load(as_global(reinterpret_cast<const u32x2 *>(vc + o)));
         }
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {
@@ -463,8 +466,8 @@ __device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint
             const uint32_t o = c * 512 + lane * 8;
             u32x2 mw, vw;
             requant8<true, KEYTAB, MODE == ERI_ADAM8_MODE_BNB>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
-            *as_global(reinterpret_cast<u32x2 *>(mc + o)) = mw;
-            *as_global(reinterpret_cast<u32x2 *>(vc + o)) = vw;
+            __builtin_nontemporal_store(mw, as_global(reinterpret_cast<u32x2 *>(mc + o)));
+            __builtin_nontemporal_store(vw, as_global(reinterpret_cast<u32x2 *>(vc + o)));
         }
     } else {
 #pragma unroll
@@ -472,8 +475,8 @@ __device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint
             const uint32_t o = c * 512 + lane * 8;
             u32x2 mw, vw;
             requant8<false, KEYTAB, MODE == ERI_ADAM8_MODE_BNB>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
-            *as_global(reinterpret_cast<u32x2 *>(mc + o)) = mw;
-            *as_global(reinterpret_cast<u32x2 *>(vc + o)) = vw;
+            __builtin_nontemporal_store(mw, as_global(reinterpret_cast<u32x2 *>(mc + o)));
+            __builtin_nontemporal_store(vw, as_global(reinterpret_cast<u32x2 *>(vc + o)));
         }
     }
 }
@@ -1015,35 +1018,50 @@ __global__ __launch_bounds__(256) void grad_sumsq_kernel(const DevTensor *__rest
         total += (double)wave_sum(acc);
         bad += (double)wave_sum(nf);
     }
-    uint32_t ti = 0;
+    // full blocks, one load ahead: the next block's four words are in flight while this one is reduced
     const BlockWalk walk(total_blocks, chunks);
-    for (uint32_t blk = walk.first; blk < walk.end; blk += walk.stride) {
-        ti = find_row(rows, n_rows, ti, blk);
-        const DevTensor t = rows[ti];
-        const size_t e0 = (size_t)(blk - t.full_start) * kBlock;
+    if (walk.first < walk.end) {
+        uint32_t ti = find_row(rows, n_rows, 0, walk.first);
         Raw8<BF16> raw[4];
+        {
+            const DevTensor t = rows[ti];
+            const size_t e0 = (size_t)(walk.first - t.full_start) * kBlock;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) raw[c].load(static_cast<const char *>(t.g) + e0 * (BF16 ? 2 : 4), c * 512 + lane * 8);
-        float acc = 0.0f;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            float g[8];
-            raw[c].unpack(g);
-#pragma unroll
-            for (int k = 0; k < 8; ++k) acc += g[k] * g[k];
+            for (int c = 0; c < 4; ++c) raw[c].load(static_cast<const char *>(t.g) + e0 * (BF16 ? 2 : 4), c * 512 + lane * 8);
         }
-        const float block_sum = wave_sum(acc);
-        total += (double)block_sum;
-        if (not_finite(block_sum) != 0.0f) { // rare: count the NaN / infinite elements of this block
-            float nf = 0.0f;
+        for (uint32_t blk = walk.first; blk < walk.end; blk += walk.stride) {
+            Raw8<BF16> cur[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) cur[c] = raw[c];
+            const uint32_t nblk = blk + walk.stride;
+            if (nblk < walk.end) {
+                ti = find_row(rows, n_rows, ti, nblk);
+                const DevTensor t = rows[ti];
+                const size_t e0 = (size_t)(nblk - t.full_start) * kBlock;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) raw[c].load(static_cast<const char *>(t.g) + e0 * (BF16 ? 2 : 4), c * 512 + lane * 8);
+            }
+            float acc = 0.0f;
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 float g[8];
-                raw[c].unpack(g);
+                cur[c].unpack(g);
 #pragma unroll
-                for (int k = 0; k < 8; ++k) nf += not_finite(g[k]);
+                for (int k = 0; k < 8; ++k) acc += g[k] * g[k];
             }
-            bad += (double)wave_sum(nf);
+            const float block_sum = wave_sum(acc);
+            total += (double)block_sum;
+            if (not_finite(block_sum) != 0.0f) { // rare: count the NaN / infinite elements of this block
+                float nf = 0.0f;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    float g[8];
+                    cur[c].unpack(g);
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) nf += not_finite(g[k]);
+                }
+                bad += (double)wave_sum(nf);
+            }
         }
     }
     if (lane == 0) {
