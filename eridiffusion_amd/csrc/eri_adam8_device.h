@@ -74,12 +74,13 @@ int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_bloc
 extern int g_kernel_variant;
 extern int g_chunks;
 extern int g_pipelined_waves;
+extern int g_norm_waves;
 /* Sum of |moment - dequantised moment| of the coming step, per row: err[2r] first moment, err[2r+1] second. */
 int launch_quant_error(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_blocks, int dtype_tag,
                        const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale, double *err,
                        uint32_t grid, void *stream);
 /* Gradient norm: one f64 partial per wave (grid * 4 of them), then norm and clip factor into out[0], out[1]. */
-constexpr uint32_t kNormWavesPerWg = 4;
+constexpr uint32_t kNormWavesPerCu = 32; // persistent waves of the gradient-norm pass per compute unit
 int launch_grad_sumsq(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_blocks, int dtype_tag,
                       double *partial, uint32_t grid, void *stream);
 int launch_grad_norm_finish(const double *partial, uint32_t n, float max_norm, float denom_eps, float *out,

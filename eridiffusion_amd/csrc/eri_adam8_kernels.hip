@@ -798,6 +798,7 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
     }
 }
 
+int g_norm_waves = 4;      // waves per workgroup of the gradient-norm pass (eri_adam8_set_tuning key 4)
 int g_pipelined_waves = 0; // measurement switch: waves per workgroup of the pipelined kernel (0 = 12)
 int g_chunks = 8; // contiguous ranges of the block list (BlockWalk); 8 = one per accelerator die
 /* The chunked walk needs the same number of workgroups in every chunk. */
@@ -996,7 +997,7 @@ __device__ __forceinline__ float wave_sum(float x) {
 }
 
 template <bool BF16>
-__global__ __launch_bounds__(256) void grad_sumsq_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
+__global__ __launch_bounds__(1024) void grad_sumsq_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
                                                          uint32_t total_blocks, double *__restrict__ partial,
                                                          uint32_t chunks) {
     // persistent: every wave adds the fp32 sums of its blocks in f64 and leaves one partial
@@ -1105,9 +1106,9 @@ int launch_grad_sumsq(const DevTensor *rows, uint32_t n_rows, uint32_t total_blo
                       uint32_t grid, void *stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype_tag == ERI_DTYPE_F32)
-        hipLaunchKernelGGL(grad_sumsq_kernel<false>, dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, partial, chunks_for(grid));
+        hipLaunchKernelGGL(grad_sumsq_kernel<false>, dim3(grid), dim3(g_norm_waves * kWave), 0, s, rows, n_rows, total_blocks, partial, chunks_for(grid));
     else
-        hipLaunchKernelGGL(grad_sumsq_kernel<true>, dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, partial, chunks_for(grid));
+        hipLaunchKernelGGL(grad_sumsq_kernel<true>, dim3(grid), dim3(g_norm_waves * kWave), 0, s, rows, n_rows, total_blocks, partial, chunks_for(grid));
     return (int)hipGetLastError();
 }
 

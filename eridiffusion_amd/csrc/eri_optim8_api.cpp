@@ -493,6 +493,11 @@ int eri_hip_mem_info(size_t *free_bytes, size_t *total_bytes) {
 static int g_grid_override = 0; // measurement switch: persistent workgroups of the step (0 = one per slot)
 
 int eri_adam8_set_tuning(int key, int value) {
+    if (key == 4) {
+        if (value != 1 && value != 2 && value != 4 && value != 8 && value != 16) return fail(ERI_ERR_ARG, "waves per workgroup must be 1, 2, 4, 8 or 16");
+        eri::g_norm_waves = value;
+        return 0;
+    }
     if (key == 3) {
         if (value < 0 || value > 12) return fail(ERI_ERR_ARG, "waves per workgroup out of range");
         eri::g_pipelined_waves = value;
@@ -703,21 +708,22 @@ int eri_adam8_grad_norm(EriAdam8Table *t, float max_norm, float denom_eps, void 
     DeviceCtx *ctx = nullptr;
     int rc = get_ctx(&ctx);
     if (rc) return rc;
-    const uint32_t grid_cap = ctx->cus * 8; // persistent: 8 workgroups of 4 waves per compute unit
+    const uint32_t wpw = (uint32_t)eri::g_norm_waves;
+    const uint32_t grid_cap = ctx->cus * eri::kNormWavesPerCu / wpw; // persistent
     if (!t->partial) {
         // two groups at most, and per wave a sum of squares and a count
-        ERI_HIP(hipMalloc((void **)&t->partial, sizeof(double) * 2 * 2 * grid_cap * eri::kNormWavesPerWg));
+        ERI_HIP(hipMalloc((void **)&t->partial, sizeof(double) * 2 * 2 * ctx->cus * eri::kNormWavesPerCu));
         ERI_HIP(hipMalloc((void **)&t->norm_out, sizeof(float) * 4)); // norm, scale, 64-bit count
     }
     uint32_t off = 0;
     for (auto &g : t->groups) {
         if (g.n == 0) continue;
         const uint32_t work = g.total_blocks > g.n ? g.total_blocks : g.n;
-        uint32_t grid = (work + eri::kNormWavesPerWg - 1) / eri::kNormWavesPerWg;
+        uint32_t grid = (work + wpw - 1) / wpw;
         if (grid > grid_cap) grid = grid_cap;
         rc = eri::launch_grad_sumsq(g.dev, g.n, g.total_blocks, g.dtype, t->partial + 2 * off, grid, stream);
         if (rc) return hip_fail((hipError_t)rc, "gradient sum-of-squares launch");
-        off += grid * eri::kNormWavesPerWg;
+        off += grid * wpw;
     }
     t->n_partial = off;
     rc = eri::launch_grad_norm_finish(t->partial, t->n_partial, max_norm, denom_eps, t->norm_out, stream);

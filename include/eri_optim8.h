@@ -145,7 +145,8 @@ int eri_adam8_init(void);
 /* Measurement switches, not part of the optimizer's behaviour (all settings give identical results):
  * key 0 = store schedule of the bf16 step kernel (0 = shipped), key 1 = number of persistent workgroups
  * (0 = one per compute unit), key 2 = contiguous ranges the block list is cut into (8 = shipped, one per
- * accelerator die; 1 = plain grid stride), key 3 = waves per workgroup of the bf16 step kernel (0 = 12). */
+ * accelerator die; 1 = plain grid stride), key 3 = waves per workgroup of the bf16 step kernel (0 = 12), key 4 = waves per workgroup of the
+ * gradient-norm pass (4 = shipped; set before a table's first norm). */
 int eri_adam8_set_tuning(int key, int value);
 
 /* The two 256-entry maps (code -> value in [-1, 1] / [0, 1]) the states are expressed in. */
