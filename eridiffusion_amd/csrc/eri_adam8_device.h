@@ -75,6 +75,24 @@ extern int g_kernel_variant;
 extern int g_chunks;
 extern int g_pipelined_waves;
 extern int g_norm_waves;
+
+/* The chunked walk (BlockWalk) needs the same number of workgroups in every chunk. */
+inline uint32_t chunks_for(uint32_t grid) {
+    return (g_chunks > 1 && grid % (uint32_t)g_chunks == 0) ? (uint32_t)g_chunks : 1u;
+}
+
+/* The step's kernels live in translation units of their own (they build in parallel); launch_step
+ * picks one.  wd / gs / keytab / exact select template instances: decay present, gradient scale present,
+ * slot-table (rather than binary-search) requantisation, IEEE square root and division on bf16. */
+int launch_step_plain_f32(int mode, bool wd, bool gs, bool keytab, const DevTensor *rows, uint32_t n_rows,
+                          uint32_t total_blocks, const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale,
+                          uint32_t grid, uint32_t wg, void *stream);
+int launch_step_plain_bf16(int mode, bool exact, bool wd, bool gs, bool keytab, const DevTensor *rows, uint32_t n_rows,
+                           uint32_t total_blocks, const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale,
+                           uint32_t grid, uint32_t wg, void *stream);
+int launch_step_pipelined(int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
+                          uint32_t total_blocks, const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale,
+                          uint32_t grid, uint32_t wg, void *stream);
 /* Sum of |moment - dequantised moment| of the coming step, per row: err[2r] first moment, err[2r+1] second. */
 int launch_quant_error(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_blocks, int dtype_tag,
                        const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale, double *err,

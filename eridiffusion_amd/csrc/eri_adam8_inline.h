@@ -1,0 +1,578 @@
+#ifndef ERI_ADAM8_INLINE_H
+#define ERI_ADAM8_INLINE_H
+/*
+ * Device code shared by the gfx950 kernels of the blockwise 8-bit AdamW step (everything here is
+ * inline or a template; the kernels themselves are in the eri_adam8_*.hip files).
+ *
+ * Work decomposition: one 64-lane wavefront owns one 2048-element quantisation block from its
+ * first load to its last store, so the per-block absmax needs nothing but a DPP reduction inside
+ * the wave -- no barrier, no cross-wave exchange.  A block is read in four 512-element passes;
+ * lane l of pass c holds elements c*512 + 8*l .. +7, which makes every access a contiguous
+ * 128-bit (params, grads) or 64-bit (codes) load per lane.  The fp32 moments of the whole block
+ * stay in registers (32 + 32 per lane) between the update and the requantisation, so each byte of
+ * p, g, m, v crosses HBM once in each direction.
+ *
+ * The grid is persistent: workgroups stage the lookup tables into LDS once, then their waves walk
+ * the global block list -- cut into one contiguous range per accelerator die, see BlockWalk -- with
+ * the stride of their die's waves, so consecutive waves touch consecutive blocks.
+ * The tensor that owns a block is found by a scalar binary search over the launch table.
+ *
+ * Arithmetic: every fp32 operation of the update is written as its own statement and the file is
+ * compiled with -ffp-contract=off, because the reference runs each as a separate tensor op
+ * (src/trainers/adam8bit_enhanced.rs:252-275).  fmaf appears only inside the exactly rounded
+ * division below.
+ */
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "eri_adam8_device.h"
+
+namespace eri {
+
+// ------------------------------------------------------------------------------------------
+// small device helpers
+// ------------------------------------------------------------------------------------------
+
+/* Pointers read from the launch table have no known address space; every one of them is device
+ * memory, and saying so turns flat_load/flat_store (which also tick the LDS counter and so
+ * serialise with the table lookups) into global_load/global_store. */
+#define ERI_GLOBAL __attribute__((address_space(1)))
+template <typename T>
+__device__ __forceinline__ ERI_GLOBAL T *as_global(T *p) {
+    return (ERI_GLOBAL T *)p;
+}
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint32_t f2u(float x) { return __builtin_bit_cast(uint32_t, x); }
+__device__ __forceinline__ float u2f(uint32_t x) { return __builtin_bit_cast(float, x); }
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_mov(float x) {
+    return u2f((uint32_t)__builtin_amdgcn_update_dpp((int)f2u(x), (int)f2u(x), CTRL, ROW_MASK, 0xf, false));
+}
+
+/* Maximum over the 64 lanes of non-negative, NaN-free values, returned wave-uniform.  Such floats
+ * order like their bit patterns, so the steps are unsigned integer maxima with the lane permutation
+ * folded into the instruction (v_max_u32_dpp); lanes a step does not write keep their value.  A DPP
+ * read of a register needs two wait states after the vector instruction that wrote it, and the
+ * assembler text below is opaque to the compiler's hazard handling, hence the explicit s_nop. */
+#define ERI_DPP_MAX(reg, ctrl) "v_max_u32_dpp " reg ", " reg ", " reg " " ctrl " bank_mask:0xf\n"
+__device__ __forceinline__ float wave_max(float x) {
+    uint32_t u = f2u(x);
+    asm volatile("s_nop 1\n"
+                 ERI_DPP_MAX("%0", "quad_perm:[1,0,3,2] row_mask:0xf") "s_nop 1\n"
+                 ERI_DPP_MAX("%0", "quad_perm:[2,3,0,1] row_mask:0xf") "s_nop 1\n"
+                 ERI_DPP_MAX("%0", "row_half_mirror row_mask:0xf") "s_nop 1\n"
+                 ERI_DPP_MAX("%0", "row_mirror row_mask:0xf") "s_nop 1\n" // every lane holds its row's maximum
+                 ERI_DPP_MAX("%0", "row_bcast:15 row_mask:0xa") "s_nop 1\n" // into rows 1 and 3
+                 ERI_DPP_MAX("%0", "row_bcast:31 row_mask:0xc") "s_nop 1\n" // into rows 2 and 3
+                 : "+v"(u));
+    return u2f((uint32_t)__builtin_amdgcn_readlane((int)u, 63));
+}
+/* Two reductions at once: each chain's instruction fills one of the other's wait states. */
+__device__ __forceinline__ void wave_max2(float &a, float &b) {
+    uint32_t u = f2u(a), w = f2u(b);
+#define ERI_DPP_MAX2(ctrl) ERI_DPP_MAX("%0", ctrl) ERI_DPP_MAX("%1", ctrl) "s_nop 0\n"
+    asm volatile("s_nop 1\n"
+                 ERI_DPP_MAX2("quad_perm:[1,0,3,2] row_mask:0xf")
+                 ERI_DPP_MAX2("quad_perm:[2,3,0,1] row_mask:0xf")
+                 ERI_DPP_MAX2("row_half_mirror row_mask:0xf")
+                 ERI_DPP_MAX2("row_mirror row_mask:0xf")
+                 ERI_DPP_MAX2("row_bcast:15 row_mask:0xa")
+                 ERI_DPP_MAX2("row_bcast:31 row_mask:0xc")
+                 : "+v"(u), "+v"(w));
+#undef ERI_DPP_MAX2
+    a = u2f((uint32_t)__builtin_amdgcn_readlane((int)u, 63));
+    b = u2f((uint32_t)__builtin_amdgcn_readlane((int)w, 63));
+}
+
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return u2f(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return u2f(w & 0xffff0000u); }
+
+/* fp32 -> bf16 bits, round to nearest even, NaN kept quiet. */
+__device__ __forceinline__ uint32_t bf16_bits(float f) {
+    __bf16 b = (__bf16)f;
+    return (uint32_t)__builtin_bit_cast(uint16_t, b);
+}
+/* Two fp32 -> one dword of two bf16 (lo in the low half): a single v_cvt_pk_bf16_f32. */
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t bf16_pair(float lo, float hi) {
+    const f32x2 f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+}
+__device__ __forceinline__ float bf16_round(float f) { return u2f(bf16_bits(f) << 16); }
+
+/*
+ * SCALE * (m / a) for a divisor shared by a whole block, SCALE a power of two.  With
+ * ra = RN(1/a), q0 = RN(m*ra) is within an ulp or two of the quotient, the remainder m - q0*a is
+ * exact in one fma, and one correction gives the correctly rounded quotient (Markstein); folding
+ * the power of two into ra (and its inverse into a) scales every intermediate exactly.  `fast`
+ * excludes the divisors for which that argument needs care (zero, subnormal-range or huge values,
+ * an all-ones significand), and those blocks use the hardware-assisted IEEE division instead.
+ * Both produce the same bits.
+ */
+struct BlockDiv {
+    float a, as, ras, scale;
+    bool fast;
+    __device__ __forceinline__ explicit BlockDiv(float a_, float scale_ = 1.0f, float scale_inv = 1.0f)
+        : a(a_), scale(scale_) {
+        fast = (a_ >= 0x1p-60f) && (a_ <= 0x1p60f) && ((f2u(a_) & 0x7fffffu) != 0x7fffffu);
+        const float ra = fast ? 1.0f / a_ : 0.0f;
+        ras = ra * scale_;
+        as = a_ * scale_inv;
+    }
+    __device__ __forceinline__ float div_fast(float m) const {
+        float q0 = m * ras;
+        float r = __builtin_fmaf(-q0, as, m);
+        return __builtin_fmaf(r, ras, q0);
+    }
+    /* div_fast for a numerator that is not tied to the divisor (the bias corrections of the functional
+     * update divide moments by 1 - beta^s).  The correction step is exact only while nothing overflows
+     * or underflows: an infinite numerator or an overflowing quotient leaves NaN in it, and below
+     * 2^-100 the remainder loses bits (one quotient in fifteen then differs from the IEEE result).
+     * Those cases take the IEEE division; zero passes through.  Checked on the CPU against IEEE division
+     * on 6e8 uniformly random bit patterns and the special values, no difference. */
+    __device__ __forceinline__ float div_fast_unbounded(float m) const {
+        const float q = div_fast(m);
+        const float am = __builtin_fabsf(m), aq = __builtin_fabsf(q);
+        const bool ok = aq <= 3.4028234e38f && aq >= 0x1p-100f && am >= 0x1p-100f;
+        return ok ? q : (am == 0.0f ? m * scale : m / a * scale);
+    }
+    __device__ __forceinline__ float div_slow(float m) const {
+        float q = a == 0.0f ? 0.0f : m / a;
+        return q * scale;
+    }
+};
+
+struct Lds {
+    const float *map_s, *map_u, *mid_s, *mid_u;
+    const char *key_s, *key_u;
+};
+
+__device__ __forceinline__ uint32_t half_key(float xs) {
+    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)xs); // v_cvt_f16_f32, round to nearest even
+}
+
+/* xs = kKeyScale * x.  The slot address is the half pattern with its low bits cleared. */
+__device__ __forceinline__ uint32_t code_signed_key(float xs, const char *key_s) {
+    const KeySlot s = *reinterpret_cast<const KeySlot *>(key_s + (half_key(xs) & 0xfff0u));
+    return s.lo + (xs > s.mid ? 1u : 0u);
+}
+
+__device__ __forceinline__ uint32_t code_unsigned_key(float xs, const char *key_u) {
+    const KeySlot s = *reinterpret_cast<const KeySlot *>(key_u + (half_key(xs) & 0x7ff8u));
+    return s.lo + (xs > s.mid ? 1u : 0u);
+}
+
+/* Number of midpoints below x by binary search of the 255-entry LDS table (entry 255 is +inf). */
+__device__ __forceinline__ uint32_t code_bsearch(float x, const float *mid) {
+    uint32_t idx = 0;
+#pragma unroll
+    for (uint32_t s = 128; s >= 1; s >>= 1) idx += (x > mid[idx + s - 1]) ? s : 0u;
+    return idx;
+}
+
+// ------------------------------------------------------------------------------------------
+// the update of one element
+// ------------------------------------------------------------------------------------------
+
+template <int MODE, bool EXACT, bool BF16, bool WD, bool GS>
+__device__ __forceinline__ void adam_elem(float p, float g, float m_old, float v_old, const EriAdam8Hyper &h,
+                                          float gscale, const BlockDiv &dbc1, const BlockDiv &dbc2, float &m,
+                                          float &v, float &pn) {
+    if (GS) g = g * gscale;
+    if (MODE == ERI_ADAM8_MODE_L2 && WD) { // adam8bit.rs:113-120
+        float pw = p * h.weight_decay;
+        g = g + pw;
+    }
+    float t1 = m_old * h.beta1; // adam8bit_enhanced.rs:256
+    float t2 = g * h.omb1;
+    m = t1 + t2;
+    float gg = g * g; // :259-260
+    float t3 = v_old * h.beta2;
+    float t4 = gg * h.omb2;
+    v = t3 + t4;
+    if (MODE == ERI_ADAM8_MODE_L2) {
+        float mh = dbc1.fast ? dbc1.div_fast_unbounded(m) : m / dbc1.a; // adam8bit.rs:170
+        float vh = dbc2.fast ? dbc2.div_fast_unbounded(v) : v / dbc2.a; // :178
+        vh = fmaxf(vh, 0.0f);                                  // :181-182
+        float upd;
+        if (EXACT) {
+            float den = sqrtf(vh) + h.eps; // :187
+            upd = mh / den;
+        } else {
+            float den = __builtin_amdgcn_sqrtf(vh) + h.eps;
+            upd = mh * __builtin_amdgcn_rcpf(den);
+        }
+        float us = upd * h.step_size; // :196
+        if (BF16) us = bf16_round(us); // :197-198
+        pn = p - us;                   // :205
+    } else if (MODE == ERI_ADAM8_MODE_BNB) { // h.eps carries sqrt(bc2), h.weight_decay is the factor 1 - lr*wd
+        float den = sqrtf(v) + h.eps;
+        float r = m / den;
+        float us = r * h.step_size;
+        pn = p - us;
+        if (WD) pn = pn * h.weight_decay;
+    } else {
+        if (EXACT) {
+            float den = sqrtf(v) + h.eps; // adam8bit_enhanced.rs:263
+            float r = m / den;            // :264
+            float u = r;
+            if (WD) { // :267-271
+                float pw = p * h.weight_decay;
+                u = r + pw;
+            }
+            float us = u * h.step_size; // :274
+            pn = p - us;                // :275
+        } else {
+            // bf16 parameters: hardware square root and reciprocal (1 ulp each) and two fused
+            // multiply-adds; the fp32 result is within a few ulp of the exact chain, which moves
+            // the bf16 rounding of p by at most one step, rarely
+            float den = __builtin_amdgcn_sqrtf(v) + h.eps;
+            float r = m * __builtin_amdgcn_rcpf(den);
+            float u = WD ? __builtin_fmaf(p, h.weight_decay, r) : r;
+            pn = __builtin_fmaf(-u, h.step_size, p);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// 8 consecutive elements per lane: loads and stores
+// ------------------------------------------------------------------------------------------
+
+/* Eight consecutive elements of one lane as they come from memory: one 128-bit word of bf16, or
+ * two of fp32.  Loading and unpacking are separate so that a block's loads can all be issued
+ * before the first value is needed. */
+template <bool BF16>
+struct Raw8;
+template <>
+struct Raw8<true> {
+    u32x4 w;
+    __device__ __forceinline__ void load(const void *base, uint32_t elem) {
+        // every byte these kernels stream is touched once per launch: non-temporal throughout
+        w = __builtin_nontemporal_load(as_global(reinterpret_cast<const u32x4 *>(static_cast<const uint16_t *>(base) + elem)));
+    }
+    __device__ __forceinline__ void unpack(float (&out)[8]) const {
+        out[0] = bf16_lo(w.x); out[1] = bf16_hi(w.x); out[2] = bf16_lo(w.y); out[3] = bf16_hi(w.y);
+        out[4] = bf16_lo(w.z); out[5] = bf16_hi(w.z); out[6] = bf16_lo(w.w); out[7] = bf16_hi(w.w);
+    }
+};
+template <>
+struct Raw8<false> {
+    f32x4 a, b;
+    __device__ __forceinline__ void load(const void *base, uint32_t elem) {
+        ERI_GLOBAL const f32x4 *q = as_global(reinterpret_cast<const f32x4 *>(static_cast<const float *>(base) + elem));
+        // a lane's two words share cache lines with its neighbours' across the two instructions, so these
+        // stay ordinary loads: streamed, the second instruction would fetch every line again
+        a = q[0];
+        b = q[1];
+    }
+    __device__ __forceinline__ void unpack(float (&out)[8]) const {
+        out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w;
+        out[4] = b.x; out[5] = b.y; out[6] = b.z; out[7] = b.w;
+    }
+};
+
+template <bool BF16>
+__device__ __forceinline__ void store8(void *base, uint32_t elem, const float (&v)[8]) {
+    if (BF16) {
+        u32x4 w;
+        w.x = bf16_pair(v[0], v[1]);
+        w.y = bf16_pair(v[2], v[3]);
+        w.z = bf16_pair(v[4], v[5]);
+        w.w = bf16_pair(v[6], v[7]);
+        __builtin_nontemporal_store(w, as_global(reinterpret_cast<u32x4 *>(static_cast<uint16_t *>(base) + elem)));
+    } else {
+        ERI_GLOBAL f32x4 *q = as_global(reinterpret_cast<f32x4 *>(static_cast<float *>(base) + elem));
+        q[0] = f32x4{v[0], v[1], v[2], v[3]}; // half a line per instruction: left to the cache to merge
+        q[1] = f32x4{v[4], v[5], v[6], v[7]};
+    }
+}
+
+__device__ __forceinline__ uint32_t byte_of(const u32x2 w, int k) {
+    const uint32_t d = k < 4 ? w.x : w.y;
+    return (d >> (8 * (k & 3))) & 0xffu;
+}
+
+/* 4 * (byte k of the eight packed codes): the LDS byte offset of a float table entry, in one
+ * sub-dword-addressed shift (v_lshlrev_b32 with an SDWA byte select) instead of an extract and a
+ * shift.  k must be a compile-time constant after unrolling. */
+__device__ __forceinline__ uint32_t code_offset(const u32x2 w, int k) {
+    const uint32_t d = k < 4 ? w.x : w.y;
+    const uint32_t two = 2u;
+    uint32_t r;
+    switch (k & 3) {
+    case 0:
+        asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_0" : "=v"(r) : "v"(two), "v"(d));
+        break;
+    case 1:
+        asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_1" : "=v"(r) : "v"(two), "v"(d));
+        break;
+    case 2:
+        asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_2" : "=v"(r) : "v"(two), "v"(d));
+        break;
+    default:
+        asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_3" : "=v"(r) : "v"(two), "v"(d));
+        break;
+    }
+    return r;
+}
+__device__ __forceinline__ float lds_float_at(const float *table, uint32_t byte_offset) {
+    return *reinterpret_cast<const float *>(reinterpret_cast<const char *>(table) + byte_offset);
+}
+
+// ------------------------------------------------------------------------------------------
+// a full 2048-element block, one wavefront
+// ------------------------------------------------------------------------------------------
+
+/*
+ * acc.byte[k] = lo + (xs > mid): the compare, the add and the insertion into the packed word of four
+ * codes in two instructions -- a carry-in add whose SDWA destination select writes one byte and
+ * preserves the others.  Every block opens with the compare, so two byte writes into the same
+ * register are never adjacent (the sub-dword write needs one instruction before its result is
+ * read); the last byte is followed by an s_nop before the store consumes the word.
+ * k must be a compile-time constant after unrolling.
+ */
+__device__ __forceinline__ void pack_code(uint32_t &acc, int k, float xs, float mid, uint32_t lo) {
+    const uint32_t zero = 0u;
+    switch (k & 3) {
+    case 0:
+        asm("v_cmp_gt_f32 vcc, %1, %2\n\t"
+            "v_addc_co_u32_sdwa %0, vcc, %3, %4, vcc dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:DWORD"
+            : "=v"(acc) : "v"(xs), "v"(mid), "v"(lo), "v"(zero) : "vcc");
+        break;
+    case 1:
+        asm("v_cmp_gt_f32 vcc, %1, %2\n\t"
+            "v_addc_co_u32_sdwa %0, vcc, %3, %4, vcc dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD"
+            : "+v"(acc) : "v"(xs), "v"(mid), "v"(lo), "v"(zero) : "vcc");
+        break;
+    case 2:
+        asm("v_cmp_gt_f32 vcc, %1, %2\n\t"
+            "v_addc_co_u32_sdwa %0, vcc, %3, %4, vcc dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD"
+            : "+v"(acc) : "v"(xs), "v"(mid), "v"(lo), "v"(zero) : "vcc");
+        break;
+    default:
+        asm("v_cmp_gt_f32 vcc, %1, %2\n\t"
+            "v_addc_co_u32_sdwa %0, vcc, %3, %4, vcc dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD\n\t"
+            "s_nop 0"
+            : "+v"(acc) : "v"(xs), "v"(mid), "v"(lo), "v"(zero) : "vcc");
+        break;
+    }
+}
+
+/* Mode BNB: a first-moment code whose map value has the other sign than the moment moves one entry
+ * toward the moment's sign.  The signed map is negative below entry 127, zero at 127 and positive
+ * above, and the quotient has the moment's sign, so the only case is a negative moment that
+ * rounds to the zero entry: it takes entry 126, the negative value nearest zero. */
+__device__ __forceinline__ uint32_t keep_sign(uint32_t code, float m, float absmax) {
+    return (code == 127u && (f2u(m) >> 31) != 0u && absmax != 0.0f) ? 126u : code;
+}
+
+template <bool FAST_DIV, bool KEYTAB, bool KEEP_SIGN = false>
+__device__ __forceinline__ void requant8(const float *mf, const float *vf, const BlockDiv &dm, const BlockDiv &dv,
+                                         const Lds &L, u32x2 &mw, u32x2 &vw) {
+    if (KEYTAB && FAST_DIV && !KEEP_SIGN) { // the hot path: slot lookup, codes packed by byte-select writes
+        uint32_t am[2], av[2];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const float xm = dm.div_fast(mf[k]); // times kKeyScale
+            const float xv = dv.div_fast(vf[k]);
+            const KeySlot sm = *reinterpret_cast<const KeySlot *>(L.key_s + (half_key(xm) & 0xfff0u));
+            const KeySlot sv = *reinterpret_cast<const KeySlot *>(L.key_u + (half_key(xv) & 0x7ff8u));
+            pack_code(am[k >> 2], k, xm, sm.mid, sm.lo);
+            pack_code(av[k >> 2], k, xv, sv.mid, sv.lo);
+        }
+        mw.x = am[0]; mw.y = am[1];
+        vw.x = av[0]; vw.y = av[1];
+        return;
+    }
+    uint32_t cm[8], cv[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const float xm = FAST_DIV ? dm.div_fast(mf[k]) : dm.div_slow(mf[k]); // times dm.scale
+        const float xv = FAST_DIV ? dv.div_fast(vf[k]) : dv.div_slow(vf[k]);
+        cm[k] = KEYTAB ? code_signed_key(xm, L.key_s) : code_bsearch(xm, L.mid_s);
+        if (KEEP_SIGN) cm[k] = keep_sign(cm[k], mf[k], dm.a);
+        cv[k] = KEYTAB ? code_unsigned_key(xv, L.key_u) : code_bsearch(xv, L.mid_u);
+    }
+    mw.x = cm[0] | (cm[1] << 8) | (cm[2] << 16) | (cm[3] << 24);
+    mw.y = cm[4] | (cm[5] << 8) | (cm[6] << 16) | (cm[7] << 24);
+    vw.x = cv[0] | (cv[1] << 8) | (cv[2] << 16) | (cv[3] << 24);
+    vw.y = cv[4] | (cv[5] << 8) | (cv[6] << 16) | (cv[7] << 24);
+}
+
+template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB>
+__device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint32_t lane, const EriAdam8Hyper &h,
+                                           float gscale, const BlockDiv &dbc1, const BlockDiv &dbc2, const Lds &L) {
+    const size_t e0 = (size_t)lb * kBlock;
+    const size_t esz = BF16 ? 2 : 4;
+    char *p = static_cast<char *>(t.p) + e0 * esz;
+    const char *g = static_cast<const char *>(t.g) + e0 * esz;
+    uint8_t *mc = t.m + e0;
+    uint8_t *vc = t.v + e0;
+    const float a_m = as_global(t.absmax_m)[lb];
+    const float a_v = as_global(t.absmax_v)[lb];
+
+    float mf[32], vf[32];
+    float lm = 0.0f, lv = 0.0f;
+    // Issue the loads of DEPTH passes before touching the first value: the wave then waits once per
+    // DEPTH passes, with 48 * DEPTH bytes per lane in flight (bf16; fp32 holds twice the registers).
+    constexpr int DEPTH = BF16 ? 4 : 2;
+#pragma unroll
+    for (int c0 = 0; c0 < 4; c0 += DEPTH) {
+        Raw8<BF16> pr[DEPTH], gr[DEPTH];
+        u32x2 mr[DEPTH], vr[DEPTH];
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const uint32_t o = (c0 + d) * 512 + lane * 8;
+            pr[d].load(p, o);
+            gr[d].load(g, o);
+            mr[d] = __builtin_nontemporal_load(as_global(reinterpret_cast<const u32x2 *>(mc + o)));
+            vr[d] = __builtin_nontemporal_load(as_global(reinterpret_cast<const u32x2 *>(vc + o)));
+        }
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const int c = c0 + d;
+            const uint32_t o = c * 512 + lane * 8;
+            float pv[8], gv[8], pn[8];
+            pr[d].unpack(pv);
+            gr[d].unpack(gv);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const float m_old = L.map_s[byte_of(mr[d], k)] * a_m;
+                const float v_old = L.map_u[byte_of(vr[d], k)] * a_v;
+                float m, v;
+                adam_elem<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], m_old, v_old, h, gscale, dbc1, dbc2, m, v, pn[k]);
+                mf[c * 8 + k] = m;
+                vf[c * 8 + k] = v;
+                lm = fmaxf(lm, __builtin_fabsf(m));
+                lv = fmaxf(lv, __builtin_fabsf(v));
+            }
+            store8<BF16>(p, o, pn);
+        }
+    }
+    float nam = lm, nav = lv;
+    wave_max2(nam, nav);
+    if (lane == 0) {
+        as_global(t.absmax_m)[lb] = nam;
+        as_global(t.absmax_v)[lb] = nav;
+    }
+    constexpr float ks = KEYTAB ? kKeyScale : 1.0f, ksi = KEYTAB ? kKeyScaleInv : 1.0f;
+    const BlockDiv dm(nam, ks, ksi), dv(nav, ks, ksi);
+    if (dm.fast && dv.fast) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t o = c * 512 + lane * 8;
+            u32x2 mw, vw;
+            requant8<true, KEYTAB, MODE == ERI_ADAM8_MODE_BNB>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
+            __builtin_nontemporal_store(mw, as_global(reinterpret_cast<u32x2 *>(mc + o)));
+            __builtin_nontemporal_store(vw, as_global(reinterpret_cast<u32x2 *>(vc + o)));
+        }
+    } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t o = c * 512 + lane * 8;
+            u32x2 mw, vw;
+            requant8<false, KEYTAB, MODE == ERI_ADAM8_MODE_BNB>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
+            __builtin_nontemporal_store(mw, as_global(reinterpret_cast<u32x2 *>(mc + o)));
+            __builtin_nontemporal_store(vw, as_global(reinterpret_cast<u32x2 *>(vc + o)));
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// the last, partial block of a tensor: element-wise, bounds-checked, moments recomputed in the
+// second sweep instead of being held (n < 2048 elements, once per tensor at most)
+// ------------------------------------------------------------------------------------------
+
+template <bool BF16>
+__device__ __forceinline__ float load1(const void *base, size_t i) {
+    if (BF16) return u2f((uint32_t)as_global(static_cast<const uint16_t *>(base))[i] << 16);
+    return as_global(static_cast<const float *>(base))[i];
+}
+
+template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB>
+__device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint32_t n, uint32_t lane,
+                                        const EriAdam8Hyper &h, float gscale, const BlockDiv &dbc1,
+                                        const BlockDiv &dbc2, const Lds &L) {
+    const size_t e0 = (size_t)lb * kBlock;
+    ERI_GLOBAL uint8_t *mc = as_global(t.m);
+    ERI_GLOBAL uint8_t *vc = as_global(t.v);
+    const float a_m = as_global(t.absmax_m)[lb];
+    const float a_v = as_global(t.absmax_v)[lb];
+    float lm = 0.0f, lv = 0.0f;
+    for (uint32_t i = lane; i < n; i += kWave) {
+        const size_t e = e0 + i;
+        float m, v, pn;
+        adam_elem<MODE, EXACT, BF16, WD, GS>(load1<BF16>(t.p, e), load1<BF16>(t.g, e), L.map_s[mc[e]] * a_m,
+                                             L.map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn);
+        lm = fmaxf(lm, __builtin_fabsf(m));
+        lv = fmaxf(lv, __builtin_fabsf(v));
+    }
+    float nam = lm, nav = lv;
+    wave_max2(nam, nav);
+    constexpr float ks = KEYTAB ? kKeyScale : 1.0f, ksi = KEYTAB ? kKeyScaleInv : 1.0f;
+    const BlockDiv dm(nam, ks, ksi), dv(nav, ks, ksi);
+    for (uint32_t i = lane; i < n; i += kWave) {
+        const size_t e = e0 + i;
+        float m, v, pn;
+        adam_elem<MODE, EXACT, BF16, WD, GS>(load1<BF16>(t.p, e), load1<BF16>(t.g, e), L.map_s[mc[e]] * a_m,
+                                             L.map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn);
+        const float xm = dm.div_slow(m);
+        const float xv = dv.div_slow(v);
+        uint32_t cm = KEYTAB ? code_signed_key(xm, L.key_s) : code_bsearch(xm, L.mid_s);
+        if (MODE == ERI_ADAM8_MODE_BNB) cm = keep_sign(cm, m, nam);
+        mc[e] = (uint8_t)cm;
+        vc[e] = (uint8_t)(KEYTAB ? code_unsigned_key(xv, L.key_u) : code_bsearch(xv, L.mid_u));
+        if (BF16) as_global(static_cast<uint16_t *>(t.p))[e] = (uint16_t)bf16_bits(pn);
+        else as_global(static_cast<float *>(t.p))[e] = pn;
+    }
+    if (lane == 0) {
+        as_global(t.absmax_m)[lb] = nam;
+        as_global(t.absmax_v)[lb] = nav;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// the step kernel
+// ------------------------------------------------------------------------------------------
+
+/* The table image, staged once per workgroup.  A static array: its LDS address is a compile-time
+ * constant, so table offsets fold into the ds_read immediates. */
+#define ERI_LDS_IMAGE __shared__ uint4 lds_raw[kLdsImageBytes / 16]
+
+/* Row owning full block `blk`: the last row whose full_start is <= blk (rows without full blocks
+ * share their successor's full_start and are skipped by taking the last).  All wave-uniform. */
+__device__ __forceinline__ uint32_t find_row(const DevTensor *rows, uint32_t n_rows, uint32_t from, uint32_t blk) {
+    uint32_t lo = from, hi = n_rows; // rows[lo].full_start <= blk
+    while (hi - lo > 1) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (rows[mid].full_start <= blk) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
+/* The full blocks one wave walks.  Workgroup i of a launch runs on accelerator die (XCD) i mod 8.  The
+ * block list is cut into `chunks` contiguous ranges and workgroup i walks range i mod chunks, so with
+ * chunks == 8 each die sweeps its own part of every buffer instead of all dies advancing through one
+ * common window; on MI355X that made the sweep both a little faster and much less dependent on where
+ * the buffers happen to lie physically.  chunks == 1 is the plain grid-stride walk. */
+struct BlockWalk {
+    uint32_t first, end, stride;
+    __device__ __forceinline__ BlockWalk(uint32_t total_blocks, uint32_t chunks) {
+        const uint32_t waves_per_wg = blockDim.x / kWave;
+        const uint32_t per_chunk = (total_blocks + chunks - 1) / chunks;
+        const uint32_t lo = (blockIdx.x % chunks) * per_chunk;
+        end = lo + per_chunk < total_blocks ? lo + per_chunk : total_blocks;
+        stride = (gridDim.x / chunks) * waves_per_wg;
+        first = __builtin_amdgcn_readfirstlane(lo + (blockIdx.x / chunks) * waves_per_wg + threadIdx.x / kWave);
+    }
+};
+
+
+} // namespace eri
+#endif /* ERI_ADAM8_INLINE_H */

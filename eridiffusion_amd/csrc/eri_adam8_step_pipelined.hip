@@ -1,0 +1,231 @@
+/* The software-pipelined step kernel for bf16 tensors: the benchmark kernel. */
+#include "eri_adam8_inline.h"
+
+namespace eri {
+
+// ------------------------------------------------------------------------------------------
+// software-pipelined step kernel for bf16 tensors
+//
+// Same arithmetic as adam8_step_kernel, but a wave issues the loads of its NEXT block after the
+// update half of the current block (when the raw words of the current block are dead) and before
+// the requantisation half, so it always has 48 bytes per lane in flight while it computes.  The
+// registers of the raw words are the ones just freed, so the pipeline costs no copies; it needs
+// 48 (raw) + 64 (moments) + temporaries at its peak, hence three waves per SIMD (768 threads).
+// ------------------------------------------------------------------------------------------
+
+struct RawBlock {
+    u32x4 p[4], g[4];
+    u32x2 m[4], v[4];
+    float a_m, a_v;
+    __device__ __forceinline__ void issue(const DevTensor &t, uint32_t lb, uint32_t lane) {
+        const size_t e0 = (size_t)lb * kBlock;
+        ERI_GLOBAL const u32x4 *pp = as_global(reinterpret_cast<const u32x4 *>(static_cast<const uint16_t *>(t.p) + e0));
+        ERI_GLOBAL const u32x4 *gp = as_global(reinterpret_cast<const u32x4 *>(static_cast<const uint16_t *>(t.g) + e0));
+        ERI_GLOBAL const u32x2 *mp = as_global(reinterpret_cast<const u32x2 *>(t.m + e0));
+        ERI_GLOBAL const u32x2 *vp = as_global(reinterpret_cast<const u32x2 *>(t.v + e0));
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            p[c] = __builtin_nontemporal_load(&pp[c * 64 + lane]); // each byte is touched once per step
+            g[c] = __builtin_nontemporal_load(&gp[c * 64 + lane]);
+            m[c] = __builtin_nontemporal_load(&mp[c * 64 + lane]);
+            v[c] = __builtin_nontemporal_load(&vp[c * 64 + lane]);
+        }
+        a_m = as_global(t.absmax_m)[lb];
+        a_v = as_global(t.absmax_v)[lb];
+    }
+};
+
+template <int MODE, bool EXACT, bool WD, bool GS, int V = 0>
+__global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTensor *__restrict__ rows,
+                                                                   uint32_t n_rows, uint32_t total_blocks,
+                                                                   EriAdam8Hyper h,
+                                                                   const uint4 *__restrict__ lds_image,
+                                                                   const float *__restrict__ dev_scale,
+                                                                   uint32_t chunks) {
+    ERI_LDS_IMAGE;
+    // clip factor left on the device by the gradient-norm pass (1.0 when there is none)
+    const float tscale = (GS && dev_scale) ? *dev_scale : 1.0f;
+    for (uint32_t i = threadIdx.x; i < kLdsImageBytes / 16; i += blockDim.x) lds_raw[i] = lds_image[i];
+    __syncthreads();
+    const char *base = reinterpret_cast<const char *>(lds_raw);
+    Lds L;
+    L.map_s = reinterpret_cast<const float *>(base + kOffMapS);
+    L.map_u = reinterpret_cast<const float *>(base + kOffMapU);
+    L.mid_s = reinterpret_cast<const float *>(base + kOffMidS);
+    L.mid_u = reinterpret_cast<const float *>(base + kOffMidU);
+    L.key_s = base + kOffKeyS;
+    L.key_u = base + kOffKeyU;
+
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t waves_per_wg = blockDim.x / kWave;
+    const uint32_t stride = gridDim.x * waves_per_wg;
+    const BlockDiv dbc1(h.bc1), dbc2(h.bc2);
+
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
+    // partial last blocks first: one per row at most, handed out from the last wave backwards -- the
+    // waves at the end of each range are the ones that get one full block fewer when the blocks do not
+    // divide evenly, so the slower element-wise tail lands where there is slack
+    for (uint32_t r = stride - 1 - wave; r < n_rows; r += stride) {
+        const DevTensor t = rows[r];
+        const uint32_t n = (uint32_t)(t.numel % kBlock);
+        if (n != 0) {
+            const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
+            tail_block<true, MODE, EXACT, WD, GS, true>(t, (uint32_t)(t.numel / kBlock), n, lane, h, gscale, dbc1, dbc2, L);
+        }
+    }
+    const BlockWalk walk(total_blocks, chunks);
+    uint32_t blk = walk.first;
+    if (blk >= walk.end) return;
+
+    uint32_t ti = find_row(rows, n_rows, 0, blk);
+    DevTensor t = rows[ti];
+    RawBlock raw;
+    raw.issue(t, blk - t.full_start, lane);
+    while (true) {
+        // the block after this one; past the end the wave re-reads its last block (the loads must
+        // stay unconditional so that the raw registers have a single definition in the loop)
+        const uint32_t nblk = blk + walk.stride;
+        const bool more = nblk < walk.end;
+        const uint32_t pblk = more ? nblk : blk;
+        const uint32_t nti = find_row(rows, n_rows, ti, pblk);
+        const DevTensor nt = rows[nti];
+
+        const uint32_t lb = blk - t.full_start;
+        const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
+        const size_t e0 = (size_t)lb * kBlock;
+        char *p = static_cast<char *>(t.p) + e0 * 2;
+        uint8_t *mc = t.m + e0;
+        uint8_t *vc = t.v + e0;
+        float mf[32], vf[32];
+        u32x4 pw[4]; // updated parameters, packed, stored after the next block's loads are out
+        float lm = 0.0f, lv = 0.0f;
+        const float a_m = raw.a_m, a_v = raw.a_v;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            Raw8<true> pr, gr;
+            pr.w = raw.p[c];
+            gr.w = raw.g[c];
+            float pv[8], gv[8], pn[8];
+            pr.unpack(pv);
+            gr.unpack(gv);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const float m_old = lds_float_at(L.map_s, code_offset(raw.m[c], k)) * a_m;
+                const float v_old = lds_float_at(L.map_u, code_offset(raw.v[c], k)) * a_v;
+                float m, v;
+                adam_elem<MODE, EXACT, true, WD, GS>(pv[k], gv[k], m_old, v_old, h, gscale, dbc1, dbc2, m, v, pn[k]);
+                mf[c * 8 + k] = m;
+                vf[c * 8 + k] = v;
+                lm = fmaxf(lm, __builtin_fabsf(m));
+                lv = fmaxf(lv, __builtin_fabsf(v));
+            }
+            pw[c].x = bf16_pair(pn[0], pn[1]);
+            pw[c].y = bf16_pair(pn[2], pn[3]);
+            pw[c].z = bf16_pair(pn[4], pn[5]);
+            pw[c].w = bf16_pair(pn[6], pn[7]);
+            if (V == 1) __builtin_nontemporal_store(pw[c], as_global(reinterpret_cast<u32x4 *>(p) + c * 64 + lane));
+        }
+        float nam = lm, nav = lv;
+        wave_max2(nam, nav);
+        if (lane == 0) {
+            as_global(t.absmax_m)[lb] = nam;
+            as_global(t.absmax_v)[lb] = nav;
+        }
+        raw.issue(nt, pblk - nt.full_start, lane); // prefetch: in flight during the requantisation
+        if (V == 0 || V == 3) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                __builtin_nontemporal_store(pw[c], as_global(reinterpret_cast<u32x4 *>(p) + c * 64 + lane));
+        }
+        const BlockDiv dm(nam, kKeyScale, kKeyScaleInv), dv(nav, kKeyScale, kKeyScaleInv);
+        if (dm.fast && dv.fast) {
+            u32x2 mws[4], vws[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint32_t o = c * 512 + lane * 8;
+                requant8<true, true>(mf + c * 8, vf + c * 8, dm, dv, L, mws[c], vws[c]);
+                if (V != 3) {
+                    __builtin_nontemporal_store(mws[c], as_global(reinterpret_cast<u32x2 *>(mc + o)));
+                    __builtin_nontemporal_store(vws[c], as_global(reinterpret_cast<u32x2 *>(vc + o)));
+                }
+            }
+            if (V == 3) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const uint32_t o = c * 512 + lane * 8;
+                    __builtin_nontemporal_store(mws[c], as_global(reinterpret_cast<u32x2 *>(mc + o)));
+                    __builtin_nontemporal_store(vws[c], as_global(reinterpret_cast<u32x2 *>(vc + o)));
+                }
+            }
+            if (V == 2) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    __builtin_nontemporal_store(pw[c], as_global(reinterpret_cast<u32x4 *>(p) + c * 64 + lane));
+            }
+        } else {
+            if (V == 2) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    __builtin_nontemporal_store(pw[c], as_global(reinterpret_cast<u32x4 *>(p) + c * 64 + lane));
+            }
+            for (int c = 0; c < 4; ++c) {
+                const uint32_t o = c * 512 + lane * 8;
+                u32x2 mw, vw;
+                requant8<false, true>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
+                __builtin_nontemporal_store(mw, as_global(reinterpret_cast<u32x2 *>(mc + o)));
+                __builtin_nontemporal_store(vw, as_global(reinterpret_cast<u32x2 *>(vc + o)));
+            }
+        }
+        if (!more) break;
+        blk = nblk;
+        ti = nti;
+        t = nt;
+    }
+}
+
+int g_pipelined_waves = 0; // measurement switch: waves per workgroup of the pipelined kernel (0 = 12)
+int g_kernel_variant = 0;  // A/B switch for measurements (eri_adam8_set_tuning); 0 is the shipped schedule
+
+namespace {
+
+template <int MODE, bool EXACT, bool WD, bool GS>
+int launch_pipelined(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
+                     const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg, hipStream_t s) {
+    auto k = adam8_step_pipelined_kernel<MODE, EXACT, WD, GS>;
+    if (MODE == ERI_ADAM8_MODE_ERI && !EXACT && WD && !GS) { // the benchmark configuration carries the variants
+        if (g_kernel_variant == 1) k = adam8_step_pipelined_kernel<MODE, EXACT, WD, GS, 1>;
+        if (g_kernel_variant == 2) k = adam8_step_pipelined_kernel<MODE, EXACT, WD, GS, 2>;
+        if (g_kernel_variant == 3) k = adam8_step_pipelined_kernel<MODE, EXACT, WD, GS, 3>;
+    }
+    if (wg > 768) wg = 768;
+    if (g_pipelined_waves >= 1 && g_pipelined_waves <= 12) wg = (uint32_t)g_pipelined_waves * kWave;
+    hipLaunchKernelGGL(k, dim3(grid), dim3(wg), 0, s, rows, n_rows, total_blocks, h,
+                       static_cast<const uint4 *>(lds_image), dev_scale, chunks_for(grid));
+    return (int)hipGetLastError();
+}
+
+template <int MODE, bool EXACT>
+int launch_flags(bool wd, bool gs, const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
+                 const void *img, const float *dev_scale, uint32_t grid, uint32_t wg, hipStream_t s) {
+    if (wd) {
+        if (gs) return launch_pipelined<MODE, EXACT, true, true>(rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s);
+        return launch_pipelined<MODE, EXACT, true, false>(rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s);
+    }
+    if (gs) return launch_pipelined<MODE, EXACT, false, true>(rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s);
+    return launch_pipelined<MODE, EXACT, false, false>(rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s);
+}
+
+} // namespace
+
+int launch_step_pipelined(int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
+                          uint32_t total_blocks, const EriAdam8Hyper &h, const void *img, const float *dev_scale,
+                          uint32_t grid, uint32_t wg, void *stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+#define ERI_ARGS wd, gs, rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s
+    if (mode == ERI_ADAM8_MODE_L2)
+        return exact ? launch_flags<ERI_ADAM8_MODE_L2, true>(ERI_ARGS) : launch_flags<ERI_ADAM8_MODE_L2, false>(ERI_ARGS);
+    return exact ? launch_flags<ERI_ADAM8_MODE_ERI, true>(ERI_ARGS) : launch_flags<ERI_ADAM8_MODE_ERI, false>(ERI_ARGS);
+#undef ERI_ARGS
+}
+
+} // namespace eri

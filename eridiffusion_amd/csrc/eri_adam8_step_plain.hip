@@ -1,0 +1,119 @@
+/*
+ * The plain step kernel (no cross-block prefetch): fp32 tensors, and bf16 tensors in mode BNB, with
+ * ERI_ADAM8_FLAG_BSEARCH or with ERI_ADAM8_FLAG_NO_PIPELINE.  Compiled twice, once per parameter dtype
+ * (-DERI_PLAIN_BF16=0|1), so that the two halves build in parallel.
+ */
+#include "eri_adam8_inline.h"
+
+#ifndef ERI_PLAIN_BF16
+#error "compile with -DERI_PLAIN_BF16=0 or 1"
+#endif
+
+namespace eri {
+
+template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB>
+__global__ __launch_bounds__(1024) void adam8_step_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
+                                                          uint32_t total_blocks, EriAdam8Hyper h,
+                                                          const uint4 *__restrict__ lds_image,
+                                                          const float *__restrict__ dev_scale, uint32_t chunks) {
+    ERI_LDS_IMAGE;
+    // clip factor left on the device by the gradient-norm pass (1.0 when there is none)
+    const float tscale = (GS && dev_scale) ? *dev_scale : 1.0f;
+    // the binary search needs the maps and midpoints only (4 KB); the slot tables are the other 96 KB
+    constexpr uint32_t staged = KEYTAB ? kLdsImageBytes : kOffKeyU;
+    for (uint32_t i = threadIdx.x; i < staged / 16; i += blockDim.x) lds_raw[i] = lds_image[i];
+    __syncthreads();
+    const char *base = reinterpret_cast<const char *>(lds_raw);
+    Lds L;
+    L.map_s = reinterpret_cast<const float *>(base + kOffMapS);
+    L.map_u = reinterpret_cast<const float *>(base + kOffMapU);
+    L.mid_s = reinterpret_cast<const float *>(base + kOffMidS);
+    L.mid_u = reinterpret_cast<const float *>(base + kOffMidU);
+    L.key_s = base + kOffKeyS;
+    L.key_u = base + kOffKeyU;
+
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t waves_per_wg = blockDim.x / kWave;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
+    const uint32_t stride = gridDim.x * waves_per_wg;
+    const BlockDiv dbc1(h.bc1), dbc2(h.bc2);
+
+    // partial last blocks first: one per row at most, handed out from the last wave backwards -- the
+    // waves at the end of each range are the ones that get one full block fewer when the blocks do not
+    // divide evenly, so the slower element-wise tail lands where there is slack
+    for (uint32_t r = stride - 1 - wave; r < n_rows; r += stride) {
+        const DevTensor t = rows[r];
+        const uint32_t n = (uint32_t)(t.numel % kBlock);
+        if (n != 0) {
+            const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
+            tail_block<BF16, MODE, EXACT, WD, GS, KEYTAB>(t, (uint32_t)(t.numel / kBlock), n, lane, h, gscale, dbc1, dbc2, L);
+        }
+    }
+    uint32_t ti = 0; // rows[ti].full_start <= blk; blk only grows, so the search restarts from ti
+    const BlockWalk walk(total_blocks, chunks);
+    for (uint32_t blk = walk.first; blk < walk.end; blk += walk.stride) {
+        ti = find_row(rows, n_rows, ti, blk);
+        const DevTensor t = rows[ti];
+        const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
+        full_block<BF16, MODE, EXACT, WD, GS, KEYTAB>(t, blk - t.full_start, lane, h, gscale, dbc1, dbc2, L);
+    }
+}
+
+namespace {
+
+constexpr bool kBf16 = ERI_PLAIN_BF16 != 0;
+
+template <int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB>
+int launch_one(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
+               const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg, hipStream_t s) {
+    auto k = adam8_step_kernel<kBf16, MODE, EXACT, WD, GS, KEYTAB>;
+    hipLaunchKernelGGL(k, dim3(grid), dim3(wg), 0, s, rows, n_rows, total_blocks, h,
+                       static_cast<const uint4 *>(lds_image), dev_scale, chunks_for(grid));
+    return (int)hipGetLastError();
+}
+
+/* BSEARCH selects the cross-check variants (binary search of the midpoint table); mode BNB has none. */
+template <int MODE, bool EXACT, bool BSEARCH>
+int launch_flags(bool wd, bool gs, bool keytab, const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks,
+                 const EriAdam8Hyper &h, const void *img, const float *dev_scale, uint32_t grid, uint32_t wg, hipStream_t s) {
+#define ERI_GO(W, G, K) return launch_one<MODE, EXACT, W, G, K>(rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s)
+    if (BSEARCH && !keytab) {
+        if (wd) { if (gs) ERI_GO(true, true, !BSEARCH); ERI_GO(true, false, !BSEARCH); }
+        if (gs) ERI_GO(false, true, !BSEARCH);
+        ERI_GO(false, false, !BSEARCH);
+    }
+    if (wd) { if (gs) ERI_GO(true, true, true); ERI_GO(true, false, true); }
+    if (gs) ERI_GO(false, true, true);
+    ERI_GO(false, false, true);
+#undef ERI_GO
+}
+
+} // namespace
+
+#if ERI_PLAIN_BF16
+int launch_step_plain_bf16(int mode, bool exact, bool wd, bool gs, bool keytab, const DevTensor *rows, uint32_t n_rows,
+                           uint32_t total_blocks, const EriAdam8Hyper &h, const void *img, const float *dev_scale,
+                           uint32_t grid, uint32_t wg, void *stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+#define ERI_ARGS wd, gs, keytab, rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s
+    if (mode == ERI_ADAM8_MODE_BNB) return launch_flags<ERI_ADAM8_MODE_BNB, true, false>(ERI_ARGS);
+    if (mode == ERI_ADAM8_MODE_L2)
+        return exact ? launch_flags<ERI_ADAM8_MODE_L2, true, true>(ERI_ARGS) : launch_flags<ERI_ADAM8_MODE_L2, false, true>(ERI_ARGS);
+    return exact ? launch_flags<ERI_ADAM8_MODE_ERI, true, true>(ERI_ARGS) : launch_flags<ERI_ADAM8_MODE_ERI, false, true>(ERI_ARGS);
+#undef ERI_ARGS
+}
+#else
+/* fp32 parameters always take the IEEE square root and division. */
+int launch_step_plain_f32(int mode, bool wd, bool gs, bool keytab, const DevTensor *rows, uint32_t n_rows,
+                          uint32_t total_blocks, const EriAdam8Hyper &h, const void *img, const float *dev_scale,
+                          uint32_t grid, uint32_t wg, void *stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+#define ERI_ARGS wd, gs, keytab, rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s
+    if (mode == ERI_ADAM8_MODE_BNB) return launch_flags<ERI_ADAM8_MODE_BNB, true, false>(ERI_ARGS);
+    if (mode == ERI_ADAM8_MODE_L2) return launch_flags<ERI_ADAM8_MODE_L2, true, true>(ERI_ARGS);
+    return launch_flags<ERI_ADAM8_MODE_ERI, true, true>(ERI_ARGS);
+#undef ERI_ARGS
+}
+#endif
+
+} // namespace eri

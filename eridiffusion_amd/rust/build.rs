@@ -28,13 +28,21 @@ fn main() {
         "-packed-fp32-ops".into(),
     ];
     let mut objects = Vec::new();
-    for (file, is_hip) in [
-        ("eri_adam8_kernels.hip", true),
-        ("eri_optim8_api.cpp", true),
-        ("eri_adam8bit_host.cpp", false),
+    // (source, object name, extra define, compiled as HIP?) -- the plain step kernel is built once per
+    // parameter dtype
+    for (file, obj_name, define, is_hip) in [
+        ("eri_adam8_kernels.hip", "kernels", "", true),
+        ("eri_adam8_step_pipelined.hip", "step_pipelined", "", true),
+        ("eri_adam8_step_plain.hip", "step_plain_bf16", "-DERI_PLAIN_BF16=1", true),
+        ("eri_adam8_step_plain.hip", "step_plain_f32", "-DERI_PLAIN_BF16=0", true),
+        ("eri_optim8_api.cpp", "api", "", true),
+        ("eri_adam8bit_host.cpp", "host", "", false),
     ] {
-        let obj = out.join(format!("{file}.o"));
+        let obj = out.join(format!("{obj_name}.o"));
         let mut cmd = Command::new(&hipcc);
+        if !define.is_empty() {
+            cmd.arg(define);
+        }
         if is_hip {
             cmd.args(&device_flags).args(["-x", "hip"]);
         } else {
@@ -54,7 +62,7 @@ fn main() {
     println!("cargo:rustc-link-search=native=/opt/rocm/lib");
     println!("cargo:rustc-link-lib=dylib=amdhip64");
     println!("cargo:rustc-link-lib=dylib=stdc++");
-    for h in ["eri_adam8_device.h", "eri_dynamic_maps.inc"] {
+    for h in ["eri_adam8_device.h", "eri_adam8_inline.h", "eri_dynamic_maps.inc"] {
         println!("cargo:rerun-if-changed=csrc/{h}");
     }
 }
