@@ -70,11 +70,12 @@ static_assert(kLdsImageBytes % 16 == 0, "the image is staged in 16-byte words");
  * hipError_t as int.  `lds_image` is the device copy of the kLdsImageBytes table image. */
 int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_blocks, int dtype_tag,
                 const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg,
-                void *stream);
+                uint32_t compute_units, void *stream);
 extern int g_kernel_variant;
 extern int g_chunks;
 extern int g_pipelined_waves;
 extern int g_norm_waves;
+extern int g_split_blocks_per_cu;
 
 /* The chunked walk (BlockWalk) needs the same number of workgroups in every chunk. */
 inline uint32_t chunks_for(uint32_t grid) {
@@ -90,6 +91,10 @@ int launch_step_plain_f32(int mode, bool wd, bool gs, bool keytab, const DevTens
 int launch_step_plain_bf16(int mode, bool exact, bool wd, bool gs, bool keytab, const DevTensor *rows, uint32_t n_rows,
                            uint32_t total_blocks, const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale,
                            uint32_t grid, uint32_t wg, void *stream);
+/* Four waves per block, for tables of few blocks; `grid` workgroups of 1024 threads. */
+int launch_step_split(bool bf16, int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
+                      uint32_t total_blocks, const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale,
+                      uint32_t grid, void *stream);
 int launch_step_pipelined(int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
                           uint32_t total_blocks, const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale,
                           uint32_t grid, uint32_t wg, void *stream);

@@ -9,12 +9,28 @@ namespace eri {
 
 int g_norm_waves = 4; // waves per workgroup of the gradient-norm pass (eri_adam8_set_tuning key 4)
 int g_chunks = 8;     // contiguous ranges of the block list (BlockWalk); 8 = one per accelerator die
+int g_split_blocks_per_cu = 4; // tables of at most this many full blocks per compute unit take the four-waves-per-block kernel
 
 int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, int dtype_tag,
                 const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg,
-                void *stream) {
+                uint32_t compute_units, void *stream) {
     const bool bf16 = dtype_tag != ERI_DTYPE_F32;
     const bool gs = (h.flags & ERI_ADAM8_FLAG_GRAD_SCALE) != 0;
+    // Few blocks: one wave per block would leave the chip idle, four waves share each block instead.
+    // The two flags that name a kernel (cross-check and A/B) keep their meaning.
+    const bool kernel_named = (h.flags & (ERI_ADAM8_FLAG_BSEARCH | ERI_ADAM8_FLAG_NO_PIPELINE)) != 0;
+    if (!kernel_named && g_split_blocks_per_cu > 0 &&
+        (uint64_t)total_blocks <= (uint64_t)compute_units * (uint64_t)g_split_blocks_per_cu) {
+        const bool bnb = h.mode == ERI_ADAM8_MODE_BNB;
+        const bool wd_s = bnb ? h.weight_decay != 1.0f : h.weight_decay > 0.0f;
+        const bool exact_s = bnb || !bf16 || (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0;
+        uint32_t need = (total_blocks + 3) / 4;
+        const uint32_t for_tails = (n_rows + 15) / 16;
+        if (need < for_tails) need = for_tails;
+        if (need > compute_units) need = compute_units;
+        if (need == 0) need = 1;
+        return launch_step_split(bf16, h.mode, exact_s, wd_s, gs, rows, n_rows, total_blocks, h, lds_image, dev_scale, need, stream);
+    }
     if (h.mode == ERI_ADAM8_MODE_BNB) { // plain kernel, slot table, IEEE arithmetic; the decay is a factor
         const bool wd = h.weight_decay != 1.0f;
         if (bf16) return launch_step_plain_bf16(h.mode, true, wd, gs, true, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);

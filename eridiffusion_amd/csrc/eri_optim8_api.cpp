@@ -493,6 +493,11 @@ int eri_hip_mem_info(size_t *free_bytes, size_t *total_bytes) {
 static int g_grid_override = 0; // measurement switch: persistent workgroups of the step (0 = one per slot)
 
 int eri_adam8_set_tuning(int key, int value) {
+    if (key == 5) {
+        if (value < 0 || value > (1 << 20)) return fail(ERI_ERR_ARG, "blocks per compute unit out of range");
+        eri::g_split_blocks_per_cu = value;
+        return 0;
+    }
     if (key == 4) {
         if (value != 1 && value != 2 && value != 4 && value != 8 && value != 16) return fail(ERI_ERR_ARG, "waves per workgroup must be 1, 2, 4, 8 or 16");
         eri::g_norm_waves = value;
@@ -697,7 +702,7 @@ int eri_adam8_step_table(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream)
                 if (!g.unit_scales) return fail(ERI_ERR_ARG, "ERI_ADAM8_FLAG_CLIP_FROM_TABLE needs per-tensor grad_scale = 1 unless ERI_ADAM8_FLAG_GRAD_SCALE is set");
             }
         }
-        rc = eri::launch_step(g.dev, g.n, g.total_blocks, g.dtype, hh, ctx->image, dev_scale, grid, waves_per_wg * eri::kWave, stream);
+        rc = eri::launch_step(g.dev, g.n, g.total_blocks, g.dtype, hh, ctx->image, dev_scale, grid, waves_per_wg * eri::kWave, ctx->cus, stream);
         if (rc) return hip_fail((hipError_t)rc, "adam8 step launch");
     }
     return 0;

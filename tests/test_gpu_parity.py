@@ -19,6 +19,17 @@ pytestmark = pytest.mark.gpu
 LR, B1, B2, EPS, WD = 1e-4, 0.9, 0.999, 1e-8, 0.01
 
 
+@pytest.fixture(autouse=True, params=["split-kernel-for-small-tables", "one-wave-per-block-kernels"])
+def which_kernels(request):
+    """The tables of these tests are small, so by default they all run on the four-waves-per-block kernel.
+    Every test therefore runs twice: as shipped, and with that kernel switched off, which sends bf16 tables
+    to the pipelined kernel and fp32 tables to the plain one."""
+    L = _lib()
+    L.check(L.lib().eri_adam8_set_tuning(5, 4 if request.param.startswith("split") else 0), "set_tuning")
+    yield request.param
+    L.check(L.lib().eri_adam8_set_tuning(5, 4), "set_tuning")
+
+
 def _lib():
     from eridiffusion_amd import _lib
     return _lib
