@@ -9,7 +9,7 @@ namespace eri {
 
 int g_norm_waves = 4; // waves per workgroup of the gradient-norm pass (eri_adam8_set_tuning key 4)
 int g_chunks = 8;     // contiguous ranges of the block list (BlockWalk); 8 = one per accelerator die
-int g_split_blocks_per_cu = 4; // tables of at most this many full blocks per compute unit take the four-waves-per-block kernel
+int g_split_blocks_per_cu = 64; // tables of at most this many full blocks per compute unit take the four-waves-per-block kernel
 
 int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, int dtype_tag,
                 const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg,

@@ -25,9 +25,9 @@ def which_kernels(request):
     Every test therefore runs twice: as shipped, and with that kernel switched off, which sends bf16 tables
     to the pipelined kernel and fp32 tables to the plain one."""
     L = _lib()
-    L.check(L.lib().eri_adam8_set_tuning(5, 4 if request.param.startswith("split") else 0), "set_tuning")
+    L.check(L.lib().eri_adam8_set_tuning(5, 64 if request.param.startswith("split") else 0), "set_tuning")
     yield request.param
-    L.check(L.lib().eri_adam8_set_tuning(5, 4), "set_tuning")
+    L.check(L.lib().eri_adam8_set_tuning(5, 64), "set_tuning")
 
 
 def _lib():
