@@ -61,7 +61,12 @@ void eri_set_last_error(const char *message);
 int eri_hip_device_count(int *count);
 int eri_hip_set_device(int device);
 int eri_hip_get_device(int *device);
-int eri_hip_malloc_zeroed(int device, size_t bytes, void **out); /* 256-byte aligned, zero-filled */
+/* 256-byte aligned, zero-filled.  Allocations of 64 MB and more are allocated, released and allocated
+ * again before they are handed out: on MI355X the first physical placement a large request receives
+ * sustains visibly less bandwidth than the one it receives after the range went back to the driver.
+ * Environment: ERI_HIP_MALLOC_RECYCLE=0 switches that off; ERI_HIP_MALLOC_CONTIGUOUS=1 asks the driver
+ * for physically contiguous memory for such allocations (falls back silently; measurement aid). */
+int eri_hip_malloc_zeroed(int device, size_t bytes, void **out);
 int eri_hip_free(void *ptr);
 void *eri_hip_host_alloc(size_t bytes);                          /* pinned; NULL on failure */
 int eri_hip_host_free(void *ptr);
