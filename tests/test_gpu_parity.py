@@ -90,6 +90,25 @@ def run_case(sizes, bf16, seed, steps=3, mode=0, flags=0, wd=WD, p_std=0.02, g_s
     return stats
 
 
+@pytest.mark.parametrize("name", ["eri_f32", "eri_bf16", "l2_f32", "l2_bf16", "bnb_f32", "bnb_bf16", "eri_bf16_gs"])
+def test_committed_step_vectors(name):
+    """tests/golden/step_vectors.npz: three steps from a zero state, bit for bit (bf16 with the exact flag)."""
+    import os
+    vec = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "step_vectors.npz"))
+    mode = {"eri": 0, "l2": 1, "bnb": 2}[name.split("_")[0]]
+    bf16 = "bf16" in name
+    gs = 0.37 if name.endswith("_gs") else None
+    p0 = vec[name + ".p0"].copy()
+    gt = hs.GpuTensors([p0], [vec[name + ".g0"].copy()], hs.oracle_states([p0.size]), bf16)
+    gpu_steps(gt, [None, [vec[name + ".g1"]], [vec[name + ".g2"]]], 1, mode, flags=2, grad_scale=gs)
+    got_p, got_st = gt.fetch()
+    raw = np.uint16 if bf16 else np.uint32
+    assert np.array_equal(got_p[0].view(raw), vec[name + ".p"].view(raw))
+    assert np.array_equal(got_st[0][0], vec[name + ".m"]) and np.array_equal(got_st[0][1], vec[name + ".v"])
+    assert np.array_equal(got_st[0][2].view(np.uint32), vec[name + ".absmax_m"].view(np.uint32))
+    assert np.array_equal(got_st[0][3].view(np.uint32), vec[name + ".absmax_v"].view(np.uint32))
+
+
 def test_config1_flat_fp32_after_ten_prior_steps():
     # benchmark configuration 1: 2**20 fp32 params ~N(0, 0.02), grads ~N(0, 1e-3), states from ten
     # prior steps, block 2048, lr 1e-4, betas (0.9, 0.999), eps 1e-8, wd 0.01; one step
