@@ -100,9 +100,11 @@ enum {
     ERI_ADAM8_FLAG_EXACT_PARAM = 1u << 1, /* IEEE sqrt and divide on the parameter update of BF16
                                              tensors too (F32 tensors always use them) */
     ERI_ADAM8_FLAG_BSEARCH = 1u << 2,     /* requantise by binary search of the LDS midpoint table
-                                             instead of the float-keyed slot table (same codes) */
-    ERI_ADAM8_FLAG_NO_PIPELINE = 1u << 3, /* BF16: use the plain kernel, not the one that prefetches
-                                             the next block (same results; for A/B measurements) */
+                                             instead of the float-keyed slot table (same codes; runs on
+                                             the plain one-wave-per-block kernel whatever the table size) */
+    ERI_ADAM8_FLAG_NO_PIPELINE = 1u << 3, /* use the plain one-wave-per-block kernel: not the one that
+                                             prefetches the next block (BF16), not the four-waves-per-
+                                             block one (small tables).  Same results; for A/B measurements */
     ERI_ADAM8_FLAG_CLIP_FROM_TABLE = 1u << 4 /* also multiply gradients by the clip factor the last
                                              eri_adam8_grad_norm left in the table (device memory) */
 };
