@@ -505,6 +505,68 @@ __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint
     const float a_m = as_global(t.absmax_m)[lb];
     const float a_v = as_global(t.absmax_v)[lb];
     float lm = 0.0f, lv = 0.0f;
+    constexpr float ks = KEYTAB ? kKeyScale : 1.0f, ksi = KEYTAB ? kKeyScaleInv : 1.0f;
+    if ((n & 7u) == 0) {
+        // The usual case (tensor sizes are multiples of eight): the same 8-elements-per-lane accesses as a
+        // full block, lanes past the end switched off.  Two sweeps, the second recomputing the moments,
+        // so that nothing but one pass of values is held -- this code is inlined into kernels whose
+        // register budget belongs to their main loop.
+        const size_t esz = BF16 ? 2 : 4;
+        char *p = static_cast<char *>(t.p) + e0 * esz;
+        const char *g = static_cast<const char *>(t.g) + e0 * esz;
+        const uint32_t passes = (n + 511) / 512;
+        for (uint32_t c = 0; c < passes; ++c) {
+            const uint32_t o = c * 512 + lane * 8;
+            if (o < n) {
+                Raw8<BF16> pr, gr;
+                pr.load(p, o);
+                gr.load(g, o);
+                const u32x2 mr = *as_global(reinterpret_cast<const u32x2 *>(t.m + e0 + o));
+                const u32x2 vr = *as_global(reinterpret_cast<const u32x2 *>(t.v + e0 + o));
+                float pv[8], gv[8];
+                pr.unpack(pv);
+                gr.unpack(gv);
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    float m, v, pn;
+                    adam_elem<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], L.map_s[byte_of(mr, k)] * a_m,
+                                                         L.map_u[byte_of(vr, k)] * a_v, h, gscale, dbc1, dbc2, m, v, pn);
+                    lm = fmaxf(lm, __builtin_fabsf(m));
+                    lv = fmaxf(lv, __builtin_fabsf(v));
+                }
+            }
+        }
+        float nam = lm, nav = lv;
+        wave_max2(nam, nav);
+        const BlockDiv dm(nam, ks, ksi), dv(nav, ks, ksi);
+        for (uint32_t c = 0; c < passes; ++c) {
+            const uint32_t o = c * 512 + lane * 8;
+            if (o < n) {
+                Raw8<BF16> pr, gr;
+                pr.load(p, o);
+                gr.load(g, o);
+                const u32x2 mr = *as_global(reinterpret_cast<const u32x2 *>(t.m + e0 + o));
+                const u32x2 vr = *as_global(reinterpret_cast<const u32x2 *>(t.v + e0 + o));
+                float pv[8], gv[8], pn[8], m[8], v[8];
+                pr.unpack(pv);
+                gr.unpack(gv);
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    adam_elem<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], L.map_s[byte_of(mr, k)] * a_m,
+                                                         L.map_u[byte_of(vr, k)] * a_v, h, gscale, dbc1, dbc2, m[k], v[k], pn[k]);
+                u32x2 mw, vw;
+                requant8<false, KEYTAB, MODE == ERI_ADAM8_MODE_BNB>(m, v, dm, dv, L, mw, vw);
+                *as_global(reinterpret_cast<u32x2 *>(t.m + e0 + o)) = mw;
+                *as_global(reinterpret_cast<u32x2 *>(t.v + e0 + o)) = vw;
+                store8<BF16>(p, o, pn);
+            }
+        }
+        if (lane == 0) {
+            as_global(t.absmax_m)[lb] = nam;
+            as_global(t.absmax_v)[lb] = nav;
+        }
+        return;
+    }
     for (uint32_t i = lane; i < n; i += kWave) {
         const size_t e = e0 + i;
         float m, v, pn;
@@ -515,7 +577,6 @@ __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint
     }
     float nam = lm, nav = lv;
     wave_max2(nam, nav);
-    constexpr float ks = KEYTAB ? kKeyScale : 1.0f, ksi = KEYTAB ? kKeyScaleInv : 1.0f;
     const BlockDiv dm(nam, ks, ksi), dv(nav, ks, ksi);
     for (uint32_t i = lane; i < n; i += kWave) {
         const size_t e = e0 + i;

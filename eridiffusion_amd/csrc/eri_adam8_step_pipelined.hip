@@ -192,7 +192,7 @@ template <int MODE, bool EXACT, bool WD, bool GS>
 int launch_pipelined(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
                      const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg, hipStream_t s) {
     auto k = adam8_step_pipelined_kernel<MODE, EXACT, WD, GS>;
-    if (MODE == ERI_ADAM8_MODE_ERI && !EXACT && WD && !GS) { // the benchmark configuration carries the variants
+    if constexpr (MODE == ERI_ADAM8_MODE_ERI && !EXACT && WD && !GS) { // only the benchmark configuration carries the variants
         if (g_kernel_variant == 1) k = adam8_step_pipelined_kernel<MODE, EXACT, WD, GS, 1>;
         if (g_kernel_variant == 2) k = adam8_step_pipelined_kernel<MODE, EXACT, WD, GS, 2>;
         if (g_kernel_variant == 3) k = adam8_step_pipelined_kernel<MODE, EXACT, WD, GS, 3>;
