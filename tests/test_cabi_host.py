@@ -176,3 +176,31 @@ def test_package_refuses_to_work_without_the_library(monkeypatch):
     monkeypatch.setattr(L, "LIB_PATH", os.path.join(ROOT, "eridiffusion_amd", "no_such_library.so"))
     with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
         L.lib()
+
+
+def test_headers_compile_as_c_and_cpp_and_agree_on_struct_sizes(tmp_path):
+    """The two headers are the boundary: they must be valid C11 and C++17 on their own, and the struct sizes a
+    C compiler sees must be the ones the ctypes table (and the Rust #[repr(C)] block) assume."""
+    import subprocess
+    inc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
+    src = tmp_path / "check.c"
+    src.write_text('''
+#include "eri_optim8.h"
+#include "eri_adam8bit.h"
+#include <stdio.h>
+int main(void) {
+    printf("%zu %zu %zu %zu %zu %zu %zu\\n", sizeof(EriAdam8Hyper), sizeof(EriAdam8Tensor), sizeof(EriAdamW32Tensor),
+           sizeof(EriAdamW32Hyper), sizeof(EriEmaTensor), sizeof(EriAdam8bitConfig), sizeof(EriOptimizerMemoryReport));
+    return 0;
+}
+''')
+    exe = tmp_path / "check"
+    subprocess.check_call(["gcc", "-std=c11", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", inc, str(src), "-o", str(exe)])
+    got = [int(x) for x in subprocess.check_output([str(exe)]).split()]
+    want = [C.sizeof(L.Hyper), C.sizeof(L.TensorRow), C.sizeof(L.AdamW32Row), C.sizeof(L.AdamW32Hyper), C.sizeof(L.EmaRow),
+            C.sizeof(L.Adam8bitConfigC), C.sizeof(L.MemoryReportC)]
+    assert got == want, (got, want)
+    cpp = tmp_path / "check.cpp"
+    cpp.write_text('#include "eri_optim8.h"\n#include "eri_adam8bit.h"\nint main() { return sizeof(EriAdam8Hyper) == 48 ? 0 : 1; }\n')
+    subprocess.check_call(["g++", "-std=c++17", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", inc, str(cpp), "-o", str(tmp_path / "checkpp")])
+    assert subprocess.call([str(tmp_path / "checkpp")]) == 0
