@@ -1,0 +1,21 @@
+"""Runs tests/cabi_parity, the parity check written in plain C against include/eri_optim8.h: device steps
+through the C ABI against the CPU oracle, bit for bit, with no Python or torch in the process."""
+import os
+import subprocess
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("mode", ["eri", "l2", "bnb"])
+def test_c_program_matches_the_oracle(dtype, mode):
+    exe = os.path.join(HERE, "cabi_parity")
+    if not os.path.exists(exe):  # normally built beforehand by __graft_entry__.build()
+        subprocess.check_call(["make", "-C", HERE, "cabi_parity"])
+    out = subprocess.run([exe, dtype, mode], capture_output=True, text=True, timeout=120)
+    print(out.stdout, out.stderr, flush=True)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert out.stdout.count("bit-exact") == 5 and out.stdout.strip().endswith("ok")
