@@ -608,13 +608,27 @@ __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint
 
 /* Row owning full block `blk`: the last row whose full_start is <= blk (rows without full blocks
  * share their successor's full_start and are skipped by taking the last).  All wave-uniform. */
-__device__ __forceinline__ uint32_t find_row(const DevTensor *rows, uint32_t n_rows, uint32_t from, uint32_t blk) {
+template <typename Row>
+__device__ __forceinline__ uint32_t find_row(const Row *rows, uint32_t n_rows, uint32_t from, uint32_t blk) {
     uint32_t lo = from, hi = n_rows; // rows[lo].full_start <= blk
     while (hi - lo > 1) {
         const uint32_t mid = (lo + hi) >> 1;
         if (rows[mid].full_start <= blk) lo = mid; else hi = mid;
     }
     return lo;
+}
+
+/* A wave's blocks only grow and a tensor usually spans many of them, so the owning row is searched for
+ * again only when a block leaves the range [t.full_start, t_end) of the row at hand (t_end = 0 forces
+ * the first search).  Saves the ten dependent scalar loads of the search on almost every block. */
+template <typename Row>
+__device__ __forceinline__ void seek_row(const Row *rows, uint32_t n_rows, uint32_t blk, uint32_t &ti, Row &t,
+                                         uint32_t &t_end) {
+    if (blk >= t_end) {
+        ti = find_row(rows, n_rows, ti, blk);
+        t = rows[ti];
+        t_end = t.full_start + (uint32_t)(t.numel / kBlock);
+    }
 }
 
 /* The full blocks one wave walks.  Workgroup i of a launch runs on accelerator die (XCD) i mod 8.  The

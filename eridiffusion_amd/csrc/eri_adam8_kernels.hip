@@ -177,10 +177,11 @@ __global__ __launch_bounds__(1024) void grad_sumsq_kernel(const DevTensor *__res
     // full blocks, one load ahead: the next block's four words are in flight while this one is reduced
     const BlockWalk walk(total_blocks, chunks);
     if (walk.first < walk.end) {
-        uint32_t ti = find_row(rows, n_rows, 0, walk.first);
+        uint32_t ti = 0, t_end = 0;
+        DevTensor t;
         Raw8<BF16> raw[4];
         {
-            const DevTensor t = rows[ti];
+            seek_row(rows, n_rows, walk.first, ti, t, t_end);
             const size_t e0 = (size_t)(walk.first - t.full_start) * kBlock;
 #pragma unroll
             for (int c = 0; c < 4; ++c) raw[c].load(static_cast<const char *>(t.g) + e0 * (BF16 ? 2 : 4), c * 512 + lane * 8);
@@ -191,8 +192,7 @@ __global__ __launch_bounds__(1024) void grad_sumsq_kernel(const DevTensor *__res
             for (int c = 0; c < 4; ++c) cur[c] = raw[c];
             const uint32_t nblk = blk + walk.stride;
             if (nblk < walk.end) {
-                ti = find_row(rows, n_rows, ti, nblk);
-                const DevTensor t = rows[ti];
+                seek_row(rows, n_rows, nblk, ti, t, t_end);
                 const size_t e0 = (size_t)(nblk - t.full_start) * kBlock;
 #pragma unroll
                 for (int c = 0; c < 4; ++c) raw[c].load(static_cast<const char *>(t.g) + e0 * (BF16 ? 2 : 4), c * 512 + lane * 8);
@@ -383,15 +383,6 @@ int launch_quant_error(const DevTensor *rows, uint32_t n_rows, uint32_t total_bl
 // AdamW bf16 22 B/param (read 2+2+4+4, write 2+4+4), fp32 28 B/param; EMA 3 x element size.
 // ------------------------------------------------------------------------------------------
 
-__device__ __forceinline__ uint32_t find_elem_row(const ElemRow *rows, uint32_t n_rows, uint32_t from, uint32_t blk) {
-    uint32_t lo = from, hi = n_rows;
-    while (hi - lo > 1) {
-        const uint32_t mid = (lo + hi) >> 1;
-        if (rows[mid].full_start <= blk) lo = mid; else hi = mid;
-    }
-    return lo;
-}
-
 /* crates/common/optim/src/adamw.rs:34-54, one rounded operation per line */
 __device__ __forceinline__ void adamw32_elem(float p, float g, float &m, float &v, const EriAdamW32Hyper &h, float omb1,
                                              float omb2, float neg_lr, float &pn) {
@@ -481,11 +472,11 @@ __global__ __launch_bounds__(256) void adamw32_kernel(const ElemRow *__restrict_
             store1<BF16>(t.a, e0 + i, pn);
         }
     }
-    uint32_t ti = 0;
+    uint32_t ti = 0, t_end = 0;
+    ElemRow t;
     const BlockWalk walk(total_blocks, chunks);
     for (uint32_t blk = walk.first; blk < walk.end; blk += walk.stride) {
-        ti = find_elem_row(rows, n_rows, ti, blk);
-        const ElemRow t = rows[ti];
+        seek_row(rows, n_rows, blk, ti, t, t_end);
         const size_t e0 = (size_t)(blk - t.full_start) * kBlock;
         if (t.e) adamw32_block<BF16, true>(t, e0, lane, h, omb1, omb2, neg_lr);
         else adamw32_block<BF16, false>(t, e0, lane, h, omb1, omb2, neg_lr);
@@ -514,11 +505,11 @@ __global__ __launch_bounds__(256) void ema_kernel(const ElemRow *__restrict__ ro
         for (uint32_t i = lane; i < n; i += kWave)
             store1<BF16>(t.a, e0 + i, ema_elem(load1<BF16>(t.a, e0 + i), load1<BF16>(t.b, e0 + i), decay, omd));
     }
-    uint32_t ti = 0;
+    uint32_t ti = 0, t_end = 0;
+    ElemRow t;
     const BlockWalk walk(total_blocks, chunks);
     for (uint32_t blk = walk.first; blk < walk.end; blk += walk.stride) {
-        ti = find_elem_row(rows, n_rows, ti, blk);
-        const ElemRow t = rows[ti];
+        seek_row(rows, n_rows, blk, ti, t, t_end);
         const size_t e0 = (size_t)(blk - t.full_start) * kBlock;
         char *s = static_cast<char *>(t.a) + e0 * (BF16 ? 2 : 4);
         const char *p = static_cast<const char *>(t.b) + e0 * (BF16 ? 2 : 4);

@@ -77,8 +77,11 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
     uint32_t blk = walk.first;
     if (blk >= walk.end) return;
 
-    uint32_t ti = find_row(rows, n_rows, 0, blk);
-    DevTensor t = rows[ti];
+    uint32_t ti = 0, t_end = 0;
+    DevTensor t;
+    seek_row(rows, n_rows, blk, ti, t, t_end);
+    uint32_t nti = ti, nt_end = t_end;
+    DevTensor nt = t;
     RawBlock raw;
     raw.issue(t, blk - t.full_start, lane);
     while (true) {
@@ -87,8 +90,7 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
         const uint32_t nblk = blk + walk.stride;
         const bool more = nblk < walk.end;
         const uint32_t pblk = more ? nblk : blk;
-        const uint32_t nti = find_row(rows, n_rows, ti, pblk);
-        const DevTensor nt = rows[nti];
+        seek_row(rows, n_rows, pblk, nti, nt, nt_end);
 
         const uint32_t lb = blk - t.full_start;
         const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
@@ -178,7 +180,6 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
         }
         if (!more) break;
         blk = nblk;
-        ti = nti;
         t = nt;
     }
 }

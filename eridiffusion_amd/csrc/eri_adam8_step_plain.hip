@@ -49,11 +49,11 @@ __global__ __launch_bounds__(1024) void adam8_step_kernel(const DevTensor *__res
             tail_block<BF16, MODE, EXACT, WD, GS, KEYTAB>(t, (uint32_t)(t.numel / kBlock), n, lane, h, gscale, dbc1, dbc2, L);
         }
     }
-    uint32_t ti = 0; // rows[ti].full_start <= blk; blk only grows, so the search restarts from ti
+    uint32_t ti = 0, t_end = 0;
+    DevTensor t;
     const BlockWalk walk(total_blocks, chunks);
     for (uint32_t blk = walk.first; blk < walk.end; blk += walk.stride) {
-        ti = find_row(rows, n_rows, ti, blk);
-        const DevTensor t = rows[ti];
+        seek_row(rows, n_rows, blk, ti, t, t_end);
         const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
         full_block<BF16, MODE, EXACT, WD, GS, KEYTAB>(t, blk - t.full_start, lane, h, gscale, dbc1, dbc2, L);
     }

@@ -38,13 +38,12 @@ __global__ __launch_bounds__(1024) void adam8_step_split_kernel(const DevTensor 
         u32x2 mr, vr;
         float a_m, a_v;
     } q;
-    uint32_t ti = 0;
+    uint32_t ti = 0, t_end = 0;
     auto request = [&](uint32_t first) {
         const uint32_t blk = first + team;
         q.active = blk < total_blocks;
         if (!q.active) return;
-        ti = find_row(rows, n_rows, ti, blk);
-        q.t = rows[ti];
+        seek_row(rows, n_rows, blk, ti, q.t, t_end);
         q.lb = blk - q.t.full_start;
         const size_t e0 = (size_t)q.lb * kBlock;
         const size_t esz = BF16 ? 2 : 4;
