@@ -84,7 +84,7 @@ struct StEntry {
 struct StFile {
     std::map<std::string, std::string> metadata;
     std::map<std::string, StEntry> tensors;
-    std::vector<char> data;
+    uint64_t data_start = 0; // file offset of the byte that data_offsets count from
 };
 
 struct JsonCursor {
@@ -119,12 +119,20 @@ struct JsonCursor {
     }
 };
 
-bool parse_safetensors(const std::vector<char> &raw, StFile &out, std::string &why) {
-    if (raw.size() < 8) { why = "file shorter than its header length"; return false; }
+/* Reads and checks the header of an open safetensors file; tensor bytes stay in the file. */
+bool parse_safetensors(std::ifstream &f, StFile &out, std::string &why) {
+    f.seekg(0, std::ios::end);
+    const std::streamoff end_pos = f.tellg();
+    f.seekg(0, std::ios::beg);
+    if (!f || end_pos < 8) { why = "file shorter than its header length"; return false; }
+    const uint64_t size = (uint64_t)end_pos;
     uint64_t hlen = 0;
-    std::memcpy(&hlen, raw.data(), 8);
-    if (hlen > raw.size() - 8) { why = "header length exceeds the file"; return false; }
-    JsonCursor c{raw.data() + 8, raw.data() + 8 + hlen};
+    f.read(reinterpret_cast<char *>(&hlen), 8);
+    if (!f || hlen > size - 8) { why = "header length exceeds the file"; return false; }
+    std::vector<char> raw((size_t)hlen);
+    f.read(raw.data(), (std::streamsize)hlen);
+    if (!f) { why = "header cannot be read"; return false; }
+    JsonCursor c{raw.data(), raw.data() + hlen};
     if (!c.eat('{')) { why = "header is not a JSON object"; return false; }
     bool first = true;
     while (c.ok && !c.peek('}')) {
@@ -162,20 +170,20 @@ bool parse_safetensors(const std::vector<char> &raw, StFile &out, std::string &w
         if (key != "__metadata__") out.tensors[key] = ent;
     }
     if (!c.ok || !c.eat('}')) { why = "malformed header"; return false; }
-    out.data.assign(raw.begin() + 8 + (std::ptrdiff_t)hlen, raw.end());
+    out.data_start = 8 + hlen;
     for (auto &kv : out.tensors)
-        if (kv.second.end < kv.second.begin || kv.second.end > out.data.size()) {
+        if (kv.second.end < kv.second.begin || kv.second.end > size - out.data_start) {
             why = "tensor '" + kv.first + "' points outside the file";
             return false;
         }
     return true;
 }
 
+/* The header is complete before any tensor byte exists: sizes alone fix the offsets, so the caller
+ * can stream the tensors behind it in the order it added them. */
 struct StWriter {
     std::ostringstream header;
-    std::vector<std::pair<const void *, uint64_t>> chunks; // host pointers
     uint64_t offset = 0;
-    bool first = true;
     void begin(const std::map<std::string, std::string> &meta) {
         header << "{\"__metadata__\":{";
         bool f = true;
@@ -185,25 +193,83 @@ struct StWriter {
         }
         header << "}";
     }
-    void add(const std::string &name, const char *dtype, uint64_t count, const void *host, uint64_t bytes) {
+    void add(const std::string &name, const char *dtype, uint64_t count, uint64_t bytes) {
         header << ",\"" << name << "\":{\"dtype\":\"" << dtype << "\",\"shape\":[" << count << "],\"data_offsets\":["
                << offset << "," << offset + bytes << "]}";
-        chunks.emplace_back(host, bytes);
         offset += bytes;
     }
-    bool write(const std::string &path) {
+    bool write_header(std::ofstream &f) {
         header << "}";
         std::string h = header.str();
         while (h.size() % 8) h.push_back(' ');
-        std::ofstream f(path, std::ios::binary | std::ios::trunc);
-        if (!f) return false;
         const uint64_t hl = h.size();
         f.write(reinterpret_cast<const char *>(&hl), 8);
         f.write(h.data(), (std::streamsize)h.size());
-        for (auto &c : chunks) f.write(static_cast<const char *>(c.first), (std::streamsize)c.second);
         return (bool)f;
     }
 };
+
+/* Pinned host memory in two halves, through which state moves between the device and a file in
+ * bounded pieces: one half is in a device copy while the other is read or written. */
+struct Bounce {
+    static constexpr uint64_t kHalf = (uint64_t)32 << 20;
+    char *host = nullptr;
+    int which = 0;
+    int ensure() {
+        if (host) return 0;
+        host = static_cast<char *>(eri_hip_host_alloc(2 * kHalf));
+        return host ? 0 : ERI_ERR_INTERNAL; // the allocator has set the message
+    }
+    char *next() { which ^= 1; return host + which * kHalf; }
+    ~Bounce() { if (host) eri_hip_host_free(host); }
+};
+
+/* device -> file.  The copy of piece i+1 is queued before piece i is written. */
+int stream_out(std::ofstream &f, const void *dev, uint64_t bytes, Bounce &b, void *stream) {
+    const char *src = static_cast<const char *>(dev);
+    char *cur = nullptr;
+    uint64_t cur_n = 0;
+    for (uint64_t done = 0; done < bytes || cur;) {
+        char *nxt = nullptr;
+        uint64_t nxt_n = 0;
+        if (done < bytes) {
+            nxt = b.next();
+            nxt_n = bytes - done < Bounce::kHalf ? bytes - done : Bounce::kHalf;
+            int rc = eri_hip_memcpy_async(nxt, src + done, nxt_n, 2, stream);
+            if (rc) return rc;
+            done += nxt_n;
+        }
+        if (cur) {
+            f.write(cur, (std::streamsize)cur_n);
+            if (!f) return fail(ERI_ERR_ARG, "InvalidOperation: Failed to save optimizer: write failed");
+        }
+        if (nxt) {
+            int rc = eri_hip_stream_sync(stream);
+            if (rc) return rc;
+        }
+        cur = nxt;
+        cur_n = nxt_n;
+    }
+    return 0;
+}
+
+/* file -> device.  Piece i+1 is read from the file while piece i is in its copy. */
+int stream_in(std::ifstream &f, uint64_t file_offset, void *dev, uint64_t bytes, Bounce &b, void *stream) {
+    f.seekg((std::streamoff)file_offset, std::ios::beg);
+    char *dst = static_cast<char *>(dev);
+    for (uint64_t done = 0; done < bytes;) {
+        char *buf = b.next();
+        const uint64_t n = bytes - done < Bounce::kHalf ? bytes - done : Bounce::kHalf;
+        f.read(buf, (std::streamsize)n);
+        if (!f) return fail(ERI_ERR_ARG, "InvalidOperation: Failed to read optimizer: file ends inside a tensor");
+        int rc = eri_hip_stream_sync(stream); // the other half's copy; this half's was waited for a round ago
+        if (rc) return rc;
+        rc = eri_hip_memcpy_async(dst + done, buf, n, 1, stream);
+        if (rc) return rc;
+        done += n;
+    }
+    return eri_hip_stream_sync(stream);
+}
 
 } // namespace
 
@@ -240,11 +306,22 @@ struct EriAdam8bit {
     std::vector<EriAdam8Tensor> table_rows;  // rows as last uploaded
 };
 
+/* One named state of the functional flavour with its own one-row launch table: updates of many
+ * names in turn then cost a pointer comparison each, not a table rebuild. */
+struct FnState : State8 {
+    EriAdam8Table *table = nullptr;
+    EriAdam8Tensor row;
+    FnState() { std::memset(&row, 0, sizeof row); }
+    ~FnState() {
+        if (table) eri_adam8_table_destroy(table);
+    }
+};
+
 struct EriAdam8bitFn {
     double lr = 1e-4, beta1 = 0.9, beta2 = 0.999, eps = 1e-8, wd = 0.01;
     uint64_t step = 0;
     void *stream = nullptr;
-    std::map<std::string, std::unique_ptr<State8>> states;
+    std::map<std::string, std::unique_ptr<FnState>> states;
 };
 
 extern "C" {
@@ -513,8 +590,7 @@ int eri_adam8bit_state_ptrs(const EriAdam8bit *o, uint32_t index, uint8_t **m, u
 
 int eri_adam8bit_save_state(EriAdam8bit *o, const char *path) {
     if (!o || !path) return fail(ERI_ERR_NULL, "optimizer or path is NULL");
-    // stage every state to host memory, then write one safetensors file
-    std::vector<std::vector<char>> host;
+    // header from the sizes alone, then every state streamed behind it through pinned memory
     StWriter w;
     char buf[64];
     std::map<std::string, std::string> meta;
@@ -525,6 +601,26 @@ int eri_adam8bit_save_state(EriAdam8bit *o, const char *path) {
     std::snprintf(buf, sizeof buf, "%.17g", o->lr);
     meta["learning_rate"] = buf;
     w.begin(meta);
+    bool any = false;
+    for (uint32_t i = 0; i < o->states.size(); ++i) {
+        const State8 *s = o->states[i].get();
+        if (!s) continue;
+        any = true;
+        const uint64_t nb = blocks_of(s->numel);
+        const std::string base = "optimizer.param_" + std::to_string(i);
+        w.add(base + ".m", "U8", s->numel, s->numel);
+        w.add(base + ".v", "U8", s->numel, s->numel);
+        w.add(base + ".absmax_m", "F32", nb, nb * 4);
+        w.add(base + ".absmax_v", "F32", nb, nb * 4);
+    }
+    Bounce bounce;
+    if (any) {
+        int rc = bounce.ensure();
+        if (rc) return rc;
+    }
+    std::ofstream f(path, std::ios::binary | std::ios::trunc);
+    if (!f || !w.write_header(f))
+        return fail(ERI_ERR_ARG, std::string("InvalidOperation: Failed to save optimizer: cannot write ") + path);
     for (uint32_t i = 0; i < o->states.size(); ++i) {
         const State8 *s = o->states[i].get();
         if (!s) continue;
@@ -532,26 +628,12 @@ int eri_adam8bit_save_state(EriAdam8bit *o, const char *path) {
         const uint64_t sizes[4] = {s->numel, s->numel, nb * 4, nb * 4};
         const void *src[4] = {s->m, s->v, s->absmax_m, s->absmax_v};
         for (int k = 0; k < 4; ++k) {
-            host.emplace_back(sizes[k]);
-            int rc = eri_hip_memcpy_async(host.back().data(), src[k], sizes[k], 2, o->stream);
+            int rc = stream_out(f, src[k], sizes[k], bounce, o->stream);
             if (rc) return rc;
         }
     }
-    int rc = eri_hip_stream_sync(o->stream);
-    if (rc) return rc;
-    size_t h = 0;
-    for (uint32_t i = 0; i < o->states.size(); ++i) {
-        const State8 *s = o->states[i].get();
-        if (!s) continue;
-        const uint64_t nb = blocks_of(s->numel);
-        const std::string base = "optimizer.param_" + std::to_string(i);
-        w.add(base + ".m", "U8", s->numel, host[h].data(), s->numel);
-        w.add(base + ".v", "U8", s->numel, host[h + 1].data(), s->numel);
-        w.add(base + ".absmax_m", "F32", nb, host[h + 2].data(), nb * 4);
-        w.add(base + ".absmax_v", "F32", nb, host[h + 3].data(), nb * 4);
-        h += 4;
-    }
-    if (!w.write(path)) return fail(ERI_ERR_ARG, std::string("InvalidOperation: Failed to save optimizer: cannot write ") + path);
+    f.flush();
+    if (!f) return fail(ERI_ERR_ARG, std::string("InvalidOperation: Failed to save optimizer: cannot write ") + path);
     return 0;
 }
 
@@ -559,10 +641,9 @@ int eri_adam8bit_load_state(EriAdam8bit *o, const char *path) {
     if (!o || !path) return fail(ERI_ERR_NULL, "optimizer or path is NULL");
     std::ifstream f(path, std::ios::binary);
     if (!f) return fail(ERI_ERR_ARG, std::string("InvalidOperation: Failed to read optimizer: cannot open ") + path);
-    std::vector<char> raw((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
     StFile st;
     std::string why;
-    if (!parse_safetensors(raw, st, why))
+    if (!parse_safetensors(f, st, why))
         return fail(ERI_ERR_ARG, "InvalidOperation: Failed to deserialize optimizer: " + why);
     if (!st.metadata.count("step") || !st.metadata.count("learning_rate"))
         return fail(ERI_ERR_ARG, "InvalidOperation: Failed to deserialize optimizer: step / learning_rate missing");
@@ -585,20 +666,24 @@ int eri_adam8bit_load_state(EriAdam8bit *o, const char *path) {
                 return fail(ERI_ERR_ARG, "InvalidOperation: Failed to deserialize optimizer: size or dtype mismatch for " + base);
         items.push_back({i, {e[0], e[1], e[2], e[3]}});
     }
+    // the new states are complete before the first one replaces an old one: a failure half way
+    // through the file leaves the optimizer as it was
+    Bounce bounce;
+    std::vector<std::unique_ptr<State8>> fresh;
     for (auto &it : items) {
-        EriParameter *p = o->params[it.idx];
+        int rc = bounce.ensure();
+        if (rc) return rc;
         std::unique_ptr<State8> s(new State8());
-        int rc = s->allocate(p->numel, o->stream);
+        rc = s->allocate(o->params[it.idx]->numel, o->stream);
         if (rc) return rc;
         void *dst[4] = {s->m, s->v, s->absmax_m, s->absmax_v};
         for (int k = 0; k < 4; ++k) {
-            rc = eri_hip_memcpy_async(dst[k], st.data.data() + it.e[k]->begin, it.e[k]->end - it.e[k]->begin, 1, o->stream);
+            rc = stream_in(f, st.data_start + it.e[k]->begin, dst[k], it.e[k]->end - it.e[k]->begin, bounce, o->stream);
             if (rc) return rc;
         }
-        rc = eri_hip_stream_sync(o->stream); // st.data is pageable and goes out of scope with this call
-        if (rc) return rc;
-        o->states[it.idx] = std::move(s);
+        fresh.push_back(std::move(s));
     }
+    for (size_t k = 0; k < items.size(); ++k) o->states[items[k].idx] = std::move(fresh[k]);
     o->step = std::strtoull(st.metadata["step"].c_str(), nullptr, 10);
     o->lr = std::strtod(st.metadata["learning_rate"].c_str(), nullptr);
     if (o->table) { // state pointers changed
@@ -763,7 +848,7 @@ int eri_adam8bit_fn_update(EriAdam8bitFn *o, const char *name, const void *param
         return fail(ERI_ERR_DTYPE, "Unsupported: 8-bit Adam takes F32 or BF16 parameters");
     auto it = o->states.find(name);
     if (it == o->states.end()) { // adam8bit.rs:126-130
-        std::unique_ptr<State8> s(new State8());
+        std::unique_ptr<FnState> s(new FnState());
         int rc = s->allocate(numel, o->stream);
         if (rc) return rc;
         it = o->states.emplace(name, std::move(s)).first;
@@ -775,7 +860,7 @@ int eri_adam8bit_fn_update(EriAdam8bitFn *o, const char *name, const void *param
         rc = eri_hip_memcpy_async(out, param, numel * (dtype_tag == ERI_DTYPE_F32 ? 4 : 2), 3, o->stream);
         if (rc) return rc;
     }
-    State8 &s = *it->second;
+    FnState &s = *it->second;
     EriAdam8Tensor r;
     std::memset(&r, 0, sizeof r);
     r.p = out;
@@ -793,7 +878,22 @@ int eri_adam8bit_fn_update(EriAdam8bitFn *o, const char *name, const void *param
     rc = eri_adam8_hyper_pack(o->lr, o->beta1, o->beta2, o->eps, o->wd, o->step, ERI_ADAM8_MODE_L2,
                               ERI_ADAM8_FLAG_EXACT_PARAM, &h);
     if (rc) return rc;
-    return eri_adam8_step_multi(&r, 1, &h, o->stream);
+    if (!s.table) {
+        rc = eri_adam8_table_create(&r, 1, o->stream, &s.table);
+        if (rc) return rc;
+        s.row = r;
+    } else if (std::memcmp(&r, &s.row, sizeof r) != 0) { // same size by the check above; new pointers or dtype
+        if (r.dtype_tag != s.row.dtype_tag) {
+            eri_adam8_table_destroy(s.table);
+            s.table = nullptr;
+            rc = eri_adam8_table_create(&r, 1, o->stream, &s.table);
+        } else {
+            rc = eri_adam8_table_update(s.table, &r, 1, o->stream);
+        }
+        if (rc) return rc;
+        s.row = r;
+    }
+    return eri_adam8_step_table(s.table, &h, o->stream);
 }
 
 int eri_adam8bit_fn_step(EriAdam8bitFn *o) {
@@ -840,7 +940,7 @@ int eri_adam8bit_fn_load_state_fp32(EriAdam8bitFn *o, const char *name, const fl
                                     uint64_t numel) {
     if (!o || !name || !m || !v) return fail(ERI_ERR_NULL, "NULL argument");
     if (numel == 0) return fail(ERI_ERR_EMPTY, "InvalidOperation: Empty tensor for quantization");
-    std::unique_ptr<State8> s(new State8());
+    std::unique_ptr<FnState> s(new FnState());
     int rc = s->allocate(numel, o->stream);
     if (rc) return rc;
     rc = eri_adam8_quantize(m, 1, numel, s->m, s->absmax_m, o->stream);

@@ -220,11 +220,32 @@ int get_ctx(DeviceCtx **out) {
         c.wg = (uint32_t)env_u32("ERI_ADAM8_WG", 64, 1024, 1024) & ~63u;
         c.wg_per_cu = (uint32_t)env_u32("ERI_ADAM8_WG_PER_CU", 1, 16, 1);
         eri::g_chunks = env_u32("ERI_ADAM8_CHUNKS", 1, 4096, 8);
-        ERI_HIP(hipMalloc(&c.image, eri::kLdsImageBytes));
-        ERI_HIP(hipMemcpy(c.image, t.image.data(), eri::kLdsImageBytes, hipMemcpyHostToDevice));
+        void *image = nullptr;
+        ERI_HIP(hipMalloc(&image, eri::kLdsImageBytes));
+        const hipError_t e = hipMemcpy(image, t.image.data(), eri::kLdsImageBytes, hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            (void)hipFree(image);
+            return hip_fail(e, "upload of the quantisation tables");
+        }
+        c.image = image;
         c.ready = true;
     }
     *out = &c;
+    return 0;
+}
+
+/* The context of the current device, which must be the one the table was created on: its rows and
+ * the table image are addresses of that device. */
+int get_ctx_on(int table_device, DeviceCtx **out) {
+    int rc = get_ctx(out);
+    if (rc) return rc;
+    if (*out != &g_ctx[table_device]) {
+        int dev = 0;
+        (void)hipGetDevice(&dev);
+        char buf[96];
+        std::snprintf(buf, sizeof buf, "table belongs to device %d, current device is %d", table_device, dev);
+        return fail(ERI_ERR_ARG, buf);
+    }
     return 0;
 }
 
@@ -676,8 +697,16 @@ int eri_adam8_step_table(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream)
     if (h->mode != ERI_ADAM8_MODE_ERI && h->mode != ERI_ADAM8_MODE_L2 && h->mode != ERI_ADAM8_MODE_BNB)
         return fail(ERI_ERR_ARG, "unknown mode");
     DeviceCtx *ctx = nullptr;
-    int rc = get_ctx(&ctx);
+    int rc = get_ctx_on(t->device, &ctx);
     if (rc) return rc;
+    const bool clip = (h->flags & ERI_ADAM8_FLAG_CLIP_FROM_TABLE) != 0;
+    const bool scaled = (h->flags & ERI_ADAM8_FLAG_GRAD_SCALE) != 0;
+    if (clip) { // checked for every group before the first launch: a refused step changes nothing
+        if (!t->norm_out) return fail(ERI_ERR_ARG, "ERI_ADAM8_FLAG_CLIP_FROM_TABLE without a prior eri_adam8_grad_norm");
+        for (auto &g : t->groups)
+            if (g.n && !scaled && !g.unit_scales)
+                return fail(ERI_ERR_ARG, "ERI_ADAM8_FLAG_CLIP_FROM_TABLE needs per-tensor grad_scale = 1 unless ERI_ADAM8_FLAG_GRAD_SCALE is set");
+    }
     for (auto &g : t->groups) {
         if (g.n == 0) continue;
         // One wavefront per block.  A small table gets smaller workgroups so that its blocks still
@@ -693,13 +722,11 @@ int eri_adam8_step_table(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream)
         if (grid == 0) grid = 1;
         EriAdam8Hyper hh = *h;
         const float *dev_scale = nullptr;
-        if (hh.flags & ERI_ADAM8_FLAG_CLIP_FROM_TABLE) {
-            if (!t->norm_out) return fail(ERI_ERR_ARG, "ERI_ADAM8_FLAG_CLIP_FROM_TABLE without a prior eri_adam8_grad_norm");
+        if (clip) {
             dev_scale = t->norm_out + 1;
-            if (!(hh.flags & ERI_ADAM8_FLAG_GRAD_SCALE)) { // the scale path is needed; neutral host-side factors
+            if (!scaled) { // the scale path is needed; neutral host-side factors
                 hh.flags |= ERI_ADAM8_FLAG_GRAD_SCALE;
                 hh.grad_scale = 1.0f;
-                if (!g.unit_scales) return fail(ERI_ERR_ARG, "ERI_ADAM8_FLAG_CLIP_FROM_TABLE needs per-tensor grad_scale = 1 unless ERI_ADAM8_FLAG_GRAD_SCALE is set");
             }
         }
         rc = eri::launch_step(g.dev, g.n, g.total_blocks, g.dtype, hh, ctx->image, dev_scale, grid, waves_per_wg * eri::kWave, ctx->cus, stream);
@@ -711,15 +738,13 @@ int eri_adam8_step_table(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream)
 int eri_adam8_grad_norm(EriAdam8Table *t, float max_norm, float denom_eps, void *stream) {
     if (!t) return fail(ERI_ERR_NULL, "table is NULL");
     DeviceCtx *ctx = nullptr;
-    int rc = get_ctx(&ctx);
+    int rc = get_ctx_on(t->device, &ctx);
     if (rc) return rc;
     const uint32_t wpw = (uint32_t)eri::g_norm_waves;
     const uint32_t grid_cap = ctx->cus * eri::kNormWavesPerCu / wpw; // persistent
-    if (!t->partial) {
-        // two groups at most, and per wave a sum of squares and a count
-        ERI_HIP(hipMalloc((void **)&t->partial, sizeof(double) * 2 * 2 * ctx->cus * eri::kNormWavesPerCu));
-        ERI_HIP(hipMalloc((void **)&t->norm_out, sizeof(float) * 4)); // norm, scale, 64-bit count
-    }
+    // two groups at most, and per wave a sum of squares and a count
+    if (!t->partial) ERI_HIP(hipMalloc((void **)&t->partial, sizeof(double) * 2 * 2 * ctx->cus * eri::kNormWavesPerCu));
+    if (!t->norm_out) ERI_HIP(hipMalloc((void **)&t->norm_out, sizeof(float) * 4)); // norm, scale, 64-bit count
     uint32_t off = 0;
     for (auto &g : t->groups) {
         if (g.n == 0) continue;
@@ -762,7 +787,7 @@ int eri_adam8_quant_error(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream
     if (h->mode != ERI_ADAM8_MODE_ERI && h->mode != ERI_ADAM8_MODE_L2)
         return fail(ERI_ERR_ARG, "the quantisation error pass knows the modes ERI and L2");
     DeviceCtx *ctx = nullptr;
-    int rc = get_ctx(&ctx);
+    int rc = get_ctx_on(t->device, &ctx);
     if (rc) return rc;
     if (!t->qerr) ERI_HIP(hipMalloc((void **)&t->qerr, sizeof(double) * 2 * t->n));
     uint32_t off = 0;
@@ -891,24 +916,39 @@ struct ElemCache {
              const void *extra) {
         int dev = 0;
         ERI_HIP(hipGetDevice(&dev));
+        if (dev != device) { // the thread moved to another device: nothing cached is an address there
+            if (pending) (void)hipEventSynchronize(ev);
+            pending = false;
+            for (auto &g : groups) {
+                if (g.dev) (void)hipFree(g.dev);
+                if (g.pinned) (void)hipHostFree(g.pinned);
+                g.dev = g.pinned = nullptr;
+                g.cap = 0;
+            }
+            if (ev) (void)hipEventDestroy(ev);
+            ev = nullptr;
+            device = dev;
+        }
         if (!ev) ERI_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
         for (int gi = 0; gi < 2; ++gi) {
             Group &g = groups[gi];
             const uint32_t n = (uint32_t)g.rows.size();
             if (n == 0) continue;
-            bool same = dev == device && g.cap >= n && std::memcmp(g.pinned, g.rows.data(), n * sizeof(eri::ElemRow)) == 0;
+            bool same = g.cap >= n && std::memcmp(g.pinned, g.rows.data(), n * sizeof(eri::ElemRow)) == 0;
             if (!same) {
                 if (pending) {
                     ERI_HIP(hipEventSynchronize(ev));
                     pending = false;
                 }
-                if (g.cap < n || dev != device) {
+                if (g.cap < n) {
                     if (g.dev) (void)hipFree(g.dev);
                     if (g.pinned) (void)hipHostFree(g.pinned);
                     g.dev = g.pinned = nullptr;
-                    g.cap = n + n / 2 + 16;
-                    ERI_HIP(hipMalloc((void **)&g.dev, sizeof(eri::ElemRow) * g.cap));
-                    ERI_HIP(hipHostMalloc((void **)&g.pinned, sizeof(eri::ElemRow) * g.cap, hipHostMallocDefault));
+                    g.cap = 0; // stays 0 if an allocation below fails: the next call starts over
+                    const uint32_t cap = n + n / 2 + 16;
+                    ERI_HIP(hipMalloc((void **)&g.dev, sizeof(eri::ElemRow) * cap));
+                    ERI_HIP(hipHostMalloc((void **)&g.pinned, sizeof(eri::ElemRow) * cap, hipHostMallocDefault));
+                    g.cap = cap;
                 }
                 std::memcpy(g.pinned, g.rows.data(), n * sizeof(eri::ElemRow));
                 ERI_HIP(hipMemcpyAsync(g.dev, g.pinned, n * sizeof(eri::ElemRow), hipMemcpyHostToDevice,
@@ -924,7 +964,6 @@ struct ElemCache {
             int rc = launch(g.dev, n, total, gi == 0 ? ERI_DTYPE_F32 : ERI_DTYPE_BF16, grid, stream, extra);
             if (rc) return hip_fail((hipError_t)rc, "element-wise sweep launch");
         }
-        device = dev;
         return 0;
     }
 };

@@ -41,7 +41,7 @@ typedef enum EriStatus {
     ERI_ERR_BLOCK_START = -5, /* block_start is not the running sum of ceil(numel / 2048) */
     ERI_ERR_ARG = -6,         /* any other bad argument (mode, count, size, kind) */
     ERI_ERR_TOO_LARGE = -7,   /* more than 2^31 - 1 blocks in one table */
-    ERI_ERR_INTERNAL = -8     /* the lookup tables failed their self-check */
+    ERI_ERR_INTERNAL = -8     /* the lookup tables failed their self-check, or pinned staging memory is unavailable */
 } EriStatus;
 
 /* Message for the last failing call on this thread ("" if none).  Never NULL. */

@@ -154,6 +154,123 @@ def test_save_and_load_state_round_trip(tmp_path):
     L.lib().eri_adam8bit_destroy(opt2)
 
 
+def test_state_larger_than_the_staging_buffer_round_trips(tmp_path):
+    """The file is written and read in 32 MiB pieces through pinned memory; a 72 Mi-element state takes
+    three pieces per moment, the last one partial, and a second small parameter follows it in the file.
+    The device state is filled with a known byte pattern so that a misplaced piece shows."""
+    import torch
+    from safetensors import safe_open
+    L = _L()
+    big = 72 * (1 << 20) + 12345
+    sizes = [big, 5000]
+    dev = torch.device("cuda:0")
+    p = [torch.zeros(n, dtype=torch.bfloat16, device=dev) for n in sizes]
+    g = [torch.full((n,), 1e-3, dtype=torch.bfloat16, device=dev) for n in sizes]
+    handles = (C.c_void_p * 2)()
+    for i in range(2):
+        h = C.c_void_p()
+        L.check(L.lib().eri_param_create(p[i].data_ptr(), sizes[i], 2, C.byref(h)), "param_create")
+        L.check(L.lib().eri_param_set_grad(h, g[i].data_ptr()), "set_grad")
+        handles[i] = h
+
+    def new_opt():
+        opt = C.c_void_p()
+        L.check(L.lib().eri_adam8bit_new(handles, 2, None, None, C.byref(opt)), "adam8bit_new")
+        return opt
+
+    def state_views(opt, i):
+        ptrs = [C.c_void_p() for _ in range(4)]
+        L.check(L.lib().eri_adam8bit_state_ptrs(opt, i, *[C.byref(q) for q in ptrs]), "state_ptrs")
+        return ptrs
+
+    opt = new_opt()
+    L.check(L.lib().eri_adam8bit_step(opt, None), "step")  # creates the states
+    _sync()
+    want = []
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(99)
+    for i, n in enumerate(sizes):
+        nb = (n + 2047) // 2048
+        ptrs = state_views(opt, i)
+        arrs = []
+        for q, (nbytes, dt) in zip(ptrs, ((n, torch.uint8), (n, torch.uint8), (4 * nb, torch.float32), (4 * nb, torch.float32))):
+            if dt is torch.uint8:
+                src = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device=dev, generator=gen)
+            else:
+                src = torch.rand(nbytes // 4, dtype=torch.float32, device=dev, generator=gen)
+            L.check(L.lib().eri_hip_memcpy_async(q.value, src.data_ptr(), nbytes, 3, None), "fill")
+            arrs.append(src.cpu().numpy())
+        want.append(arrs)
+    _sync()
+    path = str(tmp_path / "big.safetensors")
+    L.check(L.lib().eri_adam8bit_save_state(opt, path.encode()), "save_state")
+    with safe_open(path, framework="np") as f:
+        for i in range(2):
+            base = "optimizer.param_%d" % i
+            for k, name in enumerate((".m", ".v", ".absmax_m", ".absmax_v")):
+                got = f.get_tensor(base + name)
+                assert np.array_equal(got.view(np.uint8), want[i][k].view(np.uint8)), base + name
+    opt2 = new_opt()
+    L.check(L.lib().eri_adam8bit_load_state(opt2, path.encode()), "load_state")
+    assert L.lib().eri_adam8bit_get_step(opt2) == 1
+    for i, n in enumerate(sizes):
+        nb = (n + 2047) // 2048
+        for q, w, nbytes in zip(state_views(opt2, i), want[i], (n, n, 4 * nb, 4 * nb)):
+            back = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            L.check(L.lib().eri_hip_memcpy_async(back.data_ptr(), q.value, nbytes, 3, None), "read")
+            _sync()
+            assert np.array_equal(back.cpu().numpy(), w.view(np.uint8))
+    # a file cut inside the big tensor is refused and leaves the optimizer as it was
+    cut = tmp_path / "cut.safetensors"
+    with open(path, "rb") as f:
+        blob = f.read(40 * (1 << 20))
+    cut.write_bytes(blob)
+    before = [q.value for q in state_views(opt2, 0)]
+    assert L.lib().eri_adam8bit_load_state(opt2, str(cut).encode()) == -6
+    assert [q.value for q in state_views(opt2, 0)] == before
+    L.lib().eri_adam8bit_destroy(opt)
+    L.lib().eri_adam8bit_destroy(opt2)
+    for h in handles:
+        L.lib().eri_param_release(h)
+
+
+def test_functional_updates_of_several_names_in_turn():
+    """Three names of different sizes and dtypes updated in turn for three rounds, each call writing
+    into a fresh output buffer: every name keeps its own launch table, re-pointed when the addresses
+    change."""
+    import torch
+    L = _L()
+    names = [(b"a.lora_down", 2048 * 2 + 9, True), (b"b.lora_up", 700, True), (b"c.bias", 2048 * 5, False)]
+    dev = torch.device("cuda:0")
+    opt = C.c_void_p()
+    L.check(L.lib().eri_adam8bit_fn_with_params(1e-4, B1, B2, EPS, WD, None, C.byref(opt)), "with_params")
+    host = {}
+    for k, (name, n, bf16) in enumerate(names):
+        ps, gs = hs.make_inputs([n], bf16, 300 + k)
+        host[name] = [ps, gs, hs.oracle_states([n]), torch.from_numpy(ps[0].view(np.uint8).copy()).to(dev)]
+    keep = []
+    for rnd in range(3):
+        for name, n, bf16 in names:
+            ps, gs, states, cur = host[name]
+            g_dev = torch.from_numpy(gs[0].view(np.uint8).copy()).to(dev)
+            out = torch.zeros(n * (2 if bf16 else 4), dtype=torch.uint8, device=dev)
+            keep += [g_dev, out, cur]
+            L.check(L.lib().eri_adam8bit_fn_update(opt, name, cur.data_ptr(), g_dev.data_ptr(), n, 2 if bf16 else 0,
+                                                   out.data_ptr()), "fn_update")
+            host[name][3] = out
+            hs.oracle_step(ps, gs, states, (1e-4, B1, B2, EPS, WD, rnd), bf16, mode=oc.MODE_L2)
+        L.check(L.lib().eri_adam8bit_fn_step(opt), "fn_step")
+    _sync()
+    for name, n, bf16 in names:
+        ps, gs, states, cur = host[name]
+        bits = np.uint16 if bf16 else np.uint32
+        assert np.array_equal(cur.cpu().numpy().view(bits), ps[0].view(bits)), name
+    cnt, nbytes = C.c_uint64(), C.c_uint64()
+    L.check(L.lib().eri_adam8bit_fn_memory_stats(opt, C.byref(cnt), C.byref(nbytes)), "memory_stats")
+    assert cnt.value == 3
+    L.lib().eri_adam8bit_fn_destroy(opt)
+
+
 @pytest.mark.parametrize("bf16", [True, False])
 def test_functional_update_returns_a_new_tensor(bf16):
     import torch
