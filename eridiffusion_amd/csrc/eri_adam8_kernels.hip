@@ -16,11 +16,13 @@ int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, i
                 uint32_t compute_units, void *stream) {
     const bool bf16 = dtype_tag != ERI_DTYPE_F32;
     const bool gs = (h.flags & ERI_ADAM8_FLAG_GRAD_SCALE) != 0;
-    // Few blocks: one wave per block would leave the chip idle, four waves share each block instead.
+    // Four waves share each block where that is the faster kernel: few blocks (one wave per block would
+    // leave the chip idle) and fp32 parameters (measured ahead of the one-wave kernel from 64 Ki to
+    // 3 Mi blocks).
     // The two flags that name a kernel (cross-check and A/B) keep their meaning.
     const bool kernel_named = (h.flags & (ERI_ADAM8_FLAG_BSEARCH | ERI_ADAM8_FLAG_NO_PIPELINE)) != 0;
-    if (!kernel_named && g_split_blocks_per_cu > 0 &&
-        (uint64_t)total_blocks <= (uint64_t)compute_units * (uint64_t)g_split_blocks_per_cu) {
+    const bool few = (uint64_t)total_blocks <= (uint64_t)compute_units * (uint64_t)g_split_blocks_per_cu;
+    if (!kernel_named && g_split_blocks_per_cu > 0 && (few || !bf16)) {
         const bool bnb = h.mode == ERI_ADAM8_MODE_BNB;
         const bool wd_s = bnb ? h.weight_decay != 1.0f : h.weight_decay > 0.0f;
         const bool exact_s = bnb || !bf16 || (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0;
@@ -40,8 +42,8 @@ int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, i
     const bool exact = (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0;
     const bool keytab = (h.flags & ERI_ADAM8_FLAG_BSEARCH) == 0;
     if (!bf16) return launch_step_plain_f32(h.mode, wd, gs, keytab, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
-    if (keytab && (h.flags & ERI_ADAM8_FLAG_NO_PIPELINE) == 0)
-        return launch_step_pipelined(h.mode, exact, wd, gs, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
+    if (keytab && h.mode == ERI_ADAM8_MODE_ERI && (h.flags & ERI_ADAM8_FLAG_NO_PIPELINE) == 0)
+        return launch_step_pipelined(exact, wd, gs, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
     return launch_step_plain_bf16(h.mode, exact, wd, gs, keytab, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
 }
 

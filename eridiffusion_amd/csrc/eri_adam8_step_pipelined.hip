@@ -218,13 +218,14 @@ int launch_flags(bool wd, bool gs, const DevTensor *rows, uint32_t n_rows, uint3
 
 } // namespace
 
-int launch_step_pipelined(int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
+/* Mode ERI only.  The coupled-decay mode needs more live values per element than this kernel's
+ * register budget holds (its instantiations spilled 80-232 B per lane) and runs faster on the kernel
+ * without the prefetch; the dispatcher sends it there. */
+int launch_step_pipelined(bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
                           uint32_t total_blocks, const EriAdam8Hyper &h, const void *img, const float *dev_scale,
                           uint32_t grid, uint32_t wg, void *stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define ERI_ARGS wd, gs, rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s
-    if (mode == ERI_ADAM8_MODE_L2)
-        return exact ? launch_flags<ERI_ADAM8_MODE_L2, true>(ERI_ARGS) : launch_flags<ERI_ADAM8_MODE_L2, false>(ERI_ARGS);
     return exact ? launch_flags<ERI_ADAM8_MODE_ERI, true>(ERI_ARGS) : launch_flags<ERI_ADAM8_MODE_ERI, false>(ERI_ARGS);
 #undef ERI_ARGS
 }

@@ -154,7 +154,8 @@ int eri_adam8_init(void);
  * (0 = one per compute unit), key 2 = contiguous ranges the block list is cut into (8 = shipped, one per
  * accelerator die; 1 = plain grid stride), key 3 = waves per workgroup of the bf16 step kernel (0 = 12), key 4 = waves per workgroup of the
  * gradient-norm pass (4 = shipped; set before a table's first norm), key 5 = largest table, in full blocks
- * per compute unit, that takes the four-waves-per-block kernel (64 = shipped, 0 = never). */
+ * per compute unit, that takes the four-waves-per-block kernel (64 = shipped, 0 = never; fp32 tables
+ * take that kernel at every size unless this is 0). */
 int eri_adam8_set_tuning(int key, int value);
 
 /* The two 256-entry maps (code -> value in [-1, 1] / [0, 1]) the states are expressed in. */
