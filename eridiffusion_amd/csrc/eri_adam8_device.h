@@ -95,7 +95,7 @@ int launch_step_plain_bf16(int mode, bool exact, bool wd, bool gs, bool keytab, 
 int launch_step_split(bool bf16, int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
                       uint32_t total_blocks, const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale,
                       uint32_t grid, void *stream);
-int launch_step_pipelined(bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
+int launch_step_pipelined(int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
                           uint32_t total_blocks, const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale,
                           uint32_t grid, uint32_t wg, void *stream);
 /* Sum of |moment - dequantised moment| of the coming step, per row: err[2r] first moment, err[2r+1] second. */

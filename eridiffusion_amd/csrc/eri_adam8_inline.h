@@ -180,10 +180,36 @@ __device__ __forceinline__ uint32_t code_bsearch(float x, const float *mid) {
 // the update of one element
 // ------------------------------------------------------------------------------------------
 
+/* The parameter update from finished moments, one rounded operation per line: what EXACT computes for
+ * the modes ERI and BNB. */
+template <int MODE, bool WD>
+__device__ __forceinline__ float param_exact(float p, float m, float v, const EriAdam8Hyper &h) {
+    float den = sqrtf(v) + h.eps; // adam8bit_enhanced.rs:263
+    float r = m / den;            // :264
+    if (MODE == ERI_ADAM8_MODE_BNB) {
+        float us = r * h.step_size;
+        float pn = p - us;
+        if (WD) pn = pn * h.weight_decay;
+        return pn;
+    }
+    float u = r;
+    if (WD) { // :267-271
+        float pw = p * h.weight_decay;
+        u = r + pw;
+    }
+    float us = u * h.step_size; // :274
+    return p - us;              // :275
+}
+
+/* `cancel` collects (it is only ever set) whether the approximate chain met a subtraction that cancels:
+ * the chain's few fp32 ulp of error are measured against the size of the update, so a result more than
+ * 2^12 times smaller than the parameter it came from can land more than one bf16 step from the exact
+ * chain's.  Callers recompute such elements with param_exact (about one element in 10^5 on trained
+ * weights); with EXACT it is never set. */
 template <int MODE, bool EXACT, bool BF16, bool WD, bool GS>
 __device__ __forceinline__ void adam_elem(float p, float g, float m_old, float v_old, const EriAdam8Hyper &h,
                                           float gscale, const BlockDiv &dbc1, const BlockDiv &dbc2, float &m,
-                                          float &v, float &pn) {
+                                          float &v, float &pn, bool &cancel) {
     if (GS) g = g * gscale;
     if (MODE == ERI_ADAM8_MODE_L2 && WD) { // adam8bit.rs:113-120
         float pw = p * h.weight_decay;
@@ -200,34 +226,24 @@ __device__ __forceinline__ void adam_elem(float p, float g, float m_old, float v
         float mh = dbc1.fast ? dbc1.div_fast_unbounded(m) : m / dbc1.a; // adam8bit.rs:170
         float vh = dbc2.fast ? dbc2.div_fast_unbounded(v) : v / dbc2.a; // :178
         vh = fmaxf(vh, 0.0f);                                  // :181-182
-        float upd;
-        if (EXACT) {
-            float den = sqrtf(vh) + h.eps; // :187
-            upd = mh / den;
-        } else {
-            float den = __builtin_amdgcn_sqrtf(vh) + h.eps;
-            upd = mh * __builtin_amdgcn_rcpf(den);
-        }
+        float den = sqrtf(vh) + h.eps; // :187  (this mode always takes the IEEE chain)
+        float upd = mh / den;
         float us = upd * h.step_size; // :196
         if (BF16) us = bf16_round(us); // :197-198
         pn = p - us;                   // :205
     } else if (MODE == ERI_ADAM8_MODE_BNB) { // h.eps carries sqrt(bc2), h.weight_decay is the factor 1 - lr*wd
-        float den = sqrtf(v) + h.eps;
-        float r = m / den;
-        float us = r * h.step_size;
-        pn = p - us;
-        if (WD) pn = pn * h.weight_decay;
+        if (EXACT) {
+            pn = param_exact<MODE, WD>(p, m, v, h);
+        } else { // bf16 parameters: as in mode ERI below, at most one bf16 step away from the exact chain, rarely
+            float den = __builtin_amdgcn_sqrtf(v) + h.eps;
+            float r = m * __builtin_amdgcn_rcpf(den);
+            pn = __builtin_fmaf(-r, h.step_size, p);
+            cancel |= __builtin_fabsf(pn) * 4096.0f < __builtin_fabsf(p);
+            if (WD) pn = pn * h.weight_decay;
+        }
     } else {
         if (EXACT) {
-            float den = sqrtf(v) + h.eps; // adam8bit_enhanced.rs:263
-            float r = m / den;            // :264
-            float u = r;
-            if (WD) { // :267-271
-                float pw = p * h.weight_decay;
-                u = r + pw;
-            }
-            float us = u * h.step_size; // :274
-            pn = p - us;                // :275
+            pn = param_exact<MODE, WD>(p, m, v, h);
         } else {
             // bf16 parameters: hardware square root and reciprocal (1 ulp each) and two fused
             // multiply-adds; the fp32 result is within a few ulp of the exact chain, which moves
@@ -236,6 +252,7 @@ __device__ __forceinline__ void adam_elem(float p, float g, float m_old, float v
             float r = m * __builtin_amdgcn_rcpf(den);
             float u = WD ? __builtin_fmaf(p, h.weight_decay, r) : r;
             pn = __builtin_fmaf(-u, h.step_size, p);
+            cancel |= __builtin_fabsf(pn) * 4096.0f < __builtin_fabsf(p);
         }
     }
 }
@@ -441,16 +458,21 @@ __device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint
             float pv[8], gv[8], pn[8];
             pr[d].unpack(pv);
             gr[d].unpack(gv);
+            bool cancel = false;
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
                 const float m_old = L.map_s[byte_of(mr[d], k)] * a_m;
                 const float v_old = L.map_u[byte_of(vr[d], k)] * a_v;
                 float m, v;
-                adam_elem<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], m_old, v_old, h, gscale, dbc1, dbc2, m, v, pn[k]);
+                adam_elem<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], m_old, v_old, h, gscale, dbc1, dbc2, m, v, pn[k], cancel);
                 mf[c * 8 + k] = m;
                 vf[c * 8 + k] = v;
                 lm = fmaxf(lm, __builtin_fabsf(m));
                 lv = fmaxf(lv, __builtin_fabsf(v));
+            }
+            if (cancel) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) pn[k] = param_exact<MODE, WD>(pv[k], mf[c * 8 + k], vf[c * 8 + k], h);
             }
             store8<BF16>(p, o, pn);
         }
@@ -529,8 +551,9 @@ __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
                     float m, v, pn;
+                    bool unused = false;
                     adam_elem<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], L.map_s[byte_of(mr, k)] * a_m,
-                                                         L.map_u[byte_of(vr, k)] * a_v, h, gscale, dbc1, dbc2, m, v, pn);
+                                                         L.map_u[byte_of(vr, k)] * a_v, h, gscale, dbc1, dbc2, m, v, pn, unused);
                     lm = fmaxf(lm, __builtin_fabsf(m));
                     lv = fmaxf(lv, __builtin_fabsf(v));
                 }
@@ -550,10 +573,15 @@ __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint
                 float pv[8], gv[8], pn[8], m[8], v[8];
                 pr.unpack(pv);
                 gr.unpack(gv);
+                bool cancel = false;
 #pragma unroll
                 for (int k = 0; k < 8; ++k)
                     adam_elem<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], L.map_s[byte_of(mr, k)] * a_m,
-                                                         L.map_u[byte_of(vr, k)] * a_v, h, gscale, dbc1, dbc2, m[k], v[k], pn[k]);
+                                                         L.map_u[byte_of(vr, k)] * a_v, h, gscale, dbc1, dbc2, m[k], v[k], pn[k], cancel);
+                if (cancel) {
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) pn[k] = param_exact<MODE, WD>(pv[k], m[k], v[k], h);
+                }
                 u32x2 mw, vw;
                 requant8<false, KEYTAB, MODE == ERI_ADAM8_MODE_BNB>(m, v, dm, dv, L, mw, vw);
                 *as_global(reinterpret_cast<u32x2 *>(t.m + e0 + o)) = mw;
@@ -570,8 +598,9 @@ __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint
     for (uint32_t i = lane; i < n; i += kWave) {
         const size_t e = e0 + i;
         float m, v, pn;
+        bool unused = false;
         adam_elem<MODE, EXACT, BF16, WD, GS>(load1<BF16>(t.p, e), load1<BF16>(t.g, e), L.map_s[mc[e]] * a_m,
-                                             L.map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn);
+                                             L.map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn, unused);
         lm = fmaxf(lm, __builtin_fabsf(m));
         lv = fmaxf(lv, __builtin_fabsf(v));
     }
@@ -581,8 +610,11 @@ __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint
     for (uint32_t i = lane; i < n; i += kWave) {
         const size_t e = e0 + i;
         float m, v, pn;
-        adam_elem<MODE, EXACT, BF16, WD, GS>(load1<BF16>(t.p, e), load1<BF16>(t.g, e), L.map_s[mc[e]] * a_m,
-                                             L.map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn);
+        bool cancel = false;
+        const float p_old = load1<BF16>(t.p, e);
+        adam_elem<MODE, EXACT, BF16, WD, GS>(p_old, load1<BF16>(t.g, e), L.map_s[mc[e]] * a_m,
+                                             L.map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn, cancel);
+        if (cancel) pn = param_exact<MODE, WD>(p_old, m, v, h);
         const float xm = dm.div_slow(m);
         const float xv = dv.div_slow(v);
         uint32_t cm = KEYTAB ? code_signed_key(xm, L.key_s) : code_bsearch(xm, L.mid_s);

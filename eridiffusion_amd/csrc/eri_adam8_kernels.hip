@@ -25,7 +25,7 @@ int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, i
     if (!kernel_named && g_split_blocks_per_cu > 0 && (few || !bf16)) {
         const bool bnb = h.mode == ERI_ADAM8_MODE_BNB;
         const bool wd_s = bnb ? h.weight_decay != 1.0f : h.weight_decay > 0.0f;
-        const bool exact_s = bnb || !bf16 || (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0;
+        const bool exact_s = !bf16 || (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0;
         uint32_t need = (total_blocks + 3) / 4;
         const uint32_t for_tails = (n_rows + 15) / 16;
         if (need < for_tails) need = for_tails;
@@ -33,9 +33,12 @@ int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, i
         if (need == 0) need = 1;
         return launch_step_split(bf16, h.mode, exact_s, wd_s, gs, rows, n_rows, total_blocks, h, lds_image, dev_scale, need, stream);
     }
-    if (h.mode == ERI_ADAM8_MODE_BNB) { // plain kernel, slot table, IEEE arithmetic; the decay is a factor
+    if (h.mode == ERI_ADAM8_MODE_BNB) { // slot table only; the decay is a factor
         const bool wd = h.weight_decay != 1.0f;
-        if (bf16) return launch_step_plain_bf16(h.mode, true, wd, gs, true, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
+        const bool exact = (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0;
+        if (bf16 && !kernel_named)
+            return launch_step_pipelined(h.mode, exact, wd, gs, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
+        if (bf16) return launch_step_plain_bf16(h.mode, exact, wd, gs, true, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
         return launch_step_plain_f32(h.mode, wd, gs, true, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
     }
     const bool wd = h.weight_decay > 0.0f;
@@ -43,7 +46,7 @@ int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, i
     const bool keytab = (h.flags & ERI_ADAM8_FLAG_BSEARCH) == 0;
     if (!bf16) return launch_step_plain_f32(h.mode, wd, gs, keytab, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
     if (keytab && h.mode == ERI_ADAM8_MODE_ERI && (h.flags & ERI_ADAM8_FLAG_NO_PIPELINE) == 0)
-        return launch_step_pipelined(exact, wd, gs, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
+        return launch_step_pipelined(h.mode, exact, wd, gs, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
     return launch_step_plain_bf16(h.mode, exact, wd, gs, keytab, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
 }
 
@@ -330,8 +333,9 @@ __global__ __launch_bounds__(256) void quant_error_kernel(const DevTensor *__res
         for (uint32_t i = lane; i < n; i += kWave) {
             const size_t e = e0 + i;
             float m, v, pn;
+            bool unused = false; // the exact chain never sets it
             adam_elem<MODE, true, BF16, WD, GS>(load1<BF16>(t.p, e), load1<BF16>(t.g, e), map_s[mc[e]] * a_m,
-                                                map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn);
+                                                map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn, unused);
             lm = fmaxf(lm, __builtin_fabsf(m));
             lv = fmaxf(lv, __builtin_fabsf(v));
         }
@@ -342,8 +346,9 @@ __global__ __launch_bounds__(256) void quant_error_kernel(const DevTensor *__res
         for (uint32_t i = lane; i < n; i += kWave) {
             const size_t e = e0 + i;
             float m, v, pn;
+            bool unused = false; // the exact chain never sets it
             adam_elem<MODE, true, BF16, WD, GS>(load1<BF16>(t.p, e), load1<BF16>(t.g, e), map_s[mc[e]] * a_m,
-                                                map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn);
+                                                map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn, unused);
             const float qm = map_s[code_bsearch(dm.div_slow(m), mid_s)] * nam;
             const float qv = map_u[code_bsearch(dv.div_slow(v), mid_u)] * nav;
             em += (double)__builtin_fabsf(m - qm);

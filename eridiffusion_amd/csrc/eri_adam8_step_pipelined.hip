@@ -102,6 +102,7 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
         u32x4 pw[4]; // updated parameters, packed, stored after the next block's loads are out
         float lm = 0.0f, lv = 0.0f;
         const float a_m = raw.a_m, a_v = raw.a_v;
+        bool cancel = false;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             Raw8<true> pr, gr;
@@ -115,7 +116,7 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
                 const float m_old = lds_float_at(L.map_s, code_offset(raw.m[c], k)) * a_m;
                 const float v_old = lds_float_at(L.map_u, code_offset(raw.v[c], k)) * a_v;
                 float m, v;
-                adam_elem<MODE, EXACT, true, WD, GS>(pv[k], gv[k], m_old, v_old, h, gscale, dbc1, dbc2, m, v, pn[k]);
+                adam_elem<MODE, EXACT, true, WD, GS>(pv[k], gv[k], m_old, v_old, h, gscale, dbc1, dbc2, m, v, pn[k], cancel);
                 mf[c * 8 + k] = m;
                 vf[c * 8 + k] = v;
                 lm = fmaxf(lm, __builtin_fabsf(m));
@@ -126,6 +127,22 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
             pw[c].z = bf16_pair(pn[4], pn[5]);
             pw[c].w = bf16_pair(pn[6], pn[7]);
             if (V == 1) __builtin_nontemporal_store(pw[c], as_global(reinterpret_cast<u32x4 *>(p) + c * 64 + lane));
+        }
+        if (cancel) { // rare: a lane whose update cancelled redoes its 32 parameters with the exact chain
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                Raw8<true> pr;
+                pr.w = raw.p[c];
+                float pv[8], pn[8];
+                pr.unpack(pv);
+#pragma unroll
+                for (int k = 0; k < 8; ++k) pn[k] = param_exact<MODE, WD>(pv[k], mf[c * 8 + k], vf[c * 8 + k], h);
+                pw[c].x = bf16_pair(pn[0], pn[1]);
+                pw[c].y = bf16_pair(pn[2], pn[3]);
+                pw[c].z = bf16_pair(pn[4], pn[5]);
+                pw[c].w = bf16_pair(pn[6], pn[7]);
+                if (V == 1) __builtin_nontemporal_store(pw[c], as_global(reinterpret_cast<u32x4 *>(p) + c * 64 + lane));
+            }
         }
         float nam = lm, nav = lv;
         wave_max2(nam, nav);
@@ -145,7 +162,7 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const uint32_t o = c * 512 + lane * 8;
-                requant8<true, true>(mf + c * 8, vf + c * 8, dm, dv, L, mws[c], vws[c]);
+                requant8<true, true, MODE == ERI_ADAM8_MODE_BNB>(mf + c * 8, vf + c * 8, dm, dv, L, mws[c], vws[c]);
                 if (V != 3) {
                     __builtin_nontemporal_store(mws[c], as_global(reinterpret_cast<u32x2 *>(mc + o)));
                     __builtin_nontemporal_store(vws[c], as_global(reinterpret_cast<u32x2 *>(vc + o)));
@@ -173,7 +190,7 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
             for (int c = 0; c < 4; ++c) {
                 const uint32_t o = c * 512 + lane * 8;
                 u32x2 mw, vw;
-                requant8<false, true>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
+                requant8<false, true, MODE == ERI_ADAM8_MODE_BNB>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
                 __builtin_nontemporal_store(mw, as_global(reinterpret_cast<u32x2 *>(mc + o)));
                 __builtin_nontemporal_store(vw, as_global(reinterpret_cast<u32x2 *>(vc + o)));
             }
@@ -218,14 +235,16 @@ int launch_flags(bool wd, bool gs, const DevTensor *rows, uint32_t n_rows, uint3
 
 } // namespace
 
-/* Mode ERI only.  The coupled-decay mode needs more live values per element than this kernel's
+/* Modes ERI and BNB.  The coupled-decay mode needs more live values per element than this kernel's
  * register budget holds (its instantiations spilled 80-232 B per lane) and runs faster on the kernel
  * without the prefetch; the dispatcher sends it there. */
-int launch_step_pipelined(bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
+int launch_step_pipelined(int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
                           uint32_t total_blocks, const EriAdam8Hyper &h, const void *img, const float *dev_scale,
                           uint32_t grid, uint32_t wg, void *stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define ERI_ARGS wd, gs, rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s
+    if (mode == ERI_ADAM8_MODE_BNB)
+        return exact ? launch_flags<ERI_ADAM8_MODE_BNB, true>(ERI_ARGS) : launch_flags<ERI_ADAM8_MODE_BNB, false>(ERI_ARGS);
     return exact ? launch_flags<ERI_ADAM8_MODE_ERI, true>(ERI_ARGS) : launch_flags<ERI_ADAM8_MODE_ERI, false>(ERI_ARGS);
 #undef ERI_ARGS
 }

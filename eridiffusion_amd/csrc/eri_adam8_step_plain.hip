@@ -96,9 +96,9 @@ int launch_step_plain_bf16(int mode, bool exact, bool wd, bool gs, bool keytab, 
                            uint32_t grid, uint32_t wg, void *stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define ERI_ARGS wd, gs, keytab, rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s
-    if (mode == ERI_ADAM8_MODE_BNB) return launch_flags<ERI_ADAM8_MODE_BNB, true, false>(ERI_ARGS);
-    if (mode == ERI_ADAM8_MODE_L2)
-        return exact ? launch_flags<ERI_ADAM8_MODE_L2, true, true>(ERI_ARGS) : launch_flags<ERI_ADAM8_MODE_L2, false, true>(ERI_ARGS);
+    if (mode == ERI_ADAM8_MODE_BNB)
+        return exact ? launch_flags<ERI_ADAM8_MODE_BNB, true, false>(ERI_ARGS) : launch_flags<ERI_ADAM8_MODE_BNB, false, false>(ERI_ARGS);
+    if (mode == ERI_ADAM8_MODE_L2) return launch_flags<ERI_ADAM8_MODE_L2, true, true>(ERI_ARGS); // always the IEEE chain
     return exact ? launch_flags<ERI_ADAM8_MODE_ERI, true, true>(ERI_ARGS) : launch_flags<ERI_ADAM8_MODE_ERI, false, true>(ERI_ARGS);
 #undef ERI_ARGS
 }

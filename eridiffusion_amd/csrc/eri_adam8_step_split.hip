@@ -91,13 +91,18 @@ __global__ __launch_bounds__(1024) void adam8_step_split_kernel(const DevTensor 
             float pv[8], gv[8], pn[8];
             q.pr.unpack(pv);
             q.gr.unpack(gv);
+            bool cancel = false;
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
                 const float m_old = L.map_s[byte_of(q.mr, k)] * q.a_m;
                 const float v_old = L.map_u[byte_of(q.vr, k)] * q.a_v;
-                adam_elem<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], m_old, v_old, h, gscale, dbc1, dbc2, m[k], v[k], pn[k]);
+                adam_elem<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], m_old, v_old, h, gscale, dbc1, dbc2, m[k], v[k], pn[k], cancel);
                 nam = fmaxf(nam, __builtin_fabsf(m[k]));
                 nav = fmaxf(nav, __builtin_fabsf(v[k]));
+            }
+            if (cancel) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) pn[k] = param_exact<MODE, WD>(pv[k], m[k], v[k], h);
             }
             store8<BF16>(p, o, pn);
             wave_max2(nam, nav);
@@ -157,9 +162,9 @@ int launch_step_split(bool bf16, int mode, bool exact, bool wd, bool gs, const D
         if (mode == ERI_ADAM8_MODE_L2) return launch_flags<false, ERI_ADAM8_MODE_L2, true>(ERI_ARGS);
         return launch_flags<false, ERI_ADAM8_MODE_ERI, true>(ERI_ARGS);
     }
-    if (mode == ERI_ADAM8_MODE_BNB) return launch_flags<true, ERI_ADAM8_MODE_BNB, true>(ERI_ARGS);
-    if (mode == ERI_ADAM8_MODE_L2)
-        return exact ? launch_flags<true, ERI_ADAM8_MODE_L2, true>(ERI_ARGS) : launch_flags<true, ERI_ADAM8_MODE_L2, false>(ERI_ARGS);
+    if (mode == ERI_ADAM8_MODE_BNB)
+        return exact ? launch_flags<true, ERI_ADAM8_MODE_BNB, true>(ERI_ARGS) : launch_flags<true, ERI_ADAM8_MODE_BNB, false>(ERI_ARGS);
+    if (mode == ERI_ADAM8_MODE_L2) return launch_flags<true, ERI_ADAM8_MODE_L2, true>(ERI_ARGS); // always the IEEE chain
     return exact ? launch_flags<true, ERI_ADAM8_MODE_ERI, true>(ERI_ARGS) : launch_flags<true, ERI_ADAM8_MODE_ERI, false>(ERI_ARGS);
 #undef ERI_ARGS
 }

@@ -91,8 +91,8 @@ typedef enum EriAdam8Mode {
                                (bitsandbytes 8-bit blockwise Adam): p = (p - step_size * m / (sqrt(v) +
                                eps*sqrt(bc2))) * (1 - lr*wd), and a first-moment code whose map value has the
                                other sign than the moment moves one entry toward the moment's sign.  With
-                               wd = 0 this is the textbook Adam formula.  Moments as in ERI.  Always IEEE
-                               sqrt and divide; not available to eri_adam8_quant_error. */
+                               wd = 0 this is the textbook Adam formula.  Moments as in ERI.  Not
+                               available to eri_adam8_quant_error. */
 } EriAdam8Mode;
 
 enum {

@@ -84,7 +84,7 @@ def test_mode_bnb_with_clipping_and_statistics_through_the_python_face():
     ps, _ = hs.make_inputs(sizes, True, 15, p_std=1e-2)
     states = hs.oracle_states(sizes)
     params = [_bf16_tensor(p) for p in ps]
-    opt = Adam8bit(params, Adam8bitConfig(lr=1e-3))
+    opt = Adam8bit(params, Adam8bitConfig(lr=1e-3), flags=L.FLAG_EXACT_PARAM)  # bit-for-bit bf16 parameters
     opt.set_mode(L.MODE_BNB)
     opt.set_max_grad_norm(0.05)
     opt.track_quantization_error(True)
