@@ -8,6 +8,12 @@
  *   Adam8bit / Adam8bitConfig / OptimizerState   src/trainers/adam8bit_enhanced.rs:10-27,372-404
  *   Adam8bit (functional) / Adam8bitState        src/trainers/adam8bit.rs:15-47
  */
+#include <fcntl.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -726,8 +732,42 @@ struct Bincode {
     }
 };
 
+/* One QuantizedTensor of the file, left where it lies in the mapped file. */
 struct LegacyTensor {
-    std::vector<float> values; // dequantised
+    const int8_t *q = nullptr;
+    uint64_t n = 0;
+    float scale = 1.0f;
+    int8_t zp = 0;
+};
+
+/* A file mapped read-only: a state file of a large model is walked in place, never copied whole. */
+struct MappedFile {
+    const unsigned char *data = nullptr;
+    size_t size = 0;
+    bool open(const char *path) {
+        const int fd = ::open(path, O_RDONLY);
+        if (fd < 0) return false;
+        struct stat st;
+        if (::fstat(fd, &st) != 0 || !S_ISREG(st.st_mode)) {
+            ::close(fd);
+            return false;
+        }
+        size = (size_t)st.st_size;
+        if (size) {
+            void *m = ::mmap(nullptr, size, PROT_READ, MAP_PRIVATE, fd, 0);
+            if (m == MAP_FAILED) {
+                ::close(fd);
+                size = 0;
+                return false;
+            }
+            data = static_cast<const unsigned char *>(m);
+        }
+        ::close(fd);
+        return true;
+    }
+    ~MappedFile() {
+        if (data) ::munmap(const_cast<unsigned char *>(data), size);
+    }
 };
 
 bool read_legacy_map(Bincode &b, std::map<std::string, LegacyTensor> &out) {
@@ -750,12 +790,11 @@ bool read_legacy_map(Bincode &b, std::map<std::string, LegacyTensor> &out) {
         b.f32(); // quantization_error
         if (!b.ok) return false;
         LegacyTensor t;
-        t.values.resize(n);
-        for (uint64_t i = 0; i < n; ++i) { // to_tensor, adam8bit_enhanced.rs:117-129
-            float x = ((float)q[i] - (float)zp) * scale;
-            t.values[i] = std::isfinite(x) ? x : 0.0f;
-        }
-        out[key] = std::move(t);
+        t.q = q;
+        t.n = n;
+        t.scale = scale;
+        t.zp = zp;
+        out[key] = t;
     }
     return true;
 }
@@ -764,10 +803,9 @@ bool read_legacy_map(Bincode &b, std::map<std::string, LegacyTensor> &out) {
 
 extern "C" int eri_adam8bit_load_legacy_state(EriAdam8bit *o, const char *path) {
     if (!o || !path) return fail(ERI_ERR_NULL, "optimizer or path is NULL");
-    std::ifstream f(path, std::ios::binary);
-    if (!f) return fail(ERI_ERR_ARG, std::string("InvalidOperation: Failed to read optimizer: cannot open ") + path);
-    std::vector<unsigned char> raw((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
-    Bincode b{raw.data(), raw.data() + raw.size()};
+    MappedFile raw;
+    if (!raw.open(path)) return fail(ERI_ERR_ARG, std::string("InvalidOperation: Failed to read optimizer: cannot open ") + path);
+    Bincode b{raw.data, raw.data + raw.size};
     const uint64_t step = b.u64();
     std::map<std::string, LegacyTensor> first, second;
     if (!read_legacy_map(b, first) || !read_legacy_map(b, second))
@@ -781,34 +819,55 @@ extern "C" int eri_adam8bit_load_legacy_state(EriAdam8bit *o, const char *path) 
         const std::string key = "param_" + std::to_string(i);
         auto m = first.find(key), v = second.find(key);
         if (m == first.end() && v == second.end()) continue;
-        if (m == first.end() || v == second.end() || m->second.values.size() != o->params[i]->numel ||
-            v->second.values.size() != o->params[i]->numel)
+        if (m == first.end() || v == second.end() || m->second.n != o->params[i]->numel ||
+            v->second.n != o->params[i]->numel)
             return fail(ERI_ERR_ARG, "InvalidOperation: Failed to deserialize optimizer: state of " + key + " does not fit its parameter");
         items.push_back({i, &m->second, &v->second});
     }
+    // dequantised as the reference does (to_tensor, adam8bit_enhanced.rs:117-129) piece by piece into
+    // pinned memory, gathered in one fp32 device buffer per tensor, quantised blockwise from there;
+    // every new state is complete before the first one replaces an old one
+    uint64_t largest = 0;
+    for (auto &it : items) largest = std::max<uint64_t>(largest, o->params[it.idx]->numel);
+    void *tmp = nullptr;
+    Bounce bounce;
+    if (!items.empty()) {
+        int dev = 0;
+        int rc = eri_hip_get_device(&dev);
+        if (!rc) rc = bounce.ensure();
+        if (!rc) rc = eri_hip_malloc_zeroed(dev, largest * 4, &tmp);
+        if (rc) return rc;
+    }
+    std::vector<std::unique_ptr<State8>> fresh;
+    int rc = 0;
     for (auto &it : items) {
         const uint64_t n = o->params[it.idx]->numel;
         std::unique_ptr<State8> s(new State8());
-        int rc = s->allocate(n, o->stream);
-        if (rc) return rc;
-        void *tmp = nullptr;
-        int dev = 0;
-        rc = eri_hip_get_device(&dev);
-        if (rc) return rc;
-        rc = eri_hip_malloc_zeroed(dev, n * 4, &tmp);
-        if (rc) return rc;
+        rc = s->allocate(n, o->stream);
         for (int k = 0; k < 2 && rc == 0; ++k) {
             const LegacyTensor *src = k == 0 ? it.m : it.v;
-            rc = eri_hip_memcpy_async(tmp, src->values.data(), n * 4, 1, o->stream);
+            const uint64_t piece = Bounce::kHalf / 4;
+            for (uint64_t done = 0; done < n && rc == 0; done += piece) {
+                const uint64_t cnt = n - done < piece ? n - done : piece;
+                float *buf = reinterpret_cast<float *>(bounce.next());
+                for (uint64_t i = 0; i < cnt; ++i) {
+                    const float x = ((float)src->q[done + i] - (float)src->zp) * src->scale;
+                    buf[i] = std::isfinite(x) ? x : 0.0f;
+                }
+                rc = eri_hip_stream_sync(o->stream); // the copy out of the other half
+                if (rc == 0) rc = eri_hip_memcpy_async(static_cast<float *>(tmp) + done, buf, cnt * 4, 1, o->stream);
+            }
             if (rc == 0)
                 rc = eri_adam8_quantize(static_cast<const float *>(tmp), k == 0 ? 1 : 0, n, k == 0 ? s->m : s->v,
                                         k == 0 ? s->absmax_m : s->absmax_v, o->stream);
             if (rc == 0) rc = eri_hip_stream_sync(o->stream);
         }
-        eri_hip_free(tmp);
-        if (rc) return rc;
-        o->states[it.idx] = std::move(s);
+        if (rc) break;
+        fresh.push_back(std::move(s));
     }
+    if (tmp) eri_hip_free(tmp);
+    if (rc) return rc;
+    for (size_t k = 0; k < items.size(); ++k) o->states[items[k].idx] = std::move(fresh[k]);
     o->step = step;
     o->lr = lr;
     if (o->table) {

@@ -344,3 +344,50 @@ def test_legacy_bincode_state_is_imported_and_requantised(tmp_path):
         assert np.array_equal(got[k], codes)
         assert np.array_equal(got[2 + k].view(np.uint32), absmax.view(np.uint32))
     L.lib().eri_adam8bit_destroy(opt)
+
+
+def test_legacy_state_longer_than_one_staging_piece(tmp_path):
+    """A tensor of 8 Mi + 5000 elements is dequantised in two pieces of pinned memory (the second partial)
+    before it is quantised blockwise; a small second parameter follows."""
+    import torch
+    from test_host_objects_cpu import _bincode_state
+    L = _L()
+    sizes = [8 * (1 << 20) + 5000, 3000]
+    dev = torch.device("cuda:0")
+    p = [torch.zeros(n, dtype=torch.float32, device=dev) for n in sizes]
+    handles = (C.c_void_p * 2)()
+    for i in range(2):
+        h = C.c_void_p()
+        L.check(L.lib().eri_param_create(p[i].data_ptr(), sizes[i], 0, C.byref(h)), "param_create")
+        handles[i] = h
+    opt = C.c_void_p()
+    L.check(L.lib().eri_adam8bit_new(handles, 2, None, None, C.byref(opt)), "adam8bit_new")
+    rng = np.random.default_rng(12)
+    q = {(i, k): rng.integers(-128, 128, n, dtype=np.int8) for i, n in enumerate(sizes) for k in (0, 1)}
+    par = {(0, 0): (2e-5, 3), (0, 1): (4e-10, -128), (1, 0): (1e-4, -1), (1, 1): (7e-9, -128)}
+    first = {"param_%d" % i: (q[i, 0].tobytes(), par[i, 0][0], par[i, 0][1], [n], 0.0) for i, n in enumerate(sizes)}
+    second = {"param_%d" % i: (q[i, 1].tobytes(), par[i, 1][0], par[i, 1][1], [n], 0.0) for i, n in enumerate(sizes)}
+    path = tmp_path / "optimizer.pt"
+    path.write_bytes(_bincode_state(9, 1e-4, first, second))
+    L.check(L.lib().eri_adam8bit_load_legacy_state(opt, str(path).encode()), "load_legacy")
+    assert L.lib().eri_adam8bit_get_step(opt) == 9
+    for i, n in enumerate(sizes):
+        nb = (n + 2047) // 2048
+        ptrs = [C.c_void_p() for _ in range(4)]
+        L.check(L.lib().eri_adam8bit_state_ptrs(opt, i, *[C.byref(x) for x in ptrs]), "state_ptrs")
+        for k in (0, 1):
+            scale, zp = par[i, k]
+            x = ((q[i, k].astype(np.float32) - np.float32(zp)) * np.float32(scale)).astype(np.float32)
+            codes = np.empty(n, np.uint8)
+            absmax = np.empty(nb, np.float32)
+            oc.lib().eri_oracle_quantize(oc.ptr(x), oc.ptr(hs.MAPS[k]), n, oc.ptr(codes), oc.ptr(absmax))
+            got_c = np.empty(n, np.uint8)
+            got_a = np.empty(nb, np.float32)
+            L.check(L.lib().eri_hip_memcpy_async(got_c.ctypes.data, ptrs[k].value, n, 2, None), "d2h")
+            L.check(L.lib().eri_hip_memcpy_async(got_a.ctypes.data, ptrs[2 + k].value, 4 * nb, 2, None), "d2h")
+            L.check(L.lib().eri_hip_stream_sync(None), "sync")
+            assert np.array_equal(got_c, codes)
+            assert np.array_equal(got_a.view(np.uint32), absmax.view(np.uint32))
+    L.lib().eri_adam8bit_destroy(opt)
+    for h in handles:
+        L.lib().eri_param_release(h)

@@ -102,7 +102,8 @@ def test_functional_flavour_counters_and_errors():
 def _bincode_state(step, lr, first, second):
     """bincode 1.3 default options of the reference's OptimizerState (adam8bit_enhanced.rs:398-404)."""
     def qt(q, scale, zp, shape, err):
-        b = struct.pack("<Q", len(q)) + bytes((x & 0xFF) for x in q) + struct.pack("<f", scale) + struct.pack("<b", zp)
+        raw = bytes(q) if isinstance(q, (bytes, bytearray)) else bytes((x & 0xFF) for x in q)
+        b = struct.pack("<Q", len(raw)) + raw + struct.pack("<f", scale) + struct.pack("<b", zp)
         b += struct.pack("<Q", len(shape)) + b"".join(struct.pack("<Q", d) for d in shape) + struct.pack("<f", err)
         return b
 
