@@ -264,6 +264,27 @@ def test_scaled_model_shapes_bf16():
         run_case(sizes, True, 800 + len(sizes), steps=2, label=name + "-scaled")
 
 
+def test_hundred_steps_of_a_lora_set_stay_on_the_oracle():
+    """The rank-32 FLUX LoRA list (every sixth tensor, widths / 16) for a hundred steps with fresh
+    gradients each step, as the LoRA configurations of the benchmark prescribe: states start at zero,
+    LoRA-B weights start at zero and grow to the size of their updates.  Exact flag: states and bf16
+    parameters bit for bit after step 100 -- one wrong code early on would have spread by then."""
+    from eridiffusion_amd import workloads as w
+    sizes = [w.numel(s) for _, s in w.c3_flux_lora(scale=16)][::6]
+    ps, _ = hs.make_inputs(sizes, True, 1234, 0.02, 1e-4)
+    for i in range(1, len(ps), 2):
+        ps[i][:] = 0  # every other tensor starts at zero, as LoRA-B matrices do
+    states = hs.oracle_states(sizes)
+    all_g = [hs.fresh_grads(sizes, True, 50000 + t, 1e-4) for t in range(100)]
+    gt = hs.GpuTensors(ps, all_g[0], states, True)
+    for t, g_t in enumerate(all_g):
+        hs.oracle_step(ps, g_t, states, (LR, B1, B2, EPS, WD, t + 1), True, oc.MODE_ERI)
+    gpu_steps(gt, [None] + all_g[1:], 1, 0, 2, WD)
+    got_p, got_st = gt.fetch()
+    stats = hs.compare(got_p, got_st, ps, states, True, True, "lora-100-steps")
+    assert stats["code_mismatch"] == 0
+
+
 def test_zero_gradients_and_zero_state():
     sizes = [2048 * 2 + 9]
     ps, gs = hs.make_inputs(sizes, False, 900)
