@@ -11,8 +11,13 @@
 
 namespace eri {
 
+/* Threads per workgroup.  The coupled-decay mode holds two more divisions' worth of values per element:
+ * with the 128 registers a 1024-thread workgroup leaves each lane it spilled 28-68 bytes, with 768
+ * threads (170 registers) it does not. */
+constexpr uint32_t plain_threads(int mode) { return mode == ERI_ADAM8_MODE_L2 ? 768 : 1024; }
+
 template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB>
-__global__ __launch_bounds__(1024) void adam8_step_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
+__global__ __launch_bounds__(plain_threads(MODE)) void adam8_step_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
                                                           uint32_t total_blocks, EriAdam8Hyper h,
                                                           const uint4 *__restrict__ lds_image,
                                                           const float *__restrict__ dev_scale, uint32_t chunks) {
@@ -67,6 +72,7 @@ template <int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB>
 int launch_one(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
                const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg, hipStream_t s) {
     auto k = adam8_step_kernel<kBf16, MODE, EXACT, WD, GS, KEYTAB>;
+    if (wg > plain_threads(MODE)) wg = plain_threads(MODE);
     hipLaunchKernelGGL(k, dim3(grid), dim3(wg), 0, s, rows, n_rows, total_blocks, h,
                        static_cast<const uint4 *>(lds_image), dev_scale, chunks_for(grid));
     return (int)hipGetLastError();
