@@ -28,6 +28,7 @@ int fail(int code, const std::string &msg) {
 
 int hip_fail(hipError_t e, const char *what) {
     g_err = std::string(what) + ": " + hipGetErrorString(e);
+    (void)hipGetLastError(); // reported here: the runtime's own record must not surface in the caller's next HIP call
     return (int)e;
 }
 
