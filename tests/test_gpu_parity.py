@@ -436,7 +436,6 @@ def test_randomized_extreme_values_against_the_oracle():
         wd = float(rng.choice([0.0, 0.01]))
         mag_g = 10.0 ** rng.uniform(-30, 30) if case % 2 else 10.0 ** rng.uniform(-8, 2)
         ps, _ = hs.make_inputs(sizes, bf16, 3000 + case, p_std=float(10.0 ** rng.uniform(-4, 2)))
-        omode = {0: oc.MODE_ERI, 1: oc.MODE_L2, 2: oc.MODE_BNB}[mode]
         states = hs.oracle_states(sizes)
 
         def grads():
