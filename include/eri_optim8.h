@@ -71,6 +71,8 @@ int eri_hip_free(void *ptr);
 void *eri_hip_host_alloc(size_t bytes);                          /* pinned; NULL on failure */
 int eri_hip_host_free(void *ptr);
 int eri_hip_memcpy_async(void *dst, const void *src, size_t bytes, int kind, void *stream);
+/* Byte fill through the runtime's own memset.  Not for a stream that is being captured into a HIP graph:
+ * the optimizer calls below clear what they need with a small kernel of their own and stay capturable. */
 int eri_hip_memset_async(void *dst, int value, size_t bytes, void *stream);
 int eri_hip_stream_create(void **stream);                        /* default priority */
 int eri_hip_stream_sync(void *stream);
