@@ -33,12 +33,9 @@ def parse():
     ap.add_argument("--kernel", choices=["adam8", "adam8_clip", "grad_norm", "adamw32", "ema"], default="adam8",
                     help="what one step is: the 8-bit AdamW step (headline), the same preceded by the device-side "
                          "gradient norm, the norm alone, the 32-bit AdamW sibling, or the EMA sweep")
-    ap.add_argument("--variants", default="", help="comma-separated kernel variants to time interleaved (A/B tool)")
-    ap.add_argument("--alloc", choices=["arena", "pool", "tensor"], default="arena",
-                    help="one flat allocation per kind of buffer, or one allocation per tensor and buffer")
-    ap.add_argument("--calibrate-copy", type=int, default=0,
-                    help="instead of the benchmark, run a plain device copy of this many bytes three times "
-                         "(the known-size kernel the rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by)")
+    ap.add_argument("--alloc", choices=["arena", "tensor"], default="arena",
+                    help="one flat allocation per kind of buffer (library allocator), or one torch allocation per "
+                         "tensor and buffer (how a tensor runtime holds parameters and states)")
     ap.add_argument("--traffic-json", default=os.path.join(ROOT, "profiles", "traffic.json"),
                     help="HBM bytes per launch derived from rocprofv3 --pmc runs, if present")
     return ap.parse_args()
@@ -94,42 +91,6 @@ class Arena:
         L.lib().eri_hip_free(self.base)
 
 
-class Pool:
-    """One device allocation for everything (how a pooling allocator would hold a model): the six
-    buffers are consecutive ranges of it, each starting on a 2 MiB boundary."""
-    base = None
-    used = 0
-    capacity = 0
-
-    @classmethod
-    def reserve(cls, nbytes):
-        from eridiffusion_amd import _lib as L
-        out = C.c_void_p()
-        L.check(L.lib().eri_hip_malloc_zeroed(0, nbytes, C.byref(out)), "eri_hip_malloc_zeroed")
-        cls.base, cls.used, cls.capacity = out.value, 0, nbytes
-
-    def __init__(self, torch, sizes_bytes):
-        self.offsets = []
-        total = 0
-        for b in sizes_bytes:
-            self.offsets.append(total)
-            total += align(b)
-        self.nbytes = align(max(total, 256), 2 << 20)
-        if Pool.used + self.nbytes > Pool.capacity:
-            raise RuntimeError("pool exhausted")
-        self.base = Pool.base + Pool.used
-        Pool.used += self.nbytes
-
-    ptr = Arena.ptr
-    fill = Arena.fill
-
-    def free(self):
-        from eridiffusion_amd import _lib as L
-        if Pool.base is not None:
-            L.lib().eri_hip_free(Pool.base)
-            Pool.base = None
-
-
 def cpu_baseline(tensors, bf16, sample_params, hyper_args):
     """Times the C oracle (oracle/liberi_oracle.so) on a prefix of the same tensor list."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
@@ -174,13 +135,16 @@ def cpu_baseline(tensors, bf16, sample_params, hyper_args):
     n1 = min(sizes[big], 1 << 26)
     st1 = list(oc.state_init(n1))
     p1, g1 = p1[:n1].copy(), g1[:n1].copy()
-    t0 = time.perf_counter()
-    oc.step_tensor(p1, g1, *st1, oc.hyper_pack(*hyper_args[:5], 1), maps, dt_tag, 1)
-    single = n1 / (time.perf_counter() - t0)
-    return {"value": total / best, "unit": "params/s", "cores": threads, "kind": "port",
-            "sample": "first %d tensors of the workload (%d params), one step, C oracle with OpenMP over blocks, "
-                      "best of 2" % (len(sizes), total),
-            "single_thread_value": single, "single_thread_sample": "%d params of the sample's largest tensor, one step" % n1}
+    single = None
+    for rep in range(2):  # the second step starts from real state contents, not from the all-zero state
+        t0 = time.perf_counter()
+        oc.step_tensor(p1, g1, *st1, oc.hyper_pack(*hyper_args[:5], rep + 1), maps, dt_tag, 1)
+        single = n1 / (time.perf_counter() - t0)
+    return {"value": total / best, "unit": "params/s", "cores": threads, "host_cores": os.cpu_count(), "kind": "port",
+            "sample": "first %d tensors of the workload (%d params), one step, C oracle with OpenMP over blocks on "
+                      "%d threads, best of 2" % (len(sizes), total, threads),
+            "single_thread_value": single,
+            "single_thread_sample": "%d params of the sample's largest tensor, second of two steps" % n1}
 
 
 def main():
@@ -190,15 +154,6 @@ def main():
               "a single MI355X; rerun with --gpus 1", file=sys.stderr)
         sys.exit(2)
     import torch
-
-    if args.calibrate_copy > 0:
-        src = torch.empty(args.calibrate_copy // 4, dtype=torch.float32, device="cuda:0").fill_(1.0)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        print(json.dumps({"calibrate_copy_bytes": src.numel() * 4, "launches": 3}))
-        return
 
     from eridiffusion_amd import _lib as L
     from eridiffusion_amd import workloads as W
@@ -213,10 +168,7 @@ def main():
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream().cuda_stream
 
-    Alloc = {"arena": Arena, "pool": Pool, "tensor": PerTensor}[args.alloc]
-    if args.alloc == "pool":
-        extra_b = {"adamw32": 8, "ema": esz}.get(args.kernel, 0)
-        Pool.reserve(align(n_params * (2 * esz + 2 + extra_b) + n_blocks * 8 + 300 * len(sizes) * 8, 2 << 20) + (20 << 20))
+    Alloc = {"arena": Arena, "tensor": PerTensor}[args.alloc]
     a_p = Alloc(torch, [n * esz for n in sizes])
     a_g = Alloc(torch, [n * esz for n in sizes])
     a_m = Alloc(torch, sizes)
@@ -282,23 +234,6 @@ def main():
         h = L.hyper_pack(*hyper_args, t, L.MODE_ERI, flags)
         L.check(L.lib().eri_adam8_step_table(table, C.byref(h), stream), "step_table")
 
-    if args.variants:
-        vs = [int(x) for x in args.variants.split(",")]
-        acc = {v: [] for v in vs}
-        t = 0
-        for rep in range(args.steps):
-            for v in vs:
-                L.check(L.lib().eri_adam8_set_tuning(0, v), "set_tuning")
-                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                t += 1
-                a.record()
-                step(t)
-                b.record()
-                torch.cuda.synchronize()
-                if rep >= args.warmup:
-                    acc[v].append(a.elapsed_time(b))
-        print(json.dumps({"variants_ms": {str(v): sum(x) / len(x) for v, x in acc.items()}}))
-        return
     t = 0
     for _ in range(args.warmup):
         t += 1
@@ -343,6 +278,8 @@ def main():
                    "resident_gb": round((n_params * (2 * esz + 2) + n_blocks * 8) / 1e9, 2)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                      "frac": achieved / PEAK_HBM_GBPS, "traffic": traffic,
+                     "traffic_source": None if traffic is None else "profiles/traffic.json: FETCH_SIZE and WRITE_SIZE of "
+                                       "rocprofv3 --pmc runs of this command, not counted in this run",
                      "kernel_ms": avg_launch_s * 1e3, "kernel_ms_min": min(launch_ms), "kernel_ms_max": max(launch_ms),
                      "algorithmic_bytes": algo_bytes},
     }

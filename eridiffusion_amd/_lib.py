@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(_HERE, "liberi_optim8.so")
 BLOCK = 2048
 DTYPE_F32, DTYPE_F16, DTYPE_BF16, DTYPE_I32 = 0, 1, 2, 3
 MODE_ERI, MODE_L2, MODE_BNB = 0, 1, 2
-FLAG_GRAD_SCALE, FLAG_EXACT_PARAM, FLAG_BSEARCH, FLAG_NO_PIPELINE, FLAG_CLIP_FROM_TABLE = 1, 2, 4, 8, 16
+FLAG_GRAD_SCALE, FLAG_EXACT_PARAM, FLAG_BSEARCH, FLAG_NO_PIPELINE, FLAG_CLIP_FROM_TABLE, FLAG_ONE_WAVE = 1, 2, 4, 8, 16, 32
 
 
 class Hyper(C.Structure):
@@ -80,7 +80,6 @@ EXPORTS = {
     "eri_hip_stream_destroy": (C.c_int, [C.c_void_p]),
     "eri_hip_mem_info": (C.c_int, [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
     "eri_adam8_init": (C.c_int, []),
-    "eri_adam8_set_tuning": (C.c_int, [C.c_int, C.c_int]),
     "eri_adam8_get_maps": (C.c_int, [C.c_void_p, C.c_void_p]),
     "eri_adam8_table_image": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_size_t), C.POINTER(C.c_uint32)]),
     "eri_adam8_hyper_pack": (C.c_int, [C.c_double] * 5 + [C.c_uint64, C.c_int, C.c_uint32, C.POINTER(Hyper)]),

@@ -71,16 +71,14 @@ static_assert(kLdsImageBytes % 16 == 0, "the image is staged in 16-byte words");
 int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_blocks, int dtype_tag,
                 const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg,
                 uint32_t compute_units, void *stream);
-extern int g_kernel_variant;
-extern int g_chunks;
-extern int g_pipelined_waves;
-extern int g_norm_waves;
-extern int g_split_blocks_per_cu;
+
+constexpr uint32_t kChunks = 8;           /* contiguous ranges the block list is cut into: one per accelerator die */
+constexpr uint32_t kSplitBlocksPerCu = 64; /* tables of at most this many full blocks per compute unit take the
+                                              four-waves-per-block kernel */
+constexpr uint32_t kNormWaves = 4;        /* waves per workgroup of the gradient-norm pass */
 
 /* The chunked walk (BlockWalk) needs the same number of workgroups in every chunk. */
-inline uint32_t chunks_for(uint32_t grid) {
-    return (g_chunks > 1 && grid % (uint32_t)g_chunks == 0) ? (uint32_t)g_chunks : 1u;
-}
+inline uint32_t chunks_for(uint32_t grid) { return grid % kChunks == 0 ? kChunks : 1u; }
 
 /* The step's kernels live in translation units of their own (they build in parallel); launch_step
  * picks one.  wd / gs / keytab / exact select template instances: decay present, gradient scale present,

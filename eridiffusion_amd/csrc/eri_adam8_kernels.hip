@@ -7,10 +7,6 @@
 
 namespace eri {
 
-int g_norm_waves = 4; // waves per workgroup of the gradient-norm pass (eri_adam8_set_tuning key 4)
-int g_chunks = 8;     // contiguous ranges of the block list (BlockWalk); 8 = one per accelerator die
-int g_split_blocks_per_cu = 64; // tables of at most this many full blocks per compute unit take the four-waves-per-block kernel
-
 int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, int dtype_tag,
                 const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg,
                 uint32_t compute_units, void *stream) {
@@ -19,10 +15,11 @@ int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, i
     // Four waves share each block where that is the faster kernel: few blocks (one wave per block would
     // leave the chip idle) and fp32 parameters (measured ahead of the one-wave kernel from 64 Ki to
     // 3 Mi blocks).
-    // The two flags that name a kernel (cross-check and A/B) keep their meaning.
+    // The flags that name a kernel (cross-checks) keep their meaning.
+    const bool one_wave = (h.flags & ERI_ADAM8_FLAG_ONE_WAVE) != 0;
     const bool kernel_named = (h.flags & (ERI_ADAM8_FLAG_BSEARCH | ERI_ADAM8_FLAG_NO_PIPELINE)) != 0;
-    const bool few = (uint64_t)total_blocks <= (uint64_t)compute_units * (uint64_t)g_split_blocks_per_cu;
-    if (!kernel_named && g_split_blocks_per_cu > 0 && (few || !bf16)) {
+    const bool few = (uint64_t)total_blocks <= (uint64_t)compute_units * (uint64_t)kSplitBlocksPerCu;
+    if (!kernel_named && !one_wave && (few || !bf16)) {
         const bool bnb = h.mode == ERI_ADAM8_MODE_BNB;
         const bool wd_s = bnb ? h.weight_decay != 1.0f : h.weight_decay > 0.0f;
         const bool exact_s = !bf16 || (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0;
@@ -266,9 +263,9 @@ int launch_grad_sumsq(const DevTensor *rows, uint32_t n_rows, uint32_t total_blo
                       uint32_t grid, void *stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype_tag == ERI_DTYPE_F32)
-        hipLaunchKernelGGL(grad_sumsq_kernel<false>, dim3(grid), dim3(g_norm_waves * kWave), 0, s, rows, n_rows, total_blocks, partial, chunks_for(grid));
+        hipLaunchKernelGGL(grad_sumsq_kernel<false>, dim3(grid), dim3(kNormWaves * kWave), 0, s, rows, n_rows, total_blocks, partial, chunks_for(grid));
     else
-        hipLaunchKernelGGL(grad_sumsq_kernel<true>, dim3(grid), dim3(g_norm_waves * kWave), 0, s, rows, n_rows, total_blocks, partial, chunks_for(grid));
+        hipLaunchKernelGGL(grad_sumsq_kernel<true>, dim3(grid), dim3(kNormWaves * kWave), 0, s, rows, n_rows, total_blocks, partial, chunks_for(grid));
     return (int)hipGetLastError();
 }
 

@@ -35,7 +35,7 @@ struct RawBlock {
     }
 };
 
-template <int MODE, bool EXACT, bool WD, bool GS, int V = 0>
+template <int MODE, bool EXACT, bool WD, bool GS>
 __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTensor *__restrict__ rows,
                                                                    uint32_t n_rows, uint32_t total_blocks,
                                                                    EriAdam8Hyper h,
@@ -126,7 +126,6 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
             pw[c].y = bf16_pair(pn[2], pn[3]);
             pw[c].z = bf16_pair(pn[4], pn[5]);
             pw[c].w = bf16_pair(pn[6], pn[7]);
-            if (V == 1) __builtin_nontemporal_store(pw[c], as_global(reinterpret_cast<u32x4 *>(p) + c * 64 + lane));
         }
         if (cancel) { // rare: a lane whose update cancelled redoes its 32 parameters with the exact chain
 #pragma unroll
@@ -141,8 +140,7 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
                 pw[c].y = bf16_pair(pn[2], pn[3]);
                 pw[c].z = bf16_pair(pn[4], pn[5]);
                 pw[c].w = bf16_pair(pn[6], pn[7]);
-                if (V == 1) __builtin_nontemporal_store(pw[c], as_global(reinterpret_cast<u32x4 *>(p) + c * 64 + lane));
-            }
+                }
         }
         float nam = lm, nav = lv;
         wave_max2(nam, nav);
@@ -151,42 +149,20 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
             as_global(t.absmax_v)[lb] = nav;
         }
         raw.issue(nt, pblk - nt.full_start, lane); // prefetch: in flight during the requantisation
-        if (V == 0 || V == 3) {
 #pragma unroll
-            for (int c = 0; c < 4; ++c)
-                __builtin_nontemporal_store(pw[c], as_global(reinterpret_cast<u32x4 *>(p) + c * 64 + lane));
-        }
+        for (int c = 0; c < 4; ++c)
+            __builtin_nontemporal_store(pw[c], as_global(reinterpret_cast<u32x4 *>(p) + c * 64 + lane));
         const BlockDiv dm(nam, kKeyScale, kKeyScaleInv), dv(nav, kKeyScale, kKeyScaleInv);
         if (dm.fast && dv.fast) {
-            u32x2 mws[4], vws[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const uint32_t o = c * 512 + lane * 8;
-                requant8<true, true, MODE == ERI_ADAM8_MODE_BNB>(mf + c * 8, vf + c * 8, dm, dv, L, mws[c], vws[c]);
-                if (V != 3) {
-                    __builtin_nontemporal_store(mws[c], as_global(reinterpret_cast<u32x2 *>(mc + o)));
-                    __builtin_nontemporal_store(vws[c], as_global(reinterpret_cast<u32x2 *>(vc + o)));
-                }
-            }
-            if (V == 3) {
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    const uint32_t o = c * 512 + lane * 8;
-                    __builtin_nontemporal_store(mws[c], as_global(reinterpret_cast<u32x2 *>(mc + o)));
-                    __builtin_nontemporal_store(vws[c], as_global(reinterpret_cast<u32x2 *>(vc + o)));
-                }
-            }
-            if (V == 2) {
-#pragma unroll
-                for (int c = 0; c < 4; ++c)
-                    __builtin_nontemporal_store(pw[c], as_global(reinterpret_cast<u32x4 *>(p) + c * 64 + lane));
+                u32x2 mw, vw;
+                requant8<true, true, MODE == ERI_ADAM8_MODE_BNB>(mf + c * 8, vf + c * 8, dm, dv, L, mw, vw);
+                __builtin_nontemporal_store(mw, as_global(reinterpret_cast<u32x2 *>(mc + o)));
+                __builtin_nontemporal_store(vw, as_global(reinterpret_cast<u32x2 *>(vc + o)));
             }
         } else {
-            if (V == 2) {
-#pragma unroll
-                for (int c = 0; c < 4; ++c)
-                    __builtin_nontemporal_store(pw[c], as_global(reinterpret_cast<u32x4 *>(p) + c * 64 + lane));
-            }
             for (int c = 0; c < 4; ++c) {
                 const uint32_t o = c * 512 + lane * 8;
                 u32x2 mw, vw;
@@ -201,23 +177,13 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
     }
 }
 
-int g_pipelined_waves = 0; // measurement switch: waves per workgroup of the pipelined kernel (0 = 12)
-int g_kernel_variant = 0;  // A/B switch for measurements (eri_adam8_set_tuning); 0 is the shipped schedule
-
 namespace {
 
 template <int MODE, bool EXACT, bool WD, bool GS>
 int launch_pipelined(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
                      const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg, hipStream_t s) {
-    auto k = adam8_step_pipelined_kernel<MODE, EXACT, WD, GS>;
-    if constexpr (MODE == ERI_ADAM8_MODE_ERI && !EXACT && WD && !GS) { // only the benchmark configuration carries the variants
-        if (g_kernel_variant == 1) k = adam8_step_pipelined_kernel<MODE, EXACT, WD, GS, 1>;
-        if (g_kernel_variant == 2) k = adam8_step_pipelined_kernel<MODE, EXACT, WD, GS, 2>;
-        if (g_kernel_variant == 3) k = adam8_step_pipelined_kernel<MODE, EXACT, WD, GS, 3>;
-    }
     if (wg > 768) wg = 768;
-    if (g_pipelined_waves >= 1 && g_pipelined_waves <= 12) wg = (uint32_t)g_pipelined_waves * kWave;
-    hipLaunchKernelGGL(k, dim3(grid), dim3(wg), 0, s, rows, n_rows, total_blocks, h,
+    hipLaunchKernelGGL((adam8_step_pipelined_kernel<MODE, EXACT, WD, GS>), dim3(grid), dim3(wg), 0, s, rows, n_rows, total_blocks, h,
                        static_cast<const uint4 *>(lds_image), dev_scale, chunks_for(grid));
     return (int)hipGetLastError();
 }

@@ -198,14 +198,6 @@ struct DeviceCtx {
 DeviceCtx g_ctx[kMaxDevices];
 std::mutex g_ctx_mu;
 
-int env_u32(const char *name, uint32_t lo, uint32_t hi, uint32_t dflt) {
-    const char *s = std::getenv(name);
-    if (!s || !*s) return (int)dflt;
-    long v = std::strtol(s, nullptr, 10);
-    if (v < (long)lo || v > (long)hi) return (int)dflt;
-    return (int)v;
-}
-
 int get_ctx(DeviceCtx **out) {
     int dev = 0;
     ERI_HIP(hipGetDevice(&dev));
@@ -218,9 +210,6 @@ int get_ctx(DeviceCtx **out) {
         hipDeviceProp_t prop;
         ERI_HIP(hipGetDeviceProperties(&prop, dev));
         c.cus = (uint32_t)prop.multiProcessorCount;
-        c.wg = (uint32_t)env_u32("ERI_ADAM8_WG", 64, 1024, 1024) & ~63u;
-        c.wg_per_cu = (uint32_t)env_u32("ERI_ADAM8_WG_PER_CU", 1, 16, 1);
-        eri::g_chunks = env_u32("ERI_ADAM8_CHUNKS", 1, 4096, 8);
         void *image = nullptr;
         ERI_HIP(hipMalloc(&image, eri::kLdsImageBytes));
         const hipError_t e = hipMemcpy(image, t.image.data(), eri::kLdsImageBytes, hipMemcpyHostToDevice);
@@ -287,8 +276,12 @@ struct EriAdam8Table {
     std::vector<int32_t> dtype;
     hipEvent_t uploaded = nullptr;
     bool upload_pending = false;
+    void *upload_stream = nullptr;  // stream of the last upload
+    void *ordered_stream = nullptr; // another stream that has already been made to wait for that upload
+    bool ordered_valid = false;
     double *partial = nullptr; // one sum of squares per wave of the norm pass, per group
-    float *norm_out = nullptr; // device: {norm, clip factor}
+    float *norm_out = nullptr; // device: {norm, clip factor, 64-bit count}, owned by the table
+    float *norm_last = nullptr; // where the last norm pass left its result: norm_out, or the caller's buffer
     uint32_t n_partial = 0;
     double *qerr = nullptr;    // device: per row {sum |m - deq m|, sum |v - deq v|}, groups back to back
     bool qerr_valid = false;
@@ -362,6 +355,36 @@ int upload(EriAdam8Table *t, void *stream) {
     }
     ERI_HIP(hipEventRecord(t->uploaded, static_cast<hipStream_t>(stream)));
     t->upload_pending = true;
+    t->upload_stream = stream;
+    t->ordered_valid = false;
+    return 0;
+}
+
+/* Work that reads the device rows must run after their upload.  On the upload's own stream that is stream
+ * order; another stream is made to wait for the upload's event (no host wait).  A stream that is being
+ * captured into a graph cannot wait for an event outside the graph, so there the host waits for the
+ * upload instead, once. */
+int order_after_upload(EriAdam8Table *t, void *stream) {
+    if (!t->upload_pending || stream == t->upload_stream) return 0;
+    if (t->ordered_valid && stream == t->ordered_stream) return 0;
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &cs) != hipSuccess) {
+        (void)hipGetLastError();
+        cs = hipStreamCaptureStatusNone;
+    }
+    if (cs == hipStreamCaptureStatusActive) {
+        const hipError_t e = hipEventSynchronize(t->uploaded);
+        if (e != hipSuccess) {
+            hip_fail(e, "hipEventSynchronize");
+            return fail((int)e, "the launch table was uploaded on another stream and that copy may not have finished: "
+                                "create or update the table on the stream being captured, or synchronise before the capture");
+        }
+        t->upload_pending = false;
+        return 0;
+    }
+    ERI_HIP(hipStreamWaitEvent(static_cast<hipStream_t>(stream), t->uploaded, 0));
+    t->ordered_stream = stream;
+    t->ordered_valid = true;
     return 0;
 }
 
@@ -413,15 +436,7 @@ int eri_hip_malloc_zeroed(int device, size_t bytes, void **out) {
     ERI_HIP(hipGetDevice(&prev));
     if (prev != device) ERI_HIP(hipSetDevice(device));
     void *p = nullptr;
-    static const bool contiguous = std::getenv("ERI_HIP_MALLOC_CONTIGUOUS") && std::atoi(std::getenv("ERI_HIP_MALLOC_CONTIGUOUS")) != 0;
-    auto device_alloc = [&](void **q) -> hipError_t {
-        if (contiguous && bytes >= kRecycleThreshold) {
-            hipError_t ce = hipExtMallocWithFlags(q, bytes, hipDeviceMallocContiguous);
-            if (ce == hipSuccess) return ce;
-            (void)hipGetLastError();
-        }
-        return hipMalloc(q, bytes);
-    };
+    auto device_alloc = [&](void **q) -> hipError_t { return hipMalloc(q, bytes); };
     hipError_t e = device_alloc(&p);
     // Placement conditioning.  On MI355X the first physical placement a large allocation receives
     // sustains visibly less write bandwidth than the placement the same request receives once the
@@ -511,42 +526,6 @@ int eri_hip_mem_info(size_t *free_bytes, size_t *total_bytes) {
 }
 
 // ---- optimizer ------------------------------------------------------------------------------
-
-static int g_grid_override = 0; // measurement switch: persistent workgroups of the step (0 = one per slot)
-
-int eri_adam8_set_tuning(int key, int value) {
-    if (key == 5) {
-        if (value < 0 || value > (1 << 20)) return fail(ERI_ERR_ARG, "blocks per compute unit out of range");
-        eri::g_split_blocks_per_cu = value;
-        return 0;
-    }
-    if (key == 4) {
-        if (value != 1 && value != 2 && value != 4 && value != 8 && value != 16) return fail(ERI_ERR_ARG, "waves per workgroup must be 1, 2, 4, 8 or 16");
-        eri::g_norm_waves = value;
-        return 0;
-    }
-    if (key == 3) {
-        if (value < 0 || value > 12) return fail(ERI_ERR_ARG, "waves per workgroup out of range");
-        eri::g_pipelined_waves = value;
-        return 0;
-    }
-    if (key == 2) {
-        if (value < 1 || value > 4096) return fail(ERI_ERR_ARG, "chunk count out of range");
-        eri::g_chunks = value;
-        return 0;
-    }
-    if (key == 1) {
-        if (value < 0 || value > 65536) return fail(ERI_ERR_ARG, "grid override out of range");
-        g_grid_override = value;
-        return 0;
-    }
-    if (key == 0) {
-        if (value < 0 || value > 3) return fail(ERI_ERR_ARG, "kernel variant out of range");
-        eri::g_kernel_variant = value;
-        return 0;
-    }
-    return fail(ERI_ERR_ARG, "unknown tuning key");
-}
 
 int eri_adam8_init(void) {
     DeviceCtx *c = nullptr;
@@ -703,17 +682,19 @@ int eri_adam8_step_table(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream)
     const bool clip = (h->flags & ERI_ADAM8_FLAG_CLIP_FROM_TABLE) != 0;
     const bool scaled = (h->flags & ERI_ADAM8_FLAG_GRAD_SCALE) != 0;
     if (clip) { // checked for every group before the first launch: a refused step changes nothing
-        if (!t->norm_out) return fail(ERI_ERR_ARG, "ERI_ADAM8_FLAG_CLIP_FROM_TABLE without a prior eri_adam8_grad_norm");
+        if (!t->norm_last) return fail(ERI_ERR_ARG, "ERI_ADAM8_FLAG_CLIP_FROM_TABLE without a prior eri_adam8_grad_norm");
         for (auto &g : t->groups)
             if (g.n && !scaled && !g.unit_scales)
                 return fail(ERI_ERR_ARG, "ERI_ADAM8_FLAG_CLIP_FROM_TABLE needs per-tensor grad_scale = 1 unless ERI_ADAM8_FLAG_GRAD_SCALE is set");
     }
+    rc = order_after_upload(t, stream);
+    if (rc) return rc;
     for (auto &g : t->groups) {
         if (g.n == 0) continue;
         // One wavefront per block.  A small table gets smaller workgroups so that its blocks still
         // spread over every compute unit instead of filling a few of them.
         uint32_t waves_per_wg = ctx->wg / eri::kWave;
-        const uint32_t slots = g_grid_override ? (uint32_t)g_grid_override : ctx->cus * ctx->wg_per_cu;
+        const uint32_t slots = ctx->cus * ctx->wg_per_cu;
         const uint32_t work = g.total_blocks > g.n ? g.total_blocks : g.n; // full blocks, or one tail per row
         const uint32_t per_slot = (work + slots - 1) / slots;
         if (per_slot < waves_per_wg) waves_per_wg = per_slot < 4 ? 4 : per_slot;
@@ -724,7 +705,7 @@ int eri_adam8_step_table(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream)
         EriAdam8Hyper hh = *h;
         const float *dev_scale = nullptr;
         if (clip) {
-            dev_scale = t->norm_out + 1;
+            dev_scale = t->norm_last + 1;
             if (!scaled) { // the scale path is needed; neutral host-side factors
                 hh.flags |= ERI_ADAM8_FLAG_GRAD_SCALE;
                 hh.grad_scale = 1.0f;
@@ -736,37 +717,61 @@ int eri_adam8_step_table(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream)
     return 0;
 }
 
+/* The two launches of the gradient-norm pass.  `partial` holds room for `pairs` {sum, count} pairs. */
+static int grad_norm_launch(EriAdam8Table *t, DeviceCtx *ctx, float max_norm, float denom_eps, double *partial,
+                            uint32_t pairs, float *result, void *stream) {
+    const uint32_t wpw = (uint32_t)eri::kNormWaves;
+    const uint32_t grid_cap = ctx->cus * eri::kNormWavesPerCu / wpw; // persistent
+    uint32_t grids[2] = {0, 0}, need = 0;
+    for (int gi = 0; gi < 2; ++gi) {
+        const auto &g = t->groups[gi];
+        if (g.n == 0) continue;
+        const uint32_t work = g.total_blocks > g.n ? g.total_blocks : g.n;
+        uint32_t grid = (work + wpw - 1) / wpw;
+        if (grid > grid_cap) grid = grid_cap;
+        grids[gi] = grid;
+        need += grid * wpw;
+    }
+    if (need > pairs) {
+        char buf[160];
+        std::snprintf(buf, sizeof buf, "the gradient-norm pass of this table needs %u per-wave partial sums, the scratch holds %u",
+                      need, pairs);
+        return fail(ERI_ERR_TOO_LARGE, buf);
+    }
+    int rc = order_after_upload(t, stream);
+    if (rc) return rc;
+    uint32_t off = 0;
+    for (int gi = 0; gi < 2; ++gi) {
+        auto &g = t->groups[gi];
+        if (g.n == 0) continue;
+        rc = eri::launch_grad_sumsq(g.dev, g.n, g.total_blocks, g.dtype, partial + 2 * off, grids[gi], stream);
+        if (rc) return hip_fail((hipError_t)rc, "gradient sum-of-squares launch");
+        off += grids[gi] * wpw;
+    }
+    t->n_partial = off;
+    rc = eri::launch_grad_norm_finish(partial, off, max_norm, denom_eps, result, stream);
+    if (rc) return hip_fail((hipError_t)rc, "gradient norm launch");
+    t->norm_last = result;
+    return 0;
+}
+
 int eri_adam8_grad_norm(EriAdam8Table *t, float max_norm, float denom_eps, void *stream) {
     if (!t) return fail(ERI_ERR_NULL, "table is NULL");
     DeviceCtx *ctx = nullptr;
     int rc = get_ctx_on(t->device, &ctx);
     if (rc) return rc;
-    const uint32_t wpw = (uint32_t)eri::g_norm_waves;
-    const uint32_t grid_cap = ctx->cus * eri::kNormWavesPerCu / wpw; // persistent
     // two groups at most, and per wave a sum of squares and a count
-    if (!t->partial) ERI_HIP(hipMalloc((void **)&t->partial, sizeof(double) * 2 * 2 * ctx->cus * eri::kNormWavesPerCu));
+    const uint32_t pairs = 2 * ctx->cus * eri::kNormWavesPerCu;
+    if (!t->partial) ERI_HIP(hipMalloc((void **)&t->partial, sizeof(double) * 2 * pairs));
     if (!t->norm_out) ERI_HIP(hipMalloc((void **)&t->norm_out, sizeof(float) * 4)); // norm, scale, 64-bit count
-    uint32_t off = 0;
-    for (auto &g : t->groups) {
-        if (g.n == 0) continue;
-        const uint32_t work = g.total_blocks > g.n ? g.total_blocks : g.n;
-        uint32_t grid = (work + wpw - 1) / wpw;
-        if (grid > grid_cap) grid = grid_cap;
-        rc = eri::launch_grad_sumsq(g.dev, g.n, g.total_blocks, g.dtype, t->partial + 2 * off, grid, stream);
-        if (rc) return hip_fail((hipError_t)rc, "gradient sum-of-squares launch");
-        off += grid * wpw;
-    }
-    t->n_partial = off;
-    rc = eri::launch_grad_norm_finish(t->partial, t->n_partial, max_norm, denom_eps, t->norm_out, stream);
-    if (rc) return hip_fail((hipError_t)rc, "gradient norm launch");
-    return 0;
+    return grad_norm_launch(t, ctx, max_norm, denom_eps, t->partial, pairs, t->norm_out, stream);
 }
 
 int eri_adam8_grad_norm_read(EriAdam8Table *t, float *norm, float *scale, void *stream) {
     if (!t) return fail(ERI_ERR_NULL, "table is NULL");
-    if (!t->norm_out) return fail(ERI_ERR_ARG, "no gradient norm has been computed for this table");
+    if (!t->norm_last) return fail(ERI_ERR_ARG, "no gradient norm has been computed for this table");
     float host[2] = {0.0f, 1.0f};
-    ERI_HIP(hipMemcpyAsync(host, t->norm_out, sizeof host, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream)));
+    ERI_HIP(hipMemcpyAsync(host, t->norm_last, sizeof host, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream)));
     ERI_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
     if (norm) *norm = host[0];
     if (scale) *scale = host[1];
@@ -775,9 +780,9 @@ int eri_adam8_grad_norm_read(EriAdam8Table *t, float *norm, float *scale, void *
 
 int eri_adam8_grad_nonfinite_read(EriAdam8Table *t, uint64_t *count, void *stream) {
     if (!t || !count) return fail(ERI_ERR_NULL, "table or count is NULL");
-    if (!t->norm_out) return fail(ERI_ERR_ARG, "no gradient norm has been computed for this table");
+    if (!t->norm_last) return fail(ERI_ERR_ARG, "no gradient norm has been computed for this table");
     unsigned long long host = 0;
-    ERI_HIP(hipMemcpyAsync(&host, t->norm_out + 2, sizeof host, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream)));
+    ERI_HIP(hipMemcpyAsync(&host, t->norm_last + 2, sizeof host, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream)));
     ERI_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
     *count = host;
     return 0;
@@ -791,14 +796,16 @@ int eri_adam8_quant_error(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream
     int rc = get_ctx_on(t->device, &ctx);
     if (rc) return rc;
     if (!t->qerr) ERI_HIP(hipMalloc((void **)&t->qerr, sizeof(double) * 2 * t->n));
+    rc = order_after_upload(t, stream);
+    if (rc) return rc;
     uint32_t off = 0;
     for (auto &g : t->groups) {
         if (g.n == 0) continue;
         EriAdam8Hyper hh = *h;
         const float *dev_scale = nullptr;
         if (hh.flags & ERI_ADAM8_FLAG_CLIP_FROM_TABLE) {
-            if (!t->norm_out) return fail(ERI_ERR_ARG, "ERI_ADAM8_FLAG_CLIP_FROM_TABLE without a prior eri_adam8_grad_norm");
-            dev_scale = t->norm_out + 1;
+            if (!t->norm_last) return fail(ERI_ERR_ARG, "ERI_ADAM8_FLAG_CLIP_FROM_TABLE without a prior eri_adam8_grad_norm");
+            dev_scale = t->norm_last + 1;
             if (!(hh.flags & ERI_ADAM8_FLAG_GRAD_SCALE)) {
                 hh.flags |= ERI_ADAM8_FLAG_GRAD_SCALE;
                 hh.grad_scale = 1.0f;

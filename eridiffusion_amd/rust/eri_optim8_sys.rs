@@ -17,6 +17,7 @@ pub const ERI_ADAM8_FLAG_EXACT_PARAM: u32 = 2;
 pub const ERI_ADAM8_FLAG_BSEARCH: u32 = 4;
 pub const ERI_ADAM8_FLAG_NO_PIPELINE: u32 = 8;
 pub const ERI_ADAM8_FLAG_CLIP_FROM_TABLE: u32 = 16;
+pub const ERI_ADAM8_FLAG_ONE_WAVE: u32 = 32;
 
 #[repr(C)]
 #[derive(Clone, Copy, Default)]
@@ -80,7 +81,6 @@ extern "C" {
     pub fn eri_hip_mem_info(free_bytes: *mut usize, total_bytes: *mut usize) -> c_int;
     // the step
     pub fn eri_adam8_init() -> c_int;
-    pub fn eri_adam8_set_tuning(key: c_int, value: c_int) -> c_int;
     pub fn eri_adam8_get_maps(signed256: *mut f32, unsigned256: *mut f32) -> c_int;
     pub fn eri_adam8_table_image(out: *mut c_void, cap: usize, bytes: *mut usize, offsets: *mut u32) -> c_int;
     pub fn eri_adam8_hyper_pack(lr: f64, beta1: f64, beta2: f64, eps: f64, weight_decay: f64, step: u64, mode: c_int, flags: u32, out: *mut EriAdam8Hyper) -> c_int;

@@ -64,8 +64,7 @@ int eri_hip_get_device(int *device);
 /* 256-byte aligned, zero-filled.  Allocations of 64 MB and more are allocated, released and allocated
  * again before they are handed out: on MI355X the first physical placement a large request receives
  * sustains visibly less bandwidth than the one it receives after the range went back to the driver.
- * Environment: ERI_HIP_MALLOC_RECYCLE=0 switches that off; ERI_HIP_MALLOC_CONTIGUOUS=1 asks the driver
- * for physically contiguous memory for such allocations (falls back silently; measurement aid). */
+ * Environment: ERI_HIP_MALLOC_RECYCLE=0 switches that off. */
 int eri_hip_malloc_zeroed(int device, size_t bytes, void **out);
 int eri_hip_free(void *ptr);
 void *eri_hip_host_alloc(size_t bytes);                          /* pinned; NULL on failure */
@@ -106,9 +105,13 @@ enum {
                                              the plain one-wave-per-block kernel whatever the table size) */
     ERI_ADAM8_FLAG_NO_PIPELINE = 1u << 3, /* use the plain one-wave-per-block kernel: not the one that
                                              prefetches the next block (BF16), not the four-waves-per-
-                                             block one (small tables).  Same results; for A/B measurements */
-    ERI_ADAM8_FLAG_CLIP_FROM_TABLE = 1u << 4 /* also multiply gradients by the clip factor the last
+                                             block one (small tables).  Same results; a cross-check */
+    ERI_ADAM8_FLAG_CLIP_FROM_TABLE = 1u << 4, /* also multiply gradients by the clip factor the last
                                              eri_adam8_grad_norm left in the table (device memory) */
+    ERI_ADAM8_FLAG_ONE_WAVE = 1u << 5     /* never take the four-waves-per-block kernel, which small and F32
+                                             tables get by default: a small BF16 table then runs on the
+                                             prefetching kernel.  Same results; lets tests reach every
+                                             kernel with small inputs */
 };
 
 /* Per-step scalars, already cast where the reference casts them.  Fill with eri_adam8_hyper_pack. */
@@ -151,15 +154,6 @@ typedef struct EriAdam8Table EriAdam8Table; /* device-resident copy of a launch 
 /* Loads the quantisation tables onto the current device.  Optional: the first table does it. */
 int eri_adam8_init(void);
 
-/* Measurement switches, not part of the optimizer's behaviour (all settings give identical results):
- * key 0 = store schedule of the bf16 step kernel (0 = shipped), key 1 = number of persistent workgroups
- * (0 = one per compute unit), key 2 = contiguous ranges the block list is cut into (8 = shipped, one per
- * accelerator die; 1 = plain grid stride), key 3 = waves per workgroup of the bf16 step kernel (0 = 12), key 4 = waves per workgroup of the
- * gradient-norm pass (4 = shipped; set before a table's first norm), key 5 = largest table, in full blocks
- * per compute unit, that takes the four-waves-per-block kernel (64 = shipped, 0 = never; fp32 tables
- * take that kernel at every size unless this is 0). */
-int eri_adam8_set_tuning(int key, int value);
-
 /* The two 256-entry maps (code -> value in [-1, 1] / [0, 1]) the states are expressed in. */
 int eri_adam8_get_maps(float *signed256, float *unsigned256);
 
@@ -167,7 +161,11 @@ int eri_adam8_get_maps(float *signed256, float *unsigned256);
 int eri_adam8_state_init(uint8_t *m, uint8_t *v, float *absmax_m, float *absmax_v, uint64_t numel,
                          void *stream);
 
-/* Validates `rows` and uploads them.  The steady-state step then allocates nothing. */
+/* Validates `rows` and uploads them.  The steady-state step then allocates nothing.
+ * The upload is asynchronous on `stream`.  A later call that reads the table on another stream is ordered
+ * after the upload by the library (the other stream waits for the upload's event, the host does not);
+ * only a stream that is being captured into a HIP graph cannot wait for an event outside the graph, and
+ * there the host waits for the upload once instead. */
 int eri_adam8_table_create(const EriAdam8Tensor *rows, uint32_t n, void *stream, EriAdam8Table **out);
 /* Same tensors (count, numel, dtype), new pointers / grad_scale -- e.g. fresh gradient buffers. */
 int eri_adam8_table_update(EriAdam8Table *table, const EriAdam8Tensor *rows, uint32_t n, void *stream);

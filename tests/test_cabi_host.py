@@ -35,6 +35,27 @@ def test_rust_binding_source_declares_every_symbol():
     assert bound == declared, bound ^ declared
 
 
+def test_build_rs_compiles_the_objects_of_the_makefile():
+    """The crate's build script and csrc/Makefile must build the same objects from the same sources with
+    the same defines: the Rust crate is never compiled here, so a file missing from its list would only
+    show as an undefined symbol at the maintainer's link step."""
+    csrc = os.path.join(ROOT, "eridiffusion_amd", "csrc")
+    make = open(os.path.join(csrc, "Makefile")).read().replace("\\\n", " ")
+    objs = re.search(r"^OBJS\s*:=(.*)$", make, re.M).group(1).split()
+    want = set()
+    for obj in objs:
+        rule = re.search(r"^%s:\s*(\S+).*\n\t(.*)$" % re.escape(obj), make, re.M)
+        assert rule, obj
+        define = re.search(r"(-DERI_\w+=\w+)", rule.group(2))
+        want.add((rule.group(1), define.group(1) if define else ""))
+    assert len(want) == len(objs)
+    rust = open(os.path.join(ROOT, "eridiffusion_amd", "rust", "build.rs")).read()
+    got = set(re.findall(r'\("([\w.]+\.(?:hip|cpp))",\s*"\w+",\s*"([^"]*)",\s*(?:true|false)\)', rust))
+    assert got == want, got ^ want
+    for src, _ in want:
+        assert os.path.exists(os.path.join(csrc, src)), src
+
+
 def test_struct_layouts_match_the_header():
     assert C.sizeof(L.Hyper) == 48
     assert C.sizeof(L.TensorRow) == 72
@@ -90,7 +111,8 @@ def test_table_validation_codes():
         assert rc == -4 and "dtype" in msg
     rc, msg = _create([_row(), _row(block_start=3)])
     assert rc == -5 and "expected 2" in msg
-    assert _create([_row(numel=2049), _row(block_start=2)])[0] != -5 or True
+    # a ragged row counts its partial block: these rows pass validation (what remains is the device, absent here)
+    assert _create([_row(numel=2049), _row(block_start=2)])[0] >= 0
     out = C.c_void_p()
     assert L.lib().eri_adam8_table_create(None, 1, None, C.byref(out)) == -1
     arr = (L.TensorRow * 1)(_row())

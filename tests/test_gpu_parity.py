@@ -24,10 +24,13 @@ def which_kernels(request):
     """The tables of these tests are small, so by default they all run on the four-waves-per-block kernel.
     Every test therefore runs twice: as shipped, and with that kernel switched off, which sends bf16 tables
     to the pipelined kernel and fp32 tables to the plain one."""
-    L = _lib()
-    L.check(L.lib().eri_adam8_set_tuning(5, 64 if request.param.startswith("split") else 0), "set_tuning")
+    global KERNEL_FLAGS
+    KERNEL_FLAGS = 0 if request.param.startswith("split") else _lib().FLAG_ONE_WAVE
     yield request.param
-    L.check(L.lib().eri_adam8_set_tuning(5, 64), "set_tuning")
+    KERNEL_FLAGS = 0
+
+
+KERNEL_FLAGS = 0
 
 
 def _lib():
@@ -57,7 +60,7 @@ def gpu_steps(gt, steps_grads, first_step, mode=0, flags=0, wd=WD, lr=LR, grad_s
         if gs is not None:
             gt.set_grads(gs)
         step = first_step + k
-        h = L.hyper_pack(lr, B1, B2, EPS, wd, step - 1 if mode == 1 else step, mode, flags, grad_scale)
+        h = L.hyper_pack(lr, B1, B2, EPS, wd, step - 1 if mode == 1 else step, mode, flags | KERNEL_FLAGS, grad_scale)
         if use_multi:
             L.check(L.lib().eri_adam8_step_multi(rows, len(rows), C.byref(h), _stream()), "step_multi")
         else:

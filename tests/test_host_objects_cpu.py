@@ -183,7 +183,6 @@ def test_state_file_parsers_survive_random_corruption(tmp_path):
         path.write_bytes(mutate(good_st if use_st else good_bc))
         fn = L.lib().eri_adam8bit_load_state if use_st else L.lib().eri_adam8bit_load_legacy_state
         rc = fn(opt, str(path).encode())
-        assert rc != 0 or True
         if rc == -6:
             refused += 1
             assert L.lib().eri_adam8bit_get_step(opt) == 0
