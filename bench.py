@@ -33,6 +33,14 @@ def parse():
     ap.add_argument("--kernel", choices=["adam8", "adam8_clip", "grad_norm", "adamw32", "ema"], default="adam8",
                     help="what one step is: the 8-bit AdamW step (headline), the same preceded by the device-side "
                          "gradient norm, the norm alone, the 32-bit AdamW sibling, or the EMA sweep")
+    ap.add_argument("--mode", choices=["eri", "l2"], default="eri",
+                    help="arithmetic of the table API's step: the list optimizer's (adam8bit_enhanced.rs) or the "
+                         "functional update's (adam8bit.rs, what --api functional always runs)")
+    ap.add_argument("--api", choices=["table", "functional", "functional_update"], default="table",
+                    help="table: eri_adam8_step_table on a launch table built once (headline).  functional: the "
+                         "per-name optimizer, all tensors through one eri_adam8bit_fn_update_many call per step, "
+                         "each step writing into the other of two output sets (update() returns a new tensor).  "
+                         "functional_update: the same through one batched eri_adam8bit_fn_update call per tensor")
     ap.add_argument("--alloc", choices=["arena", "tensor"], default="arena",
                     help="one flat allocation per kind of buffer (library allocator), or one torch allocation per "
                          "tensor and buffer (how a tensor runtime holds parameters and states)")
@@ -218,7 +226,43 @@ def main():
     elif args.kernel == "adam8_clip":
         bytes_per_param += esz + 4.0 / 2048
 
+    fn_opt = None
+    if args.api != "table":
+        if args.kernel != "adam8":
+            sys.exit("--api functional runs the 8-bit step only")
+        n_t = len(sizes)
+        a_p2 = Alloc(torch, [n * esz for n in sizes])  # the other output set
+        extra.append(a_p2)
+        fn_opt = C.c_void_p()
+        L.check(L.lib().eri_adam8bit_fn_with_params(*hyper_args, stream, C.byref(fn_opt)), "fn_with_params")
+        L.check(L.lib().eri_adam8bit_fn_set_batching(fn_opt, 1), "fn_set_batching")
+        tag = L.DTYPE_BF16 if bf16 else L.DTYPE_F32
+        fn_names = [name.encode() for name, _ in tensors]
+        c_names = (C.c_char_p * n_t)(*fn_names)
+        c_numels = (C.c_uint64 * n_t)(*sizes)
+        c_tags = (C.c_int32 * n_t)(*([tag] * n_t))
+        ptrs = lambda a: (C.c_void_p * n_t)(*[a.ptr(i) for i in range(n_t)])
+        c_g = ptrs(a_g)
+        sets = [(ptrs(a_p), ptrs(a_p2)), (ptrs(a_p2), ptrs(a_p))]  # (read from, write to), alternating
+        raw = [([a_p.ptr(i) for i in range(n_t)], [a_p2.ptr(i) for i in range(n_t)]),
+               ([a_p2.ptr(i) for i in range(n_t)], [a_p.ptr(i) for i in range(n_t)])]
+        g_raw = [a_g.ptr(i) for i in range(n_t)]
+
     def step(t):
+        if fn_opt is not None:
+            if args.api == "functional":
+                src, dst = sets[t & 1]
+                L.check(L.lib().eri_adam8bit_fn_update_many(fn_opt, c_names, src, c_g, c_numels, c_tags, None, dst, n_t),
+                        "fn_update_many")
+            else:
+                src, dst = raw[t & 1]
+                upd = L.lib().eri_adam8bit_fn_update
+                for i in range(n_t):
+                    rc = upd(fn_opt, fn_names[i], src[i], g_raw[i], sizes[i], tag, tag, dst[i])
+                    if rc:
+                        L.check(rc, "fn_update")
+            L.check(L.lib().eri_adam8bit_fn_step(fn_opt), "fn_step")
+            return
         if args.kernel == "adamw32":
             L.check(L.lib().eri_adamw32_step_multi(rows32, len(sizes), C.byref(h32), stream), "adamw32")
             return
@@ -231,7 +275,7 @@ def main():
             if args.kernel == "grad_norm":
                 return
             flags |= L.FLAG_CLIP_FROM_TABLE
-        h = L.hyper_pack(*hyper_args, t, L.MODE_ERI, flags)
+        h = L.hyper_pack(*hyper_args, t, L.MODE_L2 if args.mode == "l2" else L.MODE_ERI, flags)
         L.check(L.lib().eri_adam8_step_table(table, C.byref(h), stream), "step_table")
 
     t = 0
@@ -274,7 +318,8 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": args.config, "tensors": len(sizes), "params": n_params, "blocks": n_blocks,
-                   "kernel": args.kernel, "param_dtype": dt_name, "state": "uint8 m/v + fp32 absmax per 2048-block", "flags": args.flags,
+                   "kernel": args.kernel, "api": args.api, "mode": "l2" if args.api != "table" else args.mode,
+                   "param_dtype": dt_name, "state": "uint8 m/v + fp32 absmax per 2048-block", "flags": args.flags,
                    "resident_gb": round((n_params * (2 * esz + 2) + n_blocks * 8) / 1e9, 2)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                      "frac": achieved / PEAK_HBM_GBPS, "traffic": traffic,
@@ -284,6 +329,8 @@ def main():
                      "algorithmic_bytes": algo_bytes},
     }
     L.lib().eri_adam8_table_destroy(table)
+    if fn_opt is not None:
+        L.lib().eri_adam8bit_fn_destroy(fn_opt)
     for a in [a_p, a_g, a_m, a_v, a_am, a_av] + extra:
         a.free()
     if args.cpu_sample > 0:

@@ -25,7 +25,8 @@ class Hyper(C.Structure):
 class TensorRow(C.Structure):
     _fields_ = [("p", C.c_void_p), ("g", C.c_void_p), ("m", C.c_void_p), ("v", C.c_void_p),
                 ("absmax_m", C.c_void_p), ("absmax_v", C.c_void_p), ("numel", C.c_uint64),
-                ("block_start", C.c_uint64), ("dtype_tag", C.c_int32), ("grad_scale", C.c_float)]
+                ("block_start", C.c_uint64), ("dtype_tag", C.c_int32), ("grad_scale", C.c_float),
+                ("p_src", C.c_void_p), ("grad_f32", C.c_int32), ("reserved", C.c_int32)]
 
 
 class Adam8bitConfigC(C.Structure):
@@ -102,6 +103,7 @@ EXPORTS = {
     # ---- include/eri_adam8bit.h
     "eri_param_create": (C.c_int, [C.c_void_p, C.c_uint64, C.c_int, C.POINTER(C.c_void_p)]),
     "eri_param_set_grad": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "eri_param_set_grad_typed": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int]),
     "eri_param_set_data": (C.c_int, [C.c_void_p, C.c_void_p]),
     "eri_param_retain": (C.c_int, [C.c_void_p]),
     "eri_param_release": (C.c_int, [C.c_void_p]),
@@ -117,6 +119,8 @@ EXPORTS = {
     "eri_adam8bit_get_step": (C.c_uint64, [C.c_void_p]),
     "eri_adam8bit_set_grad_scale": (C.c_int, [C.c_void_p, C.c_float]),
     "eri_adam8bit_set_param_grad_scale": (C.c_int, [C.c_void_p, C.c_uint32, C.c_float]),
+    "eri_adam8bit_set_min_8bit_size": (C.c_int, [C.c_void_p, C.c_uint64]),
+    "eri_adam8bit_state32_ptrs": (C.c_int, [C.c_void_p, C.c_uint32, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p)]),
     "eri_adam8bit_set_max_grad_norm": (C.c_int, [C.c_void_p, C.c_float, C.c_float]),
     "eri_ema_new": (C.c_int, [C.c_float, C.c_int, C.c_float, C.c_void_p, C.POINTER(C.c_void_p)]),
     "eri_ema_destroy": (C.c_int, [C.c_void_p]),
@@ -144,7 +148,12 @@ EXPORTS = {
     "eri_adam8bit_state_ptrs": (C.c_int, [C.c_void_p, C.c_uint32] + [C.POINTER(C.c_void_p)] * 4),
     "eri_adam8bit_fn_with_params": (C.c_int, [C.c_double] * 5 + [C.c_void_p, C.POINTER(C.c_void_p)]),
     "eri_adam8bit_fn_destroy": (C.c_int, [C.c_void_p]),
-    "eri_adam8bit_fn_update": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_uint64, C.c_int, C.c_void_p]),
+    "eri_adam8bit_fn_update": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_uint64, C.c_int, C.c_int, C.c_void_p]),
+    "eri_adam8bit_fn_set_batching": (C.c_int, [C.c_void_p, C.c_int]),
+    "eri_adam8bit_fn_flush": (C.c_int, [C.c_void_p]),
+    "eri_adam8bit_fn_update_many": (C.c_int, [C.c_void_p, C.POINTER(C.c_char_p), C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),
+                                              C.POINTER(C.c_uint64), C.POINTER(C.c_int32), C.POINTER(C.c_int32),
+                                              C.POINTER(C.c_void_p), C.c_uint32]),
     "eri_adam8bit_fn_step": (C.c_int, [C.c_void_p]),
     "eri_adam8bit_fn_set_lr": (C.c_int, [C.c_void_p, C.c_float]),
     "eri_adam8bit_fn_get_step": (C.c_uint64, [C.c_void_p]),

@@ -25,6 +25,15 @@ def _dtype_tag(t: torch.Tensor) -> int:
     raise TypeError("Unsupported: 8-bit Adam takes float32 or bfloat16 parameters, got %s" % t.dtype)
 
 
+def _usable_grad(g: torch.Tensor, p: torch.Tensor) -> torch.Tensor:
+    """The gradient as the step reads it.  A float32 gradient of a bfloat16 parameter goes in as it is: the
+    reference casts gradients to F32 and never rounds them (adam8bit_enhanced.rs:231-235).  Any other
+    mismatch is cast to the parameter's dtype, which for bf16 -> f32 is exact."""
+    if g.dtype != p.dtype and not (p.dtype == torch.bfloat16 and g.dtype == torch.float32):
+        g = g.to(p.dtype)
+    return g.contiguous()
+
+
 def _stream_ptr() -> int:
     return torch.cuda.current_stream().cuda_stream
 
@@ -39,6 +48,7 @@ class Adam8bitConfig:
     amsgrad: bool = False
     block_wise: bool = True
     percentile_clipping: int = 99
+    min_8bit_size: int = 0  # pipeline_flux_lora_1024.rs:451 passes 4096; 0 keeps every parameter 8-bit
 
 
 class Adam8bit:
@@ -62,6 +72,8 @@ class Adam8bit:
                                      C.byref(self._opt)), "eri_adam8bit_new")
         if flags:
             check(lib().eri_adam8bit_set_flags(self._opt, flags), "eri_adam8bit_set_flags")
+        if config.min_8bit_size:
+            check(lib().eri_adam8bit_set_min_8bit_size(self._opt, config.min_8bit_size), "eri_adam8bit_set_min_8bit_size")
         self._live = []
 
     def step(self) -> int:
@@ -70,13 +82,14 @@ class Adam8bit:
         for i, p in enumerate(self.params):
             g = p.grad
             if g is not None:
-                if g.dtype != p.dtype:
-                    g = g.to(p.dtype)
-                g = g.contiguous()
+                g = _usable_grad(g, p)
                 live.append(g)
             check(lib().eri_param_set_data(self._handles[i], p.data_ptr()), "eri_param_set_data")
-            check(lib().eri_param_set_grad(self._handles[i], g.data_ptr() if g is not None else None),
-                  "eri_param_set_grad")
+            if g is None:
+                check(lib().eri_param_set_grad(self._handles[i], None), "eri_param_set_grad")
+            else:
+                check(lib().eri_param_set_grad_typed(self._handles[i], g.data_ptr(), _dtype_tag(g)),
+                      "eri_param_set_grad_typed")
         self._live = live  # cast gradients must outlive the launch
         skipped = C.c_uint32()
         check(lib().eri_adam8bit_step(self._opt, C.byref(skipped)), "eri_adam8bit_step")
@@ -155,14 +168,22 @@ class Adam8bit:
 
 
 class Adam8bitFunctional:
-    """Per-tensor flavour keyed by name: update() returns the new parameter tensor, step() only
-    bumps the counter (adam8bit.rs:89-92,101-208)."""
+    """Per-tensor flavour keyed by name: update() returns the new parameter tensor, step() ends the step
+    (adam8bit.rs:89-92,101-208).
 
-    def __init__(self, learning_rate=1e-4, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.01):
+    batched=False: every update() is one kernel launch and its result is valid at once.
+    batched=True: update() queues, and one launch over everything queued runs at step() / flush(); the
+    tensors update() returned are filled then.  Inputs are kept alive until that launch."""
+
+    def __init__(self, learning_rate=1e-4, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.01, batched=False):
         self._opt = C.c_void_p()
         check(lib().eri_adam8bit_fn_with_params(learning_rate, beta1, beta2, eps, weight_decay, _stream_ptr(),
                                                 C.byref(self._opt)), "eri_adam8bit_fn_with_params")
         self._names: List[str] = []
+        self._live: List[torch.Tensor] = []
+        self._batched = bool(batched)
+        if batched:
+            check(lib().eri_adam8bit_fn_set_batching(self._opt, 1), "eri_adam8bit_fn_set_batching")
 
     @classmethod
     def with_params(cls, learning_rate, beta1, beta2, eps, weight_decay):
@@ -170,22 +191,49 @@ class Adam8bitFunctional:
 
     def step(self) -> None:
         check(lib().eri_adam8bit_fn_step(self._opt), "eri_adam8bit_fn_step")
+        self._live = []
+
+    def flush(self) -> None:
+        check(lib().eri_adam8bit_fn_flush(self._opt), "eri_adam8bit_fn_flush")
+        self._live = []
 
     def set_lr(self, lr: float) -> None:
         check(lib().eri_adam8bit_fn_set_lr(self._opt, lr), "eri_adam8bit_fn_set_lr")
+        self._live = []
 
     def get_step(self) -> int:
         return lib().eri_adam8bit_fn_get_step(self._opt)
 
     def update(self, name: str, param: torch.Tensor, grad: torch.Tensor) -> torch.Tensor:
         p = param.detach().contiguous()
-        g = (grad if grad.dtype == p.dtype else grad.to(p.dtype)).contiguous()
+        g = _usable_grad(grad, p)
         out = torch.empty_like(p)
         check(lib().eri_adam8bit_fn_update(self._opt, name.encode(), p.data_ptr(), g.data_ptr(), p.numel(),
-                                           _dtype_tag(p), out.data_ptr()), "eri_adam8bit_fn_update")
+                                           _dtype_tag(p), _dtype_tag(g), out.data_ptr()), "eri_adam8bit_fn_update")
+        if self._batched:
+            self._live += [p, g, out]
         if name not in self._names:
             self._names.append(name)
         return out
+
+    def update_many(self, params: Dict[str, torch.Tensor], grads: Dict[str, torch.Tensor]) -> Dict[str, torch.Tensor]:
+        """Every named parameter that has a gradient, in one launch; returns the new tensors by name."""
+        names = [n for n in params if n in grads]
+        k = len(names)
+        ps = [params[n].detach().contiguous() for n in names]
+        gs = [_usable_grad(grads[n], p) for n, p in zip(names, ps)]
+        outs = [torch.empty_like(p) for p in ps]
+        c_names = (C.c_char_p * k)(*[n.encode() for n in names])
+        arr = lambda ts: (C.c_void_p * k)(*[t.data_ptr() for t in ts])
+        check(lib().eri_adam8bit_fn_update_many(self._opt, c_names, arr(ps), arr(gs),
+                                                (C.c_uint64 * k)(*[p.numel() for p in ps]),
+                                                (C.c_int32 * k)(*[_dtype_tag(p) for p in ps]),
+                                                (C.c_int32 * k)(*[_dtype_tag(g) for g in gs]), arr(outs), k),
+              "eri_adam8bit_fn_update_many")
+        for n in names:
+            if n not in self._names:
+                self._names.append(n)
+        return dict(zip(names, outs))
 
     def memory_stats(self) -> Tuple[int, int]:
         n, b = C.c_uint64(), C.c_uint64()
@@ -302,10 +350,9 @@ class EMAModel:
 
 def update_params_8bit(optimizer: Adam8bitFunctional, params: Dict[str, torch.Tensor],
                        grads: Dict[str, torch.Tensor]) -> None:
-    """adam8bit.rs:333-345: every named parameter that has a gradient is replaced by its update."""
-    for name in list(params.keys()):
-        if name in grads:
-            params[name] = optimizer.update(name, params[name], grads[name])
+    """adam8bit.rs:333-345: every named parameter that has a gradient is replaced by its update
+    (one launch for all of them instead of the reference's loop of update() calls)."""
+    params.update(optimizer.update_many(params, grads))
 
 
 def create_optimizer(optimizer_type: str, params: List[torch.Tensor], learning_rate=1e-4, weight_decay=0.01,

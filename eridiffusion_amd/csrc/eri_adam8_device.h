@@ -14,9 +14,10 @@ namespace eri {
 constexpr uint32_t kBlock = ERI_ADAM8_BLOCK; /* elements per quantisation block, one wavefront each */
 constexpr uint32_t kWave = 64;
 
-/* One tensor as the kernels see it (64 bytes, read through scalar loads). */
+/* One tensor as the kernels see it (80 bytes, read through scalar loads). */
 struct DevTensor {
-    void *p;
+    void *p;          /* new parameters are written here */
+    const void *p_in; /* old parameters are read from here: p itself for an in-place update */
     const void *g;
     uint8_t *m;
     uint8_t *v;
@@ -25,8 +26,15 @@ struct DevTensor {
     uint64_t numel;
     uint32_t full_start;  /* number of full 2048-element blocks in the rows before this one (same dtype) */
     float grad_scale;
+    uint64_t pad;
 };
-static_assert(sizeof(DevTensor) == 64, "DevTensor must stay 64 bytes");
+static_assert(sizeof(DevTensor) == 80, "DevTensor must stay 80 bytes");
+
+/* How the elements of one group of rows are stored: parameters and gradients F32, both BF16, or BF16
+ * parameters with F32 gradients (the reference casts every gradient to F32 and never rounds it). */
+enum Layout { kLayoutF32 = 0, kLayoutBF16 = 1, kLayoutBF16GradF32 = 2, kLayouts = 3 };
+inline bool layout_param_bf16(int layout) { return layout != kLayoutF32; }
+inline bool layout_grad_bf16(int layout) { return layout == kLayoutBF16; }
 
 /*
  * Requantisation without a search.  The quotient x = value / absmax in [-1, 1] is produced
@@ -68,7 +76,7 @@ static_assert(kLdsImageBytes % 16 == 0, "the image is staged in 16-byte words");
 
 /* Launchers implemented in eri_adam8_kernels.hip; `stream` is a hipStream_t.  All return a
  * hipError_t as int.  `lds_image` is the device copy of the kLdsImageBytes table image. */
-int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_blocks, int dtype_tag,
+int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_blocks, int layout,
                 const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg,
                 uint32_t compute_units, void *stream);
 
@@ -90,19 +98,19 @@ int launch_step_plain_bf16(int mode, bool exact, bool wd, bool gs, bool keytab, 
                            uint32_t total_blocks, const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale,
                            uint32_t grid, uint32_t wg, void *stream);
 /* Four waves per block, for tables of few blocks; `grid` workgroups of 1024 threads. */
-int launch_step_split(bool bf16, int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
+int launch_step_split(int layout, int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
                       uint32_t total_blocks, const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale,
                       uint32_t grid, void *stream);
 int launch_step_pipelined(int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
                           uint32_t total_blocks, const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale,
                           uint32_t grid, uint32_t wg, void *stream);
 /* Sum of |moment - dequantised moment| of the coming step, per row: err[2r] first moment, err[2r+1] second. */
-int launch_quant_error(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_blocks, int dtype_tag,
+int launch_quant_error(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_blocks, int layout,
                        const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale, double *err,
                        uint32_t grid, void *stream);
 /* Gradient norm: one f64 partial per wave (grid * 4 of them), then norm and clip factor into out[0], out[1]. */
 constexpr uint32_t kNormWavesPerCu = 32; // persistent waves of the gradient-norm pass per compute unit
-int launch_grad_sumsq(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_blocks, int dtype_tag,
+int launch_grad_sumsq(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_blocks, bool grad_bf16,
                       double *partial, uint32_t grid, void *stream);
 int launch_grad_norm_finish(const double *partial, uint32_t n, float max_norm, float denom_eps, float *out,
                             void *stream);

@@ -201,15 +201,60 @@ __device__ __forceinline__ float param_exact(float p, float m, float v, const Er
     return p - us;              // :275
 }
 
-/* `cancel` collects (it is only ever set) whether the approximate chain met a subtraction that cancels:
- * the chain's few fp32 ulp of error are measured against the size of the update, so a result more than
- * 2^12 times smaller than the parameter it came from can land more than one bf16 step from the exact
- * chain's.  Callers recompute such elements with param_exact (about one element in 10^5 on trained
- * weights); with EXACT it is never set. */
+/*
+ * bf16 parameters take the hardware square root and reciprocal (1 ulp each) and two fused multiply-adds
+ * instead of the IEEE chain of param_exact, and every element whose bf16 result that could change is
+ * flagged through `recheck` (it is only ever set); callers recompute flagged elements with param_exact.
+ *
+ * Without EXACT (the default arithmetic) the promise is "within one bf16 step of the exact chain".  The
+ * approximate chain's error is a few fp32 ulp of the *update*, so it can only exceed a bf16 step of the
+ * result where p - update cancels: a result more than 2^12 times smaller than its parameter is flagged
+ * (about one element in 10^5 on trained weights).
+ *
+ * With EXACT the promise is the exact chain's bf16 bits.  Write U = (|r| + |p| wd) * step_size for the size
+ * of the update.  Following the roundings of both chains, their results before the last rounding to fp32
+ * differ by at most 6.1 * 2^-23 * U (mode BNB: 5.1 * 2^-23 * |r| * step_size, plus one more fp32 rounding
+ * each for the decay factor).  Two fp32 values round to the same bf16 value unless a tie point of the bf16
+ * grid (the fp32 numbers whose low half is 0x8000) lies between or on them; so if the approximate result
+ * pn is further from the tie point T of its own bf16 interval than
+ *      margin = 8 * 2^-23 * U  +  |pn| * 2^-22      (the second term is at least two fp32 ulp of pn;
+ *                                                     mode BNB: 2^-21, four ulp)
+ * the exact chain's fp32 result lies strictly on the same side of T and both round to the same bf16.
+ * U is bounded without touching p again: |p| <= |pn| + U (up to roundings), hence
+ *      U <= (|r| step_size + wd step_size |pn|) / (1 - wd step_size),
+ * which turns the margin into |r| * c_r + |pn| * c_p with two constants of the launch (ExactMargin).
+ * Everything else -- about four elements in a million on trained weights, every element whose update
+ * cancels its parameter, every NaN or infinity (the comparison is written so that they fail it) -- is
+ * flagged.  The slack between 6.1 and 8 covers the use of the approximate r and the rounding of the
+ * margin's own arithmetic.
+ */
+template <int MODE, bool WD>
+struct ExactMargin {
+    float c_r, c_p;
+    __device__ __forceinline__ explicit ExactMargin(const EriAdam8Hyper &h) {
+        constexpr float kEightUlp = 0x1p-20f; // 8 * 2^-23
+        if (MODE == ERI_ADAM8_MODE_BNB) {
+            c_r = __builtin_fabsf(h.step_size) * kEightUlp;
+            c_p = 0x1p-21f;
+        } else {
+            const float ws = WD ? __builtin_fabsf(h.weight_decay * h.step_size) * 1.001f : 0.0f;
+            // a decay that moves a parameter by half of itself per step leaves no bound: flag everything
+            const float k = ws < 0.5f ? 1.001f / (1.0f - ws) : __builtin_inff();
+            c_r = __builtin_fabsf(h.step_size) * kEightUlp * k;
+            c_p = 0x1p-22f + kEightUlp * ws * k;
+        }
+    }
+    __device__ __forceinline__ bool same_bf16_as_exact(float r, float pn) const {
+        const float margin = __builtin_fmaf(__builtin_fabsf(pn), c_p, __builtin_fabsf(r) * c_r);
+        const float tie = u2f((f2u(pn) & 0xffff0000u) | 0x8000u);
+        return __builtin_fabsf(pn - tie) > margin;
+    }
+};
+
 template <int MODE, bool EXACT, bool BF16, bool WD, bool GS>
 __device__ __forceinline__ void adam_elem(float p, float g, float m_old, float v_old, const EriAdam8Hyper &h,
                                           float gscale, const BlockDiv &dbc1, const BlockDiv &dbc2, float &m,
-                                          float &v, float &pn, bool &cancel) {
+                                          float &v, float &pn, bool &recheck) {
     if (GS) g = g * gscale;
     if (MODE == ERI_ADAM8_MODE_L2 && WD) { // adam8bit.rs:113-120
         float pw = p * h.weight_decay;
@@ -231,28 +276,21 @@ __device__ __forceinline__ void adam_elem(float p, float g, float m_old, float v
         float us = upd * h.step_size; // :196
         if (BF16) us = bf16_round(us); // :197-198
         pn = p - us;                   // :205
-    } else if (MODE == ERI_ADAM8_MODE_BNB) { // h.eps carries sqrt(bc2), h.weight_decay is the factor 1 - lr*wd
-        if (EXACT) {
-            pn = param_exact<MODE, WD>(p, m, v, h);
-        } else { // bf16 parameters: as in mode ERI below, at most one bf16 step away from the exact chain, rarely
-            float den = __builtin_amdgcn_sqrtf(v) + h.eps;
-            float r = m * __builtin_amdgcn_rcpf(den);
-            pn = __builtin_fmaf(-r, h.step_size, p);
-            cancel |= __builtin_fabsf(pn) * 4096.0f < __builtin_fabsf(p);
-            if (WD) pn = pn * h.weight_decay;
-        }
-    } else {
-        if (EXACT) {
-            pn = param_exact<MODE, WD>(p, m, v, h);
+    } else if (!BF16) { // fp32 parameters: every bit of the exact chain counts
+        pn = param_exact<MODE, WD>(p, m, v, h);
+    } else { // h.eps and h.weight_decay of mode BNB carry sqrt(bc2) and the factor 1 - lr*wd
+        float den = __builtin_amdgcn_sqrtf(v) + h.eps;
+        float r = m * __builtin_amdgcn_rcpf(den);
+        if (MODE == ERI_ADAM8_MODE_BNB) {
+            float p0 = __builtin_fmaf(-r, h.step_size, p);
+            pn = WD ? p0 * h.weight_decay : p0;
+            if (EXACT) recheck |= !ExactMargin<MODE, WD>(h).same_bf16_as_exact(r, pn);
+            else recheck |= __builtin_fabsf(p0) * 4096.0f < __builtin_fabsf(p);
         } else {
-            // bf16 parameters: hardware square root and reciprocal (1 ulp each) and two fused
-            // multiply-adds; the fp32 result is within a few ulp of the exact chain, which moves
-            // the bf16 rounding of p by at most one step, rarely
-            float den = __builtin_amdgcn_sqrtf(v) + h.eps;
-            float r = m * __builtin_amdgcn_rcpf(den);
             float u = WD ? __builtin_fmaf(p, h.weight_decay, r) : r;
             pn = __builtin_fmaf(-u, h.step_size, p);
-            cancel |= __builtin_fabsf(pn) * 4096.0f < __builtin_fabsf(p);
+            if (EXACT) recheck |= !ExactMargin<MODE, WD>(h).same_bf16_as_exact(r, pn);
+            else recheck |= __builtin_fabsf(pn) * 4096.0f < __builtin_fabsf(p);
         }
     }
 }
@@ -428,6 +466,7 @@ __device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint
     const size_t e0 = (size_t)lb * kBlock;
     const size_t esz = BF16 ? 2 : 4;
     char *p = static_cast<char *>(t.p) + e0 * esz;
+    const char *p_in = static_cast<const char *>(t.p_in) + e0 * esz;
     const char *g = static_cast<const char *>(t.g) + e0 * esz;
     uint8_t *mc = t.m + e0;
     uint8_t *vc = t.v + e0;
@@ -446,7 +485,7 @@ __device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {
             const uint32_t o = (c0 + d) * 512 + lane * 8;
-            pr[d].load(p, o);
+            pr[d].load(p_in, o);
             gr[d].load(g, o);
             mr[d] = __builtin_nontemporal_load(as_global(reinterpret_cast<const u32x2 *>(mc + o)));
             vr[d] = __builtin_nontemporal_load(as_global(reinterpret_cast<const u32x2 *>(vc + o)));
@@ -517,7 +556,7 @@ __device__ __forceinline__ float load1(const void *base, size_t i) {
     return as_global(static_cast<const float *>(base))[i];
 }
 
-template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB>
+template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB, bool GBF16 = BF16>
 __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint32_t n, uint32_t lane,
                                         const EriAdam8Hyper &h, float gscale, const BlockDiv &dbc1,
                                         const BlockDiv &dbc2, const Lds &L) {
@@ -535,13 +574,15 @@ __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint
         // register budget belongs to their main loop.
         const size_t esz = BF16 ? 2 : 4;
         char *p = static_cast<char *>(t.p) + e0 * esz;
-        const char *g = static_cast<const char *>(t.g) + e0 * esz;
+        const char *p_in = static_cast<const char *>(t.p_in) + e0 * esz;
+        const char *g = static_cast<const char *>(t.g) + e0 * (GBF16 ? 2 : 4);
         const uint32_t passes = (n + 511) / 512;
         for (uint32_t c = 0; c < passes; ++c) {
             const uint32_t o = c * 512 + lane * 8;
             if (o < n) {
-                Raw8<BF16> pr, gr;
-                pr.load(p, o);
+                Raw8<BF16> pr;
+                Raw8<GBF16> gr;
+                pr.load(p_in, o);
                 gr.load(g, o);
                 const u32x2 mr = *as_global(reinterpret_cast<const u32x2 *>(t.m + e0 + o));
                 const u32x2 vr = *as_global(reinterpret_cast<const u32x2 *>(t.v + e0 + o));
@@ -565,8 +606,9 @@ __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint
         for (uint32_t c = 0; c < passes; ++c) {
             const uint32_t o = c * 512 + lane * 8;
             if (o < n) {
-                Raw8<BF16> pr, gr;
-                pr.load(p, o);
+                Raw8<BF16> pr;
+                Raw8<GBF16> gr;
+                pr.load(p_in, o);
                 gr.load(g, o);
                 const u32x2 mr = *as_global(reinterpret_cast<const u32x2 *>(t.m + e0 + o));
                 const u32x2 vr = *as_global(reinterpret_cast<const u32x2 *>(t.v + e0 + o));
@@ -599,7 +641,7 @@ __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint
         const size_t e = e0 + i;
         float m, v, pn;
         bool unused = false;
-        adam_elem<MODE, EXACT, BF16, WD, GS>(load1<BF16>(t.p, e), load1<BF16>(t.g, e), L.map_s[mc[e]] * a_m,
+        adam_elem<MODE, EXACT, BF16, WD, GS>(load1<BF16>(t.p_in, e), load1<GBF16>(t.g, e), L.map_s[mc[e]] * a_m,
                                              L.map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn, unused);
         lm = fmaxf(lm, __builtin_fabsf(m));
         lv = fmaxf(lv, __builtin_fabsf(v));
@@ -611,8 +653,8 @@ __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint
         const size_t e = e0 + i;
         float m, v, pn;
         bool cancel = false;
-        const float p_old = load1<BF16>(t.p, e);
-        adam_elem<MODE, EXACT, BF16, WD, GS>(p_old, load1<BF16>(t.g, e), L.map_s[mc[e]] * a_m,
+        const float p_old = load1<BF16>(t.p_in, e);
+        adam_elem<MODE, EXACT, BF16, WD, GS>(p_old, load1<GBF16>(t.g, e), L.map_s[mc[e]] * a_m,
                                              L.map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn, cancel);
         if (cancel) pn = param_exact<MODE, WD>(p_old, m, v, h);
         const float xm = dm.div_slow(m);

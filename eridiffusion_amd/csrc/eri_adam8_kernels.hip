@@ -7,10 +7,11 @@
 
 namespace eri {
 
-int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, int dtype_tag,
+int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, int layout,
                 const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg,
                 uint32_t compute_units, void *stream) {
-    const bool bf16 = dtype_tag != ERI_DTYPE_F32;
+    const bool bf16 = layout_param_bf16(layout);
+    const bool mixed = layout == kLayoutBF16GradF32; // only the four-waves-per-block kernel reads F32 gradients for BF16 parameters
     const bool gs = (h.flags & ERI_ADAM8_FLAG_GRAD_SCALE) != 0;
     // Four waves share each block where that is the faster kernel: few blocks (one wave per block would
     // leave the chip idle) and fp32 parameters (measured ahead of the one-wave kernel from 64 Ki to
@@ -19,7 +20,7 @@ int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, i
     const bool one_wave = (h.flags & ERI_ADAM8_FLAG_ONE_WAVE) != 0;
     const bool kernel_named = (h.flags & (ERI_ADAM8_FLAG_BSEARCH | ERI_ADAM8_FLAG_NO_PIPELINE)) != 0;
     const bool few = (uint64_t)total_blocks <= (uint64_t)compute_units * (uint64_t)kSplitBlocksPerCu;
-    if (!kernel_named && !one_wave && (few || !bf16)) {
+    if (mixed || (!kernel_named && !one_wave && (few || !bf16))) {
         const bool bnb = h.mode == ERI_ADAM8_MODE_BNB;
         const bool wd_s = bnb ? h.weight_decay != 1.0f : h.weight_decay > 0.0f;
         const bool exact_s = !bf16 || (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0;
@@ -28,7 +29,7 @@ int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, i
         if (need < for_tails) need = for_tails;
         if (need > compute_units) need = compute_units;
         if (need == 0) need = 1;
-        return launch_step_split(bf16, h.mode, exact_s, wd_s, gs, rows, n_rows, total_blocks, h, lds_image, dev_scale, need, stream);
+        return launch_step_split(layout, h.mode, exact_s, wd_s, gs, rows, n_rows, total_blocks, h, lds_image, dev_scale, need, stream);
     }
     if (h.mode == ERI_ADAM8_MODE_BNB) { // slot table only; the decay is a factor
         const bool wd = h.weight_decay != 1.0f;
@@ -259,10 +260,10 @@ __global__ __launch_bounds__(1024) void grad_norm_finish_kernel(const double *__
     }
 }
 
-int launch_grad_sumsq(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, int dtype_tag, double *partial,
+int launch_grad_sumsq(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, bool grad_bf16, double *partial,
                       uint32_t grid, void *stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dtype_tag == ERI_DTYPE_F32)
+    if (!grad_bf16)
         hipLaunchKernelGGL(grad_sumsq_kernel<false>, dim3(grid), dim3(kNormWaves * kWave), 0, s, rows, n_rows, total_blocks, partial, chunks_for(grid));
     else
         hipLaunchKernelGGL(grad_sumsq_kernel<true>, dim3(grid), dim3(kNormWaves * kWave), 0, s, rows, n_rows, total_blocks, partial, chunks_for(grid));
@@ -293,7 +294,7 @@ __global__ __launch_bounds__(256) void quant_error_kernel(const DevTensor *__res
                                                           uint32_t total_blocks, EriAdam8Hyper h,
                                                           const float *__restrict__ lds_image,
                                                           const float *__restrict__ dev_scale,
-                                                          double *__restrict__ err /* [2 * n_rows] */) {
+                                                          double *__restrict__ err /* [2 * n_rows] */, bool grad_f32) {
     __shared__ float tab[1024]; // signed map, unsigned map, signed midpoints, unsigned midpoints
     for (uint32_t i = threadIdx.x; i < 1024; i += blockDim.x) tab[i] = lds_image[i];
     __syncthreads();
@@ -331,7 +332,8 @@ __global__ __launch_bounds__(256) void quant_error_kernel(const DevTensor *__res
             const size_t e = e0 + i;
             float m, v, pn;
             bool unused = false; // the exact chain never sets it
-            adam_elem<MODE, true, BF16, WD, GS>(load1<BF16>(t.p, e), load1<BF16>(t.g, e), map_s[mc[e]] * a_m,
+            const float gr = (BF16 && !grad_f32) ? load1<true>(t.g, e) : load1<false>(t.g, e);
+            adam_elem<MODE, true, BF16, WD, GS>(load1<BF16>(t.p_in, e), gr, map_s[mc[e]] * a_m,
                                                 map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn, unused);
             lm = fmaxf(lm, __builtin_fabsf(m));
             lv = fmaxf(lv, __builtin_fabsf(v));
@@ -344,7 +346,8 @@ __global__ __launch_bounds__(256) void quant_error_kernel(const DevTensor *__res
             const size_t e = e0 + i;
             float m, v, pn;
             bool unused = false; // the exact chain never sets it
-            adam_elem<MODE, true, BF16, WD, GS>(load1<BF16>(t.p, e), load1<BF16>(t.g, e), map_s[mc[e]] * a_m,
+            const float gr = (BF16 && !grad_f32) ? load1<true>(t.g, e) : load1<false>(t.g, e);
+            adam_elem<MODE, true, BF16, WD, GS>(load1<BF16>(t.p_in, e), gr, map_s[mc[e]] * a_m,
                                                 map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn, unused);
             const float qm = map_s[code_bsearch(dm.div_slow(m), mid_s)] * nam;
             const float qv = map_u[code_bsearch(dv.div_slow(v), mid_u)] * nav;
@@ -364,15 +367,16 @@ __global__ void zero_f64_kernel(double *x, uint32_t n) {
     for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) x[i] = 0.0;
 }
 
-int launch_quant_error(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, int dtype_tag,
+int launch_quant_error(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, int layout,
                        const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale, double *err,
                        uint32_t grid, void *stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     const float *img = static_cast<const float *>(lds_image);
     hipLaunchKernelGGL(zero_f64_kernel, dim3(64), dim3(256), 0, s, err, 2 * n_rows);
-    const bool bf16 = dtype_tag != ERI_DTYPE_F32, l2 = h.mode == ERI_ADAM8_MODE_L2;
+    const bool bf16 = layout_param_bf16(layout), l2 = h.mode == ERI_ADAM8_MODE_L2;
+    const bool grad_f32 = !layout_grad_bf16(layout);
     const bool wd = h.weight_decay > 0.0f, gs = (h.flags & ERI_ADAM8_FLAG_GRAD_SCALE) != 0;
-#define ERI_QE(B, M, W, G) hipLaunchKernelGGL((quant_error_kernel<B, M, W, G>), dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, h, img, dev_scale, err)
+#define ERI_QE(B, M, W, G) hipLaunchKernelGGL((quant_error_kernel<B, M, W, G>), dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, h, img, dev_scale, err, grad_f32)
 #define ERI_QE2(B, M) do { if (wd) { if (gs) ERI_QE(B, M, true, true); else ERI_QE(B, M, true, false); } else { if (gs) ERI_QE(B, M, false, true); else ERI_QE(B, M, false, false); } } while (0)
     if (bf16) { if (l2) ERI_QE2(true, ERI_ADAM8_MODE_L2); else ERI_QE2(true, ERI_ADAM8_MODE_ERI); }
     else { if (l2) ERI_QE2(false, ERI_ADAM8_MODE_L2); else ERI_QE2(false, ERI_ADAM8_MODE_ERI); }

@@ -19,7 +19,7 @@ struct RawBlock {
     float a_m, a_v;
     __device__ __forceinline__ void issue(const DevTensor &t, uint32_t lb, uint32_t lane) {
         const size_t e0 = (size_t)lb * kBlock;
-        ERI_GLOBAL const u32x4 *pp = as_global(reinterpret_cast<const u32x4 *>(static_cast<const uint16_t *>(t.p) + e0));
+        ERI_GLOBAL const u32x4 *pp = as_global(reinterpret_cast<const u32x4 *>(static_cast<const uint16_t *>(t.p_in) + e0));
         ERI_GLOBAL const u32x4 *gp = as_global(reinterpret_cast<const u32x4 *>(static_cast<const uint16_t *>(t.g) + e0));
         ERI_GLOBAL const u32x2 *mp = as_global(reinterpret_cast<const u32x2 *>(t.m + e0));
         ERI_GLOBAL const u32x2 *vp = as_global(reinterpret_cast<const u32x2 *>(t.v + e0));

@@ -14,7 +14,7 @@
 
 namespace eri {
 
-template <bool BF16, int MODE, bool EXACT, bool WD, bool GS>
+template <bool BF16, bool GBF16, int MODE, bool EXACT, bool WD, bool GS>
 __global__ __launch_bounds__(1024) void adam8_step_split_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
                                                                 uint32_t total_blocks, EriAdam8Hyper h,
                                                                 const uint4 *__restrict__ lds_image,
@@ -34,7 +34,8 @@ __global__ __launch_bounds__(1024) void adam8_step_split_kernel(const DevTensor 
         DevTensor t;
         uint32_t lb;
         bool active;
-        Raw8<BF16> pr, gr;
+        Raw8<BF16> pr;
+        Raw8<GBF16> gr;
         u32x2 mr, vr;
         float a_m, a_v;
     } q;
@@ -47,8 +48,8 @@ __global__ __launch_bounds__(1024) void adam8_step_split_kernel(const DevTensor 
         q.lb = blk - q.t.full_start;
         const size_t e0 = (size_t)q.lb * kBlock;
         const size_t esz = BF16 ? 2 : 4;
-        q.pr.load(static_cast<const char *>(q.t.p) + e0 * esz, o);
-        q.gr.load(static_cast<const char *>(q.t.g) + e0 * esz, o);
+        q.pr.load(static_cast<const char *>(q.t.p_in) + e0 * esz, o);
+        q.gr.load(static_cast<const char *>(q.t.g) + e0 * (GBF16 ? 2 : 4), o);
         q.mr = __builtin_nontemporal_load(as_global(reinterpret_cast<const u32x2 *>(q.t.m + e0 + o)));
         q.vr = __builtin_nontemporal_load(as_global(reinterpret_cast<const u32x2 *>(q.t.v + e0 + o)));
         q.a_m = as_global(q.t.absmax_m)[q.lb];
@@ -75,7 +76,7 @@ __global__ __launch_bounds__(1024) void adam8_step_split_kernel(const DevTensor 
         const uint32_t n = (uint32_t)(t.numel % kBlock);
         if (n != 0) {
             const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
-            tail_block<BF16, MODE, EXACT, WD, GS, true>(t, (uint32_t)(t.numel / kBlock), n, lane, h, gscale, dbc1, dbc2, L);
+            tail_block<BF16, MODE, EXACT, WD, GS, true, GBF16>(t, (uint32_t)(t.numel / kBlock), n, lane, h, gscale, dbc1, dbc2, L);
         }
     }
 
@@ -135,12 +136,12 @@ __global__ __launch_bounds__(1024) void adam8_step_split_kernel(const DevTensor 
 
 namespace {
 
-template <bool BF16, int MODE, bool EXACT>
+template <bool BF16, bool GBF16, int MODE, bool EXACT>
 int launch_flags(bool wd, bool gs, const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
                  const void *img, const float *dev_scale, uint32_t grid, hipStream_t s) {
 #define ERI_GO(W, G)                                                                                                     \
     do {                                                                                                                 \
-        hipLaunchKernelGGL((adam8_step_split_kernel<BF16, MODE, EXACT, W, G>), dim3(grid), dim3(1024), 0, s, rows, n_rows, \
+        hipLaunchKernelGGL((adam8_step_split_kernel<BF16, GBF16, MODE, EXACT, W, G>), dim3(grid), dim3(1024), 0, s, rows, n_rows, \
                            total_blocks, h, static_cast<const uint4 *>(img), dev_scale);                                  \
         return (int)hipGetLastError();                                                                                   \
     } while (0)
@@ -152,20 +153,27 @@ int launch_flags(bool wd, bool gs, const DevTensor *rows, uint32_t n_rows, uint3
 
 } // namespace
 
-int launch_step_split(bool bf16, int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
+int launch_step_split(int layout, int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
                       uint32_t total_blocks, const EriAdam8Hyper &h, const void *img, const float *dev_scale, uint32_t grid,
                       void *stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define ERI_ARGS wd, gs, rows, n_rows, total_blocks, h, img, dev_scale, grid, s
-    if (!bf16) { // fp32 parameters always take the IEEE square root and division
-        if (mode == ERI_ADAM8_MODE_BNB) return launch_flags<false, ERI_ADAM8_MODE_BNB, true>(ERI_ARGS);
-        if (mode == ERI_ADAM8_MODE_L2) return launch_flags<false, ERI_ADAM8_MODE_L2, true>(ERI_ARGS);
-        return launch_flags<false, ERI_ADAM8_MODE_ERI, true>(ERI_ARGS);
+    if (layout == kLayoutF32) { // fp32 parameters always take the IEEE square root and division
+        if (mode == ERI_ADAM8_MODE_BNB) return launch_flags<false, false, ERI_ADAM8_MODE_BNB, true>(ERI_ARGS);
+        if (mode == ERI_ADAM8_MODE_L2) return launch_flags<false, false, ERI_ADAM8_MODE_L2, true>(ERI_ARGS);
+        return launch_flags<false, false, ERI_ADAM8_MODE_ERI, true>(ERI_ARGS);
     }
-    if (mode == ERI_ADAM8_MODE_BNB)
-        return exact ? launch_flags<true, ERI_ADAM8_MODE_BNB, true>(ERI_ARGS) : launch_flags<true, ERI_ADAM8_MODE_BNB, false>(ERI_ARGS);
-    if (mode == ERI_ADAM8_MODE_L2) return launch_flags<true, ERI_ADAM8_MODE_L2, true>(ERI_ARGS); // always the IEEE chain
-    return exact ? launch_flags<true, ERI_ADAM8_MODE_ERI, true>(ERI_ARGS) : launch_flags<true, ERI_ADAM8_MODE_ERI, false>(ERI_ARGS);
+    // mode L2 always takes the IEEE chain
+#define ERI_BF16(G)                                                                                                          \
+    do {                                                                                                                     \
+        if (mode == ERI_ADAM8_MODE_BNB)                                                                                      \
+            return exact ? launch_flags<true, G, ERI_ADAM8_MODE_BNB, true>(ERI_ARGS) : launch_flags<true, G, ERI_ADAM8_MODE_BNB, false>(ERI_ARGS); \
+        if (mode == ERI_ADAM8_MODE_L2) return launch_flags<true, G, ERI_ADAM8_MODE_L2, true>(ERI_ARGS);                        \
+        return exact ? launch_flags<true, G, ERI_ADAM8_MODE_ERI, true>(ERI_ARGS) : launch_flags<true, G, ERI_ADAM8_MODE_ERI, false>(ERI_ARGS); \
+    } while (0)
+    if (layout == kLayoutBF16) ERI_BF16(true);
+    ERI_BF16(false);
+#undef ERI_BF16
 #undef ERI_ARGS
 }
 

@@ -23,6 +23,7 @@
 #include <memory>
 #include <sstream>
 #include <string>
+#include <string_view>
 #include <vector>
 
 #include "../../include/eri_adam8bit.h"
@@ -77,6 +78,38 @@ struct State8 {
     State8() = default;
     State8(const State8 &) = delete;
     State8 &operator=(const State8 &) = delete;
+};
+
+/* fp32 moments of a parameter that is kept out of the 8-bit format (min_8bit_size), in one device
+ * allocation; zero-filled = the state of a zeros tensor. */
+struct State32 {
+    void *base = nullptr;
+    float *m = nullptr, *v = nullptr;
+    uint64_t numel = 0;
+    int allocate(uint64_t n) {
+        release();
+        int dev = 0;
+        int rc = eri_hip_get_device(&dev);
+        if (rc) return rc;
+        const uint64_t half = align256(n * 4);
+        rc = eri_hip_malloc_zeroed(dev, 2 * half, &base);
+        if (rc) return rc;
+        m = static_cast<float *>(base);
+        v = reinterpret_cast<float *>(static_cast<char *>(base) + half);
+        numel = n;
+        return 0;
+    }
+    void release() {
+        if (base) eri_hip_free(base);
+        base = nullptr;
+        m = v = nullptr;
+        numel = 0;
+    }
+    uint64_t nbytes() const { return 8 * numel; }
+    ~State32() { release(); }
+    State32() = default;
+    State32(const State32 &) = delete;
+    State32 &operator=(const State32 &) = delete;
 };
 
 // ---- a very small safetensors reader / writer ------------------------------------------------
@@ -288,6 +321,7 @@ struct EriParameter {
     const void *grad = nullptr;
     uint64_t numel = 0;
     int32_t dtype = 0;
+    int32_t grad_dtype = 0; // dtype of *grad: the parameter's, or F32 for a BF16 parameter
     int refs = 1;
 };
 
@@ -306,6 +340,8 @@ struct EriAdam8bit {
     bool track_qerr = false, have_qerr = false;
     std::vector<float> param_scale;
     std::vector<std::unique_ptr<State8>> states; // index = parameter index; null before the first step
+    std::vector<std::unique_ptr<State32>> states32; // fp32 moments of the parameters below min_8bit_size
+    uint64_t min_8bit_size = 0;                   // 0 = every parameter takes the 8-bit format
     void *stream = nullptr;
     EriAdam8Table *table = nullptr;
     std::vector<uint32_t> table_ids;         // parameter indices the table was built for
@@ -317,6 +353,7 @@ struct EriAdam8bit {
 struct FnState : State8 {
     EriAdam8Table *table = nullptr;
     EriAdam8Tensor row;
+    uint64_t queued_in = 0; // generation of the batch that holds a row of this state
     FnState() { std::memset(&row, 0, sizeof row); }
     ~FnState() {
         if (table) eri_adam8_table_destroy(table);
@@ -327,8 +364,23 @@ struct EriAdam8bitFn {
     double lr = 1e-4, beta1 = 0.9, beta2 = 0.999, eps = 1e-8, wd = 0.01;
     uint64_t step = 0;
     void *stream = nullptr;
-    std::map<std::string, std::unique_ptr<FnState>> states;
+    std::map<std::string, std::unique_ptr<FnState>, std::less<>> states;
+    // Batching: update() calls queue rows, one launch over all of them runs at the next flush.
+    bool batching = false;
+    uint64_t generation = 1;                 // of the batch being collected
+    std::vector<EriAdam8Tensor> pending;     // rows in call order
+    std::vector<std::pair<const std::string *, FnState *>> pending_who;
+    std::vector<std::pair<const std::string *, FnState *>> last_order; // names of the last flush, in order
+    EriAdam8Table *table = nullptr;          // launch table of the last flush
+    std::vector<EriAdam8Tensor> table_rows;
+    ~EriAdam8bitFn() {
+        if (table) eri_adam8_table_destroy(table);
+    }
 };
+
+namespace {
+int fn_flush(EriAdam8bitFn *o);
+}
 
 extern "C" {
 
@@ -342,6 +394,7 @@ int eri_param_create(void *data, uint64_t numel, int dtype_tag, EriParameter **o
     p->data = data;
     p->numel = numel;
     p->dtype = dtype_tag;
+    p->grad_dtype = dtype_tag;
     *out = p;
     return 0;
 }
@@ -349,6 +402,16 @@ int eri_param_create(void *data, uint64_t numel, int dtype_tag, EriParameter **o
 int eri_param_set_grad(EriParameter *param, const void *grad) {
     if (!param) return fail(ERI_ERR_NULL, "param is NULL");
     param->grad = grad;
+    param->grad_dtype = param->dtype;
+    return 0;
+}
+
+int eri_param_set_grad_typed(EriParameter *param, const void *grad, int grad_dtype_tag) {
+    if (!param) return fail(ERI_ERR_NULL, "param is NULL");
+    if (grad_dtype_tag != param->dtype && !(param->dtype == ERI_DTYPE_BF16 && grad_dtype_tag == ERI_DTYPE_F32))
+        return fail(ERI_ERR_DTYPE, "Unsupported: a gradient has the dtype of its parameter, or F32 for a BF16 parameter");
+    param->grad = grad;
+    param->grad_dtype = grad_dtype_tag;
     return 0;
 }
 
@@ -402,6 +465,7 @@ int eri_adam8bit_new(EriParameter *const *params, uint32_t n, const EriAdam8bitC
     o->params.assign(params, params + n);
     for (auto *p : o->params) ++p->refs; // the optimizer holds clones of the handles (:222-223)
     o->states.resize(n);
+    o->states32.resize(n);
     o->param_scale.assign(n, 1.0f);
     *out = o;
     return 0;
@@ -415,12 +479,22 @@ int eri_adam8bit_destroy(EriAdam8bit *o) {
     return 0;
 }
 
+static int adam8bit_step_impl(EriAdam8bit *o, uint32_t *skipped);
+
 int eri_adam8bit_step(EriAdam8bit *o, uint32_t *skipped) {
     if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    const uint64_t before = o->step;
+    const int rc = adam8bit_step_impl(o, skipped);
+    if (rc) o->step = before; // a refused step counts for nothing
+    return rc;
+}
+
+static int adam8bit_step_impl(EriAdam8bit *o, uint32_t *skipped) {
     o->step += 1; // :203
     uint32_t skip = 0;
     std::vector<uint32_t> ids;
     std::vector<EriAdam8Tensor> rows;
+    std::vector<EriAdamW32Tensor> rows32;
     uint64_t start = 0;
     bool scaled = o->grad_scale != 1.0f;
     for (uint32_t i = 0; i < o->params.size(); ++i) {
@@ -431,6 +505,28 @@ int eri_adam8bit_step(EriAdam8bit *o, uint32_t *skipped) {
             continue;
         }
         if (p->numel == 0) return fail(ERI_ERR_EMPTY, "InvalidOperation: Empty tensor for quantization");
+        // min_8bit_size (pipeline_flux_lora_1024.rs:451): a short tensor keeps fp32 moments and takes the same
+        // update without the quantiser, unless it already has an 8-bit state or its gradient is of another dtype
+        const bool small = o->states32[i] || (o->min_8bit_size && p->numel < o->min_8bit_size && !o->states[i] &&
+                                              p->grad_dtype == p->dtype);
+        if (small) {
+            if (!o->states32[i]) {
+                std::unique_ptr<State32> s(new State32());
+                int rc = s->allocate(p->numel);
+                if (rc) return rc;
+                o->states32[i] = std::move(s);
+            }
+            EriAdamW32Tensor r;
+            std::memset(&r, 0, sizeof r);
+            r.p = p->data;
+            r.g = p->grad;
+            r.m = o->states32[i]->m;
+            r.v = o->states32[i]->v;
+            r.numel = p->numel;
+            r.dtype_tag = p->dtype;
+            rows32.push_back(r);
+            continue;
+        }
         if (!o->states[i]) { // init_state :179-199
             std::unique_ptr<State8> s(new State8());
             int rc = s->allocate(p->numel, o->stream);
@@ -449,6 +545,7 @@ int eri_adam8bit_step(EriAdam8bit *o, uint32_t *skipped) {
         r.numel = p->numel;
         r.block_start = start;
         r.dtype_tag = p->dtype;
+        r.grad_f32 = (p->dtype == ERI_DTYPE_BF16 && p->grad_dtype == ERI_DTYPE_F32) ? 1 : 0;
         r.grad_scale = o->param_scale[i];
         scaled = scaled || o->param_scale[i] != 1.0f;
         start += blocks_of(p->numel);
@@ -456,8 +553,32 @@ int eri_adam8bit_step(EriAdam8bit *o, uint32_t *skipped) {
         rows.push_back(r);
     }
     if (skipped) *skipped = skip;
-    if (rows.empty()) return 0;
+    const bool clip = o->max_grad_norm > 0.0f;
+    if (!rows32.empty()) { // refused before anything is launched
+        for (uint32_t i = 0; i < o->params.size(); ++i) scaled = scaled || (o->states32[i] && o->param_scale[i] != 1.0f);
+        if (scaled || clip)
+            return fail(ERI_ERR_ARG, "InvalidOperation: min_8bit_size cannot be combined with gradient scaling or clipping inside the step");
+        if (o->mode != ERI_ADAM8_MODE_ERI)
+            return fail(ERI_ERR_ARG, "InvalidOperation: min_8bit_size needs mode ERI");
+    }
     int rc = 0;
+    if (!rows32.empty()) {
+        // The reference's update with fp32 moments: the 32-bit step computes
+        // p + ((m/(sqrt(v)+eps)) + p*wd) * (-lr), which with lr = the bias-corrected step size is
+        // adam8bit_enhanced.rs:252-275 bit for bit (x * (-a) = -(x * a), p + (-y) = p - y).
+        EriAdam8Hyper h8;
+        rc = eri_adam8_hyper_pack(o->lr, o->beta1, o->beta2, o->eps, o->wd, o->step, ERI_ADAM8_MODE_ERI, 0, &h8);
+        if (rc) return rc;
+        EriAdamW32Hyper h32;
+        h32.lr = h8.step_size;
+        h32.beta1 = h8.beta1;
+        h32.beta2 = h8.beta2;
+        h32.eps = h8.eps;
+        h32.weight_decay = h8.weight_decay > 0.0f ? h8.weight_decay : 0.0f; // :267: decay only if positive
+        rc = eri_adamw32_step_multi(rows32.data(), (uint32_t)rows32.size(), &h32, o->stream);
+        if (rc) return rc;
+    }
+    if (rows.empty()) return 0;
     if (!o->table || ids != o->table_ids) {
         if (o->table) eri_adam8_table_destroy(o->table);
         o->table = nullptr;
@@ -471,7 +592,6 @@ int eri_adam8bit_step(EriAdam8bit *o, uint32_t *skipped) {
         if (rc) return rc;
         o->table_rows = rows;
     }
-    const bool clip = o->max_grad_norm > 0.0f;
     if (clip) {
         rc = eri_adam8_grad_norm(o->table, o->max_grad_norm, o->clip_denom_eps, o->stream);
         if (rc) return rc;
@@ -513,8 +633,12 @@ int eri_adam8bit_set_learning_rate(EriAdam8bit *o, double lr) {
 uint64_t eri_adam8bit_quantized_memory_usage(const EriAdam8bit *o) {
     uint64_t total = 0;
     if (o)
+    {
         for (auto &s : o->states)
             if (s) total += s->nbytes();
+        for (auto &s : o->states32)
+            if (s) total += s->nbytes();
+    }
     return total;
 }
 
@@ -576,6 +700,21 @@ int eri_adam8bit_set_mode(EriAdam8bit *o, int mode) {
     return 0;
 }
 
+int eri_adam8bit_set_min_8bit_size(EriAdam8bit *o, uint64_t numel) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    o->min_8bit_size = numel;
+    return 0;
+}
+
+int eri_adam8bit_state32_ptrs(const EriAdam8bit *o, uint32_t index, float **m, float **v) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    if (index >= o->states32.size()) return fail(ERI_ERR_ARG, "parameter index out of range");
+    const State32 *s = o->states32[index].get();
+    if (m) *m = s ? s->m : nullptr;
+    if (v) *v = s ? s->v : nullptr;
+    return 0;
+}
+
 int eri_adam8bit_set_flags(EriAdam8bit *o, uint32_t flags) {
     if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
     o->flags = flags;
@@ -619,6 +758,14 @@ int eri_adam8bit_save_state(EriAdam8bit *o, const char *path) {
         w.add(base + ".absmax_m", "F32", nb, nb * 4);
         w.add(base + ".absmax_v", "F32", nb, nb * 4);
     }
+    for (uint32_t i = 0; i < o->states32.size(); ++i) { // fp32 moments of the parameters below min_8bit_size
+        const State32 *s = o->states32[i].get();
+        if (!s) continue;
+        any = true;
+        const std::string base = "optimizer.param_" + std::to_string(i);
+        w.add(base + ".m32", "F32", s->numel, s->numel * 4);
+        w.add(base + ".v32", "F32", s->numel, s->numel * 4);
+    }
     Bounce bounce;
     if (any) {
         int rc = bounce.ensure();
@@ -638,6 +785,13 @@ int eri_adam8bit_save_state(EriAdam8bit *o, const char *path) {
             if (rc) return rc;
         }
     }
+    for (uint32_t i = 0; i < o->states32.size(); ++i) {
+        const State32 *s = o->states32[i].get();
+        if (!s) continue;
+        int rc = stream_out(f, s->m, s->numel * 4, bounce, o->stream);
+        if (!rc) rc = stream_out(f, s->v, s->numel * 4, bounce, o->stream);
+        if (rc) return rc;
+    }
     f.flush();
     if (!f) return fail(ERI_ERR_ARG, std::string("InvalidOperation: Failed to save optimizer: cannot write ") + path);
     return 0;
@@ -655,9 +809,19 @@ int eri_adam8bit_load_state(EriAdam8bit *o, const char *path) {
         return fail(ERI_ERR_ARG, "InvalidOperation: Failed to deserialize optimizer: step / learning_rate missing");
     // validate everything before touching the optimizer
     struct Item { uint32_t idx; const StEntry *e[4]; };
-    std::vector<Item> items;
+    std::vector<Item> items, items32;
     for (uint32_t i = 0; i < o->params.size(); ++i) {
         const std::string base = "optimizer.param_" + std::to_string(i);
+        auto m32 = st.tensors.find(base + ".m32");
+        if (m32 != st.tensors.end()) { // fp32 moments
+            auto v32 = st.tensors.find(base + ".v32");
+            const uint64_t bytes = o->params[i]->numel * 4;
+            if (v32 == st.tensors.end() || m32->second.dtype != "F32" || v32->second.dtype != "F32" ||
+                m32->second.end - m32->second.begin != bytes || v32->second.end - v32->second.begin != bytes)
+                return fail(ERI_ERR_ARG, "InvalidOperation: Failed to deserialize optimizer: size or dtype mismatch for " + base);
+            items32.push_back({i, {&m32->second, &v32->second, nullptr, nullptr}});
+            continue;
+        }
         auto m = st.tensors.find(base + ".m");
         if (m == st.tensors.end()) continue;
         auto v = st.tensors.find(base + ".v"), am = st.tensors.find(base + ".absmax_m"), av = st.tensors.find(base + ".absmax_v");
@@ -689,7 +853,28 @@ int eri_adam8bit_load_state(EriAdam8bit *o, const char *path) {
         }
         fresh.push_back(std::move(s));
     }
-    for (size_t k = 0; k < items.size(); ++k) o->states[items[k].idx] = std::move(fresh[k]);
+    std::vector<std::unique_ptr<State32>> fresh32;
+    for (auto &it : items32) {
+        int rc = bounce.ensure();
+        if (rc) return rc;
+        std::unique_ptr<State32> s(new State32());
+        rc = s->allocate(o->params[it.idx]->numel);
+        if (rc) return rc;
+        void *dst[2] = {s->m, s->v};
+        for (int k = 0; k < 2; ++k) {
+            rc = stream_in(f, st.data_start + it.e[k]->begin, dst[k], it.e[k]->end - it.e[k]->begin, bounce, o->stream);
+            if (rc) return rc;
+        }
+        fresh32.push_back(std::move(s));
+    }
+    for (size_t k = 0; k < items.size(); ++k) {
+        o->states[items[k].idx] = std::move(fresh[k]);
+        o->states32[items[k].idx].reset();
+    }
+    for (size_t k = 0; k < items32.size(); ++k) {
+        o->states32[items32[k].idx] = std::move(fresh32[k]);
+        o->states[items32[k].idx].reset();
+    }
     o->step = std::strtoull(st.metadata["step"].c_str(), nullptr, 10);
     o->lr = std::strtod(st.metadata["learning_rate"].c_str(), nullptr);
     if (o->table) { // state pointers changed
@@ -895,34 +1080,57 @@ int eri_adam8bit_fn_with_params(double lr, double beta1, double beta2, double ep
 }
 
 int eri_adam8bit_fn_destroy(EriAdam8bitFn *o) {
+    if (!o) return 0;
+    int rc = fn_flush(o); // an update that was accepted runs
     delete o;
+    return rc;
+}
+
+} // extern "C"
+
+namespace {
+
+/* The state of `name`, created on first use (adam8bit.rs:126-130).  `hint` is the position of this update in
+ * the batch: trainers update the same names in the same order every step, so the name usually matches the
+ * one the last flush had at that position and the map is not searched. */
+int fn_state_of(EriAdam8bitFn *o, const char *name, uint64_t numel, size_t hint, const std::string **key, FnState **out) {
+    if (hint < o->last_order.size() && *o->last_order[hint].first == name) {
+        *key = o->last_order[hint].first;
+        *out = o->last_order[hint].second;
+    } else {
+        auto it = o->states.find(std::string_view(name));
+        if (it == o->states.end()) {
+            std::unique_ptr<FnState> s(new FnState());
+            int rc = s->allocate(numel, o->stream);
+            if (rc) return rc;
+            it = o->states.emplace(name, std::move(s)).first;
+        }
+        *key = &it->first;
+        *out = it->second.get();
+    }
+    if ((*out)->numel != numel) return fail(ERI_ERR_ARG, std::string("state of '") + name + "' has a different size");
     return 0;
 }
 
-int eri_adam8bit_fn_update(EriAdam8bitFn *o, const char *name, const void *param, const void *grad, uint64_t numel,
-                           int dtype_tag, void *out) {
-    if (!o || !name || !param || !grad || !out) return fail(ERI_ERR_NULL, "update with NULL argument");
+int fn_check_update(const char *name, const void *param, const void *grad, uint64_t numel, int dtype_tag,
+                    int grad_dtype_tag, const void *out) {
+    if (!name || !param || !grad || !out) return fail(ERI_ERR_NULL, "update with NULL argument");
     if (numel == 0) return fail(ERI_ERR_EMPTY, "InvalidOperation: Empty tensor for quantization");
     if (dtype_tag != ERI_DTYPE_F32 && dtype_tag != ERI_DTYPE_BF16)
         return fail(ERI_ERR_DTYPE, "Unsupported: 8-bit Adam takes F32 or BF16 parameters");
-    auto it = o->states.find(name);
-    if (it == o->states.end()) { // adam8bit.rs:126-130
-        std::unique_ptr<FnState> s(new FnState());
-        int rc = s->allocate(numel, o->stream);
-        if (rc) return rc;
-        it = o->states.emplace(name, std::move(s)).first;
-    } else if (it->second->numel != numel) {
-        return fail(ERI_ERR_ARG, std::string("state of '") + name + "' has a different size");
-    }
-    int rc = 0;
-    if (out != param) {
-        rc = eri_hip_memcpy_async(out, param, numel * (dtype_tag == ERI_DTYPE_F32 ? 4 : 2), 3, o->stream);
-        if (rc) return rc;
-    }
-    FnState &s = *it->second;
+    if (grad_dtype_tag != dtype_tag && !(dtype_tag == ERI_DTYPE_BF16 && grad_dtype_tag == ERI_DTYPE_F32))
+        return fail(ERI_ERR_DTYPE, "Unsupported: a gradient has the dtype of its parameter, or F32 for a BF16 parameter");
+    if (((uintptr_t)param | (uintptr_t)grad | (uintptr_t)out) & 15u)
+        return fail(ERI_ERR_ALIGN, "update: param, grad and out must be 16-byte aligned");
+    return 0;
+}
+
+EriAdam8Tensor fn_row(const FnState &s, const void *param, const void *grad, uint64_t numel, int dtype_tag,
+                      int grad_dtype_tag, void *out) {
     EriAdam8Tensor r;
     std::memset(&r, 0, sizeof r);
     r.p = out;
+    r.p_src = out == param ? nullptr : param; // the kernel reads the old values from param and writes out: no copy
     r.g = grad;
     r.m = s.m;
     r.v = s.v;
@@ -931,18 +1139,96 @@ int eri_adam8bit_fn_update(EriAdam8bitFn *o, const char *name, const void *param
     r.numel = numel;
     r.block_start = 0;
     r.dtype_tag = dtype_tag;
+    r.grad_f32 = (dtype_tag == ERI_DTYPE_BF16 && grad_dtype_tag == ERI_DTYPE_F32) ? 1 : 0;
     r.grad_scale = 1.0f;
-    EriAdam8Hyper h;
+    return r;
+}
+
+int fn_hyper(const EriAdam8bitFn *o, EriAdam8Hyper *h) {
     // the bias correction uses the counter as it stands; step() bumps it later (:107,:164)
-    rc = eri_adam8_hyper_pack(o->lr, o->beta1, o->beta2, o->eps, o->wd, o->step, ERI_ADAM8_MODE_L2,
-                              ERI_ADAM8_FLAG_EXACT_PARAM, &h);
+    return eri_adam8_hyper_pack(o->lr, o->beta1, o->beta2, o->eps, o->wd, o->step, ERI_ADAM8_MODE_L2,
+                                ERI_ADAM8_FLAG_EXACT_PARAM, h);
+}
+
+/* One launch over every queued row.  The launch table of the last flush is kept: the same tensors with
+ * new pointers cost one small upload, the same pointers cost nothing. */
+int fn_flush(EriAdam8bitFn *o) {
+    if (o->pending.empty()) return 0;
+    std::vector<EriAdam8Tensor> rows;
+    rows.swap(o->pending);
+    std::vector<std::pair<const std::string *, FnState *>> who;
+    who.swap(o->pending_who);
+    o->generation += 1;
+    uint64_t start = 0;
+    for (auto &r : rows) {
+        r.block_start = start;
+        start += blocks_of(r.numel);
+    }
+    EriAdam8Hyper h;
+    int rc = fn_hyper(o, &h);
+    if (rc) return rc;
+    bool same = o->table && o->table_rows.size() == rows.size();
+    for (size_t i = 0; same && i < rows.size(); ++i)
+        same = rows[i].numel == o->table_rows[i].numel && rows[i].dtype_tag == o->table_rows[i].dtype_tag &&
+               rows[i].grad_f32 == o->table_rows[i].grad_f32;
+    if (!same) {
+        if (o->table) eri_adam8_table_destroy(o->table);
+        o->table = nullptr;
+        o->table_rows.clear();
+        rc = eri_adam8_table_create(rows.data(), (uint32_t)rows.size(), o->stream, &o->table);
+    } else if (std::memcmp(rows.data(), o->table_rows.data(), rows.size() * sizeof(EriAdam8Tensor)) != 0) {
+        rc = eri_adam8_table_update(o->table, rows.data(), (uint32_t)rows.size(), o->stream);
+    }
+    if (rc) return rc;
+    o->table_rows.swap(rows);
+    o->last_order.swap(who);
+    return eri_adam8_step_table(o->table, &h, o->stream);
+}
+
+int fn_enqueue(EriAdam8bitFn *o, const char *name, const void *param, const void *grad, uint64_t numel, int dtype_tag,
+               int grad_dtype_tag, void *out) {
+    int rc = fn_check_update(name, param, grad, numel, dtype_tag, grad_dtype_tag, out);
+    if (rc) return rc;
+    const std::string *key = nullptr;
+    FnState *s = nullptr;
+    rc = fn_state_of(o, name, numel, o->pending.size(), &key, &s);
+    if (rc) return rc;
+    if (s->queued_in == o->generation) { // the same name twice in one batch: the first update must run first
+        rc = fn_flush(o);
+        if (rc) return rc;
+    }
+    s->queued_in = o->generation;
+    o->pending.push_back(fn_row(*s, param, grad, numel, dtype_tag, grad_dtype_tag, out));
+    o->pending_who.emplace_back(key, s);
+    return 0;
+}
+
+} // namespace
+
+extern "C" {
+
+int eri_adam8bit_fn_update(EriAdam8bitFn *o, const char *name, const void *param, const void *grad, uint64_t numel,
+                           int dtype_tag, int grad_dtype_tag, void *out) {
+    if (!o) return fail(ERI_ERR_NULL, "update with NULL argument");
+    if (o->batching) return fn_enqueue(o, name, param, grad, numel, dtype_tag, grad_dtype_tag, out);
+    // immediate: one launch per call through the state's own one-row table
+    int rc = fn_check_update(name, param, grad, numel, dtype_tag, grad_dtype_tag, out);
+    if (rc) return rc;
+    const std::string *key = nullptr;
+    FnState *sp = nullptr;
+    rc = fn_state_of(o, name, numel, o->last_order.size(), &key, &sp);
+    if (rc) return rc;
+    FnState &s = *sp;
+    const EriAdam8Tensor r = fn_row(s, param, grad, numel, dtype_tag, grad_dtype_tag, out);
+    EriAdam8Hyper h;
+    rc = fn_hyper(o, &h);
     if (rc) return rc;
     if (!s.table) {
         rc = eri_adam8_table_create(&r, 1, o->stream, &s.table);
         if (rc) return rc;
         s.row = r;
     } else if (std::memcmp(&r, &s.row, sizeof r) != 0) { // same size by the check above; new pointers or dtype
-        if (r.dtype_tag != s.row.dtype_tag) {
+        if (r.dtype_tag != s.row.dtype_tag || r.grad_f32 != s.row.grad_f32) {
             eri_adam8_table_destroy(s.table);
             s.table = nullptr;
             rc = eri_adam8_table_create(&r, 1, o->stream, &s.table);
@@ -955,16 +1241,53 @@ int eri_adam8bit_fn_update(EriAdam8bitFn *o, const char *name, const void *param
     return eri_adam8_step_table(s.table, &h, o->stream);
 }
 
+int eri_adam8bit_fn_update_many(EriAdam8bitFn *o, const char *const *names, const void *const *params,
+                                const void *const *grads, const uint64_t *numels, const int32_t *dtype_tags,
+                                const int32_t *grad_dtype_tags, void *const *outs, uint32_t n) {
+    if (!o || !names || !params || !grads || !numels || !dtype_tags || !outs)
+        return fail(ERI_ERR_NULL, "update_many with NULL argument");
+    int rc = fn_flush(o); // rows queued by earlier update() calls keep their place in the order of updates
+    if (rc) return rc;
+    for (uint32_t i = 0; i < n; ++i) {
+        rc = fn_enqueue(o, names[i], params[i], grads[i], numels[i], dtype_tags[i],
+                        grad_dtype_tags ? grad_dtype_tags[i] : dtype_tags[i], outs[i]);
+        if (rc) { // nothing of a refused call runs
+            o->pending.clear();
+            o->pending_who.clear();
+            o->generation += 1;
+            return rc;
+        }
+    }
+    return fn_flush(o);
+}
+
+int eri_adam8bit_fn_set_batching(EriAdam8bitFn *o, int enabled) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    if (!enabled) {
+        int rc = fn_flush(o);
+        if (rc) return rc;
+    }
+    o->batching = enabled != 0;
+    return 0;
+}
+
+int eri_adam8bit_fn_flush(EriAdam8bitFn *o) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    return fn_flush(o);
+}
+
 int eri_adam8bit_fn_step(EriAdam8bitFn *o) {
     if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    int rc = fn_flush(o); // queued updates belong to the step that ends here (:89-92)
     o->step += 1;
-    return 0;
+    return rc;
 }
 
 int eri_adam8bit_fn_set_lr(EriAdam8bitFn *o, float lr) {
     if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    int rc = fn_flush(o); // queued updates were made under the old rate
     o->lr = (double)lr; // `lr as f64`, adam8bit.rs:96
-    return 0;
+    return rc;
 }
 
 uint64_t eri_adam8bit_fn_get_step(const EriAdam8bitFn *o) { return o ? o->step : 0; }
@@ -980,17 +1303,19 @@ int eri_adam8bit_fn_memory_stats(const EriAdam8bitFn *o, uint64_t *num_params, u
 
 int eri_adam8bit_fn_state_numel(const EriAdam8bitFn *o, const char *name, uint64_t *numel) {
     if (!o || !name || !numel) return fail(ERI_ERR_NULL, "NULL argument");
-    auto it = o->states.find(name);
+    auto it = o->states.find(std::string_view(name));
     *numel = it == o->states.end() ? 0 : it->second->numel;
     return 0;
 }
 
 int eri_adam8bit_fn_get_state_fp32(EriAdam8bitFn *o, const char *name, float *m_out, float *v_out) {
     if (!o || !name || !m_out || !v_out) return fail(ERI_ERR_NULL, "NULL argument");
-    auto it = o->states.find(name);
+    int rc = fn_flush(o);
+    if (rc) return rc;
+    auto it = o->states.find(std::string_view(name));
     if (it == o->states.end()) return fail(ERI_ERR_ARG, std::string("no optimizer state named '") + name + "'");
     State8 &s = *it->second;
-    int rc = eri_adam8_dequantize(s.m, s.absmax_m, 1, s.numel, m_out, o->stream);
+    rc = eri_adam8_dequantize(s.m, s.absmax_m, 1, s.numel, m_out, o->stream);
     if (rc) return rc;
     return eri_adam8_dequantize(s.v, s.absmax_v, 0, s.numel, v_out, o->stream);
 }
@@ -999,8 +1324,11 @@ int eri_adam8bit_fn_load_state_fp32(EriAdam8bitFn *o, const char *name, const fl
                                     uint64_t numel) {
     if (!o || !name || !m || !v) return fail(ERI_ERR_NULL, "NULL argument");
     if (numel == 0) return fail(ERI_ERR_EMPTY, "InvalidOperation: Empty tensor for quantization");
+    int rc = fn_flush(o);
+    if (rc) return rc;
+    o->last_order.clear(); // it may hold the state that is replaced below
     std::unique_ptr<FnState> s(new FnState());
-    int rc = s->allocate(numel, o->stream);
+    rc = s->allocate(numel, o->stream);
     if (rc) return rc;
     rc = eri_adam8_quantize(m, 1, numel, s->m, s->absmax_m, o->stream);
     if (rc) return rc;

@@ -271,9 +271,9 @@ struct EriAdam8Table {
     uint32_t n = 0;
     uint64_t total_numel = 0;
     uint64_t total_blocks = 0;
-    Group groups[2]; // F32, BF16
+    Group groups[eri::kLayouts]; // F32, BF16, BF16 with F32 gradients
     std::vector<uint64_t> numel;
-    std::vector<int32_t> dtype;
+    std::vector<int32_t> dtype; // per row: its layout
     hipEvent_t uploaded = nullptr;
     bool upload_pending = false;
     void *upload_stream = nullptr;  // stream of the last upload
@@ -288,6 +288,11 @@ struct EriAdam8Table {
 };
 
 namespace {
+
+int layout_of(const EriAdam8Tensor &r) {
+    if (r.dtype_tag == ERI_DTYPE_F32) return eri::kLayoutF32;
+    return r.grad_f32 ? eri::kLayoutBF16GradF32 : eri::kLayoutBF16;
+}
 
 int validate_rows(const EriAdam8Tensor *rows, uint32_t n) {
     if (!rows) return fail(ERI_ERR_NULL, "rows is NULL");
@@ -309,7 +314,19 @@ int validate_rows(const EriAdam8Tensor *rows, uint32_t n) {
                           r.dtype_tag);
             return fail(ERI_ERR_DTYPE, buf);
         }
-        const uintptr_t wide = (uintptr_t)r.p | (uintptr_t)r.g | (uintptr_t)r.m | (uintptr_t)r.v;
+        if (r.grad_f32 && r.dtype_tag == ERI_DTYPE_F32) {
+            std::snprintf(buf, sizeof buf, "row %u: grad_f32 is for BF16 parameters (F32 parameters take F32 gradients anyway)", i);
+            return fail(ERI_ERR_DTYPE, buf);
+        }
+        if (r.p_src && r.p_src != r.p) {
+            const uintptr_t bytes = (uintptr_t)r.numel * (r.dtype_tag == ERI_DTYPE_F32 ? 4u : 2u);
+            const uintptr_t a = (uintptr_t)r.p, b = (uintptr_t)r.p_src;
+            if (a < b + bytes && b < a + bytes) {
+                std::snprintf(buf, sizeof buf, "row %u: p_src overlaps p without being equal to it", i);
+                return fail(ERI_ERR_ARG, buf);
+            }
+        }
+        const uintptr_t wide = (uintptr_t)r.p | (uintptr_t)r.g | (uintptr_t)r.m | (uintptr_t)r.v | (uintptr_t)r.p_src;
         const uintptr_t narrow = (uintptr_t)r.absmax_m | (uintptr_t)r.absmax_v;
         if ((wide & 15u) || (narrow & 3u)) {
             std::snprintf(buf, sizeof buf, "row %u: p/g/m/v must be 16-byte aligned, absmax 4-byte aligned", i);
@@ -334,6 +351,8 @@ void fill_group(EriAdam8Table::Group &g, const EriAdam8Tensor *rows) {
         const EriAdam8Tensor &r = rows[g.src[j]];
         eri::DevTensor &d = g.pinned[j];
         d.p = r.p;
+        d.p_in = r.p_src ? r.p_src : r.p;
+        d.pad = 0;
         d.g = r.g;
         d.m = r.m;
         d.v = r.v;
@@ -611,16 +630,15 @@ int eri_adam8_table_create(const EriAdam8Tensor *rows, uint32_t n, void *stream,
     EriAdam8Table *t = new EriAdam8Table();
     t->n = n;
     (void)hipGetDevice(&t->device);
-    t->groups[0].dtype = ERI_DTYPE_F32;
-    t->groups[1].dtype = ERI_DTYPE_BF16;
+    for (int li = 0; li < eri::kLayouts; ++li) t->groups[li].dtype = li; // a Layout
     t->numel.resize(n);
     t->dtype.resize(n);
     for (uint32_t i = 0; i < n; ++i) {
         t->numel[i] = rows[i].numel;
-        t->dtype[i] = rows[i].dtype_tag;
+        t->dtype[i] = layout_of(rows[i]);
         t->total_numel += rows[i].numel;
         t->total_blocks += blocks_of(rows[i].numel);
-        t->groups[rows[i].dtype_tag == ERI_DTYPE_F32 ? 0 : 1].src.push_back(i);
+        t->groups[layout_of(rows[i])].src.push_back(i);
     }
     hipError_t e = hipEventCreateWithFlags(&t->uploaded, hipEventDisableTiming);
     for (auto &g : t->groups) {
@@ -649,7 +667,7 @@ int eri_adam8_table_update(EriAdam8Table *t, const EriAdam8Tensor *rows, uint32_
     if (rc) return rc;
     if (n != t->n) return fail(ERI_ERR_ARG, "table_update: row count differs from the table's");
     for (uint32_t i = 0; i < n; ++i)
-        if (rows[i].numel != t->numel[i] || rows[i].dtype_tag != t->dtype[i])
+        if (rows[i].numel != t->numel[i] || layout_of(rows[i]) != t->dtype[i])
             return fail(ERI_ERR_ARG, "table_update: numel or dtype differs from the table's");
     if (t->upload_pending) { // the pinned mirror may still be the source of the previous copy
         ERI_HIP(hipEventSynchronize(t->uploaded));
@@ -722,8 +740,8 @@ static int grad_norm_launch(EriAdam8Table *t, DeviceCtx *ctx, float max_norm, fl
                             uint32_t pairs, float *result, void *stream) {
     const uint32_t wpw = (uint32_t)eri::kNormWaves;
     const uint32_t grid_cap = ctx->cus * eri::kNormWavesPerCu / wpw; // persistent
-    uint32_t grids[2] = {0, 0}, need = 0;
-    for (int gi = 0; gi < 2; ++gi) {
+    uint32_t grids[eri::kLayouts] = {0, 0, 0}, need = 0;
+    for (int gi = 0; gi < eri::kLayouts; ++gi) {
         const auto &g = t->groups[gi];
         if (g.n == 0) continue;
         const uint32_t work = g.total_blocks > g.n ? g.total_blocks : g.n;
@@ -741,10 +759,10 @@ static int grad_norm_launch(EriAdam8Table *t, DeviceCtx *ctx, float max_norm, fl
     int rc = order_after_upload(t, stream);
     if (rc) return rc;
     uint32_t off = 0;
-    for (int gi = 0; gi < 2; ++gi) {
+    for (int gi = 0; gi < eri::kLayouts; ++gi) {
         auto &g = t->groups[gi];
         if (g.n == 0) continue;
-        rc = eri::launch_grad_sumsq(g.dev, g.n, g.total_blocks, g.dtype, partial + 2 * off, grids[gi], stream);
+        rc = eri::launch_grad_sumsq(g.dev, g.n, g.total_blocks, eri::layout_grad_bf16(g.dtype), partial + 2 * off, grids[gi], stream);
         if (rc) return hip_fail((hipError_t)rc, "gradient sum-of-squares launch");
         off += grids[gi] * wpw;
     }
@@ -760,8 +778,8 @@ int eri_adam8_grad_norm(EriAdam8Table *t, float max_norm, float denom_eps, void 
     DeviceCtx *ctx = nullptr;
     int rc = get_ctx_on(t->device, &ctx);
     if (rc) return rc;
-    // two groups at most, and per wave a sum of squares and a count
-    const uint32_t pairs = 2 * ctx->cus * eri::kNormWavesPerCu;
+    // one group per layout at most, and per wave a sum of squares and a count
+    const uint32_t pairs = eri::kLayouts * ctx->cus * eri::kNormWavesPerCu;
     if (!t->partial) ERI_HIP(hipMalloc((void **)&t->partial, sizeof(double) * 2 * pairs));
     if (!t->norm_out) ERI_HIP(hipMalloc((void **)&t->norm_out, sizeof(float) * 4)); // norm, scale, 64-bit count
     return grad_norm_launch(t, ctx, max_norm, denom_eps, t->partial, pairs, t->norm_out, stream);
@@ -855,7 +873,7 @@ int eri_adam8_step_multi(const EriAdam8Tensor *rows, uint32_t n, const EriAdam8H
     bool same_shape = cache.table && cache.table->n == n && cache.table->device == dev;
     if (same_shape)
         for (uint32_t i = 0; i < n && same_shape; ++i)
-            same_shape = rows[i].numel == cache.table->numel[i] && rows[i].dtype_tag == cache.table->dtype[i];
+            same_shape = rows[i].numel == cache.table->numel[i] && layout_of(rows[i]) == cache.table->dtype[i];
     int rc = 0;
     if (!same_shape) {
         destroy_table(cache.table);

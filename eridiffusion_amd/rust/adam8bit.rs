@@ -24,6 +24,17 @@ fn check(code: i32, what: &str) -> Result<()> {
     Err(Error::InvalidOperation(format!("{what} failed with code {code}: {msg}")))
 }
 
+/// The gradient as the step reads it, with its dtype tag.  An F32 gradient of a BF16 parameter goes in as it
+/// is: the reference casts every gradient to F32 and never rounds it (adam8bit_enhanced.rs:231-235,
+/// adam8bit.rs:110).  Any other mismatch is cast to the parameter's dtype (BF16 -> F32 is exact).
+fn usable_grad(grad: &Tensor, param_dtype: DType) -> Result<(Tensor, i32)> {
+    if grad.dtype() == param_dtype || (param_dtype == DType::BF16 && grad.dtype() == DType::F32) {
+        Ok((grad.clone(), dtype_tag(grad.dtype())?))
+    } else {
+        Ok((grad.to_dtype(param_dtype)?, dtype_tag(param_dtype)?))
+    }
+}
+
 fn dtype_tag(dt: DType) -> Result<i32> {
     match dt {
         DType::F32 => Ok(sys::ERI_DTYPE_F32),
@@ -42,11 +53,14 @@ pub struct Adam8bitConfig {
     pub amsgrad: bool,
     pub block_wise: bool,
     pub percentile_clipping: usize,
+    /// Not in the reference's struct, but written by its trainers (pipeline_flux_lora_1024.rs:451,
+    /// `min_8bit_size: 4096`): tensors with fewer elements keep fp32 moments.  0 = all tensors 8-bit.
+    pub min_8bit_size: usize,
 }
 
 impl Default for Adam8bitConfig {
     fn default() -> Self {
-        Self { lr: 1e-3, betas: (0.9, 0.999), eps: 1e-8, weight_decay: 0.01, amsgrad: false, block_wise: true, percentile_clipping: 99 }
+        Self { lr: 1e-3, betas: (0.9, 0.999), eps: 1e-8, weight_decay: 0.01, amsgrad: false, block_wise: true, percentile_clipping: 99, min_8bit_size: 0 }
     }
 }
 
@@ -55,7 +69,10 @@ pub struct Adam8bit {
     pub params: Vec<Parameter>,
     handles: Vec<*mut sys::EriParameter>,
     opt: *mut sys::EriAdam8bit,
-    live_grads: Vec<Tensor>, // gradients cast to the parameter dtype must outlive the launch
+    // Gradient tensors of the step in flight.  The launch is asynchronous, so they are released only when
+    // the next step begins, which on the same stream is after the kernel that read them.
+    live_grads: Vec<Tensor>,
+    flushed: bool, // flush() has launched the step that reads live_grads
 }
 
 unsafe impl Send for Adam8bit {}
@@ -81,7 +98,10 @@ impl Adam8bit {
         };
         let mut opt = std::ptr::null_mut();
         check(unsafe { sys::eri_adam8bit_new(handles.as_ptr(), handles.len() as u32, &cfg, stream, &mut opt) }, "eri_adam8bit_new")?;
-        Ok(Self { params, handles, opt, live_grads: Vec::new() })
+        if config.min_8bit_size > 0 {
+            check(unsafe { sys::eri_adam8bit_set_min_8bit_size(opt, config.min_8bit_size as u64) }, "eri_adam8bit_set_min_8bit_size")?;
+        }
+        Ok(Self { params, handles, opt, live_grads: Vec::new(), flushed: false })
     }
 
     /// adam8bit_enhanced.rs:202-291.  One kernel launch for all parameters; parameters without a
@@ -91,14 +111,13 @@ impl Adam8bit {
         for (p, &h) in self.params.iter().zip(&self.handles) {
             let t = p.tensor()?;
             check(unsafe { sys::eri_param_set_data(h, t.cuda_ptr_mut() as *mut c_void) }, "eri_param_set_data")?;
-            let g = match p.grad() {
-                Some(g) if g.dtype() != t.dtype() => Some(g.to_dtype(t.dtype())?),
-                other => other,
-            };
-            let ptr = g.as_ref().map(|g| g.cuda_ptr() as *const c_void).unwrap_or(std::ptr::null());
-            check(unsafe { sys::eri_param_set_grad(h, ptr) }, "eri_param_set_grad")?;
-            if let Some(g) = g {
-                self.live_grads.push(g);
+            match p.grad() {
+                Some(g) => {
+                    let (g, tag) = usable_grad(&g, t.dtype())?;
+                    check(unsafe { sys::eri_param_set_grad_typed(h, g.cuda_ptr() as *const c_void, tag) }, "eri_param_set_grad_typed")?;
+                    self.live_grads.push(g);
+                }
+                None => check(unsafe { sys::eri_param_set_grad(h, std::ptr::null()) }, "eri_param_set_grad")?,
             }
         }
         check(unsafe { sys::eri_adam8bit_step(self.opt, std::ptr::null_mut()) }, "eri_adam8bit_step")
@@ -177,6 +196,10 @@ impl Drop for Adam8bit {
 pub struct Adam8bitFunctional {
     opt: *mut sys::EriAdam8bitFn,
     names: Vec<String>,
+    batched: bool,
+    // With batching, the tensors a queued update reads and writes, kept until the step after the launch.
+    live: Vec<Tensor>,
+    launched: bool,
 }
 
 unsafe impl Send for Adam8bitFunctional {}
@@ -187,11 +210,22 @@ impl Adam8bitFunctional {
     pub fn with_params(learning_rate: f64, beta1: f64, beta2: f64, eps: f64, weight_decay: f64) -> Self {
         let mut opt = std::ptr::null_mut();
         unsafe { sys::eri_adam8bit_fn_with_params(learning_rate, beta1, beta2, eps, weight_decay, std::ptr::null_mut(), &mut opt) };
-        Self { opt, names: Vec::new() }
+        Self { opt, names: Vec::new(), batched: false, live: Vec::new(), launched: false }
+    }
+    /// Queue update() calls and run them as ONE launch at step(): for trainers that only store the tensor
+    /// update() returns (`layer.lora_down.set_data(updated)`, pipeline_flux_lora_sequential.rs:767-792).
+    /// A trainer that reads the returned tensor before step() (pipeline_sdxl_lora.rs:710) keeps the
+    /// default, or moves to update_many().
+    pub fn batched(mut self, enabled: bool) -> Self {
+        unsafe { sys::eri_adam8bit_fn_set_batching(self.opt, enabled as i32) };
+        self.batched = enabled;
+        self
     }
     /// :89-92
     pub fn step(&mut self) -> Result<()> {
-        check(unsafe { sys::eri_adam8bit_fn_step(self.opt) }, "eri_adam8bit_fn_step")
+        let rc = check(unsafe { sys::eri_adam8bit_fn_step(self.opt) }, "eri_adam8bit_fn_step");
+        self.launched = true; // `live` is released when the next update arrives, after this launch in stream order
+        rc
     }
     /// :95-98
     pub fn set_lr(&mut self, lr: f32) -> Result<()> {
@@ -203,14 +237,24 @@ impl Adam8bitFunctional {
     }
     /// :101-208: returns the updated tensor, the input is left alone
     pub fn update(&mut self, name: &str, param: &Tensor, grad: &Tensor) -> Result<Tensor> {
+        if self.launched {
+            self.live.clear();
+            self.launched = false;
+        }
         let out = Tensor::zeros_dtype(param.shape().clone(), param.dtype(), param.device().clone())?;
-        let g = if grad.dtype() != param.dtype() { grad.to_dtype(param.dtype())? } else { grad.clone() };
+        let (g, g_tag) = usable_grad(grad, param.dtype())?;
         let numel: usize = param.shape().dims().iter().product();
         let c = CString::new(name).map_err(|e| Error::InvalidOperation(e.to_string()))?;
         check(unsafe {
             sys::eri_adam8bit_fn_update(self.opt, c.as_ptr(), param.cuda_ptr() as *const c_void, g.cuda_ptr() as *const c_void,
-                                        numel as u64, dtype_tag(param.dtype())?, out.cuda_ptr_mut() as *mut c_void)
+                                        numel as u64, dtype_tag(param.dtype())?, g_tag, out.cuda_ptr_mut() as *mut c_void)
         }, "eri_adam8bit_fn_update")?;
+        // the launch is asynchronous (and, batched, still to come): what it reads must not be freed under it
+        self.live.push(g);
+        if self.batched {
+            self.live.push(param.clone());
+            self.live.push(out.clone());
+        }
         if !self.names.iter().any(|n| n == name) {
             self.names.push(name.to_string());
         }
@@ -262,12 +306,51 @@ impl Drop for Adam8bitFunctional {
     }
 }
 
-/// adam8bit.rs:333-345
-pub fn update_params_8bit(optimizer: &mut Adam8bitFunctional, params: &mut HashMap<String, Tensor>, grads: &HashMap<String, Tensor>) -> Result<()> {
-    for (name, param) in params.iter_mut() {
-        if let Some(grad) = grads.get(name) {
-            *param = optimizer.update(name, param, grad)?;
+impl Adam8bitFunctional {
+    /// Every (name, param, grad) in one launch; returns the new tensors in the same order.
+    pub fn update_many(&mut self, items: &[(&str, &Tensor, &Tensor)]) -> Result<Vec<Tensor>> {
+        if self.launched {
+            self.live.clear();
+            self.launched = false;
         }
+        let n = items.len();
+        let (mut names, mut name_ptrs, mut ps, mut gs, mut outs_ptr) = (Vec::with_capacity(n), Vec::with_capacity(n), Vec::with_capacity(n), Vec::with_capacity(n), Vec::with_capacity(n));
+        let (mut numels, mut tags, mut g_tags, mut outs) = (Vec::with_capacity(n), Vec::with_capacity(n), Vec::with_capacity(n), Vec::with_capacity(n));
+        for (name, param, grad) in items {
+            let (g, g_tag) = usable_grad(grad, param.dtype())?;
+            let out = Tensor::zeros_dtype(param.shape().clone(), param.dtype(), param.device().clone())?;
+            names.push(CString::new(*name).map_err(|e| Error::InvalidOperation(e.to_string()))?);
+            ps.push(param.cuda_ptr() as *const c_void);
+            gs.push(g.cuda_ptr() as *const c_void);
+            outs_ptr.push(out.cuda_ptr_mut() as *mut c_void);
+            numels.push(param.shape().dims().iter().product::<usize>() as u64);
+            tags.push(dtype_tag(param.dtype())?);
+            g_tags.push(g_tag);
+            self.live.push(g);
+            outs.push(out);
+            if !self.names.iter().any(|k| k == name) {
+                self.names.push(name.to_string());
+            }
+        }
+        for c in &names {
+            name_ptrs.push(c.as_ptr());
+        }
+        check(unsafe {
+            sys::eri_adam8bit_fn_update_many(self.opt, name_ptrs.as_ptr(), ps.as_ptr(), gs.as_ptr(), numels.as_ptr(), tags.as_ptr(),
+                                             g_tags.as_ptr(), outs_ptr.as_ptr(), n as u32)
+        }, "eri_adam8bit_fn_update_many")?;
+        self.launched = true;
+        Ok(outs)
+    }
+}
+
+/// adam8bit.rs:333-345, as one launch instead of a loop of update() calls
+pub fn update_params_8bit(optimizer: &mut Adam8bitFunctional, params: &mut HashMap<String, Tensor>, grads: &HashMap<String, Tensor>) -> Result<()> {
+    let names: Vec<String> = params.keys().filter(|k| grads.contains_key(*k)).cloned().collect();
+    let items: Vec<(&str, &Tensor, &Tensor)> = names.iter().map(|k| (k.as_str(), &params[k], &grads[k])).collect();
+    let outs = optimizer.update_many(&items)?;
+    for (k, t) in names.iter().zip(outs) {
+        params.insert(k.clone(), t);
     }
     Ok(())
 }
@@ -297,8 +380,12 @@ impl crate::trainers::training::optimization::OptimizerTrait for Adam8bit {
         let t = param.tensor()?;
         let at = self.params.iter().position(|p| p.tensor().map(|q| q.cuda_ptr() == t.cuda_ptr()).unwrap_or(false))
             .ok_or_else(|| Error::InvalidOperation("parameter is not owned by this optimizer".into()))?;
-        let g = if grad.dtype() != t.dtype() { grad.to_dtype(t.dtype())? } else { grad.clone() };
-        check(unsafe { sys::eri_param_set_grad(self.handles[at], g.cuda_ptr() as *const c_void) }, "eri_param_set_grad")?;
+        if self.flushed {
+            self.live_grads.clear(); // the step that read them was launched before this call, on the same stream
+            self.flushed = false;
+        }
+        let (g, tag) = usable_grad(grad, t.dtype())?;
+        check(unsafe { sys::eri_param_set_grad_typed(self.handles[at], g.cuda_ptr() as *const c_void, tag) }, "eri_param_set_grad_typed")?;
         self.live_grads.push(g);
         Ok(())
     }
@@ -323,7 +410,7 @@ impl Adam8bit {
     /// Launches the step for the gradients handed over through `OptimizerTrait::step`.
     pub fn flush(&mut self) -> Result<()> {
         let rc = check(unsafe { sys::eri_adam8bit_step(self.opt, std::ptr::null_mut()) }, "eri_adam8bit_step");
-        self.live_grads.clear();
+        self.flushed = true; // live_grads stay until the next gradient arrives: the launch above still reads them
         rc
     }
 }

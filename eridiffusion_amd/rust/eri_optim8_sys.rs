@@ -32,6 +32,7 @@ pub struct EriAdam8Tensor {
     pub p: *mut c_void, pub g: *const c_void, pub m: *mut u8, pub v: *mut u8,
     pub absmax_m: *mut f32, pub absmax_v: *mut f32,
     pub numel: u64, pub block_start: u64, pub dtype_tag: i32, pub grad_scale: f32,
+    pub p_src: *const c_void, pub grad_f32: i32, pub reserved: i32,
 }
 
 #[repr(C)]
@@ -104,6 +105,7 @@ extern "C" {
     // optimizer objects
     pub fn eri_param_create(data: *mut c_void, numel: u64, dtype_tag: c_int, out: *mut *mut EriParameter) -> c_int;
     pub fn eri_param_set_grad(param: *mut EriParameter, grad: *const c_void) -> c_int;
+    pub fn eri_param_set_grad_typed(param: *mut EriParameter, grad: *const c_void, grad_dtype_tag: c_int) -> c_int;
     pub fn eri_param_set_data(param: *mut EriParameter, data: *mut c_void) -> c_int;
     pub fn eri_param_retain(param: *mut EriParameter) -> c_int;
     pub fn eri_param_release(param: *mut EriParameter) -> c_int;
@@ -118,6 +120,8 @@ extern "C" {
     pub fn eri_adam8bit_get_step(opt: *const EriAdam8bit) -> u64;
     pub fn eri_adam8bit_set_grad_scale(opt: *mut EriAdam8bit, scale: f32) -> c_int;
     pub fn eri_adam8bit_set_param_grad_scale(opt: *mut EriAdam8bit, index: u32, scale: f32) -> c_int;
+    pub fn eri_adam8bit_set_min_8bit_size(opt: *mut EriAdam8bit, numel: u64) -> c_int;
+    pub fn eri_adam8bit_state32_ptrs(opt: *const EriAdam8bit, index: u32, m: *mut *mut f32, v: *mut *mut f32) -> c_int;
     pub fn eri_adam8bit_set_max_grad_norm(opt: *mut EriAdam8bit, max_norm: f32, denom_eps: f32) -> c_int;
     pub fn eri_ema_new(decay: f32, use_bias_correction: c_int, power: f32, stream: *mut c_void, out: *mut *mut EriEmaModel) -> c_int;
     pub fn eri_ema_destroy(ema: *mut EriEmaModel) -> c_int;
@@ -145,7 +149,10 @@ extern "C" {
     pub fn eri_adam8bit_state_ptrs(opt: *const EriAdam8bit, index: u32, m: *mut *mut u8, v: *mut *mut u8, absmax_m: *mut *mut f32, absmax_v: *mut *mut f32) -> c_int;
     pub fn eri_adam8bit_fn_with_params(lr: f64, beta1: f64, beta2: f64, eps: f64, weight_decay: f64, stream: *mut c_void, out: *mut *mut EriAdam8bitFn) -> c_int;
     pub fn eri_adam8bit_fn_destroy(opt: *mut EriAdam8bitFn) -> c_int;
-    pub fn eri_adam8bit_fn_update(opt: *mut EriAdam8bitFn, name: *const c_char, param: *const c_void, grad: *const c_void, numel: u64, dtype_tag: c_int, out: *mut c_void) -> c_int;
+    pub fn eri_adam8bit_fn_update(opt: *mut EriAdam8bitFn, name: *const c_char, param: *const c_void, grad: *const c_void, numel: u64, dtype_tag: c_int, grad_dtype_tag: c_int, out: *mut c_void) -> c_int;
+    pub fn eri_adam8bit_fn_set_batching(opt: *mut EriAdam8bitFn, enabled: c_int) -> c_int;
+    pub fn eri_adam8bit_fn_flush(opt: *mut EriAdam8bitFn) -> c_int;
+    pub fn eri_adam8bit_fn_update_many(opt: *mut EriAdam8bitFn, names: *const *const c_char, params: *const *const c_void, grads: *const *const c_void, numels: *const u64, dtype_tags: *const i32, grad_dtype_tags: *const i32, outs: *const *mut c_void, n: u32) -> c_int;
     pub fn eri_adam8bit_fn_step(opt: *mut EriAdam8bitFn) -> c_int;
     pub fn eri_adam8bit_fn_set_lr(opt: *mut EriAdam8bitFn, lr: f32) -> c_int;
     pub fn eri_adam8bit_fn_get_step(opt: *const EriAdam8bitFn) -> u64;

@@ -29,7 +29,11 @@ extern "C" {
  * The handle never owns the device memory it points to (crates/core/tests/wrap_external.rs:25-30). */
 typedef struct EriParameter EriParameter;
 int eri_param_create(void *data, uint64_t numel, int dtype_tag, EriParameter **out);
-int eri_param_set_grad(EriParameter *param, const void *grad); /* NULL = no gradient this step */
+int eri_param_set_grad(EriParameter *param, const void *grad); /* NULL = no gradient this step; dtype of the parameter */
+/* A gradient of another dtype than its parameter: ERI_DTYPE_F32 for a BF16 parameter.  The reference casts
+ * every gradient to F32 and never rounds it (adam8bit_enhanced.rs:231-235), so such a gradient enters the
+ * step as it is. */
+int eri_param_set_grad_typed(EriParameter *param, const void *grad, int grad_dtype_tag);
 int eri_param_set_data(EriParameter *param, void *data);       /* Parameter::set_data */
 int eri_param_retain(EriParameter *param);                     /* Parameter::clone */
 int eri_param_release(EriParameter *param);
@@ -68,6 +72,17 @@ int eri_adam8bit_set_param_grad_scale(EriAdam8bit *opt, uint32_t index, float sc
 int eri_adam8bit_set_flags(EriAdam8bit *opt, uint32_t flags); /* ERI_ADAM8_FLAG_EXACT_PARAM etc. */
 /* ERI_ADAM8_MODE_ERI (default: the reference's update) or ERI_ADAM8_MODE_BNB for later steps. */
 int eri_adam8bit_set_mode(EriAdam8bit *opt, int mode);
+/* min_8bit_size (pipeline_flux_lora_1024.rs:451, the policy of the library the state format comes from):
+ * from the next step on, a parameter with fewer than `numel` elements that has no 8-bit state yet keeps
+ * fp32 moments instead and takes the same update, adam8bit_enhanced.rs:252-275, without the quantiser --
+ * one extra launch of the 32-bit step (eri_adamw32_step_multi) over all such parameters, with the
+ * bias-corrected step size as its learning rate.  0 (the default) keeps every parameter in the 8-bit
+ * format.  Such parameters need gradients of their own dtype, mode ERI, and no gradient scaling or clipping
+ * inside the step (a step that would combine them is refused before anything runs).  save_state / load_state
+ * carry the fp32 moments as `optimizer.param_N.m32` / `.v32`. */
+int eri_adam8bit_set_min_8bit_size(EriAdam8bit *opt, uint64_t numel);
+/* Device pointers of one parameter's fp32 moments (NULL if it has none). */
+int eri_adam8bit_state32_ptrs(const EriAdam8bit *opt, uint32_t index, float **m, float **v);
 /* Global-norm clipping inside step(): max_norm > 0 makes every step first reduce the gradients' global
  * L2 norm on the device (eri_adam8_grad_norm) and apply max_norm / (norm + denom_eps) when the norm is
  * above max_norm -- the trainers' clip_gradients (pipeline_flux_lora_sequential.rs:737,1198-1213)
@@ -106,10 +121,31 @@ int eri_adam8bit_fn_with_params(double lr, double beta1, double beta2, double ep
                                 EriAdam8bitFn **out);
 int eri_adam8bit_fn_destroy(EriAdam8bitFn *opt);
 /* update(name, param, grad) -> new tensor, :101-208.  `param` is left untouched, the new values are
- * written to `out` (numel elements of the same dtype; it may alias `param`). */
+ * written to `out` (numel elements of the same dtype; it may be `param` itself: in-place).  The kernel
+ * reads `param` and writes `out`; nothing is copied.  `grad_dtype_tag` is `dtype_tag`, or ERI_DTYPE_F32
+ * for BF16 parameters (adam8bit.rs:110 casts the gradient to F32 and does not round it).  Pointers
+ * 16-byte aligned.
+ * By default every call is one kernel launch and `out` is valid in stream order when the call returns, as
+ * the reference's callers may assume (pipeline_sdxl_lora.rs:708-724 reads the new tensor at once). */
 int eri_adam8bit_fn_update(EriAdam8bitFn *opt, const char *name, const void *param, const void *grad, uint64_t numel,
-                           int dtype_tag, void *out);
-int eri_adam8bit_fn_step(EriAdam8bitFn *opt);                   /* :89-92, only bumps the counter */
+                           int dtype_tag, int grad_dtype_tag, void *out);
+/* Batching: with it enabled, update() only queues its row, and ONE launch over all queued rows runs at the
+ * next eri_adam8bit_fn_step (which every trainer calls right after its loop of updates:
+ * pipeline_flux_lora_sequential.rs:749-794), eri_adam8bit_fn_flush, set_lr, state read or destroy.  Until
+ * then `out` is not written and `param` / `grad` must stay alive and unchanged -- a caller that reads the
+ * returned tensor, or frees the gradient, before step() must not enable it.  A second update of the same
+ * name flushes the first.  The launch table is kept between flushes: the same tensors at new addresses
+ * cost one small upload, at the same addresses nothing.  The hundreds of launches of a LoRA step become one. */
+int eri_adam8bit_fn_set_batching(EriAdam8bitFn *opt, int enabled);
+int eri_adam8bit_fn_flush(EriAdam8bitFn *opt);
+/* n updates in one call and one launch, whatever the batching setting: update(names[i], params[i], grads[i])
+ * -> outs[i] for every i (update_params_8bit, adam8bit.rs:333-345, without its loop of launches).
+ * grad_dtype_tags may be NULL (every gradient has the dtype of its parameter).  Rows queued earlier run
+ * first.  If any row is refused nothing of the call runs. */
+int eri_adam8bit_fn_update_many(EriAdam8bitFn *opt, const char *const *names, const void *const *params,
+                                const void *const *grads, const uint64_t *numels, const int32_t *dtype_tags,
+                                const int32_t *grad_dtype_tags, void *const *outs, uint32_t n);
+int eri_adam8bit_fn_step(EriAdam8bitFn *opt);                   /* :89-92: runs what is queued, bumps the counter */
 int eri_adam8bit_fn_set_lr(EriAdam8bitFn *opt, float lr);       /* :95-98 */
 uint64_t eri_adam8bit_fn_get_step(const EriAdam8bitFn *opt);    /* :311-313 */
 /* memory_stats() :253-266: number of named states and their bytes */

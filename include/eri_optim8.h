@@ -14,7 +14,7 @@
  *   - streams are passed as void* and NULL means the default stream
  *     (crates/core/src/device.rs:69-71, tensor_narrow.rs:197-201).
  *   - dtype tags are F32=0, F16=1, BF16=2, I32=3 (crates/core/src/cuda/dtype_tag.rs:3-19);
- *     the optimizer accepts F32 and BF16 parameters/gradients.
+ *     the optimizer accepts F32 and BF16 parameters, with gradients of the same dtype or F32.
  *   - nothing here synchronises the device unless its name says so; the step is stream-ordered.
  *   - the library never takes ownership of parameter, gradient or state memory.
  */
@@ -134,19 +134,29 @@ int eri_adam8_hyper_pack(double lr, double beta1, double beta2, double eps, doub
                          uint64_t step, int mode, uint32_t flags, EriAdam8Hyper *out);
 
 /* One row of the launch table: a parameter tensor, its gradient and its 8-bit state.
- * m/v hold numel codes, absmax_* hold ceil(numel / 2048) floats.  All device pointers. */
+ * m/v hold numel codes, absmax_* hold ceil(numel / 2048) floats.  All device pointers.
+ * Rows are plain data: zero the struct first, so that fields added later read as "not used". */
 typedef struct EriAdam8Tensor {
-    void *p;              /* parameters, updated in place */
-    const void *g;        /* gradients, same dtype as p */
+    void *p;              /* the updated parameters are written here */
+    const void *g;        /* gradients: the dtype of p, or F32 if grad_f32 is set */
     uint8_t *m;           /* first-moment codes (signed dynamic map) */
     uint8_t *v;           /* second-moment codes (unsigned dynamic map) */
     float *absmax_m;      /* per-block scale of m */
     float *absmax_v;      /* per-block scale of v */
     uint64_t numel;
     uint64_t block_start; /* index of this tensor's first block = sum of the blocks before it */
-    int32_t dtype_tag;    /* ERI_DTYPE_F32 or ERI_DTYPE_BF16 */
+    int32_t dtype_tag;    /* ERI_DTYPE_F32 or ERI_DTYPE_BF16: the dtype of p */
     float grad_scale;     /* per-layer multiplier (pipeline_flux_lora_sequential.rs:759-766);
                              read only with ERI_ADAM8_FLAG_GRAD_SCALE */
+    const void *p_src;    /* NULL: p is updated in place (Parameter::apply_update, adam8bit_enhanced.rs:275).
+                             Otherwise the old parameters are read from p_src (dtype of p, numel elements,
+                             not overlapping p unless equal to it) and the new ones written to p, which is
+                             Adam8bit::update(name, param, grad) -> new tensor (adam8bit.rs:101-208) without a copy */
+    int32_t grad_f32;     /* non-zero with BF16 parameters: g holds F32 elements, which enter the arithmetic
+                             unrounded -- the reference casts every gradient to F32 and never rounds it
+                             (adam8bit_enhanced.rs:231-235, adam8bit.rs:110).  Such rows run on the
+                             four-waves-per-block kernel whatever the flags say.  Must be 0 for F32 parameters */
+    int32_t reserved;     /* 0 */
 } EriAdam8Tensor;
 
 typedef struct EriAdam8Table EriAdam8Table; /* device-resident copy of a launch table */
@@ -167,7 +177,8 @@ int eri_adam8_state_init(uint8_t *m, uint8_t *v, float *absmax_m, float *absmax_
  * only a stream that is being captured into a HIP graph cannot wait for an event outside the graph, and
  * there the host waits for the upload once instead. */
 int eri_adam8_table_create(const EriAdam8Tensor *rows, uint32_t n, void *stream, EriAdam8Table **out);
-/* Same tensors (count, numel, dtype), new pointers / grad_scale -- e.g. fresh gradient buffers. */
+/* Same tensors (count, numel, dtype of parameters and gradients), new pointers / grad_scale -- e.g. fresh
+ * gradient buffers, or the fresh output tensors of a functional update. */
 int eri_adam8_table_update(EriAdam8Table *table, const EriAdam8Tensor *rows, uint32_t n, void *stream);
 int eri_adam8_table_destroy(EriAdam8Table *table);
 int eri_adam8_table_info(const EriAdam8Table *table, uint64_t *total_numel, uint64_t *total_blocks);

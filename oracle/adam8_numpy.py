@@ -90,18 +90,22 @@ def _blockwise(x, numel):
     return np.concatenate([x, np.zeros(pad, x.dtype)]).reshape(nb, BLOCK), nb
 
 
-def step_tensor(p, g, m_code, v_code, absmax_m, absmax_v, h, map_s, map_u, bf16=False):
+def step_tensor(p, g, m_code, v_code, absmax_m, absmax_v, h, map_s, map_u, bf16=False, grad_bf16=None):
     """Returns (p_new, m_code_new, v_code_new, absmax_m_new, absmax_v_new); inputs untouched.
 
-    p and g are float32 arrays, or uint16 bf16 bit patterns when bf16=True.
+    p and g are float32 arrays, or uint16 bf16 bit patterns when bf16=True.  grad_bf16=False with bf16=True
+    is a float32 gradient for bf16 parameters: the reference casts every gradient to F32 and never rounds it
+    (adam8bit_enhanced.rs:231-235).
     """
+    if grad_bf16 is None:
+        grad_bf16 = bf16
     numel = int(np.asarray(m_code).size)
     if numel == 0:
         raise ValueError("Empty tensor for quantization")
     map_s = np.asarray(map_s, F32)
     map_u = np.asarray(map_u, F32)
     pf = bf16_to_f32(p) if bf16 else np.asarray(p, F32)
-    gf = bf16_to_f32(g) if bf16 else np.asarray(g, F32)
+    gf = bf16_to_f32(g) if grad_bf16 else np.asarray(g, F32)
     blk = np.arange(numel) // BLOCK
     with np.errstate(all="ignore"):
         m_old = map_s[m_code] * absmax_m[blk]

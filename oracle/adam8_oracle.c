@@ -160,7 +160,7 @@ static inline float load_elem(const void *base, uint64_t i, int dtype) {
 }
 
 static void step_block(void *p, const void *g, uint8_t *mc, uint8_t *vc, float *am, float *av,
-                       uint64_t base, int n, int dtype, const EriOracleHyper *h,
+                       uint64_t base, int n, int dtype, int g_dtype, const EriOracleHyper *h,
                        const float *map_s, const float *map_u, const float *mid_s,
                        const float *mid_u) {
     float mbuf[ERI_ORACLE_BLOCK], vbuf[ERI_ORACLE_BLOCK];
@@ -170,7 +170,7 @@ static void step_block(void *p, const void *g, uint8_t *mc, uint8_t *vc, float *
         const uint64_t e = base + (uint64_t)i;
         float m_old = map_s[mc[e]] * a_m;
         float v_old = map_u[vc[e]] * a_v;
-        float gr = load_elem(g, e, dtype);
+        float gr = load_elem(g, e, g_dtype);            /* the gradient as F32, whatever it is stored in: :231-235 */
         float pf = load_elem(p, e, dtype);
         if (h->use_grad_scale) gr = gr * h->grad_scale;
         if (h->mode == ERI_ORACLE_MODE_L2 && h->weight_decay > 0.0f) {
@@ -241,11 +241,15 @@ static void step_block(void *p, const void *g, uint8_t *mc, uint8_t *vc, float *
  * quantise an empty tensor, adam8bit_enhanced.rs:46-50), -2 for an unsupported dtype.
  * threads <= 1 runs serially; otherwise blocks are split statically over that many threads.
  */
-int eri_oracle_step_tensor(void *p, const void *g, uint8_t *m, uint8_t *v, float *absmax_m,
-                           float *absmax_v, uint64_t numel, int dtype, const EriOracleHyper *h,
-                           const float *map_s, const float *map_u, int threads) {
+/* `g_dtype` is the storage type of the gradient, which may differ from the parameter's: the reference
+ * casts every gradient to F32 before it uses it and never rounds it back
+ * (adam8bit_enhanced.rs:231-235, adam8bit.rs:110). */
+int eri_oracle_step_tensor_g(void *p, const void *g, uint8_t *m, uint8_t *v, float *absmax_m,
+                             float *absmax_v, uint64_t numel, int dtype, int g_dtype, const EriOracleHyper *h,
+                             const float *map_s, const float *map_u, int threads) {
     if (numel == 0) return -1;
     if (dtype != ERI_ORACLE_F32 && dtype != ERI_ORACLE_BF16) return -2;
+    if (g_dtype != ERI_ORACLE_F32 && g_dtype != ERI_ORACLE_BF16) return -2;
     float mid_s[255], mid_u[255];
     eri_oracle_midpoints(map_s, mid_s);
     eri_oracle_midpoints(map_u, mid_u);
@@ -258,10 +262,17 @@ int eri_oracle_step_tensor(void *p, const void *g, uint8_t *m, uint8_t *v, float
         uint64_t base = (uint64_t)b * ERI_ORACLE_BLOCK;
         uint64_t left = numel - base;
         int n = left < ERI_ORACLE_BLOCK ? (int)left : ERI_ORACLE_BLOCK;
-        step_block(p, g, m, v, absmax_m + b, absmax_v + b, base, n, dtype, h, map_s, map_u, mid_s,
+        step_block(p, g, m, v, absmax_m + b, absmax_v + b, base, n, dtype, g_dtype, h, map_s, map_u, mid_s,
                    mid_u);
     }
     return 0;
+}
+
+/* Gradient stored in the parameter's dtype. */
+int eri_oracle_step_tensor(void *p, const void *g, uint8_t *m, uint8_t *v, float *absmax_m,
+                           float *absmax_v, uint64_t numel, int dtype, const EriOracleHyper *h,
+                           const float *map_s, const float *map_u, int threads) {
+    return eri_oracle_step_tensor_g(p, g, m, v, absmax_m, absmax_v, numel, dtype, dtype, h, map_s, map_u, threads);
 }
 
 /* Fresh state: the codes of 0.0 with absmax 0, what quantising a zeros tensor gives

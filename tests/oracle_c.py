@@ -49,6 +49,9 @@ def lib():
         L.eri_oracle_step_tensor.restype = C.c_int
         L.eri_oracle_step_tensor.argtypes = [C.c_void_p] * 6 + [C.c_uint64, C.c_int, C.POINTER(Hyper),
                                                                C.c_void_p, C.c_void_p, C.c_int]
+        L.eri_oracle_step_tensor_g.restype = C.c_int
+        L.eri_oracle_step_tensor_g.argtypes = [C.c_void_p] * 6 + [C.c_uint64, C.c_int, C.c_int, C.POINTER(Hyper),
+                                                                 C.c_void_p, C.c_void_p, C.c_int]
         L.eri_oracle_state_init.argtypes = [C.c_void_p] * 4 + [C.c_uint64]
         L.eri_oracle_dequantize.argtypes = [C.c_void_p] * 3 + [C.c_uint64, C.c_void_p]
         L.eri_oracle_quantize.argtypes = [C.c_void_p] * 2 + [C.c_uint64, C.c_void_p, C.c_void_p]
@@ -88,10 +91,11 @@ def state_init(numel):
     return m, v, am, av
 
 
-def step_tensor(p, g, m, v, am, av, h, maps, dtype, threads=1):
-    """In place on p, m, v, am, av (NumPy arrays: float32, or uint16 bit patterns for bf16)."""
+def step_tensor(p, g, m, v, am, av, h, maps, dtype, threads=1, g_dtype=None):
+    """In place on p, m, v, am, av (NumPy arrays: float32, or uint16 bit patterns for bf16).
+    g_dtype: storage type of g when it differs from the parameter's (float32 gradients for bf16 parameters)."""
     s, u = maps
     for a in (p, g, m, v, am, av):
         assert a.flags["C_CONTIGUOUS"]
-    return lib().eri_oracle_step_tensor(ptr(p), ptr(g), ptr(m), ptr(v), ptr(am), ptr(av), m.size, dtype,
-                                        C.byref(h), ptr(s), ptr(u), threads)
+    return lib().eri_oracle_step_tensor_g(ptr(p), ptr(g), ptr(m), ptr(v), ptr(am), ptr(av), m.size, dtype,
+                                          dtype if g_dtype is None else g_dtype, C.byref(h), ptr(s), ptr(u), threads)

@@ -58,9 +58,10 @@ def test_build_rs_compiles_the_objects_of_the_makefile():
 
 def test_struct_layouts_match_the_header():
     assert C.sizeof(L.Hyper) == 48
-    assert C.sizeof(L.TensorRow) == 72
+    assert C.sizeof(L.TensorRow) == 88
     assert C.sizeof(L.AdamW32Row) == 56 and C.sizeof(L.EmaRow) == 32
     assert L.TensorRow.numel.offset == 48 and L.TensorRow.dtype_tag.offset == 64
+    assert L.TensorRow.p_src.offset == 72 and L.TensorRow.grad_f32.offset == 80
 
 
 def test_maps_equal_the_fixture():

@@ -1,5 +1,7 @@
-"""Parity at the benchmark's full size: the FLUX-12B-shaped set (780 bf16 tensors, 11.9e9
-parameters, ~72 GB resident).  The oracle cannot sweep that in reasonable time, so the check is
+"""Parity at the full size of the two full fine-tune configurations: the FLUX-12B-shaped set (780 bf16
+tensors, 11.9e9 parameters, ~72 GB resident) and the SDXL-UNet-shaped set (1,680 tensors from 4 to
+29.5e6 elements, 2.57e9 parameters, 828 of them with a partial last block).  The oracle cannot sweep
+those in reasonable time, so the check is
 (a) the oracle on a sample of blocks -- first, last and partial blocks of tensors plus random ones --
 whose inputs are copied out before the step, and (b) properties that hold for every block and are
 cheap to evaluate on the device: each block's largest second moment carries code 255 and its largest
@@ -18,18 +20,27 @@ BLOCK = 2048
 
 
 def test_flux12b_full_size_sampled_blocks_and_block_properties():
+    from eridiffusion_amd import workloads as W
+    _full_size(W.c5_flux_full(), 0xE21D + 5, 11_901_408_320, 5_811_496, 80e9)
+
+
+def test_sdxl_unet_full_size_sampled_blocks_and_block_properties():
+    from eridiffusion_amd import workloads as W
+    _full_size(W.c4_sdxl_full(), 0xE21D + 4, 2_567_463_684, 1_254_022, 20e9)
+
+
+def _full_size(tensors, seed, want_numel, want_blocks, need_bytes):
     import torch
     from eridiffusion_amd import _lib as L
     from eridiffusion_amd import workloads as W
 
     free, total = torch.cuda.mem_get_info()
-    if free < 80e9:
-        pytest.skip("needs ~75 GB of free device memory")
-    tensors = W.c5_flux_full()
+    if free < need_bytes:
+        pytest.skip("needs %.0f GB of free device memory" % (need_bytes / 1e9))
     sizes = [W.numel(s) for _, s in tensors]
     dev = torch.device("cuda:0")
     gen = torch.Generator(device=dev)
-    gen.manual_seed(0xE21D + 5)
+    gen.manual_seed(seed)
     GUARD = 256  # poisoned bytes after every tensor's codes
 
     def arena(byte_sizes):
@@ -65,7 +76,7 @@ def test_flux12b_full_size_sampled_blocks_and_block_properties():
     L.check(L.lib().eri_adam8_table_create(rows, len(rows), stream, C.byref(table)), "table_create")
     total_numel, total_blocks = C.c_uint64(), C.c_uint64()
     L.check(L.lib().eri_adam8_table_info(table, C.byref(total_numel), C.byref(total_blocks)), "table_info")
-    assert total_numel.value == 11_901_408_320 and total_blocks.value == 5_811_496
+    assert total_numel.value == want_numel and total_blocks.value == want_blocks
 
     rng = np.random.default_rng(3)
     sample = set()
@@ -93,9 +104,10 @@ def test_flux12b_full_size_sampled_blocks_and_block_properties():
 
     hyper = (1e-4, 0.9, 0.999, 1e-8, 0.01)
     flips = 0
-    for t in (1, 2):
+    for t in (1, 2, 3, 4):  # two steps on the default arithmetic, then two with the IEEE chain
+        exact = t > 2
         before = grab()
-        h = L.hyper_pack(*hyper, t, L.MODE_ERI, 0)
+        h = L.hyper_pack(*hyper, t, L.MODE_ERI, L.FLAG_EXACT_PARAM if exact else 0)
         L.check(L.lib().eri_adam8_step_table(table, C.byref(h), stream), "step_table")
         torch.cuda.synchronize()
         after = grab()
@@ -107,9 +119,10 @@ def test_flux12b_full_size_sampled_blocks_and_block_properties():
             assert np.array_equal(got[4].view(np.uint32), am.view(np.uint32))
             assert np.array_equal(got[5].view(np.uint32), av.view(np.uint32))
             d = hs.bf16_ulp_distance(got[0], p)
-            assert d.max() <= 1
+            assert d.max() <= (0 if exact else 1)
             flips += int((d != 0).sum())
-    print("full-size sample: %d blocks x 2 steps, bf16 parameters one ulp off: %d" % (len(sample), flips), flush=True)
+    print("full-size sample of %d tensors: %d blocks x (2 default + 2 exact) steps, bf16 parameters one ulp off: %d" %
+          (len(sizes), len(sample), flips), flush=True)
 
     # properties of every block
     for i, n in enumerate(sizes):

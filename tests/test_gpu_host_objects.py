@@ -256,7 +256,7 @@ def test_functional_updates_of_several_names_in_turn():
             out = torch.zeros(n * (2 if bf16 else 4), dtype=torch.uint8, device=dev)
             keep += [g_dev, out, cur]
             L.check(L.lib().eri_adam8bit_fn_update(opt, name, cur.data_ptr(), g_dev.data_ptr(), n, 2 if bf16 else 0,
-                                                   out.data_ptr()), "fn_update")
+                                                   2 if bf16 else 0, out.data_ptr()), "fn_update")
             host[name][3] = out
             hs.oracle_step(ps, gs, states, (1e-4, B1, B2, EPS, WD, rnd), bf16, mode=oc.MODE_L2)
         L.check(L.lib().eri_adam8bit_fn_step(opt), "fn_step")
@@ -289,7 +289,7 @@ def test_functional_update_returns_a_new_tensor(bf16):
     for call in range(3):  # update, update, step, update: calls 1 and 2 both see counter 0 -> s = 1
         src = p_dev if call == 0 else out_dev
         L.check(L.lib().eri_adam8bit_fn_update(opt, b"layer.lora_down", src.data_ptr(), g_dev.data_ptr(), n,
-                                               2 if bf16 else 0, out_dev.data_ptr()), "fn_update")
+                                               2 if bf16 else 0, 2 if bf16 else 0, out_dev.data_ptr()), "fn_update")
         step = 0 if call < 2 else 1
         hs.oracle_step(ps, gs, states, (1e-4, B1, B2, EPS, WD, step), bf16, mode=oc.MODE_L2)
         if call == 1:
@@ -388,6 +388,104 @@ def test_legacy_state_longer_than_one_staging_piece(tmp_path):
             L.check(L.lib().eri_hip_stream_sync(None), "sync")
             assert np.array_equal(got_c, codes)
             assert np.array_equal(got_a.view(np.uint32), absmax.view(np.uint32))
+    L.lib().eri_adam8bit_destroy(opt)
+    for h in handles:
+        L.lib().eri_param_release(h)
+
+
+def test_min_8bit_size_keeps_short_tensors_in_fp32_moments(tmp_path):
+    """Parameters below min_8bit_size take the same update with fp32 moments (one launch of the 32-bit step
+    for all of them), the others the 8-bit step; both against their oracles over three steps, then a
+    save / load round trip that carries both kinds of state, and the refusals."""
+    import torch
+    L = _L()
+    sizes = [2048 * 3 + 5, 300, 4095, 4096, 64, 2048 * 2]
+    dts = [True, True, False, True, True, False]  # bf16?
+    small = [n < 4096 for n in sizes]
+    dev = torch.device("cuda:0")
+    host_p, dev_p, handles = [], [], (C.c_void_p * len(sizes))()
+    for i, (n, bf16) in enumerate(zip(sizes, dts)):
+        ps, _ = hs.make_inputs([n], bf16, 900 + i)
+        host_p.append(ps[0])
+        dev_p.append(torch.from_numpy(ps[0].view(np.uint8).copy()).to(dev))
+        h = C.c_void_p()
+        L.check(L.lib().eri_param_create(dev_p[i].data_ptr(), n, 2 if bf16 else 0, C.byref(h)), "param_create")
+        handles[i] = h
+    cfg = L.Adam8bitConfigC(1e-4, B1, B2, EPS, WD, 0, 1, 100)
+
+    def make():
+        o = C.c_void_p()
+        L.check(L.lib().eri_adam8bit_new(handles, len(sizes), C.byref(cfg), None, C.byref(o)), "new")
+        L.check(L.lib().eri_adam8bit_set_flags(o, L.FLAG_EXACT_PARAM), "set_flags")
+        L.check(L.lib().eri_adam8bit_set_min_8bit_size(o, 4096), "set_min_8bit_size")
+        return o
+
+    opt = make()
+    states8 = [list(oc.state_init(n)) for n in sizes]
+    states32 = [[np.zeros(n, np.float32), np.zeros(n, np.float32)] for n in sizes]
+    keep = []
+
+    def one_step(o, t):
+        gs = [hs.fresh_grads([n], bf16, 100 * t + i)[0] for i, (n, bf16) in enumerate(zip(sizes, dts))]
+        g_dev = [torch.from_numpy(g.view(np.uint8).copy()).to(dev) for g in gs]
+        keep.append(g_dev)
+        for i in range(len(sizes)):
+            L.check(L.lib().eri_param_set_grad(handles[i], g_dev[i].data_ptr()), "set_grad")
+        L.check(L.lib().eri_adam8bit_step(o, None), "step")
+        h = oc.hyper_pack(1e-4, B1, B2, EPS, WD, t)
+        for i, (n, bf16) in enumerate(zip(sizes, dts)):
+            dt = oc.DT_BF16 if bf16 else oc.DT_F32
+            if small[i]:
+                oc.lib().eri_oracle_adamw32_step(oc.ptr(host_p[i]), oc.ptr(gs[i]), oc.ptr(states32[i][0]), oc.ptr(states32[i][1]),
+                                                 n, dt, float(h.step_size), B1, B2, EPS, WD, None)
+            else:
+                assert oc.step_tensor(host_p[i], gs[i], *states8[i], h, hs.MAPS, dt, 2) == 0
+
+    def check(o):
+        _sync()
+        for i, (n, bf16) in enumerate(zip(sizes, dts)):
+            bits = np.uint16 if bf16 else np.uint32
+            assert np.array_equal(dev_p[i].cpu().numpy().view(bits), host_p[i].view(bits)), i
+            m32, v32 = C.c_void_p(), C.c_void_p()
+            L.check(L.lib().eri_adam8bit_state32_ptrs(o, i, C.byref(m32), C.byref(v32)), "state32_ptrs")
+            ptrs = [C.c_void_p() for _ in range(4)]
+            L.check(L.lib().eri_adam8bit_state_ptrs(o, i, *[C.byref(q) for q in ptrs]), "state_ptrs")
+            if small[i]:
+                assert m32.value and v32.value and not ptrs[0].value
+                for src, want in ((m32, states32[i][0]), (v32, states32[i][1])):
+                    got = torch.empty(n, dtype=torch.float32, device=dev)
+                    L.check(L.lib().eri_hip_memcpy_async(got.data_ptr(), src.value, 4 * n, 3, None), "memcpy")
+                    _sync()
+                    assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32)), i
+            else:
+                assert ptrs[0].value and not m32.value
+                got = torch.empty(n, dtype=torch.uint8, device=dev)
+                L.check(L.lib().eri_hip_memcpy_async(got.data_ptr(), ptrs[0].value, n, 3, None), "memcpy")
+                _sync()
+                assert np.array_equal(got.cpu().numpy(), states8[i][0]), i
+
+    for t in (1, 2, 3):
+        one_step(opt, t)
+    check(opt)
+    want_bytes = sum(8 * n if s else 2 * n + 8 * ((n + 2047) // 2048) for n, s in zip(sizes, small))
+    assert L.lib().eri_adam8bit_quantized_memory_usage(opt) == want_bytes
+    # save, load into a fresh optimizer, continue there: same trajectory
+    path = tmp_path / "mixed_state.safetensors"
+    L.check(L.lib().eri_adam8bit_save_state(opt, str(path).encode()), "save_state")
+    _sync()
+    L.lib().eri_adam8bit_destroy(opt)
+    opt = make()
+    L.check(L.lib().eri_adam8bit_load_state(opt, str(path).encode()), "load_state")
+    assert L.lib().eri_adam8bit_get_step(opt) == 3
+    one_step(opt, 4)
+    check(opt)
+    # refusals: scaling or clipping inside the step, and mode BNB, cannot be combined with fp32-moment parameters
+    L.check(L.lib().eri_adam8bit_set_grad_scale(opt, 0.5), "set_grad_scale")
+    assert L.lib().eri_adam8bit_step(opt, None) == -6
+    L.check(L.lib().eri_adam8bit_set_grad_scale(opt, 1.0), "set_grad_scale")
+    L.check(L.lib().eri_adam8bit_set_max_grad_norm(opt, 1.0, 0.0), "set_max_grad_norm")
+    assert L.lib().eri_adam8bit_step(opt, None) == -6
+    assert b"min_8bit_size" in L.lib().eri_last_error()
     L.lib().eri_adam8bit_destroy(opt)
     for h in handles:
         L.lib().eri_param_release(h)

@@ -89,10 +89,23 @@ def test_functional_flavour_counters_and_errors():
     assert L.lib().eri_adam8bit_fn_set_lr(opt, 3e-4) == 0
     n, b = C.c_uint64(5), C.c_uint64(5)
     assert L.lib().eri_adam8bit_fn_memory_stats(opt, C.byref(n), C.byref(b)) == 0 and (n.value, b.value) == (0, 0)
-    assert L.lib().eri_adam8bit_fn_update(opt, b"w", 0x1000, 0x2000, 0, L.DTYPE_BF16, 0x1000) == -3
-    assert b"Empty tensor for quantization" in L.lib().eri_last_error()
-    assert L.lib().eri_adam8bit_fn_update(opt, b"w", 0x1000, 0x2000, 16, L.DTYPE_I32, 0x1000) == -4
-    assert L.lib().eri_adam8bit_fn_update(opt, None, 0x1000, 0x2000, 16, L.DTYPE_BF16, 0x1000) == -1
+    BF, F32 = L.DTYPE_BF16, L.DTYPE_F32
+    for batching in (0, 1):  # argument errors are reported by the call that made them, queued or not
+        assert L.lib().eri_adam8bit_fn_set_batching(opt, batching) == 0
+        assert L.lib().eri_adam8bit_fn_update(opt, b"w", 0x1000, 0x2000, 0, BF, BF, 0x1000) == -3
+        assert b"Empty tensor for quantization" in L.lib().eri_last_error()
+        assert L.lib().eri_adam8bit_fn_update(opt, b"w", 0x1000, 0x2000, 16, L.DTYPE_I32, L.DTYPE_I32, 0x1000) == -4
+        assert L.lib().eri_adam8bit_fn_update(opt, b"w", 0x1000, 0x2000, 16, F32, BF, 0x1000) == -4  # F32 parameters, BF16 gradients
+        assert L.lib().eri_adam8bit_fn_update(opt, None, 0x1000, 0x2000, 16, BF, BF, 0x1000) == -1
+        assert L.lib().eri_adam8bit_fn_update(opt, b"w", 0x1000, 0x2008, 16, BF, F32, 0x1000) == -2
+        assert L.lib().eri_adam8bit_fn_flush(opt) == 0  # nothing was queued
+    names = (C.c_char_p * 1)(b"w")
+    ptrs = (C.c_void_p * 1)(0x1000)
+    numels = (C.c_uint64 * 1)(0)
+    tags = (C.c_int32 * 1)(BF)
+    assert L.lib().eri_adam8bit_fn_update_many(opt, names, ptrs, ptrs, numels, tags, None, ptrs, 1) == -3
+    assert L.lib().eri_adam8bit_fn_update_many(opt, None, ptrs, ptrs, numels, tags, None, ptrs, 1) == -1
+    assert L.lib().eri_adam8bit_fn_update_many(opt, names, ptrs, ptrs, numels, tags, None, ptrs, 0) == 0
     numel = C.c_uint64(9)
     assert L.lib().eri_adam8bit_fn_state_numel(opt, b"w", C.byref(numel)) == 0 and numel.value == 0
     assert L.lib().eri_adam8bit_fn_get_state_fp32(opt, b"w", 0x1000, 0x2000) == -6

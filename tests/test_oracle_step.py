@@ -373,3 +373,47 @@ def test_two_restatements_agree_on_randomized_cases_with_extreme_values():
                     assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), (case, t, k)
                 else:
                     assert np.array_equal(a, b), (case, t, k)
+
+
+@pytest.mark.parametrize("mode", [oc.MODE_ERI, oc.MODE_L2, oc.MODE_BNB])
+def test_f32_gradient_for_bf16_parameters_is_used_unrounded(mode):
+    """The storage type of the gradient (adam8bit_enhanced.rs:231-235: cast to F32, never rounded).
+    Pinned three ways: (1) a float32 gradient whose values are bf16 values gives exactly what the same
+    values stored as bf16 give -- the storage type alone changes nothing; (2) a float32 gradient with low
+    mantissa bits set gives what float32 *parameters* holding the same bf16 values give for the moments
+    (the moments of the modes ERI and BNB depend on the gradient only), i.e. no rounding happened on the
+    way in; (3) the C and NumPy restatements agree bit for bit."""
+    n = 3 * 2048 + 321
+    rng = np.random.default_rng(77 + mode)
+    p16 = onp.f32_to_bf16((rng.standard_normal(n) * 0.02).astype(np.float32))
+    g32 = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    assert (g32.view(np.uint32) & 0xFFFF).any()
+    step = 0 if mode == oc.MODE_L2 else 1
+    h = oc.hyper_pack(1e-4, 0.9, 0.999, 1e-8, 0.01, step, mode)
+    maps = oc.load_maps()
+
+    def run(p, g, dtype, g_dtype):
+        p = p.copy()
+        st = list(oc.state_init(n))
+        assert oc.step_tensor(p, g, *st, h, maps, dtype, 2, g_dtype=g_dtype) == 0
+        return p, st
+
+    # (1)
+    g16 = onp.f32_to_bf16(g32)
+    a_p, a_st = run(p16, g16, oc.DT_BF16, oc.DT_BF16)
+    b_p, b_st = run(p16, onp.bf16_to_f32(g16), oc.DT_BF16, oc.DT_F32)
+    assert np.array_equal(a_p, b_p) and all(np.array_equal(x.view(np.uint8), y.view(np.uint8)) for x, y in zip(a_st, b_st))
+    # (2)
+    c_p, c_st = run(p16, g32, oc.DT_BF16, oc.DT_F32)
+    assert not all(np.array_equal(x.view(np.uint8), y.view(np.uint8)) for x, y in zip(a_st, c_st))  # rounding first differs
+    if mode != oc.MODE_L2:  # (in mode L2 the decay enters the gradient, and with it the parameter's dtype does not matter either)
+        d_p, d_st = run(onp.bf16_to_f32(p16), g32, oc.DT_F32, oc.DT_F32)
+        assert all(np.array_equal(x.view(np.uint8), y.view(np.uint8)) for x, y in zip(c_st, d_st))
+        assert np.array_equal(c_p, onp.f32_to_bf16(d_p))  # one parameter update from the same fp32 values, rounded once
+    # (3)
+    modes = {oc.MODE_ERI: "eri", oc.MODE_L2: "l2", oc.MODE_BNB: "bnb"}
+    hn = onp.hyper_pack(1e-4, 0.9, 0.999, 1e-8, 0.01, step, modes[mode])
+    st0 = onp.state_init(n)
+    n_p, n_m, n_v, n_am, n_av = onp.step_tensor(p16, g32, *st0, hn, *maps, bf16=True, grad_bf16=False)
+    assert np.array_equal(n_p, c_p) and np.array_equal(n_m, c_st[0]) and np.array_equal(n_v, c_st[1])
+    assert np.array_equal(n_am.view(np.uint32), c_st[2].view(np.uint32)) and np.array_equal(n_av.view(np.uint32), c_st[3].view(np.uint32))

@@ -96,3 +96,33 @@ def test_ema_is_a_convex_combination():
     oc.lib().eri_oracle_ema_update(oc.ptr(sb), oc.ptr(pb), 1000, oc.DT_BF16, 0.9)
     want = 0.9 * onp.bf16_to_f32(onp.f32_to_bf16(s0)).astype(np.float64) + 0.1 * onp.bf16_to_f32(pb)
     assert np.all(np.abs(onp.bf16_to_f32(sb) - want) <= np.abs(want) * 2 ** -8 + 1e-30)
+
+
+def test_adamw32_with_the_bias_corrected_step_size_is_the_8bit_update_without_a_quantiser():
+    """min_8bit_size sends short tensors to the 32-bit step with lr = the step size of Adam8bit::step.  That is
+    the same update with fp32 moments: restated here in NumPy from adam8bit_enhanced.rs:252-275, one rounded
+    operation per line, it must agree with the 32-bit oracle bit for bit over several steps, bf16 and fp32."""
+    F = np.float32
+    rng = np.random.default_rng(5)
+    n = 3000
+    for bf16 in (False, True):
+        p32 = (rng.standard_normal(n) * 0.02).astype(F)
+        p = onp.f32_to_bf16(p32) if bf16 else p32.copy()
+        q = p.copy()
+        m, v = np.zeros(n, F), np.zeros(n, F)
+        mm, vv = np.zeros(n, F), np.zeros(n, F)
+        for t in range(1, 6):
+            g32 = (rng.standard_normal(n) * 1e-3).astype(F)
+            g = onp.f32_to_bf16(g32) if bf16 else g32
+            h = oc.hyper_pack(1e-4, 0.9, 0.999, 1e-8, 0.01, t)
+            adamw(p, g, m, v, oc.DT_BF16 if bf16 else oc.DT_F32, lr=float(h.step_size), b1=0.9, b2=0.999, eps=1e-8, wd=0.01)
+            gf = onp.bf16_to_f32(g) if bf16 else g
+            qf = onp.bf16_to_f32(q) if bf16 else q
+            mm = mm * F(h.beta1) + gf * F(h.omb1)            # :256
+            vv = vv * F(h.beta2) + (gf * gf) * F(h.omb2)     # :259-260
+            r = mm / (np.sqrt(vv) + F(h.eps))                # :263-264
+            u = r + qf * F(h.weight_decay)                   # :267-271
+            qn = (qf - u * F(h.step_size)).astype(F)         # :274-275
+            q = onp.f32_to_bf16(qn) if bf16 else qn
+            assert np.array_equal(m.view(np.uint32), mm.view(np.uint32)) and np.array_equal(v.view(np.uint32), vv.view(np.uint32))
+            assert np.array_equal(p.view(np.uint16 if bf16 else np.uint32), q.view(np.uint16 if bf16 else np.uint32)), (bf16, t)
