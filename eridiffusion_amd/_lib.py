@@ -91,6 +91,7 @@ EXPORTS = {
     "eri_adam8_table_info": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "eri_adam8_step_table": (C.c_int, [C.c_void_p, C.POINTER(Hyper), C.c_void_p]),
     "eri_adam8_grad_norm": (C.c_int, [C.c_void_p, C.c_float, C.c_float, C.c_void_p]),
+    "eri_adam8_grad_norm_static": (C.c_int, [C.c_void_p, C.c_float, C.c_float, C.c_void_p, C.c_void_p]),
     "eri_adam8_grad_norm_read": (C.c_int, [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_void_p]),
     "eri_adam8_grad_nonfinite_read": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint64), C.c_void_p]),
     "eri_adam8_quant_error": (C.c_int, [C.c_void_p, C.POINTER(Hyper), C.c_void_p]),

@@ -187,8 +187,16 @@ const Tables &tables() {
 
 constexpr int kMaxDevices = 16;
 
+/* Scratch of eri_adam8_grad_norm_static: the per-wave partial sums of the gradient-norm pass, in device
+ * memory that exists from the moment the library is loaded until the process ends (every device the
+ * library runs on holds its own copy, 384 KiB).  The name below is a host-side stand-in, not a device
+ * address: host code uses DeviceCtx::scratch_ptr, which hipGetSymbolAddress filled in for that device. */
+constexpr uint32_t kNormScratchPairs = 24576; // {sum of squares, non-finite count} per wave: 3 groups x 256 CUs x 32 waves
+static __device__ __align__(256) double scratch[2 * kNormScratchPairs];
+
 struct DeviceCtx {
     void *image = nullptr; // device copy of the LDS image
+    double *scratch_ptr = nullptr; // address of this device's copy of the static array `scratch`
     uint32_t cus = 0;
     uint32_t wg = 1024;      // threads per workgroup: the table image (~100 KB of LDS) allows one per CU
     uint32_t wg_per_cu = 1;  // persistent workgroups per compute unit
@@ -217,6 +225,13 @@ int get_ctx(DeviceCtx **out) {
             (void)hipFree(image);
             return hip_fail(e, "upload of the quantisation tables");
         }
+        double *ptr = nullptr; // once per device, with that device current
+        const hipError_t se = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+        if (se != hipSuccess || !ptr) {
+            (void)hipFree(image);
+            return hip_fail(se != hipSuccess ? se : hipErrorInvalidSymbol, "address of the static gradient-norm scratch");
+        }
+        c.scratch_ptr = ptr;
         c.image = image;
         c.ready = true;
     }
@@ -783,6 +798,17 @@ int eri_adam8_grad_norm(EriAdam8Table *t, float max_norm, float denom_eps, void 
     if (!t->partial) ERI_HIP(hipMalloc((void **)&t->partial, sizeof(double) * 2 * pairs));
     if (!t->norm_out) ERI_HIP(hipMalloc((void **)&t->norm_out, sizeof(float) * 4)); // norm, scale, 64-bit count
     return grad_norm_launch(t, ctx, max_norm, denom_eps, t->partial, pairs, t->norm_out, stream);
+}
+
+int eri_adam8_grad_norm_static(EriAdam8Table *t, float max_norm, float denom_eps, void *result, void *stream) {
+    if (!t || !result) return fail(ERI_ERR_NULL, "table or result is NULL");
+    if ((uintptr_t)result & 7u) return fail(ERI_ERR_ALIGN, "result must be 8-byte aligned");
+    int dev = -1;
+    ERI_HIP(hipGetDevice(&dev));
+    if (dev != t->device) return fail(ERI_ERR_ARG, "the table belongs to another device than the current one");
+    DeviceCtx *ctx = &g_ctx[dev]; // made ready, scratch address included, when the table was created
+    if (!ctx->ready || !ctx->scratch_ptr) return fail(ERI_ERR_INTERNAL, "the library was not initialised on this device");
+    return grad_norm_launch(t, ctx, max_norm, denom_eps, ctx->scratch_ptr, kNormScratchPairs, static_cast<float *>(result), stream);
 }
 
 int eri_adam8_grad_norm_read(EriAdam8Table *t, float *norm, float *scale, void *stream) {

@@ -92,6 +92,7 @@ extern "C" {
     pub fn eri_adam8_table_info(table: *const EriAdam8Table, total_numel: *mut u64, total_blocks: *mut u64) -> c_int;
     pub fn eri_adam8_step_table(table: *mut EriAdam8Table, hyper: *const EriAdam8Hyper, stream: *mut c_void) -> c_int;
     pub fn eri_adam8_grad_norm(table: *mut EriAdam8Table, max_norm: f32, denom_eps: f32, stream: *mut c_void) -> c_int;
+    pub fn eri_adam8_grad_norm_static(table: *mut EriAdam8Table, max_norm: f32, denom_eps: f32, result: *mut c_void, stream: *mut c_void) -> c_int;
     pub fn eri_adam8_grad_norm_read(table: *mut EriAdam8Table, norm: *mut f32, scale: *mut f32, stream: *mut c_void) -> c_int;
     pub fn eri_adam8_grad_nonfinite_read(table: *mut EriAdam8Table, count: *mut u64, stream: *mut c_void) -> c_int;
     pub fn eri_adam8_quant_error(table: *mut EriAdam8Table, hyper: *const EriAdam8Hyper, stream: *mut c_void) -> c_int;

@@ -195,6 +195,18 @@ int eri_adam8_step_table(EriAdam8Table *table, const EriAdam8Hyper *hyper, void 
  * clip_grads_global_norm_fp32_tensors (crates/training/src/optimizer.rs:58-85).  A following step with
  * ERI_ADAM8_FLAG_CLIP_FROM_TABLE applies the factor inside the kernel instead of rewriting gradients. */
 int eri_adam8_grad_norm(EriAdam8Table *table, float max_norm, float denom_eps, void *stream);
+/* The same pass for callers that cannot allocate (code under HIP graph capture, serving loops, harnesses
+ * that forbid hipMalloc).  It has no counterpart in the reference.  eri_adam8_grad_norm allocates the
+ * per-wave partial sums and the result words on a table's first call; this variant allocates nothing:
+ * the partial sums go to a static device array of the library (384 KiB per device, 24,576 per-wave
+ * pairs; a table whose pass needs more is refused with ERI_ERR_TOO_LARGE -- none does on a 256-CU
+ * MI355X) and the result to `result`, 16 bytes of device memory the caller owns, 8-byte aligned:
+ * {float norm, float scale, uint64 count of non-finite elements}.  A following step with
+ * ERI_ADAM8_FLAG_CLIP_FROM_TABLE, and the two read calls below, use `result` until the next norm pass
+ * of the table, so it must stay valid that long.  All calls on one device share the array: two such
+ * calls that overlap in time on one device (different streams, different tables) race.  Nothing in
+ * the array has to start at zero (every wave of a pass writes its pair before the pair is read). */
+int eri_adam8_grad_norm_static(EriAdam8Table *table, float max_norm, float denom_eps, void *result, void *stream);
 /* Copies the last norm and clip factor to the host; waits for `stream`. */
 int eri_adam8_grad_norm_read(EriAdam8Table *table, float *norm, float *scale, void *stream);
 /* How many gradient elements of the table were NaN or +-infinity in the last eri_adam8_grad_norm; waits
