@@ -30,9 +30,10 @@ def parse():
     ap.add_argument("--config", default="c5_flux12b_full")
     ap.add_argument("--flags", type=int, default=0, help="ERI_ADAM8_FLAG_* bits for the step")
     ap.add_argument("--cpu-sample", type=int, default=2 << 30, help="parameters in the CPU baseline sample (0 = skip)")
-    ap.add_argument("--kernel", choices=["adam8", "adam8_clip", "grad_norm", "adamw32", "ema"], default="adam8",
+    ap.add_argument("--kernel", choices=["adam8", "adam8_clip", "adam8_ema", "grad_norm", "adamw32", "ema"], default="adam8",
                     help="what one step is: the 8-bit AdamW step (headline), the same preceded by the device-side "
-                         "gradient norm, the norm alone, the 32-bit AdamW sibling, or the EMA sweep")
+                         "gradient norm, the same with the EMA of the parameters taken inside it, the norm alone, "
+                         "the 32-bit AdamW sibling, or the EMA sweep")
     ap.add_argument("--mode", choices=["eri", "l2"], default="eri",
                     help="arithmetic of the table API's step: the list optimizer's (adam8bit_enhanced.rs) or the "
                          "functional update's (adam8bit.rs, what --api functional always runs)")
@@ -213,6 +214,13 @@ def main():
             rows32[i].numel, rows32[i].dtype_tag = n, (L.DTYPE_BF16 if bf16 else L.DTYPE_F32)
         h32 = L.AdamW32Hyper(1e-4, 0.9, 0.999, 1e-8, 0.01)
         bytes_per_param = 3 * esz + 16
+    elif args.kernel == "adam8_ema":
+        a_sh = Alloc(torch, [n * esz for n in sizes])
+        extra.append(a_sh)
+        for i in range(len(sizes)):
+            rows[i].ema_shadow = a_sh.ptr(i)
+        L.check(L.lib().eri_adam8_table_update(table, rows, len(rows), stream), "table_update")
+        bytes_per_param += 2 * esz  # the shadow is read and written; the new parameter is still in registers
     elif args.kernel == "ema":
         a_sh = Alloc(torch, [n * esz for n in sizes])
         extra.append(a_sh)
@@ -275,7 +283,10 @@ def main():
             if args.kernel == "grad_norm":
                 return
             flags |= L.FLAG_CLIP_FROM_TABLE
+        if args.kernel == "adam8_ema":
+            flags |= L.FLAG_EMA
         h = L.hyper_pack(*hyper_args, t, L.MODE_L2 if args.mode == "l2" else L.MODE_ERI, flags)
+        h.ema_decay = 0.999
         L.check(L.lib().eri_adam8_step_table(table, C.byref(h), stream), "step_table")
 
     t = 0

@@ -12,21 +12,21 @@ LIB_PATH = os.path.join(_HERE, "liberi_optim8.so")
 BLOCK = 2048
 DTYPE_F32, DTYPE_F16, DTYPE_BF16, DTYPE_I32 = 0, 1, 2, 3
 MODE_ERI, MODE_L2, MODE_BNB = 0, 1, 2
-FLAG_GRAD_SCALE, FLAG_EXACT_PARAM, FLAG_BSEARCH, FLAG_NO_PIPELINE, FLAG_CLIP_FROM_TABLE, FLAG_ONE_WAVE = 1, 2, 4, 8, 16, 32
+FLAG_GRAD_SCALE, FLAG_EXACT_PARAM, FLAG_BSEARCH, FLAG_NO_PIPELINE, FLAG_CLIP_FROM_TABLE, FLAG_ONE_WAVE, FLAG_EMA = 1, 2, 4, 8, 16, 32, 64
 
 
 class Hyper(C.Structure):
     _fields_ = [("beta1", C.c_float), ("beta2", C.c_float), ("omb1", C.c_float), ("omb2", C.c_float),
                 ("eps", C.c_float), ("weight_decay", C.c_float), ("step_size", C.c_float),
                 ("bc1", C.c_float), ("bc2", C.c_float), ("grad_scale", C.c_float),
-                ("mode", C.c_int32), ("flags", C.c_uint32)]
+                ("mode", C.c_int32), ("flags", C.c_uint32), ("ema_decay", C.c_float), ("reserved", C.c_uint32)]
 
 
 class TensorRow(C.Structure):
     _fields_ = [("p", C.c_void_p), ("g", C.c_void_p), ("m", C.c_void_p), ("v", C.c_void_p),
                 ("absmax_m", C.c_void_p), ("absmax_v", C.c_void_p), ("numel", C.c_uint64),
                 ("block_start", C.c_uint64), ("dtype_tag", C.c_int32), ("grad_scale", C.c_float),
-                ("p_src", C.c_void_p), ("grad_f32", C.c_int32), ("reserved", C.c_int32)]
+                ("p_src", C.c_void_p), ("grad_f32", C.c_int32), ("reserved", C.c_int32), ("ema_shadow", C.c_void_p)]
 
 
 class Adam8bitConfigC(C.Structure):
@@ -120,6 +120,7 @@ EXPORTS = {
     "eri_adam8bit_get_step": (C.c_uint64, [C.c_void_p]),
     "eri_adam8bit_set_grad_scale": (C.c_int, [C.c_void_p, C.c_float]),
     "eri_adam8bit_set_param_grad_scale": (C.c_int, [C.c_void_p, C.c_uint32, C.c_float]),
+    "eri_adam8bit_attach_ema": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(C.c_char_p), C.c_uint32]),
     "eri_adam8bit_set_min_8bit_size": (C.c_int, [C.c_void_p, C.c_uint64]),
     "eri_adam8bit_state32_ptrs": (C.c_int, [C.c_void_p, C.c_uint32, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p)]),
     "eri_adam8bit_set_max_grad_norm": (C.c_int, [C.c_void_p, C.c_float, C.c_float]),

@@ -113,6 +113,17 @@ class Adam8bit:
         """MODE_ERI (the reference's update, default) or MODE_BNB."""
         check(lib().eri_adam8bit_set_mode(self._opt, mode), "eri_adam8bit_set_mode")
 
+    def attach_ema(self, ema: Optional["EMAModel"], names: Optional[List[str]] = None) -> None:
+        """From now on every step() also performs ema.update() over this optimizer's parameters (names[i] is the
+        model's name for parameter i): one launch instead of two sweeps.  attach_ema(None) detaches."""
+        if ema is None:
+            check(lib().eri_adam8bit_attach_ema(self._opt, None, None, 0), "eri_adam8bit_attach_ema")
+            self._ema = None
+            return
+        arr = (C.c_char_p * len(self.params))(*[n.encode() for n in names])
+        check(lib().eri_adam8bit_attach_ema(self._opt, ema._ema, arr, len(self.params)), "eri_adam8bit_attach_ema")
+        self._ema = ema  # keeps the model alive as long as it is attached
+
     def set_max_grad_norm(self, max_norm: float, denom_eps: float = 0.0) -> None:
         """Global-norm clipping inside step(): norm on the device, factor applied by the step kernel
         (clip_gradients, src/trainers/pipeline_flux_lora_sequential.rs:1198-1213).  <= 0 switches it off."""

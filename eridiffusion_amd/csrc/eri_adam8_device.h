@@ -26,7 +26,7 @@ struct DevTensor {
     uint64_t numel;
     uint32_t full_start;  /* number of full 2048-element blocks in the rows before this one (same dtype) */
     float grad_scale;
-    uint64_t pad;
+    void *shadow;     /* EMA shadow of the parameter, or null */
 };
 static_assert(sizeof(DevTensor) == 80, "DevTensor must stay 80 bytes");
 
@@ -101,7 +101,9 @@ int launch_step_plain_bf16(int mode, bool exact, bool wd, bool gs, bool keytab, 
 int launch_step_split(int layout, int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
                       uint32_t total_blocks, const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale,
                       uint32_t grid, void *stream);
-int launch_step_pipelined(int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
+/* Whether launch_step would run this group on the prefetching kernel with the EMA update inside it. */
+bool step_fuses_ema(uint32_t total_full_blocks, int layout, const EriAdam8Hyper &h, uint32_t compute_units);
+int launch_step_pipelined(int mode, bool exact, bool wd, bool gs, bool ema, const DevTensor *rows, uint32_t n_rows,
                           uint32_t total_blocks, const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale,
                           uint32_t grid, uint32_t wg, void *stream);
 /* Sum of |moment - dequantised moment| of the coming step, per row: err[2r] first moment, err[2r+1] second. */

@@ -180,10 +180,22 @@ __device__ __forceinline__ uint32_t code_bsearch(float x, const float *mid) {
 // the update of one element
 // ------------------------------------------------------------------------------------------
 
-/* The parameter update from finished moments, one rounded operation per line: what EXACT computes for
- * the modes ERI and BNB. */
-template <int MODE, bool WD>
-__device__ __forceinline__ float param_exact(float p, float m, float v, const EriAdam8Hyper &h) {
+/* The parameter update from finished moments, one rounded operation per line, with IEEE square root and
+ * division: what fp32 parameters always get, and bf16 parameters wherever the fast chain below cannot
+ * promise the same bits. */
+template <int MODE, bool WD, bool BF16>
+__device__ __forceinline__ float param_exact(float p, float m, float v, const EriAdam8Hyper &h, const BlockDiv &dbc1,
+                                             const BlockDiv &dbc2) {
+    if (MODE == ERI_ADAM8_MODE_L2) {
+        float mh = dbc1.fast ? dbc1.div_fast_unbounded(m) : m / dbc1.a; // adam8bit.rs:170
+        float vh = dbc2.fast ? dbc2.div_fast_unbounded(v) : v / dbc2.a; // :178
+        vh = fmaxf(vh, 0.0f);                                           // :181-182
+        float den = sqrtf(vh) + h.eps;                                  // :187
+        float upd = mh / den;
+        float us = upd * h.step_size;  // :196
+        if (BF16) us = bf16_round(us); // :197-198: the update is cast to the parameter's dtype
+        return p - us;                 // :205
+    }
     float den = sqrtf(v) + h.eps; // adam8bit_enhanced.rs:263
     float r = m / den;            // :264
     if (MODE == ERI_ADAM8_MODE_BNB) {
@@ -227,6 +239,12 @@ __device__ __forceinline__ float param_exact(float p, float m, float v, const Er
  * cancels its parameter, every NaN or infinity (the comparison is written so that they fail it) -- is
  * flagged.  The slack between 6.1 and 8 covers the use of the approximate r and the rounding of the
  * margin's own arithmetic.
+ *
+ * The functional update (mode L2) rounds the *update* to bf16 before it subtracts (adam8bit.rs:197-198), and
+ * that subtraction is a single exact-input operation, so the same argument applies to the update: the fast
+ * chain's lr * (m/bc1) / (sqrt(v/bc2) + eps) is within 6.5 * 2^-23 of the exact chain's, relative, and an
+ * update further than 8 * 2^-23 of itself from the tie point of its bf16 interval rounds to the same bf16
+ * value on both chains.  About one element in 4,000 is flagged and recomputed.
  */
 template <int MODE, bool WD>
 struct ExactMargin {
@@ -245,39 +263,56 @@ struct ExactMargin {
         }
     }
     __device__ __forceinline__ bool same_bf16_as_exact(float r, float pn) const {
-        const float margin = __builtin_fmaf(__builtin_fabsf(pn), c_p, __builtin_fabsf(r) * c_r);
+        // the floor 2^-126 flags everything down among the fp32 denormals, where the bounds above do not hold
+        const float margin = __builtin_fmaf(__builtin_fabsf(pn), c_p, __builtin_fmaf(__builtin_fabsf(r), c_r, 0x1p-126f));
         const float tie = u2f((f2u(pn) & 0xffff0000u) | 0x8000u);
         return __builtin_fabsf(pn - tie) > margin;
     }
 };
 
+/* t1 = m_old * beta1 and t3 = v_old * beta2 come in already multiplied: a kernel that holds a block's 256
+ * possible values of either product in a table of its own forms them once per code instead of once per
+ * element (same two rounded multiplications, same bits). */
+template <int MODE, bool EXACT, bool BF16, bool WD, bool GS>
+__device__ __forceinline__ void adam_elem_decayed(float p, float g, float t1, float t3, const EriAdam8Hyper &h,
+                                                  float gscale, const BlockDiv &dbc1, const BlockDiv &dbc2, float &m,
+                                                  float &v, float &pn, bool &recheck);
+
 template <int MODE, bool EXACT, bool BF16, bool WD, bool GS>
 __device__ __forceinline__ void adam_elem(float p, float g, float m_old, float v_old, const EriAdam8Hyper &h,
                                           float gscale, const BlockDiv &dbc1, const BlockDiv &dbc2, float &m,
                                           float &v, float &pn, bool &recheck) {
+    float t1 = m_old * h.beta1; // adam8bit_enhanced.rs:256
+    float t3 = v_old * h.beta2; // :260
+    adam_elem_decayed<MODE, EXACT, BF16, WD, GS>(p, g, t1, t3, h, gscale, dbc1, dbc2, m, v, pn, recheck);
+}
+
+template <int MODE, bool EXACT, bool BF16, bool WD, bool GS>
+__device__ __forceinline__ void adam_elem_decayed(float p, float g, float t1, float t3, const EriAdam8Hyper &h,
+                                                  float gscale, const BlockDiv &dbc1, const BlockDiv &dbc2, float &m,
+                                                  float &v, float &pn, bool &recheck) {
     if (GS) g = g * gscale;
     if (MODE == ERI_ADAM8_MODE_L2 && WD) { // adam8bit.rs:113-120
         float pw = p * h.weight_decay;
         g = g + pw;
     }
-    float t1 = m_old * h.beta1; // adam8bit_enhanced.rs:256
-    float t2 = g * h.omb1;
+    float t2 = g * h.omb1; // adam8bit_enhanced.rs:256
     m = t1 + t2;
     float gg = g * g; // :259-260
-    float t3 = v_old * h.beta2;
     float t4 = gg * h.omb2;
     v = t3 + t4;
-    if (MODE == ERI_ADAM8_MODE_L2) {
+    if (!BF16) { // fp32 parameters: every bit of the exact chain counts
+        pn = param_exact<MODE, WD, false>(p, m, v, h, dbc1, dbc2);
+    } else if (MODE == ERI_ADAM8_MODE_L2) { // always to the exact chain's bits (the reference rounds the update itself)
         float mh = dbc1.fast ? dbc1.div_fast_unbounded(m) : m / dbc1.a; // adam8bit.rs:170
         float vh = dbc2.fast ? dbc2.div_fast_unbounded(v) : v / dbc2.a; // :178
-        vh = fmaxf(vh, 0.0f);                                  // :181-182
-        float den = sqrtf(vh) + h.eps; // :187  (this mode always takes the IEEE chain)
-        float upd = mh / den;
-        float us = upd * h.step_size; // :196
-        if (BF16) us = bf16_round(us); // :197-198
-        pn = p - us;                   // :205
-    } else if (!BF16) { // fp32 parameters: every bit of the exact chain counts
-        pn = param_exact<MODE, WD>(p, m, v, h);
+        vh = fmaxf(vh, 0.0f);                                           // :181-182
+        float den = __builtin_amdgcn_sqrtf(vh) + h.eps;
+        float upd = mh * __builtin_amdgcn_rcpf(den);
+        float us = upd * h.step_size;
+        const float tie = u2f((f2u(us) & 0xffff0000u) | 0x8000u);
+        recheck |= !(__builtin_fabsf(us - tie) > __builtin_fmaf(__builtin_fabsf(us), 0x1p-20f, 0x1p-126f));
+        pn = p - bf16_round(us); // :197-205
     } else { // h.eps and h.weight_decay of mode BNB carry sqrt(bc2) and the factor 1 - lr*wd
         float den = __builtin_amdgcn_sqrtf(v) + h.eps;
         float r = m * __builtin_amdgcn_rcpf(den);
@@ -511,7 +546,7 @@ __device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint
             }
             if (cancel) {
 #pragma unroll
-                for (int k = 0; k < 8; ++k) pn[k] = param_exact<MODE, WD>(pv[k], mf[c * 8 + k], vf[c * 8 + k], h);
+                for (int k = 0; k < 8; ++k) pn[k] = param_exact<MODE, WD, BF16>(pv[k], mf[c * 8 + k], vf[c * 8 + k], h, dbc1, dbc2);
             }
             store8<BF16>(p, o, pn);
         }
@@ -622,7 +657,7 @@ __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint
                                                          L.map_u[byte_of(vr, k)] * a_v, h, gscale, dbc1, dbc2, m[k], v[k], pn[k], cancel);
                 if (cancel) {
 #pragma unroll
-                    for (int k = 0; k < 8; ++k) pn[k] = param_exact<MODE, WD>(pv[k], m[k], v[k], h);
+                    for (int k = 0; k < 8; ++k) pn[k] = param_exact<MODE, WD, BF16>(pv[k], m[k], v[k], h, dbc1, dbc2);
                 }
                 u32x2 mw, vw;
                 requant8<false, KEYTAB, MODE == ERI_ADAM8_MODE_BNB>(m, v, dm, dv, L, mw, vw);
@@ -656,7 +691,7 @@ __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint
         const float p_old = load1<BF16>(t.p_in, e);
         adam_elem<MODE, EXACT, BF16, WD, GS>(p_old, load1<GBF16>(t.g, e), L.map_s[mc[e]] * a_m,
                                              L.map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn, cancel);
-        if (cancel) pn = param_exact<MODE, WD>(p_old, m, v, h);
+        if (cancel) pn = param_exact<MODE, WD, BF16>(p_old, m, v, h, dbc1, dbc2);
         const float xm = dm.div_slow(m);
         const float xv = dv.div_slow(v);
         uint32_t cm = KEYTAB ? code_signed_key(xm, L.key_s) : code_bsearch(xm, L.mid_s);
@@ -692,9 +727,13 @@ __device__ __forceinline__ uint32_t find_row(const Row *rows, uint32_t n_rows, u
     return lo;
 }
 
-/* A wave's blocks only grow and a tensor usually spans many of them, so the owning row is searched for
+/* A wave's blocks only grow and a tensor usually spans many of them, so the owning row is looked up
  * again only when a block leaves the range [t.full_start, t_end) of the row at hand (t_end = 0 forces
- * the first search).  Saves the ten dependent scalar loads of the search on almost every block. */
+ * the first lookup).  A launch table carries, right behind its rows, one row index per full block
+ * (BlockRowMap): the lookup is then one scalar load and the load of the row, where the search takes ten
+ * dependent loads -- which a table of many small tensors pays on almost every block, because a wave's
+ * consecutive blocks lie a whole stride apart.  Row tables without the map (the plain element-wise sweeps)
+ * search. */
 template <typename Row>
 __device__ __forceinline__ void seek_row(const Row *rows, uint32_t n_rows, uint32_t blk, uint32_t &ti, Row &t,
                                          uint32_t &t_end) {
@@ -704,6 +743,19 @@ __device__ __forceinline__ void seek_row(const Row *rows, uint32_t n_rows, uint3
         t_end = t.full_start + (uint32_t)(t.numel / kBlock);
     }
 }
+
+struct BlockRowMap {
+    const uint32_t *row_of; // row_of[b] = index of the row that owns full block b
+    __device__ __forceinline__ BlockRowMap(const DevTensor *rows, uint32_t n_rows)
+        : row_of(reinterpret_cast<const uint32_t *>(rows + n_rows)) {}
+    __device__ __forceinline__ void seek(const DevTensor *rows, uint32_t blk, uint32_t &ti, DevTensor &t, uint32_t &t_end) const {
+        if (blk >= t_end) {
+            ti = row_of[blk];
+            t = rows[ti];
+            t_end = t.full_start + (uint32_t)(t.numel / kBlock);
+        }
+    }
+};
 
 /* The full blocks one wave walks.  Workgroup i of a launch runs on accelerator die (XCD) i mod 8.  The
  * block list is cut into `chunks` contiguous ranges and workgroup i walks range i mod chunks, so with

@@ -7,6 +7,14 @@
 
 namespace eri {
 
+/* The one case in which the EMA runs inside the step kernel: the prefetching kernel in mode ERI. */
+bool step_fuses_ema(uint32_t total_blocks, int layout, const EriAdam8Hyper &h, uint32_t compute_units) {
+    if ((h.flags & ERI_ADAM8_FLAG_EMA) == 0 || layout != kLayoutBF16 || h.mode != ERI_ADAM8_MODE_ERI) return false;
+    if (h.flags & (ERI_ADAM8_FLAG_BSEARCH | ERI_ADAM8_FLAG_NO_PIPELINE)) return false;
+    const bool few = (uint64_t)total_blocks <= (uint64_t)compute_units * (uint64_t)kSplitBlocksPerCu;
+    return (h.flags & ERI_ADAM8_FLAG_ONE_WAVE) != 0 || !few;
+}
+
 int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, int layout,
                 const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg,
                 uint32_t compute_units, void *stream) {
@@ -35,7 +43,7 @@ int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, i
         const bool wd = h.weight_decay != 1.0f;
         const bool exact = (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0;
         if (bf16 && !kernel_named)
-            return launch_step_pipelined(h.mode, exact, wd, gs, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
+            return launch_step_pipelined(h.mode, exact, wd, gs, false, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
         if (bf16) return launch_step_plain_bf16(h.mode, exact, wd, gs, true, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
         return launch_step_plain_f32(h.mode, wd, gs, true, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
     }
@@ -44,7 +52,8 @@ int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, i
     const bool keytab = (h.flags & ERI_ADAM8_FLAG_BSEARCH) == 0;
     if (!bf16) return launch_step_plain_f32(h.mode, wd, gs, keytab, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
     if (keytab && h.mode == ERI_ADAM8_MODE_ERI && (h.flags & ERI_ADAM8_FLAG_NO_PIPELINE) == 0)
-        return launch_step_pipelined(h.mode, exact, wd, gs, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
+        return launch_step_pipelined(h.mode, exact, wd, gs, step_fuses_ema(total_blocks, layout, h, compute_units), rows, n_rows,
+                                     total_blocks, h, lds_image, dev_scale, grid, wg, stream);
     return launch_step_plain_bf16(h.mode, exact, wd, gs, keytab, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
 }
 
@@ -183,8 +192,9 @@ __global__ __launch_bounds__(1024) void grad_sumsq_kernel(const DevTensor *__res
         uint32_t ti = 0, t_end = 0;
         DevTensor t;
         Raw8<BF16> raw[4];
+        const BlockRowMap map(rows, n_rows);
         {
-            seek_row(rows, n_rows, walk.first, ti, t, t_end);
+            map.seek(rows, walk.first, ti, t, t_end);
             const size_t e0 = (size_t)(walk.first - t.full_start) * kBlock;
 #pragma unroll
             for (int c = 0; c < 4; ++c) raw[c].load(static_cast<const char *>(t.g) + e0 * (BF16 ? 2 : 4), c * 512 + lane * 8);
@@ -195,7 +205,7 @@ __global__ __launch_bounds__(1024) void grad_sumsq_kernel(const DevTensor *__res
             for (int c = 0; c < 4; ++c) cur[c] = raw[c];
             const uint32_t nblk = blk + walk.stride;
             if (nblk < walk.end) {
-                seek_row(rows, n_rows, nblk, ti, t, t_end);
+                map.seek(rows, nblk, ti, t, t_end);
                 const size_t e0 = (size_t)(nblk - t.full_start) * kBlock;
 #pragma unroll
                 for (int c = 0; c < 4; ++c) raw[c].load(static_cast<const char *>(t.g) + e0 * (BF16 ? 2 : 4), c * 512 + lane * 8);

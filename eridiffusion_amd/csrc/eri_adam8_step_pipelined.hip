@@ -13,6 +13,26 @@ namespace eri {
 // 48 (raw) + 64 (moments) + temporaries at its peak, hence three waves per SIMD (768 threads).
 // ------------------------------------------------------------------------------------------
 
+/* One lane's eight shadow values of one quarter block: shadow = d*shadow + (1-d)*p', each operation rounded
+ * on its own, the result rounded to bf16. */
+__device__ __forceinline__ void ema_quarter(void *shadow, size_t e0, int c, uint32_t lane, const u32x4 &old, const u32x4 &pnew,
+                                            float decay) {
+    const float omd = 1.0f - decay; // ema_enhanced.rs:96
+    Raw8<true> so, pn;
+    so.w = old;
+    pn.w = pnew;
+    float sv[8], pv[8], out[8];
+    so.unpack(sv);
+    pn.unpack(pv);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        float a = sv[k] * decay;
+        float b = pv[k] * omd;
+        out[k] = a + b;
+    }
+    store8<true>(static_cast<char *>(shadow) + e0 * 2, c * 512 + lane * 8, out);
+}
+
 struct RawBlock {
     u32x4 p[4], g[4];
     u32x2 m[4], v[4];
@@ -35,7 +55,9 @@ struct RawBlock {
     }
 };
 
-template <int MODE, bool EXACT, bool WD, bool GS>
+/* EMA: rows that carry a shadow also get shadow = d*shadow + (1-d)*p' (src/trainers/ema_enhanced.rs:91-100),
+ * p' being the parameter as it is stored (rounded to bf16). */
+template <int MODE, bool EXACT, bool WD, bool GS, bool EMA>
 __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTensor *__restrict__ rows,
                                                                    uint32_t n_rows, uint32_t total_blocks,
                                                                    EriAdam8Hyper h,
@@ -43,6 +65,10 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
                                                                    const float *__restrict__ dev_scale,
                                                                    uint32_t chunks) {
     ERI_LDS_IMAGE;
+    // Per wave, the 2 x 256 values a state code of the block at hand can stand for, already multiplied by the
+    // block's absmax and by beta: (MAP[c] * absmax) * beta, the first two operations of both moment
+    // updates, done once per code (8 per lane) instead of once per element (64 per lane).
+    __shared__ float decayed[12][2][256];
     // clip factor left on the device by the gradient-norm pass (1.0 when there is none)
     const float tscale = (GS && dev_scale) ? *dev_scale : 1.0f;
     for (uint32_t i = threadIdx.x; i < kLdsImageBytes / 16; i += blockDim.x) lds_raw[i] = lds_image[i];
@@ -60,6 +86,9 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
     const uint32_t waves_per_wg = blockDim.x / kWave;
     const uint32_t stride = gridDim.x * waves_per_wg;
     const BlockDiv dbc1(h.bc1), dbc2(h.bc2);
+    float(*const mine)[256] = decayed[threadIdx.x / kWave];
+    const f32x4 base_s = reinterpret_cast<const f32x4 *>(L.map_s)[lane]; // codes 4*lane .. 4*lane + 3
+    const f32x4 base_u = reinterpret_cast<const f32x4 *>(L.map_u)[lane];
 
     const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
     // partial last blocks first: one per row at most, handed out from the last wave backwards -- the
@@ -71,6 +100,15 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
         if (n != 0) {
             const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
             tail_block<true, MODE, EXACT, WD, GS, true>(t, (uint32_t)(t.numel / kBlock), n, lane, h, gscale, dbc1, dbc2, L);
+            if (EMA && t.shadow != nullptr) { // the partial block's shadow, element by element, from the parameters just stored
+                const size_t e0 = (size_t)(t.numel / kBlock) * kBlock;
+                const float omd = 1.0f - h.ema_decay;
+                for (uint32_t i = lane; i < n; i += kWave) {
+                    const float a = load1<true>(t.shadow, e0 + i) * h.ema_decay;
+                    const float b = load1<true>(t.p, e0 + i) * omd;
+                    as_global(static_cast<uint16_t *>(t.shadow))[e0 + i] = (uint16_t)bf16_bits(a + b);
+                }
+            }
         }
     }
     const BlockWalk walk(total_blocks, chunks);
@@ -79,7 +117,8 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
 
     uint32_t ti = 0, t_end = 0;
     DevTensor t;
-    seek_row(rows, n_rows, blk, ti, t, t_end);
+    const BlockRowMap map(rows, n_rows);
+    map.seek(rows, blk, ti, t, t_end);
     uint32_t nti = ti, nt_end = t_end;
     DevTensor nt = t;
     RawBlock raw;
@@ -90,7 +129,7 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
         const uint32_t nblk = blk + walk.stride;
         const bool more = nblk < walk.end;
         const uint32_t pblk = more ? nblk : blk;
-        seek_row(rows, n_rows, pblk, nti, nt, nt_end);
+        map.seek(rows, pblk, nti, nt, nt_end);
 
         const uint32_t lb = blk - t.full_start;
         const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
@@ -102,6 +141,25 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
         u32x4 pw[4]; // updated parameters, packed, stored after the next block's loads are out
         float lm = 0.0f, lv = 0.0f;
         const float a_m = raw.a_m, a_v = raw.a_v;
+        {
+            f32x4 ds, du;
+            ds.x = (base_s.x * a_m) * h.beta1; ds.y = (base_s.y * a_m) * h.beta1;
+            ds.z = (base_s.z * a_m) * h.beta1; ds.w = (base_s.w * a_m) * h.beta1;
+            du.x = (base_u.x * a_v) * h.beta2; du.y = (base_u.y * a_v) * h.beta2;
+            du.z = (base_u.z * a_v) * h.beta2; du.w = (base_u.w * a_v) * h.beta2;
+            reinterpret_cast<f32x4 *>(mine[0])[lane] = ds;
+            reinterpret_cast<f32x4 *>(mine[1])[lane] = du;
+        }
+        // EMA: the shadow's words are requested first and used quarter by quarter in the update half, where the
+        // registers of the moments are still filling up (in the requantisation half, beside the next block's
+        // words, they did not fit: 104-152 bytes of scratch per lane)
+        u32x4 sh[4];
+        const bool with_shadow = EMA && t.shadow != nullptr;
+        if (EMA && with_shadow) {
+            ERI_GLOBAL const u32x4 *sp = as_global(reinterpret_cast<const u32x4 *>(static_cast<const uint16_t *>(t.shadow) + e0));
+#pragma unroll
+            for (int c = 0; c < 4; ++c) sh[c] = __builtin_nontemporal_load(&sp[c * 64 + lane]);
+        }
         bool cancel = false;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
@@ -111,21 +169,27 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
             float pv[8], gv[8], pn[8];
             pr.unpack(pv);
             gr.unpack(gv);
+            bool redo = false; // EMA: flagged elements are put right quarter by quarter, before the shadow uses them
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
-                const float m_old = lds_float_at(L.map_s, code_offset(raw.m[c], k)) * a_m;
-                const float v_old = lds_float_at(L.map_u, code_offset(raw.v[c], k)) * a_v;
+                const float t1 = lds_float_at(mine[0], code_offset(raw.m[c], k));
+                const float t3 = lds_float_at(mine[1], code_offset(raw.v[c], k));
                 float m, v;
-                adam_elem<MODE, EXACT, true, WD, GS>(pv[k], gv[k], m_old, v_old, h, gscale, dbc1, dbc2, m, v, pn[k], cancel);
+                adam_elem_decayed<MODE, EXACT, true, WD, GS>(pv[k], gv[k], t1, t3, h, gscale, dbc1, dbc2, m, v, pn[k], EMA ? redo : cancel);
                 mf[c * 8 + k] = m;
                 vf[c * 8 + k] = v;
                 lm = fmaxf(lm, __builtin_fabsf(m));
                 lv = fmaxf(lv, __builtin_fabsf(v));
             }
+            if (EMA && redo) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) pn[k] = param_exact<MODE, WD, true>(pv[k], mf[c * 8 + k], vf[c * 8 + k], h, dbc1, dbc2);
+            }
             pw[c].x = bf16_pair(pn[0], pn[1]);
             pw[c].y = bf16_pair(pn[2], pn[3]);
             pw[c].z = bf16_pair(pn[4], pn[5]);
             pw[c].w = bf16_pair(pn[6], pn[7]);
+            if (EMA && with_shadow) ema_quarter(t.shadow, e0, c, lane, sh[c], pw[c], h.ema_decay);
         }
         if (cancel) { // rare: a lane whose update cancelled redoes its 32 parameters with the exact chain
 #pragma unroll
@@ -135,7 +199,7 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
                 float pv[8], pn[8];
                 pr.unpack(pv);
 #pragma unroll
-                for (int k = 0; k < 8; ++k) pn[k] = param_exact<MODE, WD>(pv[k], mf[c * 8 + k], vf[c * 8 + k], h);
+                for (int k = 0; k < 8; ++k) pn[k] = param_exact<MODE, WD, true>(pv[k], mf[c * 8 + k], vf[c * 8 + k], h, dbc1, dbc2);
                 pw[c].x = bf16_pair(pn[0], pn[1]);
                 pw[c].y = bf16_pair(pn[2], pn[3]);
                 pw[c].z = bf16_pair(pn[4], pn[5]);
@@ -179,18 +243,28 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
 
 namespace {
 
-template <int MODE, bool EXACT, bool WD, bool GS>
+template <int MODE, bool EXACT, bool WD, bool GS, bool EMA = false>
 int launch_pipelined(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
                      const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg, hipStream_t s) {
     if (wg > 768) wg = 768;
-    hipLaunchKernelGGL((adam8_step_pipelined_kernel<MODE, EXACT, WD, GS>), dim3(grid), dim3(wg), 0, s, rows, n_rows, total_blocks, h,
+    hipLaunchKernelGGL((adam8_step_pipelined_kernel<MODE, EXACT, WD, GS, EMA>), dim3(grid), dim3(wg), 0, s, rows, n_rows, total_blocks, h,
                        static_cast<const uint4 *>(lds_image), dev_scale, chunks_for(grid));
     return (int)hipGetLastError();
 }
 
 template <int MODE, bool EXACT>
-int launch_flags(bool wd, bool gs, const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
+int launch_flags(bool wd, bool gs, bool ema, const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
                  const void *img, const float *dev_scale, uint32_t grid, uint32_t wg, hipStream_t s) {
+    if constexpr (MODE == ERI_ADAM8_MODE_ERI) { // the EMA is built into the reference's own update only
+        if (ema) {
+            if (wd) {
+                if (gs) return launch_pipelined<MODE, EXACT, true, true, true>(rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s);
+                return launch_pipelined<MODE, EXACT, true, false, true>(rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s);
+            }
+            if (gs) return launch_pipelined<MODE, EXACT, false, true, true>(rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s);
+            return launch_pipelined<MODE, EXACT, false, false, true>(rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s);
+        }
+    }
     if (wd) {
         if (gs) return launch_pipelined<MODE, EXACT, true, true>(rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s);
         return launch_pipelined<MODE, EXACT, true, false>(rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s);
@@ -204,11 +278,11 @@ int launch_flags(bool wd, bool gs, const DevTensor *rows, uint32_t n_rows, uint3
 /* Modes ERI and BNB.  The coupled-decay mode needs more live values per element than this kernel's
  * register budget holds (its instantiations spilled 80-232 B per lane) and runs faster on the kernel
  * without the prefetch; the dispatcher sends it there. */
-int launch_step_pipelined(int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
+int launch_step_pipelined(int mode, bool exact, bool wd, bool gs, bool ema, const DevTensor *rows, uint32_t n_rows,
                           uint32_t total_blocks, const EriAdam8Hyper &h, const void *img, const float *dev_scale,
                           uint32_t grid, uint32_t wg, void *stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
-#define ERI_ARGS wd, gs, rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s
+#define ERI_ARGS wd, gs, ema, rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s
     if (mode == ERI_ADAM8_MODE_BNB)
         return exact ? launch_flags<ERI_ADAM8_MODE_BNB, true>(ERI_ARGS) : launch_flags<ERI_ADAM8_MODE_BNB, false>(ERI_ARGS);
     return exact ? launch_flags<ERI_ADAM8_MODE_ERI, true>(ERI_ARGS) : launch_flags<ERI_ADAM8_MODE_ERI, false>(ERI_ARGS);

@@ -57,8 +57,9 @@ __global__ __launch_bounds__(plain_threads(MODE)) void adam8_step_kernel(const D
     uint32_t ti = 0, t_end = 0;
     DevTensor t;
     const BlockWalk walk(total_blocks, chunks);
+    const BlockRowMap map(rows, n_rows);
     for (uint32_t blk = walk.first; blk < walk.end; blk += walk.stride) {
-        seek_row(rows, n_rows, blk, ti, t, t_end);
+        map.seek(rows, blk, ti, t, t_end);
         const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
         full_block<BF16, MODE, EXACT, WD, GS, KEYTAB>(t, blk - t.full_start, lane, h, gscale, dbc1, dbc2, L);
     }

@@ -21,6 +21,9 @@ __global__ __launch_bounds__(1024) void adam8_step_split_kernel(const DevTensor 
                                                                 const float *__restrict__ dev_scale) {
     ERI_LDS_IMAGE;
     __shared__ float wave_maxima[2][4][8]; // [parity of the iteration][team][4 x first, 4 x second moment]
+    // per wave: (MAP[c] * absmax) * beta for the 2 x 256 codes of the block at hand, formed once per code
+    // (8 multiplications per lane) instead of once per element (16 per lane)
+    __shared__ float decayed[16][2][256];
     const float tscale = (GS && dev_scale) ? *dev_scale : 1.0f;
     const uint32_t lane = threadIdx.x & (kWave - 1);
     const uint32_t wave_in_wg = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -40,11 +43,12 @@ __global__ __launch_bounds__(1024) void adam8_step_split_kernel(const DevTensor 
         float a_m, a_v;
     } q;
     uint32_t ti = 0, t_end = 0;
+    const BlockRowMap map(rows, n_rows);
     auto request = [&](uint32_t first) {
         const uint32_t blk = first + team;
         q.active = blk < total_blocks;
         if (!q.active) return;
-        seek_row(rows, n_rows, blk, ti, q.t, t_end);
+        map.seek(rows, blk, ti, q.t, t_end);
         q.lb = blk - q.t.full_start;
         const size_t e0 = (size_t)q.lb * kBlock;
         const size_t esz = BF16 ? 2 : 4;
@@ -68,6 +72,9 @@ __global__ __launch_bounds__(1024) void adam8_step_split_kernel(const DevTensor 
     L.key_s = base + kOffKeyS;
     L.key_u = base + kOffKeyU;
     const BlockDiv dbc1(h.bc1), dbc2(h.bc2);
+    float(*const mine)[256] = decayed[wave_in_wg];
+    const f32x4 base_s = reinterpret_cast<const f32x4 *>(L.map_s)[lane]; // codes 4*lane .. 4*lane + 3
+    const f32x4 base_u = reinterpret_cast<const f32x4 *>(L.map_u)[lane];
 
     // partial last blocks: one wave each, no barrier involved
     const uint32_t n_waves = gridDim.x * 16;
@@ -85,25 +92,38 @@ __global__ __launch_bounds__(1024) void adam8_step_split_kernel(const DevTensor 
     for (uint32_t first = blockIdx.x * 4; first < total_blocks; first += gridDim.x * 4, parity ^= 1) {
         float m[8], v[8];
         float nam = 0.0f, nav = 0.0f;
-        if (q.active) {
-            const size_t e0 = (size_t)q.lb * kBlock;
-            char *p = static_cast<char *>(q.t.p) + e0 * (BF16 ? 2 : 4);
-            const float gscale = GS ? (h.grad_scale * q.t.grad_scale) * tscale : 1.0f;
+        // the quarter at hand; q itself is handed to the next request as soon as its raw words are used up
+        const bool active = q.active;
+        const DevTensor t = q.t;
+        const uint32_t lb = q.lb;
+        if (active) {
+            const size_t e0 = (size_t)lb * kBlock;
+            char *p = static_cast<char *>(t.p) + e0 * (BF16 ? 2 : 4);
+            const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
             float pv[8], gv[8], pn[8];
             q.pr.unpack(pv);
             q.gr.unpack(gv);
+            {
+                f32x4 ds, du;
+                ds.x = (base_s.x * q.a_m) * h.beta1; ds.y = (base_s.y * q.a_m) * h.beta1;
+                ds.z = (base_s.z * q.a_m) * h.beta1; ds.w = (base_s.w * q.a_m) * h.beta1;
+                du.x = (base_u.x * q.a_v) * h.beta2; du.y = (base_u.y * q.a_v) * h.beta2;
+                du.z = (base_u.z * q.a_v) * h.beta2; du.w = (base_u.w * q.a_v) * h.beta2;
+                reinterpret_cast<f32x4 *>(mine[0])[lane] = ds;
+                reinterpret_cast<f32x4 *>(mine[1])[lane] = du;
+            }
             bool cancel = false;
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
-                const float m_old = L.map_s[byte_of(q.mr, k)] * q.a_m;
-                const float v_old = L.map_u[byte_of(q.vr, k)] * q.a_v;
-                adam_elem<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], m_old, v_old, h, gscale, dbc1, dbc2, m[k], v[k], pn[k], cancel);
+                const float t1 = lds_float_at(mine[0], code_offset(q.mr, k));
+                const float t3 = lds_float_at(mine[1], code_offset(q.vr, k));
+                adam_elem_decayed<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], t1, t3, h, gscale, dbc1, dbc2, m[k], v[k], pn[k], cancel);
                 nam = fmaxf(nam, __builtin_fabsf(m[k]));
                 nav = fmaxf(nav, __builtin_fabsf(v[k]));
             }
             if (cancel) {
 #pragma unroll
-                for (int k = 0; k < 8; ++k) pn[k] = param_exact<MODE, WD>(pv[k], m[k], v[k], h);
+                for (int k = 0; k < 8; ++k) pn[k] = param_exact<MODE, WD, BF16>(pv[k], m[k], v[k], h, dbc1, dbc2);
             }
             store8<BF16>(p, o, pn);
             wave_max2(nam, nav);
@@ -113,24 +133,26 @@ __global__ __launch_bounds__(1024) void adam8_step_split_kernel(const DevTensor 
             }
         }
         __syncthreads();
-        if (q.active) {
+        // the next quarter's loads travel while this one is requantised
+        const uint32_t next = first + gridDim.x * 4;
+        if (next < total_blocks) request(next);
+        else q.active = false;
+        if (active) {
             const float *wm = wave_maxima[parity][team];
             nam = fmaxf(fmaxf(wm[0], wm[1]), fmaxf(wm[2], wm[3]));
             nav = fmaxf(fmaxf(wm[4], wm[5]), fmaxf(wm[6], wm[7]));
             if (quarter == 0 && lane == 0) {
-                as_global(q.t.absmax_m)[q.lb] = nam;
-                as_global(q.t.absmax_v)[q.lb] = nav;
+                as_global(t.absmax_m)[lb] = nam;
+                as_global(t.absmax_v)[lb] = nav;
             }
             const BlockDiv dm(nam, kKeyScale, kKeyScaleInv), dv(nav, kKeyScale, kKeyScaleInv);
-            const size_t e0 = (size_t)q.lb * kBlock;
+            const size_t e0 = (size_t)lb * kBlock;
             u32x2 mw, vw;
             if (dm.fast && dv.fast) requant8<true, true, MODE == ERI_ADAM8_MODE_BNB>(m, v, dm, dv, L, mw, vw);
             else requant8<false, true, MODE == ERI_ADAM8_MODE_BNB>(m, v, dm, dv, L, mw, vw);
-            __builtin_nontemporal_store(mw, as_global(reinterpret_cast<u32x2 *>(q.t.m + e0 + o)));
-            __builtin_nontemporal_store(vw, as_global(reinterpret_cast<u32x2 *>(q.t.v + e0 + o)));
+            __builtin_nontemporal_store(mw, as_global(reinterpret_cast<u32x2 *>(t.m + e0 + o)));
+            __builtin_nontemporal_store(vw, as_global(reinterpret_cast<u32x2 *>(t.v + e0 + o)));
         }
-        const uint32_t next = first + gridDim.x * 4;
-        if (next < total_blocks) request(next);
     }
 }
 

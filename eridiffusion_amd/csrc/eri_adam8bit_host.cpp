@@ -326,6 +326,57 @@ struct EriParameter {
 };
 
 // ---------------------------------------------------------------------------------------------
+// EMAModel: named shadows (defined here because the optimizer below can carry one in its step)
+// ---------------------------------------------------------------------------------------------
+
+struct EriEmaModel {
+    struct Shadow {
+        void *data = nullptr;
+        uint64_t numel = 0;
+        int32_t dtype = 0;
+    };
+    float decay = 0.999f, power = 1.0f;
+    bool bias_correction = true;
+    uint64_t step = 0;
+    void *stream = nullptr;
+    std::map<std::string, Shadow> shadows;
+    std::vector<EriEmaTensor> rows; // reused between updates
+    ~EriEmaModel() {
+        for (auto &kv : shadows)
+            if (kv.second.data) eri_hip_free(kv.second.data);
+    }
+};
+
+namespace {
+
+uint64_t elem_bytes(int32_t dtype) { return dtype == ERI_DTYPE_F32 ? 4 : 2; }
+
+// a fresh shadow holding a copy of the parameter (ema_enhanced.rs:72-73,100-103)
+int ema_adopt(EriEmaModel *e, const std::string &name, const EriParameter *p) {
+    if (!p || !p->data) return fail(ERI_ERR_NULL, "parameter without data: " + name);
+    if (p->numel == 0) return fail(ERI_ERR_EMPTY, "empty parameter: " + name);
+    if (p->dtype != ERI_DTYPE_F32 && p->dtype != ERI_DTYPE_BF16) return fail(ERI_ERR_DTYPE, "Unsupported: EMA takes F32 or BF16 parameters");
+    EriEmaModel::Shadow &s = e->shadows[name];
+    const uint64_t bytes = p->numel * elem_bytes(p->dtype);
+    if (!s.data || s.numel != p->numel || s.dtype != p->dtype) {
+        if (s.data) eri_hip_free(s.data);
+        s = EriEmaModel::Shadow();
+        int dev = 0;
+        int rc = eri_hip_get_device(&dev);
+        if (!rc) rc = eri_hip_malloc_zeroed(dev, bytes, &s.data);
+        if (rc) {
+            e->shadows.erase(name);
+            return rc;
+        }
+        s.numel = p->numel;
+        s.dtype = p->dtype;
+    }
+    return eri_hip_memcpy_async(s.data, p->data, bytes, 3, e->stream);
+}
+
+} // namespace
+
+// ---------------------------------------------------------------------------------------------
 // Adam8bit over a parameter list
 // ---------------------------------------------------------------------------------------------
 
@@ -342,6 +393,8 @@ struct EriAdam8bit {
     std::vector<std::unique_ptr<State8>> states; // index = parameter index; null before the first step
     std::vector<std::unique_ptr<State32>> states32; // fp32 moments of the parameters below min_8bit_size
     uint64_t min_8bit_size = 0;                   // 0 = every parameter takes the 8-bit format
+    EriEmaModel *ema = nullptr;                   // attached EMA model (not owned), updated inside step()
+    std::vector<std::string> ema_names;           // its name for each parameter
     void *stream = nullptr;
     EriAdam8Table *table = nullptr;
     std::vector<uint32_t> table_ids;         // parameter indices the table was built for
@@ -481,11 +534,29 @@ int eri_adam8bit_destroy(EriAdam8bit *o) {
 
 static int adam8bit_step_impl(EriAdam8bit *o, uint32_t *skipped);
 
+/* The part of an attached EMA model's update that the 8-bit step did not do itself. */
+static int adam8bit_ema_rest(EriAdam8bit *o, const std::vector<EriEmaTensor> &others, const std::vector<uint32_t> &fresh,
+                             float decay) {
+    if (!o->ema) return 0;
+    if (!others.empty()) {
+        int rc = eri_ema_update_multi(others.data(), (uint32_t)others.size(), decay, o->stream);
+        if (rc) return rc;
+    }
+    for (uint32_t i : fresh) {
+        int rc = ema_adopt(o->ema, o->ema_names[i], o->params[i]);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
 int eri_adam8bit_step(EriAdam8bit *o, uint32_t *skipped) {
     if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
-    const uint64_t before = o->step;
+    const uint64_t before = o->step, ema_before = o->ema ? o->ema->step : 0;
     const int rc = adam8bit_step_impl(o, skipped);
-    if (rc) o->step = before; // a refused step counts for nothing
+    if (rc) { // a refused step counts for nothing
+        o->step = before;
+        if (o->ema) o->ema->step = ema_before;
+    }
     return rc;
 }
 
@@ -554,6 +625,39 @@ static int adam8bit_step_impl(EriAdam8bit *o, uint32_t *skipped) {
     }
     if (skipped) *skipped = skip;
     const bool clip = o->max_grad_norm > 0.0f;
+    // Attached EMA model: EMAModel::update (ema_enhanced.rs:79-104) as part of this step.  Parameters that
+    // take the 8-bit step carry their shadow in their row (the step updates it, inside the kernel where
+    // that pays); the others -- no gradient this step, fp32 moments -- get the plain sweep afterwards, and
+    // a name seen for the first time gets a copy of its parameter as the reference does (:100-103).
+    float ema_decay = 0.0f;
+    std::vector<EriEmaTensor> ema_others;
+    std::vector<uint32_t> ema_new;
+    bool ema_rows = false;
+    if (o->ema) {
+        o->ema->step += 1;                       // :80
+        ema_decay = eri_ema_current_decay(o->ema); // :83
+        size_t k = 0;
+        for (uint32_t i = 0; i < o->params.size(); ++i) {
+            const EriParameter *p = o->params[i];
+            const bool in_table = k < ids.size() && ids[k] == i;
+            auto it = o->ema->shadows.find(o->ema_names[i]);
+            if (it == o->ema->shadows.end() || it->second.numel != p->numel || it->second.dtype != p->dtype) {
+                ema_new.push_back(i);
+            } else if (in_table) {
+                rows[k].ema_shadow = it->second.data;
+                ema_rows = true;
+            } else {
+                EriEmaTensor r;
+                r.shadow = it->second.data;
+                r.p = p->data;
+                r.numel = p->numel;
+                r.dtype_tag = p->dtype;
+                r.reserved = 0;
+                ema_others.push_back(r);
+            }
+            if (in_table) ++k;
+        }
+    }
     if (!rows32.empty()) { // refused before anything is launched
         for (uint32_t i = 0; i < o->params.size(); ++i) scaled = scaled || (o->states32[i] && o->param_scale[i] != 1.0f);
         if (scaled || clip)
@@ -578,7 +682,7 @@ static int adam8bit_step_impl(EriAdam8bit *o, uint32_t *skipped) {
         rc = eri_adamw32_step_multi(rows32.data(), (uint32_t)rows32.size(), &h32, o->stream);
         if (rc) return rc;
     }
-    if (rows.empty()) return 0;
+    if (rows.empty()) return adam8bit_ema_rest(o, ema_others, ema_new, ema_decay);
     if (!o->table || ids != o->table_ids) {
         if (o->table) eri_adam8_table_destroy(o->table);
         o->table = nullptr;
@@ -613,7 +717,13 @@ static int adam8bit_step_impl(EriAdam8bit *o, uint32_t *skipped) {
         if (rc) return rc;
         o->have_qerr = true;
     }
-    return eri_adam8_step_table(o->table, &h, o->stream);
+    if (ema_rows) {
+        h.flags |= ERI_ADAM8_FLAG_EMA;
+        h.ema_decay = ema_decay;
+    }
+    rc = eri_adam8_step_table(o->table, &h, o->stream);
+    if (rc) return rc;
+    return adam8bit_ema_rest(o, ema_others, ema_new, ema_decay);
 }
 
 int eri_adam8bit_zero_grad(EriAdam8bit *o) {
@@ -697,6 +807,26 @@ int eri_adam8bit_set_mode(EriAdam8bit *o, int mode) {
     if (mode != ERI_ADAM8_MODE_ERI && mode != ERI_ADAM8_MODE_BNB)
         return fail(ERI_ERR_ARG, "the list-of-parameters optimizer steps in mode ERI or BNB");
     o->mode = mode;
+    return 0;
+}
+
+int eri_adam8bit_attach_ema(EriAdam8bit *o, EriEmaModel *ema, const char *const *names, uint32_t n) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    if (!ema) { // detach
+        o->ema = nullptr;
+        o->ema_names.clear();
+        return 0;
+    }
+    if (!names) return fail(ERI_ERR_NULL, "names is NULL");
+    if (n != o->params.size()) return fail(ERI_ERR_ARG, "attach_ema: one name per parameter of the optimizer");
+    if (ema->stream != o->stream) return fail(ERI_ERR_ARG, "attach_ema: the EMA model and the optimizer must use the same stream");
+    std::vector<std::string> v;
+    for (uint32_t i = 0; i < n; ++i) {
+        if (!names[i]) return fail(ERI_ERR_NULL, "a name is NULL");
+        v.emplace_back(names[i]);
+    }
+    o->ema = ema;
+    o->ema_names.swap(v);
     return 0;
 }
 
@@ -1389,52 +1519,6 @@ float eri_ema_effective_decay(float decay, uint64_t step, float power, int use_b
 
 // ---- EMAModel ------------------------------------------------------------------------------------
 
-struct EriEmaModel {
-    struct Shadow {
-        void *data = nullptr;
-        uint64_t numel = 0;
-        int32_t dtype = 0;
-    };
-    float decay = 0.999f, power = 1.0f;
-    bool bias_correction = true;
-    uint64_t step = 0;
-    void *stream = nullptr;
-    std::map<std::string, Shadow> shadows;
-    std::vector<EriEmaTensor> rows; // reused between updates
-    ~EriEmaModel() {
-        for (auto &kv : shadows)
-            if (kv.second.data) eri_hip_free(kv.second.data);
-    }
-};
-
-namespace {
-
-uint64_t elem_bytes(int32_t dtype) { return dtype == ERI_DTYPE_F32 ? 4 : 2; }
-
-// a fresh shadow holding a copy of the parameter (ema_enhanced.rs:72-73,100-103)
-int ema_adopt(EriEmaModel *e, const std::string &name, const EriParameter *p) {
-    if (!p || !p->data) return fail(ERI_ERR_NULL, "parameter without data: " + name);
-    if (p->numel == 0) return fail(ERI_ERR_EMPTY, "empty parameter: " + name);
-    if (p->dtype != ERI_DTYPE_F32 && p->dtype != ERI_DTYPE_BF16) return fail(ERI_ERR_DTYPE, "Unsupported: EMA takes F32 or BF16 parameters");
-    EriEmaModel::Shadow &s = e->shadows[name];
-    const uint64_t bytes = p->numel * elem_bytes(p->dtype);
-    if (!s.data || s.numel != p->numel || s.dtype != p->dtype) {
-        if (s.data) eri_hip_free(s.data);
-        s = EriEmaModel::Shadow();
-        int dev = 0;
-        int rc = eri_hip_get_device(&dev);
-        if (!rc) rc = eri_hip_malloc_zeroed(dev, bytes, &s.data);
-        if (rc) {
-            e->shadows.erase(name);
-            return rc;
-        }
-        s.numel = p->numel;
-        s.dtype = p->dtype;
-    }
-    return eri_hip_memcpy_async(s.data, p->data, bytes, 3, e->stream);
-}
-
-} // namespace
 
 extern "C" {
 

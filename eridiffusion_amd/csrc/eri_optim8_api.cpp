@@ -277,8 +277,8 @@ struct EriAdam8Table {
         int dtype = 0;
         uint32_t n = 0;
         uint32_t total_blocks = 0; // full blocks only; a row's partial last block is handled per row
-        eri::DevTensor *dev = nullptr;
-        eri::DevTensor *pinned = nullptr;
+        eri::DevTensor *dev = nullptr;    // n rows, then one uint32 row index per full block (BlockRowMap)
+        eri::DevTensor *pinned = nullptr; // the rows only
         std::vector<uint32_t> src; // index into the caller's rows
         bool unit_scales = true;   // every row's grad_scale is exactly 1
     };
@@ -341,7 +341,8 @@ int validate_rows(const EriAdam8Tensor *rows, uint32_t n) {
                 return fail(ERI_ERR_ARG, buf);
             }
         }
-        const uintptr_t wide = (uintptr_t)r.p | (uintptr_t)r.g | (uintptr_t)r.m | (uintptr_t)r.v | (uintptr_t)r.p_src;
+        const uintptr_t wide = (uintptr_t)r.p | (uintptr_t)r.g | (uintptr_t)r.m | (uintptr_t)r.v | (uintptr_t)r.p_src |
+                               (uintptr_t)r.ema_shadow;
         const uintptr_t narrow = (uintptr_t)r.absmax_m | (uintptr_t)r.absmax_v;
         if ((wide & 15u) || (narrow & 3u)) {
             std::snprintf(buf, sizeof buf, "row %u: p/g/m/v must be 16-byte aligned, absmax 4-byte aligned", i);
@@ -367,7 +368,7 @@ void fill_group(EriAdam8Table::Group &g, const EriAdam8Tensor *rows) {
         eri::DevTensor &d = g.pinned[j];
         d.p = r.p;
         d.p_in = r.p_src ? r.p_src : r.p;
-        d.pad = 0;
+        d.shadow = r.ema_shadow;
         d.g = r.g;
         d.m = r.m;
         d.v = r.v;
@@ -659,9 +660,18 @@ int eri_adam8_table_create(const EriAdam8Tensor *rows, uint32_t n, void *stream,
     for (auto &g : t->groups) {
         g.n = (uint32_t)g.src.size();
         if (g.n == 0 || e != hipSuccess) continue;
-        e = hipMalloc((void **)&g.dev, sizeof(eri::DevTensor) * g.n);
+        uint64_t full = 0;
+        for (uint32_t j = 0; j < g.n; ++j) full += rows[g.src[j]].numel / eri::kBlock;
+        e = hipMalloc((void **)&g.dev, sizeof(eri::DevTensor) * g.n + sizeof(uint32_t) * (full ? full : 1));
         if (e == hipSuccess) e = hipHostMalloc((void **)&g.pinned, sizeof(eri::DevTensor) * g.n, hipHostMallocDefault);
         if (e == hipSuccess) fill_group(g, rows);
+        if (e == hipSuccess && full) { // which row owns which full block: fixed for the table's life
+            std::vector<uint32_t> row_of((size_t)full);
+            size_t at = 0;
+            for (uint32_t j = 0; j < g.n; ++j)
+                for (uint64_t k = rows[g.src[j]].numel / eri::kBlock; k > 0; --k) row_of[at++] = j;
+            e = hipMemcpy(g.dev + g.n, row_of.data(), sizeof(uint32_t) * (size_t)full, hipMemcpyHostToDevice);
+        }
     }
     if (e != hipSuccess) {
         destroy_table(t);
@@ -709,6 +719,8 @@ int eri_adam8_step_table(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream)
     if (!t || !h) return fail(ERI_ERR_NULL, "table or hyper is NULL");
     if (h->mode != ERI_ADAM8_MODE_ERI && h->mode != ERI_ADAM8_MODE_L2 && h->mode != ERI_ADAM8_MODE_BNB)
         return fail(ERI_ERR_ARG, "unknown mode");
+    if ((h->flags & ERI_ADAM8_FLAG_EMA) && !(h->ema_decay >= 0.0f && h->ema_decay <= 1.0f))
+        return fail(ERI_ERR_ARG, "ERI_ADAM8_FLAG_EMA needs ema_decay in [0, 1]");
     DeviceCtx *ctx = nullptr;
     int rc = get_ctx_on(t->device, &ctx);
     if (rc) return rc;
@@ -746,6 +758,25 @@ int eri_adam8_step_table(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream)
         }
         rc = eri::launch_step(g.dev, g.n, g.total_blocks, g.dtype, hh, ctx->image, dev_scale, grid, waves_per_wg * eri::kWave, ctx->cus, stream);
         if (rc) return hip_fail((hipError_t)rc, "adam8 step launch");
+        if ((hh.flags & ERI_ADAM8_FLAG_EMA) && !eri::step_fuses_ema(g.total_blocks, g.dtype, hh, ctx->cus)) {
+            // not the kernel that carries the EMA: the plain sweep over this group's shadows, right behind the step
+            std::vector<EriEmaTensor> er;
+            for (uint32_t j = 0; j < g.n; ++j) {
+                const eri::DevTensor &d = g.pinned[j];
+                if (!d.shadow) continue;
+                EriEmaTensor e;
+                e.shadow = d.shadow;
+                e.p = d.p;
+                e.numel = d.numel;
+                e.dtype_tag = eri::layout_param_bf16(g.dtype) ? ERI_DTYPE_BF16 : ERI_DTYPE_F32;
+                e.reserved = 0;
+                er.push_back(e);
+            }
+            if (!er.empty()) {
+                rc = eri_ema_update_multi(er.data(), (uint32_t)er.size(), hh.ema_decay, stream);
+                if (rc) return rc;
+            }
+        }
     }
     return 0;
 }

@@ -153,6 +153,17 @@ impl Adam8bit {
     pub fn set_grad_scale(&mut self, scale: f32) -> Result<()> {
         check(unsafe { sys::eri_adam8bit_set_grad_scale(self.opt, scale) }, "eri_adam8bit_set_grad_scale")
     }
+    /// From now on every step() also performs `ema.update(params)` (ema_enhanced.rs:79-104) over this optimizer's
+    /// parameters, `names[i]` being the model's name for parameter i; the trainer drops its own ema.update() call.
+    /// The model must outlive the optimizer or be detached with `detach_ema()`.
+    pub fn attach_ema(&mut self, ema: &mut EMAModel, names: &[&str]) -> Result<()> {
+        let c: Vec<CString> = names.iter().map(|n| CString::new(*n).unwrap()).collect();
+        let ptrs: Vec<*const std::os::raw::c_char> = c.iter().map(|n| n.as_ptr()).collect();
+        check(unsafe { sys::eri_adam8bit_attach_ema(self.opt, ema.ema, ptrs.as_ptr(), ptrs.len() as u32) }, "eri_adam8bit_attach_ema")
+    }
+    pub fn detach_ema(&mut self) {
+        unsafe { sys::eri_adam8bit_attach_ema(self.opt, std::ptr::null_mut(), std::ptr::null(), 0) };
+    }
     /// Global-norm clipping inside step(): norm on the device, factor applied by the step kernel.
     pub fn set_max_grad_norm(&mut self, max_norm: f32, denom_eps: f32) -> Result<()> {
         check(unsafe { sys::eri_adam8bit_set_max_grad_norm(self.opt, max_norm, denom_eps) }, "eri_adam8bit_set_max_grad_norm")

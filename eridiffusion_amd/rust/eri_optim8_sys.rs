@@ -18,12 +18,14 @@ pub const ERI_ADAM8_FLAG_BSEARCH: u32 = 4;
 pub const ERI_ADAM8_FLAG_NO_PIPELINE: u32 = 8;
 pub const ERI_ADAM8_FLAG_CLIP_FROM_TABLE: u32 = 16;
 pub const ERI_ADAM8_FLAG_ONE_WAVE: u32 = 32;
+pub const ERI_ADAM8_FLAG_EMA: u32 = 64;
 
 #[repr(C)]
 #[derive(Clone, Copy, Default)]
 pub struct EriAdam8Hyper {
     pub beta1: f32, pub beta2: f32, pub omb1: f32, pub omb2: f32, pub eps: f32, pub weight_decay: f32,
     pub step_size: f32, pub bc1: f32, pub bc2: f32, pub grad_scale: f32, pub mode: i32, pub flags: u32,
+    pub ema_decay: f32, pub reserved: u32,
 }
 
 #[repr(C)]
@@ -32,7 +34,7 @@ pub struct EriAdam8Tensor {
     pub p: *mut c_void, pub g: *const c_void, pub m: *mut u8, pub v: *mut u8,
     pub absmax_m: *mut f32, pub absmax_v: *mut f32,
     pub numel: u64, pub block_start: u64, pub dtype_tag: i32, pub grad_scale: f32,
-    pub p_src: *const c_void, pub grad_f32: i32, pub reserved: i32,
+    pub p_src: *const c_void, pub grad_f32: i32, pub reserved: i32, pub ema_shadow: *mut c_void,
 }
 
 #[repr(C)]
@@ -121,6 +123,7 @@ extern "C" {
     pub fn eri_adam8bit_get_step(opt: *const EriAdam8bit) -> u64;
     pub fn eri_adam8bit_set_grad_scale(opt: *mut EriAdam8bit, scale: f32) -> c_int;
     pub fn eri_adam8bit_set_param_grad_scale(opt: *mut EriAdam8bit, index: u32, scale: f32) -> c_int;
+    pub fn eri_adam8bit_attach_ema(opt: *mut EriAdam8bit, ema: *mut EriEmaModel, names: *const *const c_char, n: u32) -> c_int;
     pub fn eri_adam8bit_set_min_8bit_size(opt: *mut EriAdam8bit, numel: u64) -> c_int;
     pub fn eri_adam8bit_state32_ptrs(opt: *const EriAdam8bit, index: u32, m: *mut *mut f32, v: *mut *mut f32) -> c_int;
     pub fn eri_adam8bit_set_max_grad_norm(opt: *mut EriAdam8bit, max_norm: f32, denom_eps: f32) -> c_int;

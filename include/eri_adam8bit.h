@@ -52,6 +52,7 @@ void eri_adam8bit_config_default(EriAdam8bitConfig *cfg);
 
 /* ---- Adam8bit: step() over a parameter list --------------------------------------------------- */
 typedef struct EriAdam8bit EriAdam8bit;
+typedef struct EriEmaModel EriEmaModel; /* declared in full further down */
 /* Adam8bit::new(params, config) :161.  `stream` (NULL = default) is used by every later call. */
 int eri_adam8bit_new(EriParameter *const *params, uint32_t n, const EriAdam8bitConfig *cfg, void *stream,
                      EriAdam8bit **out);
@@ -72,6 +73,14 @@ int eri_adam8bit_set_param_grad_scale(EriAdam8bit *opt, uint32_t index, float sc
 int eri_adam8bit_set_flags(EriAdam8bit *opt, uint32_t flags); /* ERI_ADAM8_FLAG_EXACT_PARAM etc. */
 /* ERI_ADAM8_MODE_ERI (default: the reference's update) or ERI_ADAM8_MODE_BNB for later steps. */
 int eri_adam8bit_set_mode(EriAdam8bit *opt, int mode);
+/* EMA inside the step.  With a model attached, every eri_adam8bit_step also performs that model's
+ * update(params) (ema_enhanced.rs:79-104: step += 1, shadow = d*shadow + (1-d)*param with d = current_decay(),
+ * a name seen for the first time gets a copy of its parameter) over all n parameters of the optimizer, names[i]
+ * being the model's name for parameter i -- so the trainer's separate ema.update() call and its sweep go
+ * away.  For parameters that take the 8-bit step the shadow is updated by that same launch
+ * (ERI_ADAM8_FLAG_EMA); parameters without a gradient, or with fp32 moments, get the plain sweep.  The model is
+ * not owned and must outlive the optimizer or be detached (ema = NULL); both must use the same stream. */
+int eri_adam8bit_attach_ema(EriAdam8bit *opt, EriEmaModel *ema, const char *const *names, uint32_t n);
 /* min_8bit_size (pipeline_flux_lora_1024.rs:451, the policy of the library the state format comes from):
  * from the next step on, a parameter with fewer than `numel` elements that has no 8-bit state yet keeps
  * fp32 moments instead and takes the same update, adam8bit_enhanced.rs:252-275, without the quantiser --
@@ -177,7 +186,6 @@ int eri_analyze_optimizer_memory(uint64_t num_params, const char *precision, Eri
  * over every parameter already known, plus a device copy for names seen for the first time (:100-103).
  * eri_ema_new: decay outside (0, 1] is refused with "EMA decay must be in (0, 1], got ..." (:36-41);
  * the reference's defaults are use_bias_correction = 1, power = 1 (:48-50; with_config :55-64). */
-typedef struct EriEmaModel EriEmaModel;
 int eri_ema_new(float decay, int use_bias_correction, float power, void *stream, EriEmaModel **out);
 int eri_ema_destroy(EriEmaModel *ema);
 /* init_from_params :67-76: every shadow becomes a copy of its parameter. */

@@ -108,6 +108,13 @@ enum {
                                              block one (small tables).  Same results; a cross-check */
     ERI_ADAM8_FLAG_CLIP_FROM_TABLE = 1u << 4, /* also multiply gradients by the clip factor the last
                                              eri_adam8_grad_norm left in the table (device memory) */
+    ERI_ADAM8_FLAG_EMA = 1u << 6,         /* after the update, every row that has an ema_shadow also gets
+                                             shadow = ema_decay*shadow + (1 - ema_decay)*p', the EMA update of
+                                             src/trainers/ema_enhanced.rs:91-100 on the parameter as it was just
+                                             stored.  Large BF16 tables in mode ERI do it inside the step kernel
+                                             (the new parameter is still in registers: the separate sweep's read
+                                             of p is saved); every other table runs the EMA sweep right after
+                                             the step, in the same call.  Same results either way */
     ERI_ADAM8_FLAG_ONE_WAVE = 1u << 5     /* never take the four-waves-per-block kernel, which small and F32
                                              tables get by default: a small BF16 table then runs on the
                                              prefetching kernel.  Same results; lets tests reach every
@@ -126,6 +133,9 @@ typedef struct EriAdam8Hyper {
     float grad_scale;   /* used with ERI_ADAM8_FLAG_GRAD_SCALE       pipeline_flux_lora_sequential.rs:1198-1213 */
     int32_t mode;       /* EriAdam8Mode */
     uint32_t flags;     /* ERI_ADAM8_FLAG_* */
+    float ema_decay;    /* used with ERI_ADAM8_FLAG_EMA: the effective decay of this step
+                           (eri_ema_effective_decay, ema_enhanced.rs:106-127); eri_adam8_hyper_pack leaves 0 */
+    uint32_t reserved;  /* 0 */
 } EriAdam8Hyper;
 
 /* `step` is the optimizer's counter after its increment for ERI (adam8bit_enhanced.rs:203) and the
@@ -157,6 +167,8 @@ typedef struct EriAdam8Tensor {
                              (adam8bit_enhanced.rs:231-235, adam8bit.rs:110).  Such rows run on the
                              four-waves-per-block kernel whatever the flags say.  Must be 0 for F32 parameters */
     int32_t reserved;     /* 0 */
+    void *ema_shadow;     /* NULL, or the EMA shadow of this parameter (dtype of p, numel elements, 16-byte aligned):
+                             updated by steps that carry ERI_ADAM8_FLAG_EMA */
 } EriAdam8Tensor;
 
 typedef struct EriAdam8Table EriAdam8Table; /* device-resident copy of a launch table */

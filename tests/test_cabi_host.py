@@ -57,8 +57,8 @@ def test_build_rs_compiles_the_objects_of_the_makefile():
 
 
 def test_struct_layouts_match_the_header():
-    assert C.sizeof(L.Hyper) == 48
-    assert C.sizeof(L.TensorRow) == 88
+    assert C.sizeof(L.Hyper) == 56
+    assert C.sizeof(L.TensorRow) == 96
     assert C.sizeof(L.AdamW32Row) == 56 and C.sizeof(L.EmaRow) == 32
     assert L.TensorRow.numel.offset == 48 and L.TensorRow.dtype_tag.offset == 64
     assert L.TensorRow.p_src.offset == 72 and L.TensorRow.grad_f32.offset == 80
@@ -224,6 +224,6 @@ int main(void) {
             C.sizeof(L.Adam8bitConfigC), C.sizeof(L.MemoryReportC)]
     assert got == want, (got, want)
     cpp = tmp_path / "check.cpp"
-    cpp.write_text('#include "eri_optim8.h"\n#include "eri_adam8bit.h"\nint main() { return sizeof(EriAdam8Hyper) == 48 ? 0 : 1; }\n')
+    cpp.write_text('#include "eri_optim8.h"\n#include "eri_adam8bit.h"\nint main() { return sizeof(EriAdam8Hyper) == 56 && sizeof(EriAdam8Tensor) == 96 ? 0 : 1; }\n')
     subprocess.check_call(["g++", "-std=c++17", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", inc, str(cpp), "-o", str(tmp_path / "checkpp")])
     assert subprocess.call([str(tmp_path / "checkpp")]) == 0
