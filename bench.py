@@ -312,7 +312,8 @@ def main():
     if os.path.exists(args.traffic_json):
         try:
             with open(args.traffic_json) as f:
-                traffic = json.load(f).get(args.config) if args.kernel == "adam8" else None
+                key = "%s|%s|flags=%d" % (args.config, args.kernel, args.flags)
+                traffic = json.load(f).get(key) if args.api == "table" and args.mode == "eri" else None
         except Exception:
             traffic = None
     out = {

@@ -252,6 +252,36 @@ def test_l2_mode_first_call_follows_the_functional_update():
     assert np.allclose(p, want, rtol=0, atol=6e-7)  # two fp32 roundings near |p| ~ 3
 
 
+@pytest.mark.parametrize("step", [2, 7, 40])
+def test_l2_mode_bias_correction_at_later_steps(step):
+    """adam8bit.rs:164-187 beyond the first call: s = max(step, 1), m_hat = m / (1 - b1^s), v_hat = v / (1 - b2^s).
+    From a zero state one call gives m = (1-b1) g', v = (1-b2) g'^2, so the update has the closed form
+    lr * g' * [(1-b1)/(1-b1^s)] / (|g'| * sqrt((1-b2)/(1-b2^s)) + eps); a bias correction that took the wrong
+    exponent (s-1, s+1, or the other beta) is off by percents, far outside the tolerance."""
+    n = 2048
+    rng = np.random.default_rng(60 + step)
+    p0 = rng.standard_normal(n).astype(np.float32)
+    g = (rng.standard_normal(n) * 1e-2).astype(np.float32)
+    h = oc.hyper_pack(LR, 0.9, 0.999, EPS, WD, step, oc.MODE_L2)
+    assert h.bc1 == np.float32(1.0 - 0.9 ** step) and h.bc2 == np.float32(1.0 - 0.999 ** step)
+    assert h.omb1 == np.float32(1.0 - 0.9) and h.step_size == np.float32(LR)
+    p = p0.copy()
+    run_c(p, g, oc.state_init(n), step, mode=oc.MODE_L2)
+    g2 = g.astype(np.float64) + WD * p0.astype(np.float64)
+    c1 = (1 - 0.9) / (1 - 0.9 ** step)
+    c2 = np.sqrt((1 - 0.999) / (1 - 0.999 ** step))
+    want = p0 - LR * g2 * c1 / (np.abs(g2) * c2 + EPS)
+    assert np.allclose(p, want, rtol=0, atol=6e-7)
+    for wrong in (step - 1, step + 1):
+        w1 = (1 - 0.9) / (1 - 0.9 ** wrong)
+        w2 = np.sqrt((1 - 0.999) / (1 - 0.999 ** wrong))
+        assert not np.allclose(p, p0 - LR * g2 * w1 / (np.abs(g2) * w2 + EPS), rtol=0, atol=6e-7)
+    # the NumPy restatement agrees bit for bit
+    hn = onp.hyper_pack(LR, 0.9, 0.999, EPS, WD, step, "l2")
+    q = onp.step_tensor(p0, g, *onp.state_init(n), hn, *oc.load_maps())[0]
+    assert np.array_equal(q.view(np.uint32), p.view(np.uint32))
+
+
 # ---- mode BNB: eps under the bias correction, decay as a factor, sign of the first moment kept ----
 
 def test_bnb_scalars():
