@@ -42,6 +42,10 @@ def parse():
                          "per-name optimizer, all tensors through one eri_adam8bit_fn_update_many call per step, "
                          "each step writing into the other of two output sets (update() returns a new tensor).  "
                          "functional_update: the same through one batched eri_adam8bit_fn_update call per tensor")
+    ap.add_argument("--param-dtype", choices=["config", "bf16", "f32"], default="config",
+                    help="parameter dtype: the one the configuration names, or an override (the shapes stay)")
+    ap.add_argument("--grad-dtype", choices=["param", "f32"], default="param",
+                    help="gradient dtype: the parameter's, or fp32 gradients (for bf16 parameters: read unrounded)")
     ap.add_argument("--alloc", choices=["arena", "tensor"], default="arena",
                     help="one flat allocation per kind of buffer (library allocator), or one torch allocation per "
                          "tensor and buffer (how a tensor runtime holds parameters and states)")
@@ -169,8 +173,14 @@ def main():
 
     fn, dt_name = W.CONFIGS[args.config]
     tensors = fn()
+    if args.param_dtype != "config":
+        dt_name = args.param_dtype
     bf16 = dt_name == "bf16"
     esz = 2 if bf16 else 4
+    grad_f32 = bf16 and args.grad_dtype == "f32"
+    gsz = 4 if grad_f32 else esz
+    if grad_f32 and (args.kernel in ("adamw32",) or args.api != "table"):
+        sys.exit("--grad-dtype f32 is wired for the table API's 8-bit step and the gradient norm")
     sizes = [W.numel(s) for _, s in tensors]
     n_params = sum(sizes)
     n_blocks = sum((n + L.BLOCK - 1) // L.BLOCK for n in sizes)
@@ -179,7 +189,7 @@ def main():
 
     Alloc = {"arena": Arena, "tensor": PerTensor}[args.alloc]
     a_p = Alloc(torch, [n * esz for n in sizes])
-    a_g = Alloc(torch, [n * esz for n in sizes])
+    a_g = Alloc(torch, [n * gsz for n in sizes])
     a_m = Alloc(torch, sizes)
     a_v = Alloc(torch, sizes)
     a_am = Alloc(torch, [((n + 2047) // 2048) * 4 for n in sizes])
@@ -190,7 +200,7 @@ def main():
     p_std, g_std = (0.02, 1e-3)
     for i, n in enumerate(sizes):  # synthetic data: p ~ N(0, 0.02), g ~ N(0, 1e-3)
         a_p.fill(i, torch.randn(n, device="cuda:0", generator=gen).mul_(p_std).to(tdt), stream)
-        a_g.fill(i, torch.randn(n, device="cuda:0", generator=gen).mul_(g_std).to(tdt), stream)
+        a_g.fill(i, torch.randn(n, device="cuda:0", generator=gen).mul_(g_std).to(torch.float32 if grad_f32 else tdt), stream)
         L.check(L.lib().eri_adam8_state_init(a_m.ptr(i), a_v.ptr(i), a_am.ptr(i), a_av.ptr(i), n, stream), "state_init")
     rows = (L.TensorRow * len(sizes))()
     start = 0
@@ -198,11 +208,12 @@ def main():
         r = rows[i]
         r.p, r.g, r.m, r.v, r.absmax_m, r.absmax_v = a_p.ptr(i), a_g.ptr(i), a_m.ptr(i), a_v.ptr(i), a_am.ptr(i), a_av.ptr(i)
         r.numel, r.block_start, r.dtype_tag, r.grad_scale = n, start, (L.DTYPE_BF16 if bf16 else L.DTYPE_F32), 1.0
+        r.grad_f32 = 1 if grad_f32 else 0
         start += (n + L.BLOCK - 1) // L.BLOCK
     table = C.c_void_p()
     L.check(L.lib().eri_adam8_table_create(rows, len(rows), stream, C.byref(table)), "table_create")
     hyper_args = (1e-4, 0.9, 0.999, 1e-8, 0.01)
-    bytes_per_param = BYTES_PER_PARAM[dt_name]
+    bytes_per_param = BYTES_PER_PARAM[dt_name] + (gsz - esz)
     extra = []
     if args.kernel == "adamw32":
         a_m32 = Alloc(torch, [4 * n for n in sizes])
@@ -230,9 +241,9 @@ def main():
             rows_e[i].dtype_tag = L.DTYPE_BF16 if bf16 else L.DTYPE_F32
         bytes_per_param = 3 * esz
     elif args.kernel == "grad_norm":
-        bytes_per_param = esz + 4.0 / 2048
+        bytes_per_param = gsz + 4.0 / 2048
     elif args.kernel == "adam8_clip":
-        bytes_per_param += esz + 4.0 / 2048
+        bytes_per_param += gsz + 4.0 / 2048
 
     fn_opt = None
     if args.api != "table":
@@ -313,7 +324,8 @@ def main():
         try:
             with open(args.traffic_json) as f:
                 key = "%s|%s|flags=%d" % (args.config, args.kernel, args.flags)
-                traffic = json.load(f).get(key) if args.api == "table" and args.mode == "eri" else None
+                plain = args.api == "table" and args.mode == "eri" and args.param_dtype == "config" and not grad_f32
+                traffic = json.load(f).get(key) if plain else None
         except Exception:
             traffic = None
     out = {
@@ -331,8 +343,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": args.config, "tensors": len(sizes), "params": n_params, "blocks": n_blocks,
                    "kernel": args.kernel, "api": args.api, "mode": "l2" if args.api != "table" else args.mode,
-                   "param_dtype": dt_name, "state": "uint8 m/v + fp32 absmax per 2048-block", "flags": args.flags,
-                   "resident_gb": round((n_params * (2 * esz + 2) + n_blocks * 8) / 1e9, 2)},
+                   "param_dtype": dt_name, "grad_dtype": "f32" if gsz == 4 else "bf16", "state": "uint8 m/v + fp32 absmax per 2048-block", "flags": args.flags,
+                   "resident_gb": round((n_params * (esz + gsz + 2) + n_blocks * 8) / 1e9, 2)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                      "frac": achieved / PEAK_HBM_GBPS, "traffic": traffic,
                      "traffic_source": None if traffic is None else "profiles/traffic.json: FETCH_SIZE and WRITE_SIZE of "

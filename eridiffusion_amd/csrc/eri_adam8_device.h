@@ -83,6 +83,10 @@ int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_bloc
 constexpr uint32_t kChunks = 8;           /* contiguous ranges the block list is cut into: one per accelerator die */
 constexpr uint32_t kSplitBlocksPerCu = 64; /* tables of at most this many full blocks per compute unit take the
                                               four-waves-per-block kernel */
+constexpr uint32_t kPrefetchBlocksPerCu = 1024; /* bf16 tables take the prefetching kernel above this many full blocks
+                                                   per compute unit; up to it, sixteen waves without a prefetch are
+                                                   2-4 % faster than twelve with one (measured at 292-876 per unit,
+                                                   the other way round from 1,168) */
 constexpr uint32_t kNormWaves = 4;        /* waves per workgroup of the gradient-norm pass */
 
 /* The chunked walk (BlockWalk) needs the same number of workgroups in every chunk. */
@@ -94,7 +98,7 @@ inline uint32_t chunks_for(uint32_t grid) { return grid % kChunks == 0 ? kChunks
 int launch_step_plain_f32(int mode, bool wd, bool gs, bool keytab, const DevTensor *rows, uint32_t n_rows,
                           uint32_t total_blocks, const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale,
                           uint32_t grid, uint32_t wg, void *stream);
-int launch_step_plain_bf16(int mode, bool exact, bool wd, bool gs, bool keytab, const DevTensor *rows, uint32_t n_rows,
+int launch_step_plain_bf16(int mode, bool exact, bool wd, bool gs, bool keytab, bool grad_f32, const DevTensor *rows, uint32_t n_rows,
                            uint32_t total_blocks, const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale,
                            uint32_t grid, uint32_t wg, void *stream);
 /* Four waves per block, for tables of few blocks; `grid` workgroups of 1024 threads. */

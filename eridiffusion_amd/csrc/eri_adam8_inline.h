@@ -495,14 +495,14 @@ __device__ __forceinline__ void requant8(const float *mf, const float *vf, const
     vw.y = cv[4] | (cv[5] << 8) | (cv[6] << 16) | (cv[7] << 24);
 }
 
-template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB>
+template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB, bool GBF16 = BF16>
 __device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint32_t lane, const EriAdam8Hyper &h,
                                            float gscale, const BlockDiv &dbc1, const BlockDiv &dbc2, const Lds &L) {
     const size_t e0 = (size_t)lb * kBlock;
     const size_t esz = BF16 ? 2 : 4;
     char *p = static_cast<char *>(t.p) + e0 * esz;
     const char *p_in = static_cast<const char *>(t.p_in) + e0 * esz;
-    const char *g = static_cast<const char *>(t.g) + e0 * esz;
+    const char *g = static_cast<const char *>(t.g) + e0 * (GBF16 ? 2 : 4);
     uint8_t *mc = t.m + e0;
     uint8_t *vc = t.v + e0;
     const float a_m = as_global(t.absmax_m)[lb];
@@ -511,11 +511,12 @@ __device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint
     float mf[32], vf[32];
     float lm = 0.0f, lv = 0.0f;
     // Issue the loads of DEPTH passes before touching the first value: the wave then waits once per
-    // DEPTH passes, with 48 * DEPTH bytes per lane in flight (bf16; fp32 holds twice the registers).
-    constexpr int DEPTH = BF16 ? 4 : 2;
+    // DEPTH passes, with 48 * DEPTH bytes per lane in flight (bf16; fp32 values hold twice the registers).
+    constexpr int DEPTH = (BF16 && GBF16) ? 4 : 2;
 #pragma unroll
     for (int c0 = 0; c0 < 4; c0 += DEPTH) {
-        Raw8<BF16> pr[DEPTH], gr[DEPTH];
+        Raw8<BF16> pr[DEPTH];
+        Raw8<GBF16> gr[DEPTH];
         u32x2 mr[DEPTH], vr[DEPTH];
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {

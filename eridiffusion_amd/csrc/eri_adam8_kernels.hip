@@ -15,20 +15,26 @@ bool step_fuses_ema(uint32_t total_blocks, int layout, const EriAdam8Hyper &h, u
     return (h.flags & ERI_ADAM8_FLAG_ONE_WAVE) != 0 || !few;
 }
 
+/* Whether a bf16 table that qualifies for the prefetching kernel is large enough to gain from it.  A step
+ * that carries the EMA stays on the prefetching kernel at every size: it is the one that fuses it. */
+static bool prefetch_pays(uint32_t total_blocks, const EriAdam8Hyper &h, uint32_t compute_units) {
+    if (h.flags & (ERI_ADAM8_FLAG_ONE_WAVE | ERI_ADAM8_FLAG_EMA)) return true;
+    return (uint64_t)total_blocks > (uint64_t)compute_units * (uint64_t)kPrefetchBlocksPerCu;
+}
+
 int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, int layout,
                 const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg,
                 uint32_t compute_units, void *stream) {
     const bool bf16 = layout_param_bf16(layout);
-    const bool mixed = layout == kLayoutBF16GradF32; // only the four-waves-per-block kernel reads F32 gradients for BF16 parameters
+    const bool mixed = layout == kLayoutBF16GradF32; // F32 gradients for BF16 parameters
     const bool gs = (h.flags & ERI_ADAM8_FLAG_GRAD_SCALE) != 0;
-    // Four waves share each block where that is the faster kernel: few blocks (one wave per block would
-    // leave the chip idle) and fp32 parameters (measured ahead of the one-wave kernel from 64 Ki to
-    // 3 Mi blocks).
-    // The flags that name a kernel (cross-checks) keep their meaning.
+    // Four waves share each block where one wave per block would leave the chip idle: tables of few blocks.
+    // The flags that name a kernel (cross-checks) keep their meaning; bf16 parameters with fp32 gradients
+    // have no binary-search variant of the one-wave kernel and stay on this one for those flags.
     const bool one_wave = (h.flags & ERI_ADAM8_FLAG_ONE_WAVE) != 0;
     const bool kernel_named = (h.flags & (ERI_ADAM8_FLAG_BSEARCH | ERI_ADAM8_FLAG_NO_PIPELINE)) != 0;
     const bool few = (uint64_t)total_blocks <= (uint64_t)compute_units * (uint64_t)kSplitBlocksPerCu;
-    if (mixed || (!kernel_named && !one_wave && (few || !bf16))) {
+    if ((mixed && (h.flags & ERI_ADAM8_FLAG_BSEARCH) != 0) || (!kernel_named && !one_wave && few)) {
         const bool bnb = h.mode == ERI_ADAM8_MODE_BNB;
         const bool wd_s = bnb ? h.weight_decay != 1.0f : h.weight_decay > 0.0f;
         const bool exact_s = !bf16 || (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0;
@@ -39,22 +45,28 @@ int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, i
         if (need == 0) need = 1;
         return launch_step_split(layout, h.mode, exact_s, wd_s, gs, rows, n_rows, total_blocks, h, lds_image, dev_scale, need, stream);
     }
+    if (mixed) {
+        const bool wd_m = h.mode == ERI_ADAM8_MODE_BNB ? h.weight_decay != 1.0f : h.weight_decay > 0.0f;
+        return launch_step_plain_bf16(h.mode, (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0, wd_m, gs, true, true, rows, n_rows,
+                                      total_blocks, h, lds_image, dev_scale, grid, wg, stream);
+    }
     if (h.mode == ERI_ADAM8_MODE_BNB) { // slot table only; the decay is a factor
         const bool wd = h.weight_decay != 1.0f;
         const bool exact = (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0;
-        if (bf16 && !kernel_named)
+        if (bf16 && !kernel_named && prefetch_pays(total_blocks, h, compute_units))
             return launch_step_pipelined(h.mode, exact, wd, gs, false, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
-        if (bf16) return launch_step_plain_bf16(h.mode, exact, wd, gs, true, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
+        if (bf16) return launch_step_plain_bf16(h.mode, exact, wd, gs, true, false, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
         return launch_step_plain_f32(h.mode, wd, gs, true, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
     }
     const bool wd = h.weight_decay > 0.0f;
     const bool exact = (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0;
     const bool keytab = (h.flags & ERI_ADAM8_FLAG_BSEARCH) == 0;
     if (!bf16) return launch_step_plain_f32(h.mode, wd, gs, keytab, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
-    if (keytab && h.mode == ERI_ADAM8_MODE_ERI && (h.flags & ERI_ADAM8_FLAG_NO_PIPELINE) == 0)
+    if (keytab && h.mode == ERI_ADAM8_MODE_ERI && (h.flags & ERI_ADAM8_FLAG_NO_PIPELINE) == 0 &&
+        prefetch_pays(total_blocks, h, compute_units))
         return launch_step_pipelined(h.mode, exact, wd, gs, step_fuses_ema(total_blocks, layout, h, compute_units), rows, n_rows,
                                      total_blocks, h, lds_image, dev_scale, grid, wg, stream);
-    return launch_step_plain_bf16(h.mode, exact, wd, gs, keytab, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
+    return launch_step_plain_bf16(h.mode, exact, wd, gs, keytab, false, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
 }
 
 // ------------------------------------------------------------------------------------------

@@ -1,7 +1,8 @@
 /*
- * The plain step kernel (no cross-block prefetch): fp32 tensors, and bf16 tensors in mode BNB, with
- * ERI_ADAM8_FLAG_BSEARCH or with ERI_ADAM8_FLAG_NO_PIPELINE.  Compiled twice, once per parameter dtype
- * (-DERI_PLAIN_BF16=0|1), so that the two halves build in parallel.
+ * The plain step kernel (one wave per block, no cross-block prefetch): large tables of fp32 parameters and
+ * of bf16 parameters with fp32 gradients, bf16 tables in the functional update's arithmetic, and any table
+ * with ERI_ADAM8_FLAG_BSEARCH, ERI_ADAM8_FLAG_NO_PIPELINE or ERI_ADAM8_FLAG_ONE_WAVE.  Compiled twice,
+ * once per parameter dtype (-DERI_PLAIN_BF16=0|1), so that the two halves build in parallel.
  */
 #include "eri_adam8_inline.h"
 
@@ -16,7 +17,7 @@ namespace eri {
  * threads (170 registers) it does not. */
 constexpr uint32_t plain_threads(int mode) { return mode == ERI_ADAM8_MODE_L2 ? 768 : 1024; }
 
-template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB>
+template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB, bool GBF16>
 __global__ __launch_bounds__(plain_threads(MODE)) void adam8_step_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
                                                           uint32_t total_blocks, EriAdam8Hyper h,
                                                           const uint4 *__restrict__ lds_image,
@@ -51,7 +52,7 @@ __global__ __launch_bounds__(plain_threads(MODE)) void adam8_step_kernel(const D
         const uint32_t n = (uint32_t)(t.numel % kBlock);
         if (n != 0) {
             const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
-            tail_block<BF16, MODE, EXACT, WD, GS, KEYTAB>(t, (uint32_t)(t.numel / kBlock), n, lane, h, gscale, dbc1, dbc2, L);
+            tail_block<BF16, MODE, EXACT, WD, GS, KEYTAB, GBF16>(t, (uint32_t)(t.numel / kBlock), n, lane, h, gscale, dbc1, dbc2, L);
         }
     }
     uint32_t ti = 0, t_end = 0;
@@ -61,7 +62,7 @@ __global__ __launch_bounds__(plain_threads(MODE)) void adam8_step_kernel(const D
     for (uint32_t blk = walk.first; blk < walk.end; blk += walk.stride) {
         map.seek(rows, blk, ti, t, t_end);
         const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
-        full_block<BF16, MODE, EXACT, WD, GS, KEYTAB>(t, blk - t.full_start, lane, h, gscale, dbc1, dbc2, L);
+        full_block<BF16, MODE, EXACT, WD, GS, KEYTAB, GBF16>(t, blk - t.full_start, lane, h, gscale, dbc1, dbc2, L);
     }
 }
 
@@ -69,10 +70,10 @@ namespace {
 
 constexpr bool kBf16 = ERI_PLAIN_BF16 != 0;
 
-template <int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB>
+template <int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB, bool GBF16>
 int launch_one(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
                const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg, hipStream_t s) {
-    auto k = adam8_step_kernel<kBf16, MODE, EXACT, WD, GS, KEYTAB>;
+    auto k = adam8_step_kernel<kBf16, MODE, EXACT, WD, GS, KEYTAB, GBF16>;
     if (wg > plain_threads(MODE)) wg = plain_threads(MODE);
     hipLaunchKernelGGL(k, dim3(grid), dim3(wg), 0, s, rows, n_rows, total_blocks, h,
                        static_cast<const uint4 *>(lds_image), dev_scale, chunks_for(grid));
@@ -80,10 +81,10 @@ int launch_one(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, co
 }
 
 /* BSEARCH selects the cross-check variants (binary search of the midpoint table); mode BNB has none. */
-template <int MODE, bool EXACT, bool BSEARCH>
+template <int MODE, bool EXACT, bool BSEARCH, bool GBF16 = kBf16>
 int launch_flags(bool wd, bool gs, bool keytab, const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks,
                  const EriAdam8Hyper &h, const void *img, const float *dev_scale, uint32_t grid, uint32_t wg, hipStream_t s) {
-#define ERI_GO(W, G, K) return launch_one<MODE, EXACT, W, G, K>(rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s)
+#define ERI_GO(W, G, K) return launch_one<MODE, EXACT, W, G, K, GBF16>(rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s)
     if (BSEARCH && !keytab) {
         if (wd) { if (gs) ERI_GO(true, true, !BSEARCH); ERI_GO(true, false, !BSEARCH); }
         if (gs) ERI_GO(false, true, !BSEARCH);
@@ -98,11 +99,20 @@ int launch_flags(bool wd, bool gs, bool keytab, const DevTensor *rows, uint32_t 
 } // namespace
 
 #if ERI_PLAIN_BF16
-int launch_step_plain_bf16(int mode, bool exact, bool wd, bool gs, bool keytab, const DevTensor *rows, uint32_t n_rows,
-                           uint32_t total_blocks, const EriAdam8Hyper &h, const void *img, const float *dev_scale,
-                           uint32_t grid, uint32_t wg, void *stream) {
+int launch_step_plain_bf16(int mode, bool exact, bool wd, bool gs, bool keytab, bool grad_f32, const DevTensor *rows,
+                           uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h, const void *img,
+                           const float *dev_scale, uint32_t grid, uint32_t wg, void *stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define ERI_ARGS wd, gs, keytab, rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s
+    if (grad_f32) { // fp32 gradients for bf16 parameters: slot-table variants only
+        if (!keytab) return (int)hipErrorInvalidValue;
+        if (mode == ERI_ADAM8_MODE_BNB)
+            return exact ? launch_flags<ERI_ADAM8_MODE_BNB, true, false, false>(ERI_ARGS)
+                         : launch_flags<ERI_ADAM8_MODE_BNB, false, false, false>(ERI_ARGS);
+        if (mode == ERI_ADAM8_MODE_L2) return launch_flags<ERI_ADAM8_MODE_L2, true, false, false>(ERI_ARGS);
+        return exact ? launch_flags<ERI_ADAM8_MODE_ERI, true, false, false>(ERI_ARGS)
+                     : launch_flags<ERI_ADAM8_MODE_ERI, false, false, false>(ERI_ARGS);
+    }
     if (mode == ERI_ADAM8_MODE_BNB)
         return exact ? launch_flags<ERI_ADAM8_MODE_BNB, true, false>(ERI_ARGS) : launch_flags<ERI_ADAM8_MODE_BNB, false, false>(ERI_ARGS);
     if (mode == ERI_ADAM8_MODE_L2) return launch_flags<ERI_ADAM8_MODE_L2, true, true>(ERI_ARGS); // always the IEEE chain

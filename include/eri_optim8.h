@@ -104,21 +104,24 @@ enum {
                                              instead of the float-keyed slot table (same codes; runs on
                                              the plain one-wave-per-block kernel whatever the table size) */
     ERI_ADAM8_FLAG_NO_PIPELINE = 1u << 3, /* use the plain one-wave-per-block kernel: not the one that
-                                             prefetches the next block (BF16), not the four-waves-per-
-                                             block one (small tables).  Same results; a cross-check */
+                                             prefetches the next block (large BF16 tables), not the
+                                             four-waves-per-block one (small tables).  Same results; a
+                                             cross-check */
     ERI_ADAM8_FLAG_CLIP_FROM_TABLE = 1u << 4, /* also multiply gradients by the clip factor the last
                                              eri_adam8_grad_norm left in the table (device memory) */
     ERI_ADAM8_FLAG_EMA = 1u << 6,         /* after the update, every row that has an ema_shadow also gets
                                              shadow = ema_decay*shadow + (1 - ema_decay)*p', the EMA update of
                                              src/trainers/ema_enhanced.rs:91-100 on the parameter as it was just
-                                             stored.  Large BF16 tables in mode ERI do it inside the step kernel
-                                             (the new parameter is still in registers: the separate sweep's read
-                                             of p is saved); every other table runs the EMA sweep right after
-                                             the step, in the same call.  Same results either way */
-    ERI_ADAM8_FLAG_ONE_WAVE = 1u << 5     /* never take the four-waves-per-block kernel, which small and F32
-                                             tables get by default: a small BF16 table then runs on the
-                                             prefetching kernel.  Same results; lets tests reach every
-                                             kernel with small inputs */
+                                             stored.  BF16 tables in mode ERI beyond the small-table kernel's
+                                             range do it inside the step kernel (the new parameter is still in
+                                             registers: the separate sweep's read of p is saved); every other
+                                             table runs the EMA sweep right after the step, in the same call.
+                                             Same results either way */
+    ERI_ADAM8_FLAG_ONE_WAVE = 1u << 5     /* take the kernels of the largest tables whatever the size: the
+                                             prefetching kernel for BF16 parameters with BF16 gradients, the
+                                             plain one-wave-per-block kernel for F32 parameters and for F32
+                                             gradients.  Same results; lets tests reach every kernel with
+                                             small inputs */
 };
 
 /* Per-step scalars, already cast where the reference casts them.  Fill with eri_adam8_hyper_pack. */
