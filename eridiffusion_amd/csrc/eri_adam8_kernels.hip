@@ -47,6 +47,9 @@ int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, i
     }
     if (mixed) {
         const bool wd_m = h.mode == ERI_ADAM8_MODE_BNB ? h.weight_decay != 1.0f : h.weight_decay > 0.0f;
+        if (h.mode != ERI_ADAM8_MODE_L2 && (h.flags & ERI_ADAM8_FLAG_NO_PIPELINE) == 0 && prefetch_pays(total_blocks, h, compute_units))
+            return launch_step_pipelined_grad_f32(h.mode, (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0, wd_m, gs, rows, n_rows,
+                                                  total_blocks, h, lds_image, dev_scale, grid, wg, stream);
         return launch_step_plain_bf16(h.mode, (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0, wd_m, gs, true, true, rows, n_rows,
                                       total_blocks, h, lds_image, dev_scale, grid, wg, stream);
     }

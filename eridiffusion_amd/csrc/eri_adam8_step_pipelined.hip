@@ -1,7 +1,15 @@
-/* The software-pipelined step kernel for bf16 tensors: the benchmark kernel. */
+/* The software-pipelined step kernel for bf16 parameters: the benchmark kernel.  Compiled twice, once per
+ * gradient dtype (-DERI_PIPE_GRAD_BF16=1: bf16 gradients, 0: fp32 gradients), so that the two halves build
+ * in parallel. */
 #include "eri_adam8_inline.h"
 
+#ifndef ERI_PIPE_GRAD_BF16
+#error "compile with -DERI_PIPE_GRAD_BF16=0 or 1"
+#endif
+
 namespace eri {
+
+constexpr bool kGradBf16 = ERI_PIPE_GRAD_BF16 != 0;
 
 // ------------------------------------------------------------------------------------------
 // software-pipelined step kernel for bf16 tensors
@@ -11,7 +19,17 @@ namespace eri {
 // the requantisation half, so it always has 48 bytes per lane in flight while it computes.  The
 // registers of the raw words are the ones just freed, so the pipeline costs no copies; it needs
 // 48 (raw) + 64 (moments) + temporaries at its peak, hence three waves per SIMD (768 threads).
+// With fp32 gradients the raw words of a block are 64 registers, which no longer fits beside the
+// moments in the 170 registers of three waves per SIMD: that instantiation runs two waves per SIMD
+// (512 threads), each with 24 KB of its next block in flight.
 // ------------------------------------------------------------------------------------------
+
+constexpr uint32_t kPipeThreads = kGradBf16 ? 768 : 512;
+#if ERI_PIPE_GRAD_BF16
+#define ERI_PIPE_KERNEL adam8_step_pipelined_kernel
+#else
+#define ERI_PIPE_KERNEL adam8_step_pipelined_grad_f32_kernel
+#endif
 
 /* One lane's eight shadow values of one quarter block: shadow = d*shadow + (1-d)*p', each operation rounded
  * on its own, the result rounded to bf16. */
@@ -34,19 +52,27 @@ __device__ __forceinline__ void ema_quarter(void *shadow, size_t e0, int c, uint
 }
 
 struct RawBlock {
-    u32x4 p[4], g[4];
+    u32x4 p[4];
+    u32x4 g[kGradBf16 ? 4 : 8]; // bf16: one word per quarter block; fp32: two (elements 8*lane .. +3 and +4 .. +7)
     u32x2 m[4], v[4];
     float a_m, a_v;
     __device__ __forceinline__ void issue(const DevTensor &t, uint32_t lb, uint32_t lane) {
         const size_t e0 = (size_t)lb * kBlock;
         ERI_GLOBAL const u32x4 *pp = as_global(reinterpret_cast<const u32x4 *>(static_cast<const uint16_t *>(t.p_in) + e0));
-        ERI_GLOBAL const u32x4 *gp = as_global(reinterpret_cast<const u32x4 *>(static_cast<const uint16_t *>(t.g) + e0));
+        ERI_GLOBAL const u32x4 *gp = as_global(reinterpret_cast<const u32x4 *>(static_cast<const char *>(t.g) + e0 * (kGradBf16 ? 2 : 4)));
         ERI_GLOBAL const u32x2 *mp = as_global(reinterpret_cast<const u32x2 *>(t.m + e0));
         ERI_GLOBAL const u32x2 *vp = as_global(reinterpret_cast<const u32x2 *>(t.v + e0));
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             p[c] = __builtin_nontemporal_load(&pp[c * 64 + lane]); // each byte is touched once per step
-            g[c] = __builtin_nontemporal_load(&gp[c * 64 + lane]);
+            if (kGradBf16) {
+                g[c] = __builtin_nontemporal_load(&gp[c * 64 + lane]);
+            } else {
+                // a lane's two words share cache lines with its neighbours' across the two instructions, so
+                // these stay ordinary loads: streamed, the second instruction would fetch every line again
+                g[2 * c] = gp[c * 128 + 2 * lane];
+                g[2 * c + 1] = gp[c * 128 + 2 * lane + 1];
+            }
             m[c] = __builtin_nontemporal_load(&mp[c * 64 + lane]);
             v[c] = __builtin_nontemporal_load(&vp[c * 64 + lane]);
         }
@@ -58,7 +84,7 @@ struct RawBlock {
 /* EMA: rows that carry a shadow also get shadow = d*shadow + (1-d)*p' (src/trainers/ema_enhanced.rs:91-100),
  * p' being the parameter as it is stored (rounded to bf16). */
 template <int MODE, bool EXACT, bool WD, bool GS, bool EMA>
-__global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTensor *__restrict__ rows,
+__global__ __launch_bounds__(kPipeThreads) void ERI_PIPE_KERNEL(const DevTensor *__restrict__ rows,
                                                                    uint32_t n_rows, uint32_t total_blocks,
                                                                    EriAdam8Hyper h,
                                                                    const uint4 *__restrict__ lds_image,
@@ -99,7 +125,7 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
         const uint32_t n = (uint32_t)(t.numel % kBlock);
         if (n != 0) {
             const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
-            tail_block<true, MODE, EXACT, WD, GS, true>(t, (uint32_t)(t.numel / kBlock), n, lane, h, gscale, dbc1, dbc2, L);
+            tail_block<true, MODE, EXACT, WD, GS, true, kGradBf16>(t, (uint32_t)(t.numel / kBlock), n, lane, h, gscale, dbc1, dbc2, L);
             if (EMA && t.shadow != nullptr) { // the partial block's shadow, element by element, from the parameters just stored
                 const size_t e0 = (size_t)(t.numel / kBlock) * kBlock;
                 const float omd = 1.0f - h.ema_decay;
@@ -163,12 +189,19 @@ __global__ __launch_bounds__(768) void adam8_step_pipelined_kernel(const DevTens
         bool cancel = false;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            Raw8<true> pr, gr;
+            Raw8<true> pr;
             pr.w = raw.p[c];
-            gr.w = raw.g[c];
             float pv[8], gv[8], pn[8];
             pr.unpack(pv);
-            gr.unpack(gv);
+            if (kGradBf16) {
+                Raw8<true> gr;
+                gr.w = raw.g[c];
+                gr.unpack(gv);
+            } else {
+                const u32x4 ga = raw.g[kGradBf16 ? c : 2 * c], gb = raw.g[kGradBf16 ? c : 2 * c + 1];
+                gv[0] = u2f(ga.x); gv[1] = u2f(ga.y); gv[2] = u2f(ga.z); gv[3] = u2f(ga.w);
+                gv[4] = u2f(gb.x); gv[5] = u2f(gb.y); gv[6] = u2f(gb.z); gv[7] = u2f(gb.w);
+            }
             bool redo = false; // EMA: flagged elements are put right quarter by quarter, before the shadow uses them
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
@@ -246,8 +279,8 @@ namespace {
 template <int MODE, bool EXACT, bool WD, bool GS, bool EMA = false>
 int launch_pipelined(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
                      const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg, hipStream_t s) {
-    if (wg > 768) wg = 768;
-    hipLaunchKernelGGL((adam8_step_pipelined_kernel<MODE, EXACT, WD, GS, EMA>), dim3(grid), dim3(wg), 0, s, rows, n_rows, total_blocks, h,
+    if (wg > kPipeThreads) wg = kPipeThreads;
+    hipLaunchKernelGGL((ERI_PIPE_KERNEL<MODE, EXACT, WD, GS, EMA>), dim3(grid), dim3(wg), 0, s, rows, n_rows, total_blocks, h,
                        static_cast<const uint4 *>(lds_image), dev_scale, chunks_for(grid));
     return (int)hipGetLastError();
 }
@@ -255,7 +288,7 @@ int launch_pipelined(const DevTensor *rows, uint32_t n_rows, uint32_t total_bloc
 template <int MODE, bool EXACT>
 int launch_flags(bool wd, bool gs, bool ema, const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
                  const void *img, const float *dev_scale, uint32_t grid, uint32_t wg, hipStream_t s) {
-    if constexpr (MODE == ERI_ADAM8_MODE_ERI) { // the EMA is built into the reference's own update only
+    if constexpr (MODE == ERI_ADAM8_MODE_ERI && kGradBf16) { // the EMA is built into the reference's own update only
         if (ema) {
             if (wd) {
                 if (gs) return launch_pipelined<MODE, EXACT, true, true, true>(rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s);
@@ -278,9 +311,16 @@ int launch_flags(bool wd, bool gs, bool ema, const DevTensor *rows, uint32_t n_r
 /* Modes ERI and BNB.  The coupled-decay mode needs more live values per element than this kernel's
  * register budget holds (its instantiations spilled 80-232 B per lane) and runs faster on the kernel
  * without the prefetch; the dispatcher sends it there. */
+#if ERI_PIPE_GRAD_BF16
 int launch_step_pipelined(int mode, bool exact, bool wd, bool gs, bool ema, const DevTensor *rows, uint32_t n_rows,
                           uint32_t total_blocks, const EriAdam8Hyper &h, const void *img, const float *dev_scale,
                           uint32_t grid, uint32_t wg, void *stream) {
+#else
+int launch_step_pipelined_grad_f32(int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
+                                   uint32_t total_blocks, const EriAdam8Hyper &h, const void *img,
+                                   const float *dev_scale, uint32_t grid, uint32_t wg, void *stream) {
+    const bool ema = false; // rows with fp32 gradients get their EMA from the sweep
+#endif
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define ERI_ARGS wd, gs, ema, rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s
     if (mode == ERI_ADAM8_MODE_BNB)

@@ -195,18 +195,18 @@ def test_rows_that_write_to_another_tensor(mode, flags_name):
     assert L.lib().eri_adam8_table_create(rows, len(rows), None, C.byref(table)) == -6
 
 
-@pytest.mark.parametrize("kernels", ["default-kernels", "one-wave"])
+@pytest.mark.parametrize("kernels", ["default-kernels", "one-wave", "plain"])
 @pytest.mark.parametrize("mode,flags", [(0, 2), (0, 0), (1, 2), (2, 2), (2, 0)])
 def test_f32_gradients_for_bf16_parameters_in_a_mixed_table(mode, flags, kernels):
     """One table with all three layouts -- F32, BF16, and BF16 parameters with F32 gradients -- ragged sizes,
     three steps.  The F32 gradients are not representable in BF16 (their low mantissa bits are set), so a
     kernel that rounded them first would produce other moments than the oracle, which uses them as they are
     (the reference casts gradients to F32 and never rounds them, adam8bit_enhanced.rs:231-235).  Small tables
-    take the four-waves-per-block kernel; "one-wave" runs the kernels that large tables take."""
+    take the four-waves-per-block kernel; "one-wave" runs the kernels that the largest tables take (with the
+    next block's loads in flight), "plain" the one-wave kernel without them, which mid-size tables take."""
     import torch
     L = _L()
-    if kernels == "one-wave":
-        flags |= L.FLAG_ONE_WAVE
+    flags |= {"default-kernels": 0, "one-wave": L.FLAG_ONE_WAVE, "plain": L.FLAG_NO_PIPELINE}[kernels]
     sizes = [2048 * 4 + 12, 2048 * 3, 100, 2048 * 9 + 1, 640 * 16, 2048 * 2 + 1023, 5]
     p_tags = [2, 0, 2, 2, 0, 2, 2]
     g_tags = [0, 0, 0, 2, 0, 0, 2]  # rows 0, 2, 5: BF16 parameters with F32 gradients
