@@ -114,6 +114,10 @@ int launch_step_pipelined(int mode, bool exact, bool wd, bool gs, bool ema, cons
 int launch_step_pipelined_grad_f32(int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
                                    uint32_t total_blocks, const EriAdam8Hyper &h, const void *lds_image,
                                    const float *dev_scale, uint32_t grid, uint32_t wg, void *stream);
+/* The same kernel for fp32 parameters (IEEE chain throughout, no EMA inside it). */
+int launch_step_pipelined_f32(int mode, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks,
+                              const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale, uint32_t grid,
+                              uint32_t wg, void *stream);
 /* Sum of |moment - dequantised moment| of the coming step, per row: err[2r] first moment, err[2r+1] second. */
 int launch_quant_error(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_blocks, int layout,
                        const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale, double *err,

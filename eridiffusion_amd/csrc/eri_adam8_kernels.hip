@@ -59,11 +59,15 @@ int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, i
         if (bf16 && !kernel_named && prefetch_pays(total_blocks, h, compute_units))
             return launch_step_pipelined(h.mode, exact, wd, gs, false, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
         if (bf16) return launch_step_plain_bf16(h.mode, exact, wd, gs, true, false, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
+        if (!kernel_named && prefetch_pays(total_blocks, h, compute_units))
+            return launch_step_pipelined_f32(h.mode, wd, gs, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
         return launch_step_plain_f32(h.mode, wd, gs, true, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
     }
     const bool wd = h.weight_decay > 0.0f;
     const bool exact = (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0;
     const bool keytab = (h.flags & ERI_ADAM8_FLAG_BSEARCH) == 0;
+    if (!bf16 && !kernel_named && h.mode == ERI_ADAM8_MODE_ERI && prefetch_pays(total_blocks, h, compute_units))
+        return launch_step_pipelined_f32(h.mode, wd, gs, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
     if (!bf16) return launch_step_plain_f32(h.mode, wd, gs, keytab, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
     if (keytab && h.mode == ERI_ADAM8_MODE_ERI && (h.flags & ERI_ADAM8_FLAG_NO_PIPELINE) == 0 &&
         prefetch_pays(total_blocks, h, compute_units))

@@ -1,15 +1,17 @@
-/* The software-pipelined step kernel for bf16 parameters: the benchmark kernel.  Compiled twice, once per
- * gradient dtype (-DERI_PIPE_GRAD_BF16=1: bf16 gradients, 0: fp32 gradients), so that the two halves build
- * in parallel. */
+/* The software-pipelined step kernel: the benchmark kernel.  Compiled three times, once per layout of the
+ * rows (-DERI_PIPE_LAYOUT=1: bf16 parameters and gradients, 2: bf16 parameters with fp32 gradients, 0: fp32
+ * parameters and gradients), so that the three build in parallel. */
 #include "eri_adam8_inline.h"
 
-#ifndef ERI_PIPE_GRAD_BF16
-#error "compile with -DERI_PIPE_GRAD_BF16=0 or 1"
+#if !defined(ERI_PIPE_LAYOUT) || ERI_PIPE_LAYOUT < 0 || ERI_PIPE_LAYOUT > 2
+#error "compile with -DERI_PIPE_LAYOUT=0, 1 or 2"
 #endif
 
 namespace eri {
 
-constexpr bool kGradBf16 = ERI_PIPE_GRAD_BF16 != 0;
+static_assert(kLayoutF32 == 0 && kLayoutBF16 == 1 && kLayoutBF16GradF32 == 2, "ERI_PIPE_LAYOUT names a Layout");
+constexpr bool kParamBf16 = ERI_PIPE_LAYOUT != kLayoutF32;
+constexpr bool kGradBf16 = ERI_PIPE_LAYOUT == kLayoutBF16;
 
 // ------------------------------------------------------------------------------------------
 // software-pipelined step kernel for bf16 tensors
@@ -19,16 +21,18 @@ constexpr bool kGradBf16 = ERI_PIPE_GRAD_BF16 != 0;
 // the requantisation half, so it always has 48 bytes per lane in flight while it computes.  The
 // registers of the raw words are the ones just freed, so the pipeline costs no copies; it needs
 // 48 (raw) + 64 (moments) + temporaries at its peak, hence three waves per SIMD (768 threads).
-// With fp32 gradients the raw words of a block are 64 registers, which no longer fits beside the
-// moments in the 170 registers of three waves per SIMD: that instantiation runs two waves per SIMD
-// (512 threads), each with 24 KB of its next block in flight.
+// With fp32 gradients the raw words of a block are 64 registers, with fp32 parameters too 80, which no
+// longer fits beside the moments in the 170 registers of three waves per SIMD: those instantiations run
+// two waves per SIMD (512 threads), each with 24 or 20 KB of its next block in flight.
 // ------------------------------------------------------------------------------------------
 
 constexpr uint32_t kPipeThreads = kGradBf16 ? 768 : 512;
-#if ERI_PIPE_GRAD_BF16
+#if ERI_PIPE_LAYOUT == 1
 #define ERI_PIPE_KERNEL adam8_step_pipelined_kernel
-#else
+#elif ERI_PIPE_LAYOUT == 2
 #define ERI_PIPE_KERNEL adam8_step_pipelined_grad_f32_kernel
+#else
+#define ERI_PIPE_KERNEL adam8_step_pipelined_f32_kernel
 #endif
 
 /* One lane's eight shadow values of one quarter block: shadow = d*shadow + (1-d)*p', each operation rounded
@@ -52,19 +56,24 @@ __device__ __forceinline__ void ema_quarter(void *shadow, size_t e0, int c, uint
 }
 
 struct RawBlock {
-    u32x4 p[4];
-    u32x4 g[kGradBf16 ? 4 : 8]; // bf16: one word per quarter block; fp32: two (elements 8*lane .. +3 and +4 .. +7)
+    u32x4 p[kParamBf16 ? 4 : 8]; // bf16: one word per quarter block; fp32: two (elements 8*lane .. +3 and +4 .. +7)
+    u32x4 g[kGradBf16 ? 4 : 8];
     u32x2 m[4], v[4];
     float a_m, a_v;
     __device__ __forceinline__ void issue(const DevTensor &t, uint32_t lb, uint32_t lane) {
         const size_t e0 = (size_t)lb * kBlock;
-        ERI_GLOBAL const u32x4 *pp = as_global(reinterpret_cast<const u32x4 *>(static_cast<const uint16_t *>(t.p_in) + e0));
+        ERI_GLOBAL const u32x4 *pp = as_global(reinterpret_cast<const u32x4 *>(static_cast<const char *>(t.p_in) + e0 * (kParamBf16 ? 2 : 4)));
         ERI_GLOBAL const u32x4 *gp = as_global(reinterpret_cast<const u32x4 *>(static_cast<const char *>(t.g) + e0 * (kGradBf16 ? 2 : 4)));
         ERI_GLOBAL const u32x2 *mp = as_global(reinterpret_cast<const u32x2 *>(t.m + e0));
         ERI_GLOBAL const u32x2 *vp = as_global(reinterpret_cast<const u32x2 *>(t.v + e0));
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            p[c] = __builtin_nontemporal_load(&pp[c * 64 + lane]); // each byte is touched once per step
+            if (kParamBf16) {
+                p[c] = __builtin_nontemporal_load(&pp[c * 64 + lane]); // each byte is touched once per step
+            } else {
+                p[2 * c] = pp[c * 128 + 2 * lane];
+                p[2 * c + 1] = pp[c * 128 + 2 * lane + 1];
+            }
             if (kGradBf16) {
                 g[c] = __builtin_nontemporal_load(&gp[c * 64 + lane]);
             } else {
@@ -125,7 +134,7 @@ __global__ __launch_bounds__(kPipeThreads) void ERI_PIPE_KERNEL(const DevTensor 
         const uint32_t n = (uint32_t)(t.numel % kBlock);
         if (n != 0) {
             const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
-            tail_block<true, MODE, EXACT, WD, GS, true, kGradBf16>(t, (uint32_t)(t.numel / kBlock), n, lane, h, gscale, dbc1, dbc2, L);
+            tail_block<kParamBf16, MODE, EXACT, WD, GS, true, kGradBf16>(t, (uint32_t)(t.numel / kBlock), n, lane, h, gscale, dbc1, dbc2, L);
             if (EMA && t.shadow != nullptr) { // the partial block's shadow, element by element, from the parameters just stored
                 const size_t e0 = (size_t)(t.numel / kBlock) * kBlock;
                 const float omd = 1.0f - h.ema_decay;
@@ -160,7 +169,7 @@ __global__ __launch_bounds__(kPipeThreads) void ERI_PIPE_KERNEL(const DevTensor 
         const uint32_t lb = blk - t.full_start;
         const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
         const size_t e0 = (size_t)lb * kBlock;
-        char *p = static_cast<char *>(t.p) + e0 * 2;
+        char *p = static_cast<char *>(t.p) + e0 * (kParamBf16 ? 2 : 4);
         uint8_t *mc = t.m + e0;
         uint8_t *vc = t.v + e0;
         float mf[32], vf[32];
@@ -189,10 +198,16 @@ __global__ __launch_bounds__(kPipeThreads) void ERI_PIPE_KERNEL(const DevTensor 
         bool cancel = false;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            Raw8<true> pr;
-            pr.w = raw.p[c];
             float pv[8], gv[8], pn[8];
-            pr.unpack(pv);
+            if (kParamBf16) {
+                Raw8<true> pr;
+                pr.w = raw.p[c];
+                pr.unpack(pv);
+            } else {
+                const u32x4 pa = raw.p[kParamBf16 ? c : 2 * c], pb = raw.p[kParamBf16 ? c : 2 * c + 1];
+                pv[0] = u2f(pa.x); pv[1] = u2f(pa.y); pv[2] = u2f(pa.z); pv[3] = u2f(pa.w);
+                pv[4] = u2f(pb.x); pv[5] = u2f(pb.y); pv[6] = u2f(pb.z); pv[7] = u2f(pb.w);
+            }
             if (kGradBf16) {
                 Raw8<true> gr;
                 gr.w = raw.g[c];
@@ -208,7 +223,7 @@ __global__ __launch_bounds__(kPipeThreads) void ERI_PIPE_KERNEL(const DevTensor 
                 const float t1 = lds_float_at(mine[0], code_offset(raw.m[c], k));
                 const float t3 = lds_float_at(mine[1], code_offset(raw.v[c], k));
                 float m, v;
-                adam_elem_decayed<MODE, EXACT, true, WD, GS>(pv[k], gv[k], t1, t3, h, gscale, dbc1, dbc2, m, v, pn[k], EMA ? redo : cancel);
+                adam_elem_decayed<MODE, EXACT, kParamBf16, WD, GS>(pv[k], gv[k], t1, t3, h, gscale, dbc1, dbc2, m, v, pn[k], EMA ? redo : cancel);
                 mf[c * 8 + k] = m;
                 vf[c * 8 + k] = v;
                 lm = fmaxf(lm, __builtin_fabsf(m));
@@ -218,13 +233,17 @@ __global__ __launch_bounds__(kPipeThreads) void ERI_PIPE_KERNEL(const DevTensor 
 #pragma unroll
                 for (int k = 0; k < 8; ++k) pn[k] = param_exact<MODE, WD, true>(pv[k], mf[c * 8 + k], vf[c * 8 + k], h, dbc1, dbc2);
             }
-            pw[c].x = bf16_pair(pn[0], pn[1]);
-            pw[c].y = bf16_pair(pn[2], pn[3]);
-            pw[c].z = bf16_pair(pn[4], pn[5]);
-            pw[c].w = bf16_pair(pn[6], pn[7]);
+            if (kParamBf16) {
+                pw[c].x = bf16_pair(pn[0], pn[1]);
+                pw[c].y = bf16_pair(pn[2], pn[3]);
+                pw[c].z = bf16_pair(pn[4], pn[5]);
+                pw[c].w = bf16_pair(pn[6], pn[7]);
+            } else { // fp32 parameters are final here (they take the exact chain): stored quarter by quarter
+                store8<false>(p, c * 512 + lane * 8, pn);
+            }
             if (EMA && with_shadow) ema_quarter(t.shadow, e0, c, lane, sh[c], pw[c], h.ema_decay);
         }
-        if (cancel) { // rare: a lane whose update cancelled redoes its 32 parameters with the exact chain
+        if (kParamBf16 && cancel) { // rare: a lane whose update cancelled redoes its 32 parameters with the exact chain
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 Raw8<true> pr;
@@ -246,9 +265,11 @@ __global__ __launch_bounds__(kPipeThreads) void ERI_PIPE_KERNEL(const DevTensor 
             as_global(t.absmax_v)[lb] = nav;
         }
         raw.issue(nt, pblk - nt.full_start, lane); // prefetch: in flight during the requantisation
+        if (kParamBf16) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c)
-            __builtin_nontemporal_store(pw[c], as_global(reinterpret_cast<u32x4 *>(p) + c * 64 + lane));
+            for (int c = 0; c < 4; ++c)
+                __builtin_nontemporal_store(pw[c], as_global(reinterpret_cast<u32x4 *>(p) + c * 64 + lane));
+        }
         const BlockDiv dm(nam, kKeyScale, kKeyScaleInv), dv(nav, kKeyScale, kKeyScaleInv);
         if (dm.fast && dv.fast) {
 #pragma unroll
@@ -288,7 +309,7 @@ int launch_pipelined(const DevTensor *rows, uint32_t n_rows, uint32_t total_bloc
 template <int MODE, bool EXACT>
 int launch_flags(bool wd, bool gs, bool ema, const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
                  const void *img, const float *dev_scale, uint32_t grid, uint32_t wg, hipStream_t s) {
-    if constexpr (MODE == ERI_ADAM8_MODE_ERI && kGradBf16) { // the EMA is built into the reference's own update only
+    if constexpr (MODE == ERI_ADAM8_MODE_ERI && kGradBf16) { // (which implies bf16 parameters) // the EMA is built into the reference's own update only
         if (ema) {
             if (wd) {
                 if (gs) return launch_pipelined<MODE, EXACT, true, true, true>(rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s);
@@ -311,21 +332,32 @@ int launch_flags(bool wd, bool gs, bool ema, const DevTensor *rows, uint32_t n_r
 /* Modes ERI and BNB.  The coupled-decay mode needs more live values per element than this kernel's
  * register budget holds (its instantiations spilled 80-232 B per lane) and runs faster on the kernel
  * without the prefetch; the dispatcher sends it there. */
-#if ERI_PIPE_GRAD_BF16
+#if ERI_PIPE_LAYOUT == 1
 int launch_step_pipelined(int mode, bool exact, bool wd, bool gs, bool ema, const DevTensor *rows, uint32_t n_rows,
                           uint32_t total_blocks, const EriAdam8Hyper &h, const void *img, const float *dev_scale,
                           uint32_t grid, uint32_t wg, void *stream) {
-#else
+#elif ERI_PIPE_LAYOUT == 2
 int launch_step_pipelined_grad_f32(int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
                                    uint32_t total_blocks, const EriAdam8Hyper &h, const void *img,
                                    const float *dev_scale, uint32_t grid, uint32_t wg, void *stream) {
     const bool ema = false; // rows with fp32 gradients get their EMA from the sweep
+#else
+int launch_step_pipelined_f32(int mode, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks,
+                              const EriAdam8Hyper &h, const void *img, const float *dev_scale, uint32_t grid,
+                              uint32_t wg, void *stream) {
+    const bool ema = false;   // fp32 rows get their EMA from the sweep
+    constexpr bool exact = true; // fp32 parameters always take the IEEE square root and division
 #endif
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define ERI_ARGS wd, gs, ema, rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s
+#if ERI_PIPE_LAYOUT == 0
+    if (mode == ERI_ADAM8_MODE_BNB) return launch_flags<ERI_ADAM8_MODE_BNB, exact>(ERI_ARGS);
+    return launch_flags<ERI_ADAM8_MODE_ERI, exact>(ERI_ARGS);
+#else
     if (mode == ERI_ADAM8_MODE_BNB)
         return exact ? launch_flags<ERI_ADAM8_MODE_BNB, true>(ERI_ARGS) : launch_flags<ERI_ADAM8_MODE_BNB, false>(ERI_ARGS);
     return exact ? launch_flags<ERI_ADAM8_MODE_ERI, true>(ERI_ARGS) : launch_flags<ERI_ADAM8_MODE_ERI, false>(ERI_ARGS);
+#endif
 #undef ERI_ARGS
 }
 

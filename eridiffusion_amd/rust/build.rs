@@ -33,8 +33,9 @@ fn main() {
     for (file, obj_name, define, is_hip) in [
         ("eri_adam8_kernels.hip", "kernels", "", true),
         ("eri_adam8_step_split.hip", "step_split", "", true),
-        ("eri_adam8_step_pipelined.hip", "step_pipelined", "-DERI_PIPE_GRAD_BF16=1", true),
-        ("eri_adam8_step_pipelined.hip", "step_pipelined_grad_f32", "-DERI_PIPE_GRAD_BF16=0", true),
+        ("eri_adam8_step_pipelined.hip", "step_pipelined", "-DERI_PIPE_LAYOUT=1", true),
+        ("eri_adam8_step_pipelined.hip", "step_pipelined_grad_f32", "-DERI_PIPE_LAYOUT=2", true),
+        ("eri_adam8_step_pipelined.hip", "step_pipelined_f32", "-DERI_PIPE_LAYOUT=0", true),
         ("eri_adam8_step_plain.hip", "step_plain_bf16", "-DERI_PLAIN_BF16=1", true),
         ("eri_adam8_step_plain.hip", "step_plain_f32", "-DERI_PLAIN_BF16=0", true),
         ("eri_optim8_api.cpp", "api", "", true),

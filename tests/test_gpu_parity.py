@@ -19,13 +19,15 @@ pytestmark = pytest.mark.gpu
 LR, B1, B2, EPS, WD = 1e-4, 0.9, 0.999, 1e-8, 0.01
 
 
-@pytest.fixture(autouse=True, params=["split-kernel-for-small-tables", "one-wave-per-block-kernels"])
+@pytest.fixture(autouse=True, params=["split-kernel-for-small-tables", "prefetching-kernels", "plain-kernels"])
 def which_kernels(request):
     """The tables of these tests are small, so by default they all run on the four-waves-per-block kernel.
-    Every test therefore runs twice: as shipped, and with that kernel switched off, which sends bf16 tables
-    to the pipelined kernel and fp32 tables to the plain one."""
+    Every test therefore runs three times: as shipped, on the one-wave-per-block kernels that prefetch the
+    next block (what the largest tables take), and on the one-wave kernels without the prefetch (mid-size
+    tables)."""
     global KERNEL_FLAGS
-    KERNEL_FLAGS = 0 if request.param.startswith("split") else _lib().FLAG_ONE_WAVE
+    L = _lib()
+    KERNEL_FLAGS = {"split": 0, "prefe": L.FLAG_ONE_WAVE, "plain": L.FLAG_NO_PIPELINE}[request.param[:5]]
     yield request.param
     KERNEL_FLAGS = 0
 
