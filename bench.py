@@ -324,8 +324,11 @@ def main():
         try:
             with open(args.traffic_json) as f:
                 key = "%s|%s|flags=%d" % (args.config, args.kernel, args.flags)
-                plain = args.api == "table" and args.mode == "eri" and args.param_dtype == "config" and not grad_f32
-                traffic = json.load(f).get(key) if plain else None
+                if args.param_dtype != "config" and args.param_dtype != W.CONFIGS[args.config][1]:
+                    key += "|param=" + args.param_dtype
+                if grad_f32:
+                    key += "|grad=f32"
+                traffic = json.load(f).get(key) if args.api == "table" and args.mode == "eri" else None
         except Exception:
             traffic = None
     out = {
