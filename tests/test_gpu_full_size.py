@@ -29,7 +29,19 @@ def test_sdxl_unet_full_size_sampled_blocks_and_block_properties():
     _full_size(W.c4_sdxl_full(), 0xE21D + 4, 2_567_463_684, 1_254_022, 20e9)
 
 
-def _full_size(tensors, seed, want_numel, want_blocks, need_bytes):
+def test_sdxl_unet_full_size_with_f32_gradients_for_bf16_parameters():
+    """The same table with the gradients left in F32 (what the reference's upcast amounts to when autograd
+    hands back F32 gradients): the prefetching kernel's two-waves-per-SIMD variant at its real size."""
+    from eridiffusion_amd import workloads as W
+    _full_size(W.c4_sdxl_full(), 0xE21D + 41, 2_567_463_684, 1_254_022, 26e9, layout="bf16_grad_f32")
+
+
+def test_sdxl_unet_full_size_with_f32_parameters():
+    from eridiffusion_amd import workloads as W
+    _full_size(W.c4_sdxl_full(), 0xE21D + 42, 2_567_463_684, 1_254_022, 32e9, layout="f32")
+
+
+def _full_size(tensors, seed, want_numel, want_blocks, need_bytes, layout="bf16"):
     import torch
     from eridiffusion_amd import _lib as L
     from eridiffusion_amd import workloads as W
@@ -42,6 +54,13 @@ def _full_size(tensors, seed, want_numel, want_blocks, need_bytes):
     gen = torch.Generator(device=dev)
     gen.manual_seed(seed)
     GUARD = 256  # poisoned bytes after every tensor's codes
+    p_bf16 = layout != "f32"
+    g_bf16 = layout == "bf16"
+    psz, gsz = (2 if p_bf16 else 4), (2 if g_bf16 else 4)
+    p_t = torch.bfloat16 if p_bf16 else torch.float32
+    g_t = torch.bfloat16 if g_bf16 else torch.float32
+    p_np = np.uint16 if p_bf16 else np.float32
+    g_np = np.uint16 if g_bf16 else np.float32
 
     def arena(byte_sizes):
         offs, tot = [], 0
@@ -50,8 +69,8 @@ def _full_size(tensors, seed, want_numel, want_blocks, need_bytes):
             tot += (b + GUARD + 255) // 256 * 256
         return torch.empty(tot, dtype=torch.uint8, device=dev), offs
 
-    p_buf, p_off = arena([2 * n for n in sizes])
-    g_buf, g_off = arena([2 * n for n in sizes])
+    p_buf, p_off = arena([psz * n for n in sizes])
+    g_buf, g_off = arena([gsz * n for n in sizes])
     m_buf, m_off = arena(sizes)
     v_buf, v_off = arena(sizes)
     nbs = [(n + BLOCK - 1) // BLOCK for n in sizes]
@@ -63,13 +82,14 @@ def _full_size(tensors, seed, want_numel, want_blocks, need_bytes):
     rows = (L.TensorRow * len(sizes))()
     start = 0
     for i, n in enumerate(sizes):
-        p_buf[p_off[i]:p_off[i] + 2 * n].view(torch.bfloat16).copy_(torch.randn(n, device=dev, generator=gen).mul_(0.02))
-        g_buf[g_off[i]:g_off[i] + 2 * n].view(torch.bfloat16).copy_(torch.randn(n, device=dev, generator=gen).mul_(1e-3))
+        p_buf[p_off[i]:p_off[i] + psz * n].view(p_t).copy_(torch.randn(n, device=dev, generator=gen).mul_(0.02))
+        g_buf[g_off[i]:g_off[i] + gsz * n].view(g_t).copy_(torch.randn(n, device=dev, generator=gen).mul_(1e-3))
         r = rows[i]
         r.p, r.g = p_buf.data_ptr() + p_off[i], g_buf.data_ptr() + g_off[i]
         r.m, r.v = m_buf.data_ptr() + m_off[i], v_buf.data_ptr() + v_off[i]
         r.absmax_m, r.absmax_v = am_buf.data_ptr() + am_off[i], av_buf.data_ptr() + av_off[i]
-        r.numel, r.block_start, r.dtype_tag, r.grad_scale = n, start, L.DTYPE_BF16, 1.0
+        r.numel, r.block_start, r.dtype_tag, r.grad_scale = n, start, (L.DTYPE_BF16 if p_bf16 else L.DTYPE_F32), 1.0
+        r.grad_f32 = 1 if layout == "bf16_grad_f32" else 0
         start += nbs[i]
         L.check(L.lib().eri_adam8_state_init(r.m, r.v, r.absmax_m, r.absmax_v, n, stream), "state_init")
     table = C.c_void_p()
@@ -94,8 +114,8 @@ def _full_size(tensors, seed, want_numel, want_blocks, need_bytes):
         for i, b in sample:
             lo = b * BLOCK
             n = min(BLOCK, sizes[i] - lo)
-            out.append((p_buf[p_off[i] + 2 * lo:p_off[i] + 2 * (lo + n)].cpu().numpy().view(np.uint16).copy(),
-                        g_buf[g_off[i] + 2 * lo:g_off[i] + 2 * (lo + n)].cpu().numpy().view(np.uint16).copy(),
+            out.append((p_buf[p_off[i] + psz * lo:p_off[i] + psz * (lo + n)].cpu().numpy().view(p_np).copy(),
+                        g_buf[g_off[i] + gsz * lo:g_off[i] + gsz * (lo + n)].cpu().numpy().view(g_np).copy(),
                         m_buf[m_off[i] + lo:m_off[i] + lo + n].cpu().numpy().copy(),
                         v_buf[v_off[i] + lo:v_off[i] + lo + n].cpu().numpy().copy(),
                         am_buf[am_off[i] + 4 * b:am_off[i] + 4 * b + 4].cpu().numpy().view(np.float32).copy(),
@@ -113,16 +133,20 @@ def _full_size(tensors, seed, want_numel, want_blocks, need_bytes):
         after = grab()
         ho = oc.hyper_pack(*hyper, t)
         for (p, g, m, v, am, av), got in zip(before, after):
-            rc = oc.step_tensor(p, g, m, v, am, av, ho, hs.MAPS, oc.DT_BF16, 1)
+            rc = oc.step_tensor(p, g, m, v, am, av, ho, hs.MAPS, oc.DT_BF16 if p_bf16 else oc.DT_F32, 1,
+                                g_dtype=oc.DT_BF16 if g_bf16 else oc.DT_F32)
             assert rc == 0
             assert np.array_equal(got[2], m) and np.array_equal(got[3], v)
             assert np.array_equal(got[4].view(np.uint32), am.view(np.uint32))
             assert np.array_equal(got[5].view(np.uint32), av.view(np.uint32))
-            d = hs.bf16_ulp_distance(got[0], p)
-            assert d.max() <= (0 if exact else 1)
-            flips += int((d != 0).sum())
-    print("full-size sample of %d tensors: %d blocks x (2 default + 2 exact) steps, bf16 parameters one ulp off: %d" %
-          (len(sizes), len(sample), flips), flush=True)
+            if p_bf16:
+                d = hs.bf16_ulp_distance(got[0], p)
+                assert d.max() <= (0 if exact else 1)
+                flips += int((d != 0).sum())
+            else:  # fp32 parameters take the IEEE chain whatever the flag says
+                assert np.array_equal(got[0].view(np.uint32), p.view(np.uint32))
+    print("full-size sample of %d tensors (%s): %d blocks x (2 default + 2 exact) steps, bf16 parameters one ulp off: %d" %
+          (len(sizes), layout, len(sample), flips), flush=True)
 
     # properties of every block
     for i, n in enumerate(sizes):
