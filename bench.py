@@ -37,8 +37,10 @@ def parse():
     ap.add_argument("--mode", choices=["eri", "l2"], default="eri",
                     help="arithmetic of the table API's step: the list optimizer's (adam8bit_enhanced.rs) or the "
                          "functional update's (adam8bit.rs, what --api functional always runs)")
-    ap.add_argument("--api", choices=["table", "functional", "functional_update"], default="table",
-                    help="table: eri_adam8_step_table on a launch table built once (headline).  functional: the "
+    ap.add_argument("--api", choices=["table", "object", "functional", "functional_update"], default="table",
+                    help="table: eri_adam8_step_table on a launch table built once (headline).  object: the list "
+                         "optimizer of the reference's API (eri_adam8bit_new over parameter handles, which owns its "
+                         "states; one eri_adam8bit_step call per step).  functional: the "
                          "per-name optimizer, all tensors through one eri_adam8bit_fn_update_many call per step, "
                          "each step writing into the other of two output sets (update() returns a new tensor).  "
                          "functional_update: the same through one batched eri_adam8bit_fn_update call per tensor")
@@ -179,8 +181,8 @@ def main():
     esz = 2 if bf16 else 4
     grad_f32 = bf16 and args.grad_dtype == "f32"
     gsz = 4 if grad_f32 else esz
-    if grad_f32 and (args.kernel in ("adamw32",) or args.api != "table"):
-        sys.exit("--grad-dtype f32 is wired for the table API's 8-bit step and the gradient norm")
+    if grad_f32 and (args.kernel in ("adamw32",) or args.api not in ("table", "object")):
+        sys.exit("--grad-dtype f32 is wired for the 8-bit step of the table and object APIs and for the gradient norm")
     sizes = [W.numel(s) for _, s in tensors]
     n_params = sum(sizes)
     n_blocks = sum((n + L.BLOCK - 1) // L.BLOCK for n in sizes)
@@ -246,7 +248,25 @@ def main():
         bytes_per_param += gsz + 4.0 / 2048
 
     fn_opt = None
-    if args.api != "table":
+    obj_opt, obj_params = None, []
+    if args.api == "object":
+        if args.kernel != "adam8" or args.mode != "eri":
+            sys.exit("--api object runs the 8-bit step of the list optimizer only")
+        cfg = L.Adam8bitConfigC()
+        L.lib().eri_adam8bit_config_default(C.byref(cfg))
+        cfg.lr, cfg.beta1, cfg.beta2, cfg.eps, cfg.weight_decay = hyper_args
+        handles = (C.c_void_p * len(sizes))()
+        for i, n in enumerate(sizes):
+            hnd = C.c_void_p()
+            L.check(L.lib().eri_param_create(a_p.ptr(i), n, L.DTYPE_BF16 if bf16 else L.DTYPE_F32, C.byref(hnd)), "param_create")
+            L.check(L.lib().eri_param_set_grad_typed(hnd, a_g.ptr(i), L.DTYPE_F32 if gsz == 4 else L.DTYPE_BF16), "set_grad")
+            handles[i] = hnd.value
+            obj_params.append(hnd)
+        obj_opt = C.c_void_p()
+        L.check(L.lib().eri_adam8bit_new(handles, len(sizes), C.byref(cfg), stream, C.byref(obj_opt)), "adam8bit_new")
+        if args.flags:
+            L.check(L.lib().eri_adam8bit_set_flags(obj_opt, args.flags), "set_flags")
+    elif args.api != "table":
         if args.kernel != "adam8":
             sys.exit("--api functional runs the 8-bit step only")
         n_t = len(sizes)
@@ -268,6 +288,9 @@ def main():
         g_raw = [a_g.ptr(i) for i in range(n_t)]
 
     def step(t):
+        if obj_opt is not None:
+            L.check(L.lib().eri_adam8bit_step(obj_opt, None), "adam8bit_step")
+            return
         if fn_opt is not None:
             if args.api == "functional":
                 src, dst = sets[t & 1]
@@ -345,7 +368,7 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": args.config, "tensors": len(sizes), "params": n_params, "blocks": n_blocks,
-                   "kernel": args.kernel, "api": args.api, "mode": "l2" if args.api != "table" else args.mode,
+                   "kernel": args.kernel, "api": args.api, "mode": args.mode if args.api in ("table", "object") else "l2",
                    "param_dtype": dt_name, "grad_dtype": "f32" if gsz == 4 else "bf16", "state": "uint8 m/v + fp32 absmax per 2048-block", "flags": args.flags,
                    "resident_gb": round((n_params * (esz + gsz + 2) + n_blocks * 8) / 1e9, 2)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
@@ -358,6 +381,10 @@ def main():
     L.lib().eri_adam8_table_destroy(table)
     if fn_opt is not None:
         L.lib().eri_adam8bit_fn_destroy(fn_opt)
+    if obj_opt is not None:
+        L.lib().eri_adam8bit_destroy(obj_opt)
+        for hnd in obj_params:
+            L.lib().eri_param_release(hnd)
     for a in [a_p, a_g, a_m, a_v, a_am, a_av] + extra:
         a.free()
     if args.cpu_sample > 0:
