@@ -241,10 +241,13 @@ __device__ __forceinline__ float param_exact(float p, float m, float v, const Er
  * margin's own arithmetic.
  *
  * The functional update (mode L2) rounds the *update* to bf16 before it subtracts (adam8bit.rs:197-198), and
- * that subtraction is a single exact-input operation, so the same argument applies to the update: the fast
- * chain's lr * (m/bc1) / (sqrt(v/bc2) + eps) is within 6.5 * 2^-23 of the exact chain's, relative, and an
- * update further than 8 * 2^-23 of itself from the tie point of its bf16 interval rounds to the same bf16
- * value on both chains.  About one element in 4,000 is flagged and recomputed.
+ * that subtraction is a single exact-input operation, so the same argument applies to the update.  The fast
+ * chain multiplies by the rounded reciprocals of the two bias corrections instead of dividing (1.5 * 2^-23
+ * each, relative to the exact quotient), takes the hardware square root and reciprocal (2^-23 each) and rounds
+ * six times: its lr * (m/bc1) / (sqrt(v/bc2) + eps) is within 7.75 * 2^-23 of the exact chain's, relative, and
+ * an update further than 16 * 2^-23 of itself from the tie point of its bf16 interval rounds to the same bf16
+ * value on both chains.  About one element in 2,000 is flagged and recomputed, and so is every element with a
+ * moment below 2^-100, where the products lose relative accuracy to the denormal grid.
  */
 template <int MODE, bool WD>
 struct ExactMargin {
@@ -304,14 +307,21 @@ __device__ __forceinline__ void adam_elem_decayed(float p, float g, float t1, fl
     if (!BF16) { // fp32 parameters: every bit of the exact chain counts
         pn = param_exact<MODE, WD, false>(p, m, v, h, dbc1, dbc2);
     } else if (MODE == ERI_ADAM8_MODE_L2) { // always to the exact chain's bits (the reference rounds the update itself)
-        float mh = dbc1.fast ? dbc1.div_fast_unbounded(m) : m / dbc1.a; // adam8bit.rs:170
-        float vh = dbc2.fast ? dbc2.div_fast_unbounded(v) : v / dbc2.a; // :178
-        vh = fmaxf(vh, 0.0f);                                           // :181-182
+        // fast chain: the two bias corrections as products with the rounded reciprocals, hardware square root
+        // and reciprocal; param_exact redoes whatever the test below cannot vouch for
+        float mh = m * dbc1.ras;              // adam8bit.rs:170
+        float vh = fmaxf(v * dbc2.ras, 0.0f); // :178, :181-182
         float den = __builtin_amdgcn_sqrtf(vh) + h.eps;
         float upd = mh * __builtin_amdgcn_rcpf(den);
         float us = upd * h.step_size;
         const float tie = u2f((f2u(us) & 0xffff0000u) | 0x8000u);
-        recheck |= !(__builtin_fabsf(us - tie) > __builtin_fmaf(__builtin_fabsf(us), 0x1p-20f, 0x1p-126f));
+        recheck |= !(__builtin_fabsf(us - tie) > __builtin_fmaf(__builtin_fabsf(us), 0x1p-19f, 0x1p-126f));
+        // a non-zero moment near the denormal range loses relative accuracy in the product (the exact chain's
+        // division rounds on the same grid but not to the same point).  For the second moment that only shows
+        // when eps is too small to swallow its square root.  NaN and infinity fail the comparison above.
+        recheck |= (__builtin_fabsf(m) < 0x1p-100f) & (m != 0.0f);
+        if (h.eps < 0x1p-36f) recheck |= (v < 0x1p-100f) & (v != 0.0f);
+        recheck |= !(dbc1.fast && dbc2.fast);
         pn = p - bf16_round(us); // :197-205
     } else { // h.eps and h.weight_decay of mode BNB carry sqrt(bc2) and the factor 1 - lr*wd
         float den = __builtin_amdgcn_sqrtf(v) + h.eps;

@@ -260,6 +260,76 @@ def test_l2_mode_bias_correction_with_tiny_huge_and_infinite_moments(bf16):
     assert stats["code_mismatch"] == 0
 
 
+@pytest.mark.parametrize("eps", [1e-8, 0.0])
+def test_l2_mode_with_every_moment_of_a_block_near_the_denormal_range(eps):
+    """Whole blocks of gradients between 1e-44 and 1e-28: the block maxima are tiny too, so the dequantised
+    moments stay non-zero down to the denormal range instead of rounding to the zero entry.  The fast chain of
+    the functional update multiplies by reciprocals of the bias corrections, which is not the division's
+    rounding there (the kernel sends such elements to the division); with eps = 0 nothing swallows the second
+    moment's square root either.  The oracle's bits, bf16 parameters, three steps."""
+    L = _lib()
+    n = 2048 * 3 + 300
+    rng = np.random.default_rng(4242)
+    ps, _ = hs.make_inputs([n], True, 77, p_std=0.0)  # parameters at zero: the first result is the rounded update itself
+    states = hs.oracle_states([n])
+
+    def grads(lo, hi):
+        g = (rng.standard_normal(n) * 10.0 ** rng.uniform(lo, hi, n)).astype(np.float32)
+        g[::53] = 0.0
+        return [onp.f32_to_bf16(g)]
+
+    all_g = [grads(-40, -28), grads(-44, -30), grads(-38, -28)]
+    gt = hs.GpuTensors(ps, all_g[0], states, True)
+    rows = gt.rows(None)
+    table = C.c_void_p()
+    L.check(L.lib().eri_adam8_table_create(rows, len(rows), _stream(), C.byref(table)), "table_create")
+    with np.errstate(all="ignore"):
+        for k, g_k in enumerate(all_g):
+            hs.oracle_step(ps, g_k, states, (LR, B1, B2, eps, 0.0, k), True, oc.MODE_L2)
+            if k:
+                gt.set_grads(g_k)
+            h = L.hyper_pack(LR, B1, B2, eps, 0.0, k, 1, 2 | KERNEL_FLAGS)
+            L.check(L.lib().eri_adam8_step_table(table, C.byref(h), _stream()), "step_table")
+    _sync()
+    L.lib().eri_adam8_table_destroy(table)
+    got_p, got_st = gt.fetch()
+    assert any((a.view(np.uint32) != 0).any() for a in (states[0][2], states[0][3]))  # the block maxima are not all zero
+    stats = hs.compare(got_p, got_st, ps, states, True, True, "l2-denormal-range eps=%g" % eps)
+    assert stats["code_mismatch"] == 0
+
+
+def test_l2_mode_with_first_moments_of_a_few_denormal_steps():
+    """States built by hand: first moments of 10 to 100,000 denormal steps (absmax 1e-44 to 1e-40), ordinary
+    second moments, zero gradients, and a learning rate large enough to lift the update out of the denormal
+    range.  m / (1 - beta1^s) then has few significant bits, where a product with the rounded reciprocal can
+    land a whole step of that coarse grid away from the quotient (a host search finds a few such first moments
+    per 10^5 and none among 2 * 10^7 that also changes the rounded update, so this is coverage of the regime,
+    not a case that fails without the kernel's fallback to the division)."""
+    L = _lib()
+    n = 2048 * 96
+    rng = np.random.default_rng(99)
+    ps, _ = hs.make_inputs([n], True, 78, p_std=0.0)
+    states = hs.oracle_states([n])
+    m, v, am, av = states[0]
+    m[:] = rng.integers(0, 256, n, dtype=np.uint8)
+    v[:] = rng.integers(1, 256, n, dtype=np.uint8)
+    m[::2048] = 255
+    v[::2048] = 255
+    am[:] = (10.0 ** rng.uniform(-44, -40, am.size)).astype(np.float32)
+    av[:] = np.float32(1e-6)
+    gs = [onp.f32_to_bf16(np.zeros(n, np.float32))]
+    gt = hs.GpuTensors(ps, gs, states, True)
+    lr = 1e12
+    for step in (3, 4):
+        with np.errstate(all="ignore"):
+            hs.oracle_step(ps, gs, states, (lr, B1, B2, EPS, 0.0, step), True, oc.MODE_L2)
+        gpu_steps(gt, [None], step + 1, mode=1, flags=2, wd=0.0, lr=lr)
+    got_p, got_st = gt.fetch()
+    assert np.count_nonzero(ps[0] & 0x7FFF) > n // 2  # the updates are visible in the parameters
+    stats = hs.compare(got_p, got_st, ps, states, True, True, "l2-few-denormal-steps")
+    assert stats["code_mismatch"] == 0
+
+
 def test_no_weight_decay_variant():
     run_case([2048 * 9 + 3, 640], True, 400, steps=3, wd=0.0, flags=2, label="wd0")
     run_case([2048 * 9 + 3, 640], False, 401, steps=3, wd=0.0, label="wd0-fp32")
