@@ -543,21 +543,27 @@ __device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint
             float pv[8], gv[8], pn[8];
             pr[d].unpack(pv);
             gr[d].unpack(gv);
-            bool cancel = false;
+            // one flag per element: the exact chain then runs for the flagged positions only, and a position
+            // is skipped altogether when no lane of the wave has it flagged
+            bool redo[8];
+            bool any = false;
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
                 const float m_old = L.map_s[byte_of(mr[d], k)] * a_m;
                 const float v_old = L.map_u[byte_of(vr[d], k)] * a_v;
                 float m, v;
-                adam_elem<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], m_old, v_old, h, gscale, dbc1, dbc2, m, v, pn[k], cancel);
+                redo[k] = false;
+                adam_elem<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], m_old, v_old, h, gscale, dbc1, dbc2, m, v, pn[k], redo[k]);
+                any |= redo[k];
                 mf[c * 8 + k] = m;
                 vf[c * 8 + k] = v;
                 lm = fmaxf(lm, __builtin_fabsf(m));
                 lv = fmaxf(lv, __builtin_fabsf(v));
             }
-            if (cancel) {
+            if (any) {
 #pragma unroll
-                for (int k = 0; k < 8; ++k) pn[k] = param_exact<MODE, WD, BF16>(pv[k], mf[c * 8 + k], vf[c * 8 + k], h, dbc1, dbc2);
+                for (int k = 0; k < 8; ++k)
+                    if (redo[k]) pn[k] = param_exact<MODE, WD, BF16>(pv[k], mf[c * 8 + k], vf[c * 8 + k], h, dbc1, dbc2);
             }
             store8<BF16>(p, o, pn);
         }

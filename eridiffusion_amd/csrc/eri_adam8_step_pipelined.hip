@@ -195,7 +195,6 @@ __global__ __launch_bounds__(kPipeThreads) void ERI_PIPE_KERNEL(const DevTensor 
 #pragma unroll
             for (int c = 0; c < 4; ++c) sh[c] = __builtin_nontemporal_load(&sp[c * 64 + lane]);
         }
-        bool cancel = false;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             float pv[8], gv[8], pn[8];
@@ -217,21 +216,28 @@ __global__ __launch_bounds__(kPipeThreads) void ERI_PIPE_KERNEL(const DevTensor 
                 gv[0] = u2f(ga.x); gv[1] = u2f(ga.y); gv[2] = u2f(ga.z); gv[3] = u2f(ga.w);
                 gv[4] = u2f(gb.x); gv[5] = u2f(gb.y); gv[6] = u2f(gb.z); gv[7] = u2f(gb.w);
             }
-            bool redo = false; // EMA: flagged elements are put right quarter by quarter, before the shadow uses them
+            // one flag per element: flagged elements are put right quarter by quarter (before the shadow uses
+            // them), the exact chain runs for the flagged positions only, and a position is skipped when no
+            // lane of the wave has it flagged
+            bool redo[8];
+            bool any = false;
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
                 const float t1 = lds_float_at(mine[0], code_offset(raw.m[c], k));
                 const float t3 = lds_float_at(mine[1], code_offset(raw.v[c], k));
                 float m, v;
-                adam_elem_decayed<MODE, EXACT, kParamBf16, WD, GS>(pv[k], gv[k], t1, t3, h, gscale, dbc1, dbc2, m, v, pn[k], EMA ? redo : cancel);
+                redo[k] = false;
+                adam_elem_decayed<MODE, EXACT, kParamBf16, WD, GS>(pv[k], gv[k], t1, t3, h, gscale, dbc1, dbc2, m, v, pn[k], redo[k]);
+                any |= redo[k];
                 mf[c * 8 + k] = m;
                 vf[c * 8 + k] = v;
                 lm = fmaxf(lm, __builtin_fabsf(m));
                 lv = fmaxf(lv, __builtin_fabsf(v));
             }
-            if (EMA && redo) {
+            if (kParamBf16 && any) {
 #pragma unroll
-                for (int k = 0; k < 8; ++k) pn[k] = param_exact<MODE, WD, true>(pv[k], mf[c * 8 + k], vf[c * 8 + k], h, dbc1, dbc2);
+                for (int k = 0; k < 8; ++k)
+                    if (redo[k]) pn[k] = param_exact<MODE, WD, true>(pv[k], mf[c * 8 + k], vf[c * 8 + k], h, dbc1, dbc2);
             }
             if (kParamBf16) {
                 pw[c].x = bf16_pair(pn[0], pn[1]);
@@ -242,21 +248,6 @@ __global__ __launch_bounds__(kPipeThreads) void ERI_PIPE_KERNEL(const DevTensor 
                 store8<false>(p, c * 512 + lane * 8, pn);
             }
             if (EMA && with_shadow) ema_quarter(t.shadow, e0, c, lane, sh[c], pw[c], h.ema_decay);
-        }
-        if (kParamBf16 && cancel) { // rare: a lane whose update cancelled redoes its 32 parameters with the exact chain
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                Raw8<true> pr;
-                pr.w = raw.p[c];
-                float pv[8], pn[8];
-                pr.unpack(pv);
-#pragma unroll
-                for (int k = 0; k < 8; ++k) pn[k] = param_exact<MODE, WD, true>(pv[k], mf[c * 8 + k], vf[c * 8 + k], h, dbc1, dbc2);
-                pw[c].x = bf16_pair(pn[0], pn[1]);
-                pw[c].y = bf16_pair(pn[2], pn[3]);
-                pw[c].z = bf16_pair(pn[4], pn[5]);
-                pw[c].w = bf16_pair(pn[6], pn[7]);
-                }
         }
         float nam = lm, nav = lv;
         wave_max2(nam, nav);
