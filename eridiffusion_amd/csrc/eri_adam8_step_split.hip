@@ -112,18 +112,22 @@ __global__ __launch_bounds__(1024) void adam8_step_split_kernel(const DevTensor 
                 reinterpret_cast<f32x4 *>(mine[0])[lane] = ds;
                 reinterpret_cast<f32x4 *>(mine[1])[lane] = du;
             }
-            bool cancel = false;
+            bool redo[8]; // per element: the exact chain runs for the flagged positions only
+            bool any = false;
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
                 const float t1 = lds_float_at(mine[0], code_offset(q.mr, k));
                 const float t3 = lds_float_at(mine[1], code_offset(q.vr, k));
-                adam_elem_decayed<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], t1, t3, h, gscale, dbc1, dbc2, m[k], v[k], pn[k], cancel);
+                redo[k] = false;
+                adam_elem_decayed<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], t1, t3, h, gscale, dbc1, dbc2, m[k], v[k], pn[k], redo[k]);
+                any |= redo[k];
                 nam = fmaxf(nam, __builtin_fabsf(m[k]));
                 nav = fmaxf(nav, __builtin_fabsf(v[k]));
             }
-            if (cancel) {
+            if (any) {
 #pragma unroll
-                for (int k = 0; k < 8; ++k) pn[k] = param_exact<MODE, WD, BF16>(pv[k], m[k], v[k], h, dbc1, dbc2);
+                for (int k = 0; k < 8; ++k)
+                    if (redo[k]) pn[k] = param_exact<MODE, WD, BF16>(pv[k], m[k], v[k], h, dbc1, dbc2);
             }
             store8<BF16>(p, o, pn);
             wave_max2(nam, nav);
