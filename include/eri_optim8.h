@@ -98,8 +98,11 @@ typedef enum EriAdam8Mode {
 
 enum {
     ERI_ADAM8_FLAG_GRAD_SCALE = 1u << 0,  /* multiply gradients by hyper.grad_scale * tensor.grad_scale */
-    ERI_ADAM8_FLAG_EXACT_PARAM = 1u << 1, /* IEEE sqrt and divide on the parameter update of BF16
-                                             tensors too (F32 tensors always use them) */
+    ERI_ADAM8_FLAG_EXACT_PARAM = 1u << 1, /* BF16 parameters come out with the bits of the chain of individually
+                                             rounded IEEE operations (F32 parameters always do): every element
+                                             whose rounding the faster arithmetic cannot vouch for is recomputed
+                                             with IEEE sqrt and divide.  Without the flag BF16 parameters are
+                                             within one BF16 unit in the last place of those bits */
     ERI_ADAM8_FLAG_BSEARCH = 1u << 2,     /* requantise by binary search of the LDS midpoint table
                                              instead of the float-keyed slot table (same codes; runs on
                                              the plain one-wave-per-block kernel whatever the table size) */
