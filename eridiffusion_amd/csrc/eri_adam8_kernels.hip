@@ -47,7 +47,7 @@ int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, i
     }
     if (mixed) {
         const bool wd_m = h.mode == ERI_ADAM8_MODE_BNB ? h.weight_decay != 1.0f : h.weight_decay > 0.0f;
-        if (h.mode != ERI_ADAM8_MODE_L2 && (h.flags & ERI_ADAM8_FLAG_NO_PIPELINE) == 0 && prefetch_pays(total_blocks, h, compute_units))
+        if ((h.flags & ERI_ADAM8_FLAG_NO_PIPELINE) == 0 && prefetch_pays(total_blocks, h, compute_units))
             return launch_step_pipelined_grad_f32(h.mode, (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0, wd_m, gs, rows, n_rows,
                                                   total_blocks, h, lds_image, dev_scale, grid, wg, stream);
         return launch_step_plain_bf16(h.mode, (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0, wd_m, gs, true, true, rows, n_rows,
@@ -66,11 +66,10 @@ int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, i
     const bool wd = h.weight_decay > 0.0f;
     const bool exact = (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0;
     const bool keytab = (h.flags & ERI_ADAM8_FLAG_BSEARCH) == 0;
-    if (!bf16 && !kernel_named && h.mode == ERI_ADAM8_MODE_ERI && prefetch_pays(total_blocks, h, compute_units))
+    if (!bf16 && !kernel_named && prefetch_pays(total_blocks, h, compute_units))
         return launch_step_pipelined_f32(h.mode, wd, gs, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
     if (!bf16) return launch_step_plain_f32(h.mode, wd, gs, keytab, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);
-    if (keytab && h.mode == ERI_ADAM8_MODE_ERI && (h.flags & ERI_ADAM8_FLAG_NO_PIPELINE) == 0 &&
-        prefetch_pays(total_blocks, h, compute_units))
+    if (keytab && (h.flags & ERI_ADAM8_FLAG_NO_PIPELINE) == 0 && prefetch_pays(total_blocks, h, compute_units))
         return launch_step_pipelined(h.mode, exact, wd, gs, step_fuses_ema(total_blocks, layout, h, compute_units), rows, n_rows,
                                      total_blocks, h, lds_image, dev_scale, grid, wg, stream);
     return launch_step_plain_bf16(h.mode, exact, wd, gs, keytab, false, rows, n_rows, total_blocks, h, lds_image, dev_scale, grid, wg, stream);

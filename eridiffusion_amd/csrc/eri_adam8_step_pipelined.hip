@@ -320,9 +320,8 @@ int launch_flags(bool wd, bool gs, bool ema, const DevTensor *rows, uint32_t n_r
 
 } // namespace
 
-/* Modes ERI and BNB.  The coupled-decay mode needs more live values per element than this kernel's
- * register budget holds (its instantiations spilled 80-232 B per lane) and runs faster on the kernel
- * without the prefetch; the dispatcher sends it there. */
+/* All three modes.  (The coupled-decay mode fits the register budget since its bias corrections became
+ * products in the fast chain: 168 registers, no scratch; with the two divisions it spilled 80-232 B per lane.) */
 #if ERI_PIPE_LAYOUT == 1
 int launch_step_pipelined(int mode, bool exact, bool wd, bool gs, bool ema, const DevTensor *rows, uint32_t n_rows,
                           uint32_t total_blocks, const EriAdam8Hyper &h, const void *img, const float *dev_scale,
@@ -342,9 +341,11 @@ int launch_step_pipelined_f32(int mode, bool wd, bool gs, const DevTensor *rows,
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define ERI_ARGS wd, gs, ema, rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s
 #if ERI_PIPE_LAYOUT == 0
+    if (mode == ERI_ADAM8_MODE_L2) return launch_flags<ERI_ADAM8_MODE_L2, exact>(ERI_ARGS);
     if (mode == ERI_ADAM8_MODE_BNB) return launch_flags<ERI_ADAM8_MODE_BNB, exact>(ERI_ARGS);
     return launch_flags<ERI_ADAM8_MODE_ERI, exact>(ERI_ARGS);
 #else
+    if (mode == ERI_ADAM8_MODE_L2) return launch_flags<ERI_ADAM8_MODE_L2, true>(ERI_ARGS); // its fast chain always checks itself
     if (mode == ERI_ADAM8_MODE_BNB)
         return exact ? launch_flags<ERI_ADAM8_MODE_BNB, true>(ERI_ARGS) : launch_flags<ERI_ADAM8_MODE_BNB, false>(ERI_ARGS);
     return exact ? launch_flags<ERI_ADAM8_MODE_ERI, true>(ERI_ARGS) : launch_flags<ERI_ADAM8_MODE_ERI, false>(ERI_ARGS);
