@@ -107,7 +107,7 @@ enum {
                                              instead of the float-keyed slot table (same codes; runs on
                                              the plain one-wave-per-block kernel whatever the table size) */
     ERI_ADAM8_FLAG_NO_PIPELINE = 1u << 3, /* use the plain one-wave-per-block kernel: not the one that
-                                             prefetches the next block (large BF16 tables), not the
+                                             prefetches the next block (large tables), not the
                                              four-waves-per-block one (small tables).  Same results; a
                                              cross-check */
     ERI_ADAM8_FLAG_CLIP_FROM_TABLE = 1u << 4, /* also multiply gradients by the clip factor the last
@@ -120,11 +120,9 @@ enum {
                                              registers: the separate sweep's read of p is saved); every other
                                              table runs the EMA sweep right after the step, in the same call.
                                              Same results either way */
-    ERI_ADAM8_FLAG_ONE_WAVE = 1u << 5     /* take the kernels of the largest tables whatever the size: the
-                                             prefetching kernel for BF16 parameters with BF16 gradients, the
-                                             plain one-wave-per-block kernel for F32 parameters and for F32
-                                             gradients.  Same results; lets tests reach every kernel with
-                                             small inputs */
+    ERI_ADAM8_FLAG_ONE_WAVE = 1u << 5     /* take the kernel of the largest tables whatever the size: one
+                                             wave per block with the next block's loads in flight.  Same
+                                             results; lets tests reach every kernel with small inputs */
 };
 
 /* Per-step scalars, already cast where the reference casts them.  Fill with eri_adam8_hyper_pack. */
