@@ -505,9 +505,14 @@ __device__ __forceinline__ void requant8(const float *mf, const float *vf, const
     vw.y = cv[4] | (cv[5] << 8) | (cv[6] << 16) | (cv[7] << 24);
 }
 
+/* `mine` is the wave's own pair of 256-entry tables in LDS.  The block opens by filling them with
+ * (MAP[c] * absmax) * beta for every code c -- the first two operations of both moment updates, done once
+ * per code (eight per lane) instead of once per element (64 per lane); a wave's LDS operations complete in
+ * order, so its reads below see its own writes without a barrier. */
 template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB, bool GBF16 = BF16>
 __device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint32_t lane, const EriAdam8Hyper &h,
-                                           float gscale, const BlockDiv &dbc1, const BlockDiv &dbc2, const Lds &L) {
+                                           float gscale, const BlockDiv &dbc1, const BlockDiv &dbc2, const Lds &L,
+                                           float (*mine)[256]) {
     const size_t e0 = (size_t)lb * kBlock;
     const size_t esz = BF16 ? 2 : 4;
     char *p = static_cast<char *>(t.p) + e0 * esz;
@@ -517,6 +522,17 @@ __device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint
     uint8_t *vc = t.v + e0;
     const float a_m = as_global(t.absmax_m)[lb];
     const float a_v = as_global(t.absmax_v)[lb];
+    {
+        const f32x4 bs = reinterpret_cast<const f32x4 *>(L.map_s)[lane]; // codes 4*lane .. 4*lane + 3
+        const f32x4 bu = reinterpret_cast<const f32x4 *>(L.map_u)[lane];
+        f32x4 ds, du;
+        ds.x = (bs.x * a_m) * h.beta1; ds.y = (bs.y * a_m) * h.beta1;
+        ds.z = (bs.z * a_m) * h.beta1; ds.w = (bs.w * a_m) * h.beta1;
+        du.x = (bu.x * a_v) * h.beta2; du.y = (bu.y * a_v) * h.beta2;
+        du.z = (bu.z * a_v) * h.beta2; du.w = (bu.w * a_v) * h.beta2;
+        reinterpret_cast<f32x4 *>(mine[0])[lane] = ds;
+        reinterpret_cast<f32x4 *>(mine[1])[lane] = du;
+    }
 
     float mf[32], vf[32];
     float lm = 0.0f, lv = 0.0f;
@@ -549,11 +565,11 @@ __device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint
             bool any = false;
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
-                const float m_old = L.map_s[byte_of(mr[d], k)] * a_m;
-                const float v_old = L.map_u[byte_of(vr[d], k)] * a_v;
+                const float t1 = lds_float_at(mine[0], code_offset(mr[d], k));
+                const float t3 = lds_float_at(mine[1], code_offset(vr[d], k));
                 float m, v;
                 redo[k] = false;
-                adam_elem<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], m_old, v_old, h, gscale, dbc1, dbc2, m, v, pn[k], redo[k]);
+                adam_elem_decayed<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], t1, t3, h, gscale, dbc1, dbc2, m, v, pn[k], redo[k]);
                 any |= redo[k];
                 mf[c * 8 + k] = m;
                 vf[c * 8 + k] = v;

@@ -23,6 +23,7 @@ __global__ __launch_bounds__(plain_threads(MODE)) void adam8_step_kernel(const D
                                                           const uint4 *__restrict__ lds_image,
                                                           const float *__restrict__ dev_scale, uint32_t chunks) {
     ERI_LDS_IMAGE;
+    __shared__ float decayed[16][2][256]; // per wave: the values its block's state codes stand for, decayed
     // clip factor left on the device by the gradient-norm pass (1.0 when there is none)
     const float tscale = (GS && dev_scale) ? *dev_scale : 1.0f;
     // the binary search needs the maps and midpoints only (4 KB); the slot tables are the other 96 KB
@@ -62,7 +63,8 @@ __global__ __launch_bounds__(plain_threads(MODE)) void adam8_step_kernel(const D
     for (uint32_t blk = walk.first; blk < walk.end; blk += walk.stride) {
         map.seek(rows, blk, ti, t, t_end);
         const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
-        full_block<BF16, MODE, EXACT, WD, GS, KEYTAB, GBF16>(t, blk - t.full_start, lane, h, gscale, dbc1, dbc2, L);
+        full_block<BF16, MODE, EXACT, WD, GS, KEYTAB, GBF16>(t, blk - t.full_start, lane, h, gscale, dbc1, dbc2, L,
+                                                             decayed[threadIdx.x / kWave]);
     }
 }
 
