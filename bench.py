@@ -48,9 +48,11 @@ def parse():
                     help="parameter dtype: the one the configuration names, or an override (the shapes stay)")
     ap.add_argument("--grad-dtype", choices=["param", "f32"], default="param",
                     help="gradient dtype: the parameter's, or fp32 gradients (for bf16 parameters: read unrounded)")
-    ap.add_argument("--alloc", choices=["arena", "tensor"], default="arena",
-                    help="one flat allocation per kind of buffer (library allocator), or one torch allocation per "
-                         "tensor and buffer (how a tensor runtime holds parameters and states)")
+    ap.add_argument("--alloc", choices=["arena", "tensor", "spread"], default="arena",
+                    help="one flat allocation per kind of buffer (library allocator), one torch allocation per "
+                         "tensor and buffer (how a tensor runtime holds parameters and states), or the flat arrays "
+                         "placed an eighth of the device memory apart inside one allocation (what a pool allocator "
+                         "can arrange)")
     ap.add_argument("--traffic-json", default=os.path.join(ROOT, "profiles", "traffic.json"),
                     help="HBM bytes per launch derived from rocprofv3 --pmc runs, if present")
     return ap.parse_args()
@@ -104,6 +106,43 @@ class Arena:
     def free(self):
         from eridiffusion_amd import _lib as L
         L.lib().eri_hip_free(self.base)
+
+
+class Spread(Arena):
+    """The arenas of Arena, but carved out of ONE large allocation at equal distances (an eighth of it, 30 GiB
+    and more on an empty MI355X): what a pool allocator can do that separate allocations cannot, namely keep the
+    parameter, gradient and state arrays far from each other in device memory."""
+
+    pool = None
+    pool_base = 0
+    stride = 0
+    next_slot = 0
+    SLOTS = 8
+
+    def __init__(self, torch, sizes_bytes):
+        from eridiffusion_amd import _lib as L
+        cls = Spread
+        self.offsets = []
+        total = 0
+        for b in sizes_bytes:
+            self.offsets.append(total)
+            total += align(b)
+        self.nbytes = max(total, 256)
+        if cls.pool is None:
+            free, _ = torch.cuda.mem_get_info()
+            cls.stride = int(free * 0.92) // cls.SLOTS // (2 << 20) * (2 << 20)
+            cls.pool = torch.empty(cls.stride * cls.SLOTS, dtype=torch.uint8, device="cuda:0")
+            cls.pool_base = cls.pool.data_ptr()
+            cls.next_slot = 0
+        if self.nbytes > cls.stride or cls.next_slot >= cls.SLOTS:
+            sys.exit("--alloc spread: this workload's arrays do not fit an eighth of the device memory each")
+        self.base = cls.pool_base + cls.next_slot * cls.stride
+        cls.next_slot += 1
+        # the library's allocator hands out zeroed memory; so does this one
+        cls.pool[self.base - cls.pool_base:self.base - cls.pool_base + self.nbytes].zero_()
+
+    def free(self):
+        pass  # the pool goes with the process
 
 
 def cpu_baseline(tensors, bf16, sample_params, hyper_args):
@@ -189,7 +228,7 @@ def main():
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream().cuda_stream
 
-    Alloc = {"arena": Arena, "tensor": PerTensor}[args.alloc]
+    Alloc = {"arena": Arena, "tensor": PerTensor, "spread": Spread}[args.alloc]
     a_p = Alloc(torch, [n * esz for n in sizes])
     a_g = Alloc(torch, [n * gsz for n in sizes])
     a_m = Alloc(torch, sizes)
@@ -368,7 +407,7 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": args.config, "tensors": len(sizes), "params": n_params, "blocks": n_blocks,
-                   "kernel": args.kernel, "api": args.api, "mode": args.mode if args.api in ("table", "object") else "l2",
+                   "kernel": args.kernel, "api": args.api, "alloc": args.alloc, "mode": args.mode if args.api in ("table", "object") else "l2",
                    "param_dtype": dt_name, "grad_dtype": "f32" if gsz == 4 else "bf16", "state": "uint8 m/v + fp32 absmax per 2048-block", "flags": args.flags,
                    "resident_gb": round((n_params * (esz + gsz + 2) + n_blocks * 8) / 1e9, 2)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
