@@ -48,11 +48,11 @@ def parse():
                     help="parameter dtype: the one the configuration names, or an override (the shapes stay)")
     ap.add_argument("--grad-dtype", choices=["param", "f32"], default="param",
                     help="gradient dtype: the parameter's, or fp32 gradients (for bf16 parameters: read unrounded)")
-    ap.add_argument("--alloc", choices=["arena", "tensor", "spread"], default="arena",
-                    help="one flat allocation per kind of buffer (library allocator), one torch allocation per "
-                         "tensor and buffer (how a tensor runtime holds parameters and states), or the flat arrays "
-                         "placed an eighth of the device memory apart inside one allocation (what a pool allocator "
-                         "can arrange)")
+    ap.add_argument("--alloc", choices=["arena", "tensor", "pool"], default="arena",
+                    help="arena: one flat allocation per kind of buffer (eri_hip_malloc_zeroed).  tensor: one torch "
+                         "allocation per tensor and buffer (how a tensor runtime holds parameters and states).  pool: "
+                         "the flat buffers out of the library's lane pool (eri_hip_pool_*), one 48 GiB lane per kind, "
+                         "which keeps the 8-bit states far from the parameters in device memory")
     ap.add_argument("--traffic-json", default=os.path.join(ROOT, "profiles", "traffic.json"),
                     help="HBM bytes per launch derived from rocprofv3 --pmc runs, if present")
     return ap.parse_args()
@@ -108,41 +108,40 @@ class Arena:
         L.lib().eri_hip_free(self.base)
 
 
-class Spread(Arena):
-    """The arenas of Arena, but carved out of ONE large allocation at equal distances (an eighth of it, 30 GiB
-    and more on an empty MI355X): what a pool allocator can do that separate allocations cannot, namely keep the
-    parameter, gradient and state arrays far from each other in device memory."""
+class Pool(Arena):
+    """The arenas of Arena out of the library's lane pool (eri_hip_pool_*): one device allocation, one lane per
+    kind of array -- parameters, gradients, first and second moments, anything else -- so that the 8-bit states
+    lie far from the parameters and gradients in device memory.  What a runtime with a pool allocator (the
+    reference's MemoryPool) gets by backing it with that pool."""
 
-    pool = None
-    pool_base = 0
-    stride = 0
-    next_slot = 0
-    SLOTS = 8
+    handle = None
+    next_lane = 0
 
     def __init__(self, torch, sizes_bytes):
         from eridiffusion_amd import _lib as L
-        cls = Spread
+        cls = Pool
         self.offsets = []
         total = 0
         for b in sizes_bytes:
             self.offsets.append(total)
             total += align(b)
         self.nbytes = max(total, 256)
-        if cls.pool is None:
-            free, _ = torch.cuda.mem_get_info()
-            cls.stride = int(free * 0.92) // cls.SLOTS // (2 << 20) * (2 << 20)
-            cls.pool = torch.empty(cls.stride * cls.SLOTS, dtype=torch.uint8, device="cuda:0")
-            cls.pool_base = cls.pool.data_ptr()
-            cls.next_slot = 0
-        if self.nbytes > cls.stride or cls.next_slot >= cls.SLOTS:
-            sys.exit("--alloc spread: this workload's arrays do not fit an eighth of the device memory each")
-        self.base = cls.pool_base + cls.next_slot * cls.stride
-        cls.next_slot += 1
-        # the library's allocator hands out zeroed memory; so does this one
-        cls.pool[self.base - cls.pool_base:self.base - cls.pool_base + self.nbytes].zero_()
+        if cls.handle is None:
+            cls.handle = C.c_void_p()
+            L.check(L.lib().eri_hip_pool_create(0, 0, 0, C.byref(cls.handle)), "eri_hip_pool_create")
+        out = C.c_void_p()
+        lanes = C.c_uint32()
+        L.check(L.lib().eri_hip_pool_info(cls.handle, C.byref(lanes), None), "eri_hip_pool_info")
+        for attempt in range(lanes.value):  # the next lane, or the first one after it that still has room
+            rc = L.lib().eri_hip_pool_alloc_zeroed(cls.handle, cls.next_lane + attempt, self.nbytes, C.byref(out))
+            if rc == 0:
+                break
+        L.check(rc, "eri_hip_pool_alloc_zeroed")
+        cls.next_lane += 1
+        self.base = out.value
 
     def free(self):
-        pass  # the pool goes with the process
+        pass  # pieces go back with the pool, the pool with the process
 
 
 def cpu_baseline(tensors, bf16, sample_params, hyper_args):
@@ -228,7 +227,7 @@ def main():
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream().cuda_stream
 
-    Alloc = {"arena": Arena, "tensor": PerTensor, "spread": Spread}[args.alloc]
+    Alloc = {"arena": Arena, "tensor": PerTensor, "pool": Pool}[args.alloc]
     a_p = Alloc(torch, [n * esz for n in sizes])
     a_g = Alloc(torch, [n * gsz for n in sizes])
     a_m = Alloc(torch, sizes)
@@ -305,6 +304,8 @@ def main():
         L.check(L.lib().eri_adam8bit_new(handles, len(sizes), C.byref(cfg), stream, C.byref(obj_opt)), "adam8bit_new")
         if args.flags:
             L.check(L.lib().eri_adam8bit_set_flags(obj_opt, args.flags), "set_flags")
+        if args.alloc == "pool":  # the optimizer's own states out of the lane of the first-moment arena
+            L.check(L.lib().eri_adam8bit_set_state_pool(obj_opt, Pool.handle, 2), "set_state_pool")
     elif args.api != "table":
         if args.kernel != "adam8":
             sys.exit("--api functional runs the 8-bit step only")

@@ -80,6 +80,12 @@ EXPORTS = {
     "eri_hip_stream_sync": (C.c_int, [C.c_void_p]),
     "eri_hip_stream_destroy": (C.c_int, [C.c_void_p]),
     "eri_hip_mem_info": (C.c_int, [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
+    "eri_hip_pool_create": (C.c_int, [C.c_int, C.c_size_t, C.c_uint32, C.POINTER(C.c_void_p)]),
+    "eri_hip_pool_alloc_zeroed": (C.c_int, [C.c_void_p, C.c_uint32, C.c_size_t, C.POINTER(C.c_void_p)]),
+    "eri_hip_pool_info": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint32), C.POINTER(C.c_size_t)]),
+    "eri_hip_pool_lane_used": (C.c_int, [C.c_void_p, C.c_uint32, C.POINTER(C.c_size_t)]),
+    "eri_hip_pool_reset": (C.c_int, [C.c_void_p]),
+    "eri_hip_pool_destroy": (C.c_int, [C.c_void_p]),
     "eri_adam8_init": (C.c_int, []),
     "eri_adam8_get_maps": (C.c_int, [C.c_void_p, C.c_void_p]),
     "eri_adam8_table_image": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_size_t), C.POINTER(C.c_uint32)]),
@@ -122,6 +128,7 @@ EXPORTS = {
     "eri_adam8bit_set_param_grad_scale": (C.c_int, [C.c_void_p, C.c_uint32, C.c_float]),
     "eri_adam8bit_attach_ema": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(C.c_char_p), C.c_uint32]),
     "eri_adam8bit_set_min_8bit_size": (C.c_int, [C.c_void_p, C.c_uint64]),
+    "eri_adam8bit_set_state_pool": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint32]),
     "eri_adam8bit_state32_ptrs": (C.c_int, [C.c_void_p, C.c_uint32, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p)]),
     "eri_adam8bit_set_max_grad_norm": (C.c_int, [C.c_void_p, C.c_float, C.c_float]),
     "eri_ema_new": (C.c_int, [C.c_float, C.c_int, C.c_float, C.c_void_p, C.POINTER(C.c_void_p)]),
@@ -152,6 +159,7 @@ EXPORTS = {
     "eri_adam8bit_fn_destroy": (C.c_int, [C.c_void_p]),
     "eri_adam8bit_fn_update": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_uint64, C.c_int, C.c_int, C.c_void_p]),
     "eri_adam8bit_fn_set_batching": (C.c_int, [C.c_void_p, C.c_int]),
+    "eri_adam8bit_fn_set_state_pool": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint32]),
     "eri_adam8bit_fn_flush": (C.c_int, [C.c_void_p]),
     "eri_adam8bit_fn_update_many": (C.c_int, [C.c_void_p, C.POINTER(C.c_char_p), C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),
                                               C.POINTER(C.c_uint64), C.POINTER(C.c_int32), C.POINTER(C.c_int32),

@@ -38,6 +38,38 @@ def _stream_ptr() -> int:
     return torch.cuda.current_stream().cuda_stream
 
 
+class DevicePool:
+    """One device allocation cut into equal lanes (eri_hip_pool_*): tensors of different kinds taken from
+    different lanes lie far apart in device memory, which is what the optimizer step wants of its 8-bit states
+    and the parameters.  alloc() returns a zero-filled torch tensor viewing pool memory; the pool must outlive it."""
+
+    def __init__(self, nbytes: int = 0, lanes: int = 0, device: int = 0):
+        self._pool = C.c_void_p()
+        check(lib().eri_hip_pool_create(device, nbytes, lanes, C.byref(self._pool)), "eri_hip_pool_create")
+        n, b = C.c_uint32(), C.c_size_t()
+        check(lib().eri_hip_pool_info(self._pool, C.byref(n), C.byref(b)), "eri_hip_pool_info")
+        self.lanes, self.lane_bytes = n.value, b.value
+
+    def alloc_ptr(self, lane: int, nbytes: int) -> int:
+        out = C.c_void_p()
+        check(lib().eri_hip_pool_alloc_zeroed(self._pool, lane, nbytes, C.byref(out)), "eri_hip_pool_alloc_zeroed")
+        return out.value
+
+    def reset(self) -> None:
+        check(lib().eri_hip_pool_reset(self._pool), "eri_hip_pool_reset")
+
+    def close(self) -> None:
+        if self._pool:
+            lib().eri_hip_pool_destroy(self._pool)
+            self._pool = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 @dataclass
 class Adam8bitConfig:
     """adam8bit_enhanced.rs:372-395; amsgrad, block_wise and percentile_clipping are carried only."""
@@ -112,6 +144,11 @@ class Adam8bit:
     def set_mode(self, mode: int) -> None:
         """MODE_ERI (the reference's update, default) or MODE_BNB."""
         check(lib().eri_adam8bit_set_mode(self._opt, mode), "eri_adam8bit_set_mode")
+
+    def set_state_pool(self, pool: Optional[DevicePool], lane: int = 0) -> None:
+        """States created from now on (at the first step of their parameter) come out of `lane` of the pool."""
+        check(lib().eri_adam8bit_set_state_pool(self._opt, pool._pool if pool else None, lane), "eri_adam8bit_set_state_pool")
+        self._pool = pool  # keeps the pool alive as long as the optimizer
 
     def attach_ema(self, ema: Optional["EMAModel"], names: Optional[List[str]] = None) -> None:
         """From now on every step() also performs ema.update() over this optimizer's parameters (names[i] is the
@@ -199,6 +236,11 @@ class Adam8bitFunctional:
     @classmethod
     def with_params(cls, learning_rate, beta1, beta2, eps, weight_decay):
         return cls(learning_rate, beta1, beta2, eps, weight_decay)
+
+    def set_state_pool(self, pool: Optional[DevicePool], lane: int = 0) -> None:
+        """States of names not seen yet come out of `lane` of the pool."""
+        check(lib().eri_adam8bit_fn_set_state_pool(self._opt, pool._pool if pool else None, lane), "eri_adam8bit_fn_set_state_pool")
+        self._pool = pool
 
     def step(self) -> None:
         check(lib().eri_adam8bit_fn_step(self._opt), "eri_adam8bit_fn_step")

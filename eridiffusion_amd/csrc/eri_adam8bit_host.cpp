@@ -40,14 +40,15 @@ int fail(int code, const std::string &msg) {
     return code;
 }
 
-/* uint8 codes and per-block absmax of both moments, in one device allocation. */
+/* uint8 codes and per-block absmax of both moments, in one device allocation or one piece of a memory pool. */
 struct State8 {
     void *base = nullptr;
+    bool pooled = false; // the piece belongs to a pool and goes back with it
     uint8_t *m = nullptr, *v = nullptr;
     float *absmax_m = nullptr, *absmax_v = nullptr;
     uint64_t numel = 0;
 
-    int allocate(uint64_t n, void *stream) {
+    int allocate(uint64_t n, void *stream, EriHipPool *pool = nullptr, uint32_t lane = 0) {
         release();
         const uint64_t nb = blocks_of(n);
         const uint64_t o_v = align256(n), o_am = o_v + align256(n), o_av = o_am + align256(nb * 4);
@@ -55,8 +56,9 @@ struct State8 {
         int dev = 0;
         int rc = eri_hip_get_device(&dev);
         if (rc) return rc;
-        rc = eri_hip_malloc_zeroed(dev, total, &base);
+        rc = pool ? eri_hip_pool_alloc_zeroed(pool, lane, total, &base) : eri_hip_malloc_zeroed(dev, total, &base);
         if (rc) return rc;
+        pooled = pool != nullptr;
         char *b = static_cast<char *>(base);
         m = reinterpret_cast<uint8_t *>(b);
         v = reinterpret_cast<uint8_t *>(b + o_v);
@@ -67,8 +69,9 @@ struct State8 {
         return eri_adam8_state_init(m, v, absmax_m, absmax_v, n, stream);
     }
     void release() {
-        if (base) eri_hip_free(base);
+        if (base && !pooled) eri_hip_free(base);
         base = nullptr;
+        pooled = false;
         m = v = nullptr;
         absmax_m = absmax_v = nullptr;
         numel = 0;
@@ -396,6 +399,8 @@ struct EriAdam8bit {
     EriEmaModel *ema = nullptr;                   // attached EMA model (not owned), updated inside step()
     std::vector<std::string> ema_names;           // its name for each parameter
     void *stream = nullptr;
+    EriHipPool *state_pool = nullptr;        // where states not yet created will come from (not owned)
+    uint32_t state_lane = 0;
     EriAdam8Table *table = nullptr;
     std::vector<uint32_t> table_ids;         // parameter indices the table was built for
     std::vector<EriAdam8Tensor> table_rows;  // rows as last uploaded
@@ -417,6 +422,8 @@ struct EriAdam8bitFn {
     double lr = 1e-4, beta1 = 0.9, beta2 = 0.999, eps = 1e-8, wd = 0.01;
     uint64_t step = 0;
     void *stream = nullptr;
+    EriHipPool *state_pool = nullptr; // where states not yet created will come from (not owned)
+    uint32_t state_lane = 0;
     std::map<std::string, std::unique_ptr<FnState>, std::less<>> states;
     // Batching: update() calls queue rows, one launch over all of them runs at the next flush.
     bool batching = false;
@@ -600,7 +607,7 @@ static int adam8bit_step_impl(EriAdam8bit *o, uint32_t *skipped) {
         }
         if (!o->states[i]) { // init_state :179-199
             std::unique_ptr<State8> s(new State8());
-            int rc = s->allocate(p->numel, o->stream);
+            int rc = s->allocate(p->numel, o->stream, o->state_pool, o->state_lane);
             if (rc) return rc;
             o->states[i] = std::move(s);
         }
@@ -830,6 +837,13 @@ int eri_adam8bit_attach_ema(EriAdam8bit *o, EriEmaModel *ema, const char *const 
     return 0;
 }
 
+int eri_adam8bit_set_state_pool(EriAdam8bit *o, EriHipPool *pool, uint32_t lane) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    o->state_pool = pool;
+    o->state_lane = lane;
+    return 0;
+}
+
 int eri_adam8bit_set_min_8bit_size(EriAdam8bit *o, uint64_t numel) {
     if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
     o->min_8bit_size = numel;
@@ -974,7 +988,7 @@ int eri_adam8bit_load_state(EriAdam8bit *o, const char *path) {
         int rc = bounce.ensure();
         if (rc) return rc;
         std::unique_ptr<State8> s(new State8());
-        rc = s->allocate(o->params[it.idx]->numel, o->stream);
+        rc = s->allocate(o->params[it.idx]->numel, o->stream, o->state_pool, o->state_lane);
         if (rc) return rc;
         void *dst[4] = {s->m, s->v, s->absmax_m, s->absmax_v};
         for (int k = 0; k < 4; ++k) {
@@ -1158,7 +1172,7 @@ extern "C" int eri_adam8bit_load_legacy_state(EriAdam8bit *o, const char *path) 
     for (auto &it : items) {
         const uint64_t n = o->params[it.idx]->numel;
         std::unique_ptr<State8> s(new State8());
-        rc = s->allocate(n, o->stream);
+        rc = s->allocate(n, o->stream, o->state_pool, o->state_lane);
         for (int k = 0; k < 2 && rc == 0; ++k) {
             const LegacyTensor *src = k == 0 ? it.m : it.v;
             const uint64_t piece = Bounce::kHalf / 4;
@@ -1231,7 +1245,7 @@ int fn_state_of(EriAdam8bitFn *o, const char *name, uint64_t numel, size_t hint,
         auto it = o->states.find(std::string_view(name));
         if (it == o->states.end()) {
             std::unique_ptr<FnState> s(new FnState());
-            int rc = s->allocate(numel, o->stream);
+            int rc = s->allocate(numel, o->stream, o->state_pool, o->state_lane);
             if (rc) return rc;
             it = o->states.emplace(name, std::move(s)).first;
         }
@@ -1391,6 +1405,13 @@ int eri_adam8bit_fn_update_many(EriAdam8bitFn *o, const char *const *names, cons
     return fn_flush(o);
 }
 
+int eri_adam8bit_fn_set_state_pool(EriAdam8bitFn *o, EriHipPool *pool, uint32_t lane) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    o->state_pool = pool;
+    o->state_lane = lane;
+    return 0;
+}
+
 int eri_adam8bit_fn_set_batching(EriAdam8bitFn *o, int enabled) {
     if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
     if (!enabled) {
@@ -1458,7 +1479,7 @@ int eri_adam8bit_fn_load_state_fp32(EriAdam8bitFn *o, const char *name, const fl
     if (rc) return rc;
     o->last_order.clear(); // it may hold the state that is replaced below
     std::unique_ptr<FnState> s(new FnState());
-    rc = s->allocate(numel, o->stream);
+    rc = s->allocate(numel, o->stream, o->state_pool, o->state_lane);
     if (rc) return rc;
     rc = eri_adam8_quantize(m, 1, numel, s->m, s->absmax_m, o->stream);
     if (rc) return rc;

@@ -499,6 +499,107 @@ int eri_hip_free(void *ptr) {
     return 0;
 }
 
+} // extern "C"
+
+struct EriHipPool {
+    int device = 0;
+    char *base = nullptr;
+    size_t lane_bytes = 0;
+    std::vector<size_t> used; // per lane
+    std::mutex lock;
+};
+
+extern "C" {
+
+int eri_hip_pool_create(int device, size_t bytes, uint32_t lanes, EriHipPool **out) {
+    if (!out) return fail(ERI_ERR_NULL, "out is NULL");
+    *out = nullptr;
+    int prev = 0;
+    ERI_HIP(hipGetDevice(&prev));
+    if (prev != device) ERI_HIP(hipSetDevice(device));
+    hipError_t e = hipSuccess;
+    if (bytes == 0) {
+        size_t free_b = 0, total_b = 0;
+        e = hipMemGetInfo(&free_b, &total_b);
+        bytes = free_b / 10 * 9;
+    }
+    constexpr size_t kGrain = (size_t)2 << 20;       // lanes start on 2 MiB boundaries
+    constexpr size_t kDefaultLane = (size_t)48 << 30; // the distance at which the step ran fastest
+    size_t lane_bytes;
+    if (lanes == 0) { // as many 48 GiB lanes as fit; a smaller pool is one lane
+        lanes = (uint32_t)(bytes / kDefaultLane);
+        lane_bytes = lanes ? kDefaultLane : bytes / kGrain * kGrain;
+        if (lanes == 0) lanes = 1;
+    } else {
+        lane_bytes = bytes / lanes / kGrain * kGrain;
+    }
+    void *p = nullptr;
+    if (e == hipSuccess && lane_bytes == 0) e = hipErrorInvalidValue;
+    if (e == hipSuccess) e = hipMalloc(&p, lane_bytes * lanes);
+    if (prev != device) (void)hipSetDevice(prev);
+    if (e != hipSuccess) return hip_fail(e, "memory pool allocation");
+    EriHipPool *pool = new EriHipPool();
+    pool->device = device;
+    pool->base = static_cast<char *>(p);
+    pool->lane_bytes = lane_bytes;
+    pool->used.assign(lanes, 0);
+    *out = pool;
+    return 0;
+}
+
+int eri_hip_pool_alloc_zeroed(EriHipPool *pool, uint32_t lane, size_t bytes, void **out) {
+    if (!pool || !out) return fail(ERI_ERR_NULL, "pool or out is NULL");
+    *out = nullptr;
+    if (bytes == 0) return fail(ERI_ERR_EMPTY, "pool allocation of zero bytes");
+    const size_t need = (bytes + 255) / 256 * 256;
+    char *p = nullptr;
+    {
+        std::lock_guard<std::mutex> g(pool->lock);
+        lane %= (uint32_t)pool->used.size();
+        if (need > pool->lane_bytes - pool->used[lane])
+            return fail(ERI_ERR_ARG, "memory pool: the lane is full");
+        p = pool->base + (size_t)lane * pool->lane_bytes + pool->used[lane];
+        pool->used[lane] += need;
+    }
+    int prev = 0;
+    ERI_HIP(hipGetDevice(&prev));
+    if (prev != pool->device) ERI_HIP(hipSetDevice(pool->device));
+    const hipError_t e = hipMemset(p, 0, bytes);
+    if (prev != pool->device) (void)hipSetDevice(prev);
+    if (e != hipSuccess) return hip_fail(e, "hipMemset");
+    *out = p;
+    return 0;
+}
+
+int eri_hip_pool_info(const EriHipPool *pool, uint32_t *lanes, size_t *lane_bytes) {
+    if (!pool) return fail(ERI_ERR_NULL, "pool is NULL");
+    if (lanes) *lanes = (uint32_t)pool->used.size();
+    if (lane_bytes) *lane_bytes = pool->lane_bytes;
+    return 0;
+}
+
+int eri_hip_pool_lane_used(const EriHipPool *pool, uint32_t lane, size_t *used_bytes) {
+    if (!pool || !used_bytes) return fail(ERI_ERR_NULL, "pool or used_bytes is NULL");
+    std::lock_guard<std::mutex> g(const_cast<EriHipPool *>(pool)->lock);
+    *used_bytes = pool->used[lane % pool->used.size()];
+    return 0;
+}
+
+int eri_hip_pool_reset(EriHipPool *pool) {
+    if (!pool) return fail(ERI_ERR_NULL, "pool is NULL");
+    std::lock_guard<std::mutex> g(pool->lock);
+    for (auto &u : pool->used) u = 0;
+    return 0;
+}
+
+int eri_hip_pool_destroy(EriHipPool *pool) {
+    if (!pool) return 0;
+    const hipError_t e = hipFree(pool->base);
+    delete pool;
+    if (e != hipSuccess) return hip_fail(e, "hipFree");
+    return 0;
+}
+
 void *eri_hip_host_alloc(size_t bytes) {
     void *p = nullptr;
     hipError_t e = hipHostMalloc(&p, bytes, hipHostMallocPortable);

@@ -61,6 +61,7 @@ pub struct EriOptimizerMemoryReport { pub num_params: u64, pub param_memory_gb: 
 
 pub enum EriEmaModel {}
 pub enum EriAdam8Table {}
+pub enum EriHipPool {}
 pub enum EriParameter {}
 pub enum EriAdam8bit {}
 pub enum EriAdam8bitFn {}
@@ -82,6 +83,12 @@ extern "C" {
     pub fn eri_hip_stream_sync(stream: *mut c_void) -> c_int;
     pub fn eri_hip_stream_destroy(stream: *mut c_void) -> c_int;
     pub fn eri_hip_mem_info(free_bytes: *mut usize, total_bytes: *mut usize) -> c_int;
+    pub fn eri_hip_pool_create(device: c_int, bytes: usize, lanes: u32, out: *mut *mut EriHipPool) -> c_int;
+    pub fn eri_hip_pool_alloc_zeroed(pool: *mut EriHipPool, lane: u32, bytes: usize, out: *mut *mut c_void) -> c_int;
+    pub fn eri_hip_pool_info(pool: *const EriHipPool, lanes: *mut u32, lane_bytes: *mut usize) -> c_int;
+    pub fn eri_hip_pool_lane_used(pool: *const EriHipPool, lane: u32, used_bytes: *mut usize) -> c_int;
+    pub fn eri_hip_pool_reset(pool: *mut EriHipPool) -> c_int;
+    pub fn eri_hip_pool_destroy(pool: *mut EriHipPool) -> c_int;
     // the step
     pub fn eri_adam8_init() -> c_int;
     pub fn eri_adam8_get_maps(signed256: *mut f32, unsigned256: *mut f32) -> c_int;
@@ -125,6 +132,7 @@ extern "C" {
     pub fn eri_adam8bit_set_param_grad_scale(opt: *mut EriAdam8bit, index: u32, scale: f32) -> c_int;
     pub fn eri_adam8bit_attach_ema(opt: *mut EriAdam8bit, ema: *mut EriEmaModel, names: *const *const c_char, n: u32) -> c_int;
     pub fn eri_adam8bit_set_min_8bit_size(opt: *mut EriAdam8bit, numel: u64) -> c_int;
+    pub fn eri_adam8bit_set_state_pool(opt: *mut EriAdam8bit, pool: *mut EriHipPool, lane: u32) -> c_int;
     pub fn eri_adam8bit_state32_ptrs(opt: *const EriAdam8bit, index: u32, m: *mut *mut f32, v: *mut *mut f32) -> c_int;
     pub fn eri_adam8bit_set_max_grad_norm(opt: *mut EriAdam8bit, max_norm: f32, denom_eps: f32) -> c_int;
     pub fn eri_ema_new(decay: f32, use_bias_correction: c_int, power: f32, stream: *mut c_void, out: *mut *mut EriEmaModel) -> c_int;
@@ -155,6 +163,7 @@ extern "C" {
     pub fn eri_adam8bit_fn_destroy(opt: *mut EriAdam8bitFn) -> c_int;
     pub fn eri_adam8bit_fn_update(opt: *mut EriAdam8bitFn, name: *const c_char, param: *const c_void, grad: *const c_void, numel: u64, dtype_tag: c_int, grad_dtype_tag: c_int, out: *mut c_void) -> c_int;
     pub fn eri_adam8bit_fn_set_batching(opt: *mut EriAdam8bitFn, enabled: c_int) -> c_int;
+    pub fn eri_adam8bit_fn_set_state_pool(opt: *mut EriAdam8bitFn, pool: *mut EriHipPool, lane: u32) -> c_int;
     pub fn eri_adam8bit_fn_flush(opt: *mut EriAdam8bitFn) -> c_int;
     pub fn eri_adam8bit_fn_update_many(opt: *mut EriAdam8bitFn, names: *const *const c_char, params: *const *const c_void, grads: *const *const c_void, numels: *const u64, dtype_tags: *const i32, grad_dtype_tags: *const i32, outs: *const *mut c_void, n: u32) -> c_int;
     pub fn eri_adam8bit_fn_step(opt: *mut EriAdam8bitFn) -> c_int;

@@ -1,0 +1,136 @@
+"""The lane pool of the storage seam and the optimizers' states inside it."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import harness as hs
+import oracle_c as oc
+from oracle import adam8_numpy as onp
+
+pytestmark = pytest.mark.gpu
+LR, B1, B2, EPS, WD = 1e-3, 0.9, 0.999, 1e-8, 0.01
+MiB = 1 << 20
+
+
+def _L():
+    from eridiffusion_amd import _lib
+    return _lib
+
+
+def _pool(nbytes, lanes):
+    L = _L()
+    h = C.c_void_p()
+    L.check(L.lib().eri_hip_pool_create(0, nbytes, lanes, C.byref(h)), "pool_create")
+    return h
+
+
+def test_lanes_are_equal_parts_of_one_allocation_and_pieces_come_zeroed():
+    import torch
+    L = _L()
+    pool = _pool(64 * MiB, 4)
+    lanes, lane_bytes = C.c_uint32(), C.c_size_t()
+    L.check(L.lib().eri_hip_pool_info(pool, C.byref(lanes), C.byref(lane_bytes)), "pool_info")
+    assert lanes.value == 4 and lane_bytes.value == 16 * MiB
+    a, b, c, d = (C.c_void_p() for _ in range(4))
+    L.check(L.lib().eri_hip_pool_alloc_zeroed(pool, 0, 1000, C.byref(a)), "alloc")
+    L.check(L.lib().eri_hip_pool_alloc_zeroed(pool, 0, 5, C.byref(b)), "alloc")
+    L.check(L.lib().eri_hip_pool_alloc_zeroed(pool, 3, 4 * MiB, C.byref(c)), "alloc")
+    L.check(L.lib().eri_hip_pool_alloc_zeroed(pool, 6, 256, C.byref(d)), "alloc")  # lane 6 of 4 is lane 2
+    assert b.value - a.value == 1024 and a.value % 256 == 0          # 256-byte steps inside a lane
+    assert c.value - a.value == 3 * lane_bytes.value                 # lanes are lane_bytes apart
+    assert d.value - a.value == 2 * lane_bytes.value
+    used = C.c_size_t()
+    L.check(L.lib().eri_hip_pool_lane_used(pool, 0, C.byref(used)), "lane_used")
+    assert used.value == 1024 + 256
+    # dirty a piece, reset, take it again: zero-filled again
+    host = np.full(4 * MiB, 0xAB, np.uint8)
+    L.check(L.lib().eri_hip_memcpy_async(c.value, host.ctypes.data, host.size, 1, None), "memcpy")
+    torch.cuda.synchronize()
+    L.check(L.lib().eri_hip_pool_reset(pool), "reset")
+    e = C.c_void_p()
+    L.check(L.lib().eri_hip_pool_alloc_zeroed(pool, 3, 4 * MiB, C.byref(e)), "alloc")
+    assert e.value == c.value
+    back = np.empty(4 * MiB, np.uint8)
+    L.check(L.lib().eri_hip_memcpy_async(back.ctypes.data, e.value, back.size, 2, None), "memcpy")
+    torch.cuda.synchronize()
+    assert not back.any()
+    # a lane that is full says so and leaves the pool usable
+    f = C.c_void_p()
+    assert L.lib().eri_hip_pool_alloc_zeroed(pool, 3, 13 * MiB, C.byref(f)) == -6
+    assert b"lane is full" in L.lib().eri_last_error()
+    L.check(L.lib().eri_hip_pool_alloc_zeroed(pool, 3, 12 * MiB, C.byref(f)), "alloc")
+    assert L.lib().eri_hip_pool_alloc_zeroed(None, 0, 16, C.byref(f)) == -1
+    assert L.lib().eri_hip_pool_alloc_zeroed(pool, 0, 0, C.byref(f)) == -3
+    L.check(L.lib().eri_hip_pool_destroy(pool), "destroy")
+
+
+@pytest.mark.parametrize("bf16", [True, False])
+def test_list_optimizer_with_pooled_states_matches_the_oracle(bf16):
+    """The same steps as with states of its own allocation: bit-exact states and (exact flag) parameters; the state
+    pointers lie inside the lane that was named."""
+    import torch
+    from eridiffusion_amd.adam8bit import Adam8bit, Adam8bitConfig, DevicePool
+    L = _L()
+    sizes = [2048 * 5 + 77, 300, 2048 * 2, 4099]
+    ps, gs = hs.make_inputs(sizes, bf16, 321)
+    states = hs.oracle_states(sizes)
+    dt = torch.bfloat16 if bf16 else torch.float32
+    to_t = lambda a: (torch.from_numpy(a.view(np.int16)).cuda().view(torch.bfloat16) if bf16 else torch.from_numpy(a.copy()).cuda())
+    params = [to_t(p) for p in ps]
+    pool = DevicePool(48 * MiB, 3)
+    opt = Adam8bit(params, Adam8bitConfig(lr=LR, betas=(B1, B2), eps=EPS, weight_decay=WD), flags=L.FLAG_EXACT_PARAM)
+    opt.set_state_pool(pool, 2)
+    for t in (1, 2, 3):
+        g_t = hs.fresh_grads(sizes, bf16, 400 + t, 1e-3)
+        for p, g in zip(params, g_t):
+            p.grad = to_t(g)
+        opt.step()
+        hs.oracle_step(ps, g_t, states, (LR, B1, B2, EPS, WD, t), bf16)
+    torch.cuda.synchronize()
+    lane0 = pool.alloc_ptr(0, 256)
+    for i, n in enumerate(sizes):
+        ptrs = [C.c_void_p() for _ in range(4)]
+        L.check(L.lib().eri_adam8bit_state_ptrs(opt._opt, i, *[C.byref(q) for q in ptrs]), "state_ptrs")
+        nb = (n + 2047) // 2048
+        arrs = []
+        for q, (cnt, dtp) in zip(ptrs, ((n, np.uint8), (n, np.uint8), (nb, np.float32), (nb, np.float32))):
+            host = np.empty(cnt, dtp)
+            L.check(L.lib().eri_hip_memcpy_async(host.ctypes.data, q.value, host.nbytes, 2, None), "d2h")
+            L.check(L.lib().eri_hip_stream_sync(None), "sync")
+            arrs.append(host)
+        m, v, am, av = arrs
+        assert np.array_equal(m, states[i][0]) and np.array_equal(v, states[i][1])
+        assert np.array_equal(am.view(np.uint32), states[i][2].view(np.uint32))
+        assert np.array_equal(av.view(np.uint32), states[i][3].view(np.uint32))
+        got = params[i].view(torch.int16).cpu().numpy().view(np.uint16) if bf16 else params[i].cpu().numpy()
+        assert np.array_equal(got.view(np.uint16 if bf16 else np.uint32), ps[i].view(np.uint16 if bf16 else np.uint32))
+        ptr = ptrs[0].value
+        assert lane0 + 2 * pool.lane_bytes <= ptr < lane0 + 3 * pool.lane_bytes
+    del opt
+    pool.close()
+
+
+def test_functional_optimizer_with_pooled_states_matches_the_oracle():
+    import torch
+    from eridiffusion_amd.adam8bit import Adam8bitFunctional, DevicePool
+    sizes = [2048 * 3 + 9, 640 * 16, 77]
+    ps, _ = hs.make_inputs(sizes, True, 654)
+    states = hs.oracle_states(sizes)
+    to_t = lambda a: torch.from_numpy(a.view(np.int16)).cuda().view(torch.bfloat16)
+    cur = {"t%d" % i: to_t(p) for i, p in enumerate(ps)}
+    pool = DevicePool(32 * MiB, 2)
+    opt = Adam8bitFunctional(LR, B1, B2, EPS, WD, batched=True)
+    opt.set_state_pool(pool, 1)
+    for t in range(3):
+        g_t = hs.fresh_grads(sizes, True, 700 + t, 1e-3)
+        grads = {"t%d" % i: to_t(g) for i, g in enumerate(g_t)}
+        cur = opt.update_many(cur, grads)
+        opt.step()
+        hs.oracle_step(ps, g_t, states, (LR, B1, B2, EPS, WD, t), True, oc.MODE_L2)
+    torch.cuda.synchronize()
+    for i in range(len(sizes)):
+        got = cur["t%d" % i].view(torch.int16).cpu().numpy().view(np.uint16)
+        assert np.array_equal(got, ps[i])
+    del opt
+    pool.close()
