@@ -48,11 +48,13 @@ def parse():
                     help="parameter dtype: the one the configuration names, or an override (the shapes stay)")
     ap.add_argument("--grad-dtype", choices=["param", "f32"], default="param",
                     help="gradient dtype: the parameter's, or fp32 gradients (for bf16 parameters: read unrounded)")
-    ap.add_argument("--alloc", choices=["arena", "tensor", "pool"], default="arena",
-                    help="arena: one flat allocation per kind of buffer (eri_hip_malloc_zeroed).  tensor: one torch "
-                         "allocation per tensor and buffer (how a tensor runtime holds parameters and states).  pool: "
-                         "the flat buffers out of the library's lane pool (eri_hip_pool_*), one 48 GiB lane per kind, "
-                         "which keeps the 8-bit states far from the parameters in device memory")
+    ap.add_argument("--alloc", choices=["pool", "arena", "tensor"], default="pool",
+                    help="pool: one flat buffer per kind of array out of the library's lane pool (eri_hip_pool_*), one "
+                         "48 GiB lane per kind, which keeps the 8-bit states far from the parameters in device memory "
+                         "and the placement the same in every process; if the pool cannot be created the run goes on "
+                         "as arena and says so.  arena: the same flat buffers, each a device allocation of its own "
+                         "(eri_hip_malloc_zeroed).  tensor: one torch allocation per tensor and buffer (how a tensor "
+                         "runtime holds parameters and states)")
     ap.add_argument("--traffic-json", default=os.path.join(ROOT, "profiles", "traffic.json"),
                     help="HBM bytes per launch derived from rocprofv3 --pmc runs, if present")
     return ap.parse_args()
@@ -127,8 +129,7 @@ class Pool(Arena):
             total += align(b)
         self.nbytes = max(total, 256)
         if cls.handle is None:
-            cls.handle = C.c_void_p()
-            L.check(L.lib().eri_hip_pool_create(0, 0, 0, C.byref(cls.handle)), "eri_hip_pool_create")
+            L.check(cls.open(), "eri_hip_pool_create")
         out = C.c_void_p()
         lanes = C.c_uint32()
         L.check(L.lib().eri_hip_pool_info(cls.handle, C.byref(lanes), None), "eri_hip_pool_info")
@@ -139,6 +140,16 @@ class Pool(Arena):
         L.check(rc, "eri_hip_pool_alloc_zeroed")
         cls.next_lane += 1
         self.base = out.value
+
+    @classmethod
+    def open(cls):
+        """Creates the pool (nine tenths of the free device memory, 48 GiB lanes); the library's return code."""
+        from eridiffusion_amd import _lib as L
+        handle = C.c_void_p()
+        rc = L.lib().eri_hip_pool_create(0, 0, 0, C.byref(handle))
+        if rc == 0:
+            cls.handle = handle
+        return rc
 
     def free(self):
         pass  # pieces go back with the pool, the pool with the process
@@ -227,6 +238,13 @@ def main():
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream().cuda_stream
 
+    if args.alloc == "pool" and args.kernel == "adamw32" and n_params * 4 > (20 << 30):
+        # fp32 moments of the large sets fill a 48 GiB lane each and leave no room for the other arrays
+        args.alloc = "arena"
+    if args.alloc == "pool" and Pool.open() != 0:
+        print("bench.py: no lane pool (%s); the flat buffers become allocations of their own (--alloc arena)"
+              % L.lib().eri_last_error().decode("utf-8", "replace"), file=sys.stderr)
+        args.alloc = "arena"
     Alloc = {"arena": Arena, "tensor": PerTensor, "pool": Pool}[args.alloc]
     a_p = Alloc(torch, [n * esz for n in sizes])
     a_g = Alloc(torch, [n * gsz for n in sizes])

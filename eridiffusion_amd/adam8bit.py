@@ -41,7 +41,8 @@ def _stream_ptr() -> int:
 class DevicePool:
     """One device allocation cut into equal lanes (eri_hip_pool_*): tensors of different kinds taken from
     different lanes lie far apart in device memory, which is what the optimizer step wants of its 8-bit states
-    and the parameters.  alloc() returns a zero-filled torch tensor viewing pool memory; the pool must outlive it."""
+    and the parameters.  alloc_ptr() returns the device address of zero-filled, 256-byte aligned pool memory; the
+    pool must outlive every use of it (an optimizer given the pool keeps it alive)."""
 
     def __init__(self, nbytes: int = 0, lanes: int = 0, device: int = 0):
         self._pool = C.c_void_p()

@@ -26,7 +26,7 @@ def test_more_than_one_gpu_is_refused_with_a_message():
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("extra", [[], ["--api", "object"], ["--api", "functional"], ["--kernel", "adam8_ema"],
-                                   ["--grad-dtype", "f32"], ["--alloc", "tensor"]])
+                                   ["--grad-dtype", "f32"], ["--alloc", "tensor"], ["--alloc", "arena"]])
 def test_one_small_run_prints_the_contract_line(extra):
     cmd = [sys.executable, BENCH, "--config", "c1_flat_fp32" if not extra or extra[0] == "--alloc" else "c2_sdxl_lora_r16",
            "--steps", "3", "--warmup", "1", "--cpu-sample", "1048576"] + extra
