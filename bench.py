@@ -49,9 +49,10 @@ def parse():
     ap.add_argument("--grad-dtype", choices=["param", "f32"], default="param",
                     help="gradient dtype: the parameter's, or fp32 gradients (for bf16 parameters: read unrounded)")
     ap.add_argument("--alloc", choices=["pool", "arena", "tensor"], default="pool",
-                    help="pool: one flat buffer per kind of array out of the library's lane pool (eri_hip_pool_*), one "
-                         "48 GiB lane per kind, which keeps the 8-bit states far from the parameters in device memory "
-                         "and the placement the same in every process; if the pool cannot be created the run goes on "
+                    help="pool: one flat buffer per kind of array out of the library's lane pool (eri_hip_pool_*): "
+                         "parameters, gradients and optimizer state each in a 48 GiB lane of their own, which keeps "
+                         "the 8-bit states far from the parameters in device memory and the placement the same in "
+                         "every process; if the pool cannot be created the run goes on "
                          "as arena and says so.  arena: the same flat buffers, each a device allocation of its own "
                          "(eri_hip_malloc_zeroed).  tensor: one torch allocation per tensor and buffer (how a tensor "
                          "runtime holds parameters and states)")
@@ -67,7 +68,7 @@ def align(n, a=256):
 class PerTensor:
     """One device allocation per tensor (how a tensor runtime holds parameters and states)."""
 
-    def __init__(self, torch, sizes_bytes):
+    def __init__(self, torch, sizes_bytes, lane=0):
         self.bufs = [torch.empty(max(b, 16), dtype=torch.uint8, device="cuda:0") for b in sizes_bytes]
 
     def ptr(self, i):
@@ -84,7 +85,7 @@ class Arena:
     """One flat device allocation per kind of buffer, from the library's allocator
     (eri_hip_malloc_zeroed); every tensor starts on a 256-byte boundary."""
 
-    def __init__(self, torch, sizes_bytes):
+    def __init__(self, torch, sizes_bytes, lane=0):
         from eridiffusion_amd import _lib as L
         self.offsets = []
         total = 0
@@ -111,15 +112,14 @@ class Arena:
 
 
 class Pool(Arena):
-    """The arenas of Arena out of the library's lane pool (eri_hip_pool_*): one device allocation, one lane per
-    kind of array -- parameters, gradients, first and second moments, anything else -- so that the 8-bit states
-    lie far from the parameters and gradients in device memory.  What a runtime with a pool allocator (the
+    """The arenas of Arena out of the library's lane pool (eri_hip_pool_*): one device allocation, one 48 GiB lane
+    per kind of tensor -- parameters, gradients, optimizer state, anything else -- so that the 8-bit states lie
+    far from the parameters and gradients in device memory.  What a runtime with a pool allocator (the
     reference's MemoryPool) gets by backing it with that pool."""
 
     handle = None
-    next_lane = 0
 
-    def __init__(self, torch, sizes_bytes):
+    def __init__(self, torch, sizes_bytes, lane=0):
         from eridiffusion_amd import _lib as L
         cls = Pool
         self.offsets = []
@@ -133,12 +133,11 @@ class Pool(Arena):
         out = C.c_void_p()
         lanes = C.c_uint32()
         L.check(L.lib().eri_hip_pool_info(cls.handle, C.byref(lanes), None), "eri_hip_pool_info")
-        for attempt in range(lanes.value):  # the next lane, or the first one after it that still has room
-            rc = L.lib().eri_hip_pool_alloc_zeroed(cls.handle, cls.next_lane + attempt, self.nbytes, C.byref(out))
+        for attempt in range(lanes.value):  # the lane of its kind, or the first one after it that still has room
+            rc = L.lib().eri_hip_pool_alloc_zeroed(cls.handle, lane + attempt, self.nbytes, C.byref(out))
             if rc == 0:
                 break
         L.check(rc, "eri_hip_pool_alloc_zeroed")
-        cls.next_lane += 1
         self.base = out.value
 
     @classmethod
@@ -246,12 +245,13 @@ def main():
               % L.lib().eri_last_error().decode("utf-8", "replace"), file=sys.stderr)
         args.alloc = "arena"
     Alloc = {"arena": Arena, "tensor": PerTensor, "pool": Pool}[args.alloc]
-    a_p = Alloc(torch, [n * esz for n in sizes])
-    a_g = Alloc(torch, [n * gsz for n in sizes])
-    a_m = Alloc(torch, sizes)
-    a_v = Alloc(torch, sizes)
-    a_am = Alloc(torch, [((n + 2047) // 2048) * 4 for n in sizes])
-    a_av = Alloc(torch, [((n + 2047) // 2048) * 4 for n in sizes])
+    LANE_PARAM, LANE_GRAD, LANE_STATE, LANE_OTHER = 0, 1, 2, 3  # the pool's lanes, one per kind of tensor
+    a_p = Alloc(torch, [n * esz for n in sizes], LANE_PARAM)
+    a_g = Alloc(torch, [n * gsz for n in sizes], LANE_GRAD)
+    a_m = Alloc(torch, sizes, LANE_STATE)
+    a_v = Alloc(torch, sizes, LANE_STATE)
+    a_am = Alloc(torch, [((n + 2047) // 2048) * 4 for n in sizes], LANE_STATE)
+    a_av = Alloc(torch, [((n + 2047) // 2048) * 4 for n in sizes], LANE_STATE)
     tdt = torch.bfloat16 if bf16 else torch.float32
     gen = torch.Generator(device="cuda:0")
     gen.manual_seed(0xE21D + 5)
@@ -274,8 +274,8 @@ def main():
     bytes_per_param = BYTES_PER_PARAM[dt_name] + (gsz - esz)
     extra = []
     if args.kernel == "adamw32":
-        a_m32 = Alloc(torch, [4 * n for n in sizes])
-        a_v32 = Alloc(torch, [4 * n for n in sizes])
+        a_m32 = Alloc(torch, [4 * n for n in sizes], LANE_STATE)
+        a_v32 = Alloc(torch, [4 * n for n in sizes], LANE_STATE)
         extra += [a_m32, a_v32]
         rows32 = (L.AdamW32Row * len(sizes))()
         for i, n in enumerate(sizes):
@@ -284,14 +284,14 @@ def main():
         h32 = L.AdamW32Hyper(1e-4, 0.9, 0.999, 1e-8, 0.01)
         bytes_per_param = 3 * esz + 16
     elif args.kernel == "adam8_ema":
-        a_sh = Alloc(torch, [n * esz for n in sizes])
+        a_sh = Alloc(torch, [n * esz for n in sizes], LANE_OTHER)
         extra.append(a_sh)
         for i in range(len(sizes)):
             rows[i].ema_shadow = a_sh.ptr(i)
         L.check(L.lib().eri_adam8_table_update(table, rows, len(rows), stream), "table_update")
         bytes_per_param += 2 * esz  # the shadow is read and written; the new parameter is still in registers
     elif args.kernel == "ema":
-        a_sh = Alloc(torch, [n * esz for n in sizes])
+        a_sh = Alloc(torch, [n * esz for n in sizes], LANE_OTHER)
         extra.append(a_sh)
         rows_e = (L.EmaRow * len(sizes))()
         for i, n in enumerate(sizes):
@@ -322,13 +322,13 @@ def main():
         L.check(L.lib().eri_adam8bit_new(handles, len(sizes), C.byref(cfg), stream, C.byref(obj_opt)), "adam8bit_new")
         if args.flags:
             L.check(L.lib().eri_adam8bit_set_flags(obj_opt, args.flags), "set_flags")
-        if args.alloc == "pool":  # the optimizer's own states out of the lane of the first-moment arena
-            L.check(L.lib().eri_adam8bit_set_state_pool(obj_opt, Pool.handle, 2), "set_state_pool")
+        if args.alloc == "pool":  # the optimizer's own states out of the state lane
+            L.check(L.lib().eri_adam8bit_set_state_pool(obj_opt, Pool.handle, LANE_STATE), "set_state_pool")
     elif args.api != "table":
         if args.kernel != "adam8":
             sys.exit("--api functional runs the 8-bit step only")
         n_t = len(sizes)
-        a_p2 = Alloc(torch, [n * esz for n in sizes])  # the other output set
+        a_p2 = Alloc(torch, [n * esz for n in sizes], LANE_OTHER)  # the other output set
         extra.append(a_p2)
         fn_opt = C.c_void_p()
         L.check(L.lib().eri_adam8bit_fn_with_params(*hyper_args, stream, C.byref(fn_opt)), "fn_with_params")

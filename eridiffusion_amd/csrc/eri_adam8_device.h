@@ -39,7 +39,7 @@ inline bool layout_grad_bf16(int layout) { return layout == kLayoutBF16; }
 /*
  * Requantisation without a search.  The quotient x = value / absmax in [-1, 1] is produced
  * already multiplied by kKeyScale (a power of two, so nothing is rounded differently), converted
- * to binary16 with round-to-nearest-even, and the top bits of that half float -- sign, exponent
+ * to binary16 rounded toward zero (both moments in one v_cvt_pkrtz_f16_f32), and the top bits of that half float -- sign, exponent
  * and the leading mantissa bits -- select a slot.  The slots are narrow enough that at most one
  * midpoint of the map lies inside any of them, so
  *     code(x) = slot.lo + (x * kKeyScale > slot.mid)

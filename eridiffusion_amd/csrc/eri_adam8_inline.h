@@ -153,9 +153,13 @@ struct Lds {
     const char *key_s, *key_u;
 };
 
-__device__ __forceinline__ uint32_t half_key(float xs) {
-    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)xs); // v_cvt_f16_f32, round to nearest even
+/* Two scaled quotients as binary16 patterns in one dword (a in the low half), rounded toward zero: a single
+ * v_cvt_pkrtz_f16_f32.  The slot tables are built for this rounding. */
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t half_key2(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a, b));
 }
+__device__ __forceinline__ uint32_t half_key(float xs) { return half_key2(xs, xs) & 0xffffu; }
 
 /* xs = kKeyScale * x.  The slot address is the half pattern with its low bits cleared. */
 __device__ __forceinline__ uint32_t code_signed_key(float xs, const char *key_s) {
@@ -481,8 +485,9 @@ __device__ __forceinline__ void requant8(const float *mf, const float *vf, const
         for (int k = 0; k < 8; ++k) {
             const float xm = dm.div_fast(mf[k]); // times kKeyScale
             const float xv = dv.div_fast(vf[k]);
-            const KeySlot sm = *reinterpret_cast<const KeySlot *>(L.key_s + (half_key(xm) & 0xfff0u));
-            const KeySlot sv = *reinterpret_cast<const KeySlot *>(L.key_u + (half_key(xv) & 0x7ff8u));
+            const uint32_t keys = half_key2(xm, xv); // both slot addresses out of one conversion
+            const KeySlot sm = *reinterpret_cast<const KeySlot *>(L.key_s + (keys & 0xfff0u));
+            const KeySlot sv = *reinterpret_cast<const KeySlot *>(L.key_u + ((keys >> 16) & 0x7ff8u));
             pack_code(am[k >> 2], k, xm, sm.mid, sm.lo);
             pack_code(av[k >> 2], k, xv, sv.mid, sv.lo);
         }

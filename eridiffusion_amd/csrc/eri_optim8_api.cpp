@@ -62,26 +62,20 @@ uint32_t count_below(const float *mid, float x) { // the definition the slots mu
     return n;
 }
 
-/* binary32 -> binary16 bit pattern, round to nearest even (what v_cvt_f16_f32 does). */
+/* binary32 -> binary16 bit pattern, rounded toward zero (what v_cvt_pkrtz_f16_f32 does). */
 uint16_t half_bits(float f) {
     uint32_t u;
     std::memcpy(&u, &f, 4);
     const uint32_t sign = (u >> 16) & 0x8000u;
     const uint32_t abs = u & 0x7fffffffu;
     if (abs > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);  // NaN
-    if (abs >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u); // rounds to infinity (>= 65520)
-    if (abs < 0x33000001u) return (uint16_t)sign;              // below half the smallest denormal
-    int exp = (int)(abs >> 23) - 127;
-    uint32_t mant = (abs & 0x7fffffu) | 0x800000u;
-    int shift = (exp < -14) ? (13 + (-14 - exp)) : 13; // bits to drop
-    uint32_t kept = mant >> shift;
-    const uint32_t rem = mant & ((1u << shift) - 1u);
-    const uint32_t half = 1u << (shift - 1);
-    if (rem > half || (rem == half && (kept & 1u))) kept += 1;
-    uint32_t out;
-    if (exp < -14) out = kept; // denormal (a carry into bit 10 becomes the smallest normal)
-    else out = ((uint32_t)(exp + 15) << 10) + (kept - 0x400u); // a mantissa carry bumps the exponent
-    return (uint16_t)(sign | out);
+    if (abs == 0x7f800000u) return (uint16_t)(sign | 0x7c00u); // infinity stays infinity
+    if (abs >= 0x477fe000u) return (uint16_t)(sign | 0x7bffu); // everything from 65504 up truncates to it
+    const int exp = (int)(abs >> 23) - 127;
+    if (exp < -24) return (uint16_t)sign;                      // below the smallest denormal
+    const uint32_t mant = (abs & 0x7fffffu) | 0x800000u;
+    if (exp < -14) return (uint16_t)(sign | (mant >> (13 + (-14 - exp)))); // denormal
+    return (uint16_t)(sign | (((uint32_t)(exp + 15) << 10) + ((mant >> 13) - 0x400u)));
 }
 
 /*

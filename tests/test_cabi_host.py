@@ -151,10 +151,12 @@ KEY_SCALE = np.float32(4096.0)
 
 def _replay(x, img, offs, signed):
     """The kernel's slot lookup (code_signed_key / code_unsigned_key), in NumPy: scale the quotient,
-    convert to binary16 (round to nearest even), mask the pattern into a byte address."""
+    convert to binary16 (rounded toward zero, as v_cvt_pkrtz_f16_f32 does), mask the pattern into a byte address."""
     xs = (x * KEY_SCALE).astype(np.float32)
     with np.errstate(over="ignore", invalid="ignore"):
-        h = xs.astype(np.float16).view(np.uint16).astype(np.uint32)
+        h16 = xs.astype(np.float16)  # nearest even; one pattern closer to zero wherever that rounded away from it
+        away = np.abs(h16.astype(np.float32)) > np.abs(xs)
+        h = (h16.view(np.uint16) - away.astype(np.uint16)).astype(np.uint32)
     addr = (h & 0xFFF0) if signed else (h & 0x7FF8)
     base = offs[4] if signed else offs[5]
     mid = np.empty(x.size, np.float32)
