@@ -313,17 +313,20 @@ __device__ __forceinline__ void adam_elem_decayed(float p, float g, float t1, fl
     } else if (MODE == ERI_ADAM8_MODE_L2) { // always to the exact chain's bits (the reference rounds the update itself)
         // fast chain: the two bias corrections as products with the rounded reciprocals, hardware square root
         // and reciprocal; param_exact redoes whatever the test below cannot vouch for
-        float mh = m * dbc1.ras;              // adam8bit.rs:170
-        float vh = fmaxf(v * dbc2.ras, 0.0f); // :178, :181-182
+        float mh = m * dbc1.ras; // adam8bit.rs:170
+        // :178; the clamp at zero (:181-182) only ever acts on NaN here (v is a sum of non-negative terms), and
+        // NaN fails the comparison below and is redone by the exact chain, clamp included
+        float vh = v * dbc2.ras;
         float den = __builtin_amdgcn_sqrtf(vh) + h.eps;
         float upd = mh * __builtin_amdgcn_rcpf(den);
         float us = upd * h.step_size;
         const float tie = u2f((f2u(us) & 0xffff0000u) | 0x8000u);
         recheck |= !(__builtin_fabsf(us - tie) > __builtin_fmaf(__builtin_fabsf(us), 0x1p-19f, 0x1p-126f));
-        // a non-zero moment near the denormal range loses relative accuracy in the product (the exact chain's
-        // division rounds on the same grid but not to the same point).  For the second moment that only shows
-        // when eps is too small to swallow its square root.  NaN and infinity fail the comparison above.
-        recheck |= (__builtin_fabsf(m) < 0x1p-100f) & (m != 0.0f);
+        // a moment near the denormal range loses relative accuracy in the product (the exact chain's division
+        // rounds on the same grid but not to the same point).  For the second moment that only shows when eps is
+        // too small to swallow its square root.  NaN and infinity fail the comparison above, and so does a
+        // zero update (the margin's floor), so a zero moment needs no exception here.
+        recheck |= __builtin_fabsf(m) < 0x1p-100f;
         if (h.eps < 0x1p-36f) recheck |= (v < 0x1p-100f) & (v != 0.0f);
         recheck |= !(dbc1.fast && dbc2.fast);
         pn = p - bf16_round(us); // :197-205
