@@ -244,6 +244,20 @@ def main():
         print("bench.py: no lane pool (%s); the flat buffers become allocations of their own (--alloc arena)"
               % L.lib().eri_last_error().decode("utf-8", "replace"), file=sys.stderr)
         args.alloc = "arena"
+    if args.alloc == "pool":  # four lanes, each wide enough for its kind of tensor (little free memory gives fewer)
+        lanes, lane_bytes = C.c_uint32(), C.c_size_t()
+        L.check(L.lib().eri_hip_pool_info(Pool.handle, C.byref(lanes), C.byref(lane_bytes)), "eri_hip_pool_info")
+        state_bytes = 2 * n_params + 8 * n_blocks + 1024 * len(sizes)
+        if args.api == "object":
+            state_bytes *= 2  # the optimizer's own states beside the (unused) flat ones
+        widest = max(n_params * max(esz, gsz) + 256 * len(sizes), state_bytes)
+        if lanes.value < 4 or widest > lane_bytes.value:
+            print("bench.py: the lane pool has %d lanes of %.1f GiB, too few or too narrow for this workload; the "
+                  "flat buffers become allocations of their own (--alloc arena)" % (lanes.value, lane_bytes.value / 2**30),
+                  file=sys.stderr)
+            L.lib().eri_hip_pool_destroy(Pool.handle)
+            Pool.handle = None
+            args.alloc = "arena"
     Alloc = {"arena": Arena, "tensor": PerTensor, "pool": Pool}[args.alloc]
     LANE_PARAM, LANE_GRAD, LANE_STATE, LANE_OTHER = 0, 1, 2, 3  # the pool's lanes, one per kind of tensor
     a_p = Alloc(torch, [n * esz for n in sizes], LANE_PARAM)
