@@ -104,13 +104,13 @@ __global__ __launch_bounds__(kPipeThreads) void ERI_PIPE_KERNEL(const DevTensor 
                                                                    const float *__restrict__ dev_scale,
                                                                    uint32_t chunks) {
     ERI_LDS_IMAGE;
-    // Where the next block's loads go out.  The instantiations of the reference's own update on bf16 parameters
-    // request each quarter of the next block as soon as the same quarter of this one has been consumed (its
-    // registers are free from then on), so every load has a whole block's time to arrive; measured 1-4 %
-    // faster on 2.6 B parameters, 1 % with fp32 gradients, 0.6-0.9 % with the exact chain, neutral on 12 B with
-    // default flags.  With the EMA or another mode inside the loop that order costs registers (12-80 bytes of
-    // scratch per lane) and time: those request the whole block after the update half.
-    constexpr bool kEarly = MODE == ERI_ADAM8_MODE_ERI && !EMA && kParamBf16;
+    // Where the next block's loads go out.  The instantiations of the reference's own update request each quarter
+    // of the next block as soon as the same quarter of this one has been consumed (its registers are free from
+    // then on), so every load has a whole block's time to arrive; measured 1-4 % faster on 2.6 B parameters,
+    // 1 % with fp32 gradients, 1.2-1.6 % with fp32 parameters, 0.6-0.9 % with the exact chain, neutral on 12 B
+    // bf16 parameters with default flags.  With the EMA or another mode inside the loop that order costs
+    // registers (12-80 bytes of scratch per lane) and time: those request the whole block after the update half.
+    constexpr bool kEarly = MODE == ERI_ADAM8_MODE_ERI && !EMA;
     // Per wave, the 2 x 256 values a state code of the block at hand can stand for, already multiplied by the
     // block's absmax and by beta: (MAP[c] * absmax) * beta, the first two operations of both moment
     // updates, done once per code (8 per lane) instead of once per element (64 per lane).
