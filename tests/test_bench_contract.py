@@ -41,6 +41,9 @@ def test_one_small_run_prints_the_contract_line(extra):
     assert d["n_gpus"] == 1 and d["steps"] == 3 and d["warmup"] == 1 and d["vs_baseline"] is None
     assert d["unit"] == "params/s" and d["higher_is_better"] is True and d["data"] == "synthetic"
     assert "workload" in d["config"] and "model" not in d["config"]
+    # the placement the run really used: the lane pool unless another was asked for (or the pool did not fit)
+    want = extra[1] if extra and extra[0] == "--alloc" else "pool"
+    assert d["config"]["alloc"] == want or (want == "pool" and d["config"]["alloc"] == "arena" and "lane pool" in out.stderr)
     r = d["roofline"]
     assert r["bound"] == "hbm" and r["peak"] == 8000.0 and r["unit"] == "GB/s"
     assert abs(r["frac"] - r["achieved"] / r["peak"]) < 1e-9 and 0 < r["frac"] < 1
