@@ -6,11 +6,18 @@ already resident in HBM.  Default workload: the FLUX-12B-shaped full fine-tune s
 tensors, 11,901,408,320 parameters, 8-bit m/v + fp32 absmax per 2048-block, ~72 GB resident).
 Prints one JSON line: params/s, the HBM roofline fraction of the step kernel (algorithmic bytes /
 measured launch duration / 8 TB/s) and, beside it, the CPU oracle timed on this host's cores.
+
+The default command also times, after the headline and in the same process, the other benchmark
+configurations and the other ways into the same step (the functional update the LoRA trainers call, the
+bit-exact flag, one allocation per tensor) and reports them as `configs`: one row each with ms per step,
+the kernel's duration and its roofline fraction.  Any other command line measures just what it names
+(`--rows all` adds the rows, `--rows none` leaves them out).
 """
 import argparse
 import ctypes as C
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -20,6 +27,25 @@ sys.path.insert(0, ROOT)
 PEAK_HBM_GBPS = 8000.0
 # algorithmic bytes per parameter: read p, g, m, v and write p, m, v, plus 16 bytes of absmax per block
 BYTES_PER_PARAM = {"bf16": 2 + 2 + 1 + 1 + 2 + 1 + 1 + 16.0 / 2048, "f32": 4 + 4 + 1 + 1 + 4 + 1 + 1 + 16.0 / 2048}
+# the type the arithmetic of each kernel is carried out in, whatever the parameters are stored as: every one of
+# them widens its inputs to fp32 and rounds each operation to fp32 (the gradient norm adds its fp32 block sums in f64)
+ARITHMETIC = {"adam8": "f32", "adam8_clip": "f32", "adam8_ema": "f32", "grad_norm": "f32", "adamw32": "f32", "ema": "f32"}
+
+HEADLINE = dict(config="c5_flux12b_full", flags=0, kernel="adam8", mode="eri", api="table", param_dtype="config",
+                grad_dtype="param", alloc="pool")
+# (what changes against the headline's options, timed steps, warm-up steps); the LoRA sets run the 100 steps
+# the benchmark configurations name
+ROWS = [
+    (dict(config="c1_flat_fp32"), 100, 10),
+    (dict(config="c2_sdxl_lora_r16"), 100, 10),
+    (dict(config="c2_sdxl_lora_r16", api="functional"), 100, 10),
+    (dict(config="c3_flux_lora_r32"), 100, 10),
+    (dict(config="c3_flux_lora_r32", api="functional"), 100, 10),
+    (dict(config="c4_sdxl_unet_full"), 20, 3),
+    (dict(config="c5_flux12b_full", flags=2), 20, 3),
+    (dict(config="c5_flux12b_full", mode="l2"), 20, 3),
+    (dict(config="c5_flux12b_full", alloc="tensor"), 20, 3),
+]
 
 
 def parse():
@@ -27,10 +53,10 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--config", default="c5_flux12b_full")
+    ap.add_argument("--config", default=HEADLINE["config"])
     ap.add_argument("--flags", type=int, default=0, help="ERI_ADAM8_FLAG_* bits for the step")
-    ap.add_argument("--cpu-sample", type=int, default=2 << 30, help="parameters in the CPU baseline sample (0 = skip)")
-    ap.add_argument("--kernel", choices=["adam8", "adam8_clip", "adam8_ema", "grad_norm", "adamw32", "ema"], default="adam8",
+    ap.add_argument("--cpu-sample", type=int, default=1 << 30, help="parameters in the CPU baseline sample (0 = skip)")
+    ap.add_argument("--kernel", choices=sorted(ARITHMETIC), default="adam8",
                     help="what one step is: the 8-bit AdamW step (headline), the same preceded by the device-side "
                          "gradient norm, the same with the EMA of the parameters taken inside it, the norm alone, "
                          "the 32-bit AdamW sibling, or the EMA sweep")
@@ -56,6 +82,11 @@ def parse():
                          "as arena and says so.  arena: the same flat buffers, each a device allocation of its own "
                          "(eri_hip_malloc_zeroed).  tensor: one torch allocation per tensor and buffer (how a tensor "
                          "runtime holds parameters and states)")
+    ap.add_argument("--rows", choices=["auto", "all", "none"], default="auto",
+                    help="the `configs` rows (the other configurations and entry points, timed after the headline in "
+                         "the same process): auto = only when the command line is the default one")
+    ap.add_argument("--rows-max-params", type=int, default=0,
+                    help="leave out the `configs` rows of configurations with more parameters than this (0 = keep all)")
     ap.add_argument("--traffic-json", default=os.path.join(ROOT, "profiles", "traffic.json"),
                     help="HBM bytes per launch derived from rocprofv3 --pmc runs, if present")
     return ap.parse_args()
@@ -142,20 +173,32 @@ class Pool(Arena):
 
     @classmethod
     def open(cls):
-        """Creates the pool (nine tenths of the free device memory, 48 GiB lanes); the library's return code."""
+        """Creates the pool (nine tenths of the free device memory, 48 GiB lanes) unless it exists; the library's
+        return code."""
         from eridiffusion_amd import _lib as L
+        if cls.handle is not None:
+            return 0
         handle = C.c_void_p()
         rc = L.lib().eri_hip_pool_create(0, 0, 0, C.byref(handle))
         if rc == 0:
             cls.handle = handle
         return rc
 
+    @classmethod
+    def close(cls):
+        from eridiffusion_amd import _lib as L
+        if cls.handle is not None:
+            L.lib().eri_hip_pool_destroy(cls.handle)
+            cls.handle = None
+
     def free(self):
-        pass  # pieces go back with the pool, the pool with the process
+        pass  # pieces go back when the pool is reset (after every measurement) or destroyed
 
 
-def cpu_baseline(tensors, bf16, sample_params, hyper_args):
-    """Times the C oracle (oracle/liberi_oracle.so) on a prefix of the same tensor list."""
+def cpu_baseline(tensors, bf16, sample_params, hyper_args, reps=5, single_thread=True):
+    """Times the C oracle (oracle/liberi_oracle.so) on a prefix of the same tensor list (the whole list when it
+    has no more than `sample_params` parameters): one untimed step that warms the pages and gives the states real
+    contents, then `reps` timed steps, the median reported."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import numpy as np
 
@@ -171,6 +214,7 @@ def cpu_baseline(tensors, bf16, sample_params, hyper_args):
         n = min(n, sample_params)
         sizes.append(n)
         total += n
+    whole = len(sizes) == len(tensors) and total == sum(numel(s) for _, s in tensors)
     rng = np.random.default_rng(7)
     tile = 1 << 22
     base_p = (rng.standard_normal(tile) * 0.02).astype(np.float32)
@@ -181,43 +225,44 @@ def cpu_baseline(tensors, bf16, sample_params, hyper_args):
     maps = oc.load_maps()
     bufs = []
     for n in sizes:
-        reps = (n + tile - 1) // tile
-        bufs.append((np.tile(base_p, reps)[:n].copy(), np.tile(base_g, reps)[:n].copy(), list(oc.state_init(n))))
+        reps_n = (n + tile - 1) // tile
+        bufs.append((np.tile(base_p, reps_n)[:n].copy(), np.tile(base_g, reps_n)[:n].copy(), list(oc.state_init(n))))
     dt_tag = oc.DT_BF16 if bf16 else oc.DT_F32
-    best = None
-    for rep in range(2):  # first pass warms the pages and gives the states real contents
+    times = []
+    for rep in range(reps + 1):
         h = oc.hyper_pack(*hyper_args[:5], rep + 1)
         t0 = time.perf_counter()
         for p, g, st in bufs:
             oc.step_tensor(p, g, *st, h, maps, dt_tag, threads)
-        dt = time.perf_counter() - t0
-        best = dt if best is None else min(best, dt)
-    # the same code on one thread, on the largest tensor of the sample only
-    big = max(range(len(sizes)), key=lambda i: sizes[i])
-    p1, g1, st1 = bufs[big]
-    n1 = min(sizes[big], 1 << 26)
-    st1 = list(oc.state_init(n1))
-    p1, g1 = p1[:n1].copy(), g1[:n1].copy()
-    single = None
-    for rep in range(2):  # the second step starts from real state contents, not from the all-zero state
-        t0 = time.perf_counter()
-        oc.step_tensor(p1, g1, *st1, oc.hyper_pack(*hyper_args[:5], rep + 1), maps, dt_tag, 1)
-        single = n1 / (time.perf_counter() - t0)
-    return {"value": total / best, "unit": "params/s", "cores": threads, "host_cores": os.cpu_count(), "kind": "port",
-            "sample": "first %d tensors of the workload (%d params), one step, C oracle with OpenMP over blocks on "
-                      "%d threads, best of 2" % (len(sizes), total, threads),
-            "single_thread_value": single,
-            "single_thread_sample": "%d params of the sample's largest tensor, second of two steps" % n1}
+        if rep > 0:
+            times.append(time.perf_counter() - t0)
+    out = {"value": total / statistics.median(times), "unit": "params/s", "cores": threads, "host_cores": os.cpu_count(),
+           "kind": "port",
+           "sample": "%s (%d tensors, %d params), C oracle with OpenMP over blocks on %d threads, one warm-up step, "
+                     "median of %d timed steps" % ("the whole workload" if whole else "the first tensors of the workload",
+                                                   len(sizes), total, threads, reps)}
+    if single_thread:  # the same code on one thread, on the largest tensor of the sample only
+        big = max(range(len(sizes)), key=lambda i: sizes[i])
+        p1, g1, st1 = bufs[big]
+        n1 = min(sizes[big], 1 << 25)
+        st1 = list(oc.state_init(n1))
+        p1, g1 = p1[:n1].copy(), g1[:n1].copy()
+        single = []
+        for rep in range(4):  # the first step starts from the all-zero state and is not timed
+            t0 = time.perf_counter()
+            oc.step_tensor(p1, g1, *st1, oc.hyper_pack(*hyper_args[:5], rep + 1), maps, dt_tag, 1)
+            if rep > 0:
+                single.append(n1 / (time.perf_counter() - t0))
+        out["single_thread_value"] = statistics.median(single)
+        out["single_thread_sample"] = "%d params of the sample's largest tensor, median of steps 2-4" % n1
+    return out
 
 
-def main():
-    args = parse()
-    if args.gpus != 1:
-        print("bench.py measures one GPU: the 8-bit AdamW step has no cross-GPU exchange and this build runs on "
-              "a single MI355X; rerun with --gpus 1", file=sys.stderr)
-        sys.exit(2)
-    import torch
-
+def measure(args, torch, separate_events=False):
+    """One configuration: allocates, fills, times `args.steps` steps after `args.warmup`, frees; the JSON object of
+    the run (without the CPU baseline).  separate_events: the wall clock is taken over steps without events around
+    them and the kernel's duration over as many further steps with them (for steps of a few microseconds, where
+    recording two events per step shows in the wall clock)."""
     from eridiffusion_amd import _lib as L
     from eridiffusion_amd import workloads as W
 
@@ -236,15 +281,18 @@ def main():
     n_blocks = sum((n + L.BLOCK - 1) // L.BLOCK for n in sizes)
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream().cuda_stream
+    alloc = args.alloc
 
-    if args.alloc == "pool" and args.kernel == "adamw32" and n_params * 4 > (20 << 30):
+    if alloc == "pool" and args.kernel == "adamw32" and n_params * 4 > (20 << 30):
         # fp32 moments of the large sets fill a 48 GiB lane each and leave no room for the other arrays
-        args.alloc = "arena"
-    if args.alloc == "pool" and Pool.open() != 0:
+        alloc = "arena"
+    if alloc != "pool":
+        Pool.close()  # the pool holds nine tenths of the device memory
+    elif Pool.open() != 0:
         print("bench.py: no lane pool (%s); the flat buffers become allocations of their own (--alloc arena)"
               % L.lib().eri_last_error().decode("utf-8", "replace"), file=sys.stderr)
-        args.alloc = "arena"
-    if args.alloc == "pool":  # four lanes, each wide enough for its kind of tensor (little free memory gives fewer)
+        alloc = "arena"
+    if alloc == "pool":  # four lanes, each wide enough for its kind of tensor (little free memory gives fewer)
         lanes, lane_bytes = C.c_uint32(), C.c_size_t()
         L.check(L.lib().eri_hip_pool_info(Pool.handle, C.byref(lanes), C.byref(lane_bytes)), "eri_hip_pool_info")
         state_bytes = 2 * n_params + 8 * n_blocks + 1024 * len(sizes)
@@ -255,10 +303,9 @@ def main():
             print("bench.py: the lane pool has %d lanes of %.1f GiB, too few or too narrow for this workload; the "
                   "flat buffers become allocations of their own (--alloc arena)" % (lanes.value, lane_bytes.value / 2**30),
                   file=sys.stderr)
-            L.lib().eri_hip_pool_destroy(Pool.handle)
-            Pool.handle = None
-            args.alloc = "arena"
-    Alloc = {"arena": Arena, "tensor": PerTensor, "pool": Pool}[args.alloc]
+            Pool.close()
+            alloc = "arena"
+    Alloc = {"arena": Arena, "tensor": PerTensor, "pool": Pool}[alloc]
     LANE_PARAM, LANE_GRAD, LANE_STATE, LANE_OTHER = 0, 1, 2, 3  # the pool's lanes, one per kind of tensor
     a_p = Alloc(torch, [n * esz for n in sizes], LANE_PARAM)
     a_g = Alloc(torch, [n * gsz for n in sizes], LANE_GRAD)
@@ -269,8 +316,8 @@ def main():
     tdt = torch.bfloat16 if bf16 else torch.float32
     gen = torch.Generator(device="cuda:0")
     gen.manual_seed(0xE21D + 5)
-    p_std, g_std = (0.02, 1e-3)
-    for i, n in enumerate(sizes):  # synthetic data: p ~ N(0, 0.02), g ~ N(0, 1e-3)
+    for i, (n, (name, shape)) in enumerate(zip(sizes, tensors)):  # synthetic data, the spread the configuration names
+        p_std, g_std = W.init_std(args.config, name, shape)
         a_p.fill(i, torch.randn(n, device="cuda:0", generator=gen).mul_(p_std).to(tdt), stream)
         a_g.fill(i, torch.randn(n, device="cuda:0", generator=gen).mul_(g_std).to(torch.float32 if grad_f32 else tdt), stream)
         L.check(L.lib().eri_adam8_state_init(a_m.ptr(i), a_v.ptr(i), a_am.ptr(i), a_av.ptr(i), n, stream), "state_init")
@@ -336,7 +383,7 @@ def main():
         L.check(L.lib().eri_adam8bit_new(handles, len(sizes), C.byref(cfg), stream, C.byref(obj_opt)), "adam8bit_new")
         if args.flags:
             L.check(L.lib().eri_adam8bit_set_flags(obj_opt, args.flags), "set_flags")
-        if args.alloc == "pool":  # the optimizer's own states out of the state lane
+        if alloc == "pool":  # the optimizer's own states out of the state lane
             L.check(L.lib().eri_adam8bit_set_state_pool(obj_opt, Pool.handle, LANE_STATE), "set_state_pool")
     elif args.api != "table":
         if args.kernel != "adam8":
@@ -347,6 +394,8 @@ def main():
         fn_opt = C.c_void_p()
         L.check(L.lib().eri_adam8bit_fn_with_params(*hyper_args, stream, C.byref(fn_opt)), "fn_with_params")
         L.check(L.lib().eri_adam8bit_fn_set_batching(fn_opt, 1), "fn_set_batching")
+        if alloc == "pool":
+            L.check(L.lib().eri_adam8bit_fn_set_state_pool(fn_opt, Pool.handle, LANE_STATE), "fn_set_state_pool")
         tag = L.DTYPE_BF16 if bf16 else L.DTYPE_F32
         fn_names = [name.encode() for name, _ in tensors]
         c_names = (C.c_char_p * n_t)(*fn_names)
@@ -401,14 +450,28 @@ def main():
         step(t)
     torch.cuda.synchronize()
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-    t0 = time.perf_counter()
-    for k in range(args.steps):
-        t += 1
-        ev[k][0].record()
-        step(t)
-        ev[k][1].record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
+    if separate_events:
+        t0 = time.perf_counter()
+        for k in range(args.steps):
+            t += 1
+            step(t)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        for k in range(args.steps):
+            t += 1
+            ev[k][0].record()
+            step(t)
+            ev[k][1].record()
+        torch.cuda.synchronize()
+    else:
+        t0 = time.perf_counter()
+        for k in range(args.steps):
+            t += 1
+            ev[k][0].record()
+            step(t)
+            ev[k][1].record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
     launch_ms = [a.elapsed_time(b) for a, b in ev]
     avg_launch_s = sum(launch_ms) / len(launch_ms) / 1e3
 
@@ -437,10 +500,10 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": ARITHMETIC[args.kernel],
         "data": "synthetic",
         "config": {"workload": args.config, "tensors": len(sizes), "params": n_params, "blocks": n_blocks,
-                   "kernel": args.kernel, "api": args.api, "alloc": args.alloc, "mode": args.mode if args.api in ("table", "object") else "l2",
+                   "kernel": args.kernel, "api": args.api, "alloc": alloc, "mode": args.mode if args.api in ("table", "object") else "l2",
                    "param_dtype": dt_name, "grad_dtype": "f32" if gsz == 4 else "bf16", "state": "uint8 m/v + fp32 absmax per 2048-block", "flags": args.flags,
                    "resident_gb": round((n_params * (esz + gsz + 2) + n_blocks * 8) / 1e9, 2)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
@@ -459,8 +522,63 @@ def main():
             L.lib().eri_param_release(hnd)
     for a in [a_p, a_g, a_m, a_v, a_am, a_av] + extra:
         a.free()
+    if Pool.handle is not None:
+        torch.cuda.synchronize()
+        L.lib().eri_hip_pool_reset(Pool.handle)  # every piece of this measurement goes back
+    torch.cuda.empty_cache()
+    return out, tensors, bf16, hyper_args
+
+
+def row_of(out):
+    """The short form of a measurement for the `configs` list."""
+    c, r = out["config"], out["roofline"]
+    return {"workload": c["workload"], "api": c["api"], "mode": c["mode"], "flags": c["flags"], "alloc": c["alloc"],
+            "param_dtype": c["param_dtype"], "params": c["params"], "tensors": c["tensors"], "steps": out["steps"],
+            "warmup": out["warmup"], "ms_per_step": out["ms_per_step"], "params_per_s": out["value"],
+            "kernel_ms": r["kernel_ms"], "kernel_ms_min": r["kernel_ms_min"], "frac": r["frac"],
+            "frac_of_step": r["algorithmic_bytes"] / (out["ms_per_step"] * 1e-3) / 1e9 / PEAK_HBM_GBPS}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the 8-bit AdamW step has no cross-GPU exchange and this build runs on "
+              "a single MI355X; rerun with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    is_headline = all(getattr(args, k) == v for k, v in HEADLINE.items())
+    out, tensors, bf16, hyper_args = measure(args, torch)
     if args.cpu_sample > 0:
         out["cpu_baseline"] = cpu_baseline(tensors, bf16, args.cpu_sample, hyper_args)
+    if args.rows == "all" or (args.rows == "auto" and is_headline):
+        from eridiffusion_amd import workloads as W
+        rows = []
+        for change, steps, warmup in ROWS:
+            if args.rows_max_params and W.total_params(W.CONFIGS[change["config"]][0]()) > args.rows_max_params:
+                continue
+            a = argparse.Namespace(**vars(args))
+            for k, v in HEADLINE.items():
+                setattr(a, k, v)
+            for k, v in change.items():
+                setattr(a, k, v)
+            a.steps, a.warmup = steps, warmup
+            try:
+                o, tens, b16, hy = measure(a, torch, separate_events=True)
+            except SystemExit:
+                raise
+            except Exception as e:  # a row that cannot run must not take the headline with it
+                rows.append({"workload": a.config, "api": a.api, "mode": a.mode, "flags": a.flags, "alloc": a.alloc,
+                             "error": "%s: %s" % (type(e).__name__, e)})
+                continue
+            row = row_of(o)
+            small = W.total_params(tens) <= (1 << 28)
+            if args.cpu_sample > 0 and small and a.api == "table" and a.mode == "eri" and a.flags == 0:
+                cb = cpu_baseline(tens, b16, 1 << 62, hy, single_thread=False)  # the whole configuration
+                row["cpu_params_per_s"], row["cpu_sample"] = cb["value"], cb["sample"]
+            rows.append(row)
+        out["configs"] = rows
+    Pool.close()
     print(json.dumps(out), flush=True)
 
 

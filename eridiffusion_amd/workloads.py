@@ -187,6 +187,16 @@ def c4_sdxl_full(scale=1):
     return out
 
 
+def init_std(config, name, shape):
+    """(standard deviation of the parameters, of the gradients) the benchmark configuration names for a tensor.
+    LoRA sets: A ~ N(0, 1/in), B zero-initialised then perturbed ~ N(0, 1e-4), gradients ~ N(0, 1e-4); the flat
+    tensor and the full fine-tune sets: parameters ~ N(0, 0.02), gradients ~ N(0, 1e-3)."""
+    if config in ("c2_sdxl_lora_r16", "c3_flux_lora_r32"):
+        is_a = name.endswith(".down") or name.endswith(".lora_A")
+        return (float(shape[1]) ** -0.5 if is_a else 1e-4), 1e-4
+    return 0.02, 1e-3
+
+
 CONFIGS = {
     "c1_flat_fp32": (c1_flat, "f32"),
     "c2_sdxl_lora_r16": (c2_sdxl_lora, "bf16"),
