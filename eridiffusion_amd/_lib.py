@@ -37,7 +37,7 @@ class Adam8bitConfigC(C.Structure):
 
 class AdamW32Row(C.Structure):
     _fields_ = [("p", C.c_void_p), ("g", C.c_void_p), ("m", C.c_void_p), ("v", C.c_void_p), ("master", C.c_void_p),
-                ("numel", C.c_uint64), ("dtype_tag", C.c_int32), ("reserved", C.c_int32)]
+                ("numel", C.c_uint64), ("dtype_tag", C.c_int32), ("grad_scale", C.c_float)]
 
 
 class AdamW32Hyper(C.Structure):
@@ -82,6 +82,8 @@ EXPORTS = {
     "eri_hip_mem_info": (C.c_int, [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
     "eri_hip_pool_create": (C.c_int, [C.c_int, C.c_size_t, C.c_uint32, C.POINTER(C.c_void_p)]),
     "eri_hip_pool_alloc_zeroed": (C.c_int, [C.c_void_p, C.c_uint32, C.c_size_t, C.POINTER(C.c_void_p)]),
+    "eri_hip_pool_alloc_zeroed_async": (C.c_int, [C.c_void_p, C.c_uint32, C.c_size_t, C.c_void_p, C.POINTER(C.c_void_p)]),
+    "eri_hip_pool_release": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "eri_hip_pool_info": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint32), C.POINTER(C.c_size_t)]),
     "eri_hip_pool_lane_used": (C.c_int, [C.c_void_p, C.c_uint32, C.POINTER(C.c_size_t)]),
     "eri_hip_pool_reset": (C.c_int, [C.c_void_p]),
@@ -97,6 +99,9 @@ EXPORTS = {
     "eri_adam8_table_info": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "eri_adam8_step_table": (C.c_int, [C.c_void_p, C.POINTER(Hyper), C.c_void_p]),
     "eri_adam8_grad_norm": (C.c_int, [C.c_void_p, C.c_float, C.c_float, C.c_void_p]),
+    "eri_adam8_grad_table_create": (C.c_int, [C.POINTER(TensorRow), C.c_uint32, C.c_void_p, C.POINTER(C.c_void_p)]),
+    "eri_adam8_grad_norm_joint": (C.c_int, [C.c_void_p, C.c_void_p, C.c_float, C.c_float, C.c_void_p]),
+    "eri_adam8_grad_norm_scale_ptr": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p)]),
     "eri_adam8_grad_norm_static": (C.c_int, [C.c_void_p, C.c_float, C.c_float, C.c_void_p, C.c_void_p]),
     "eri_adam8_grad_norm_read": (C.c_int, [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_void_p]),
     "eri_adam8_grad_nonfinite_read": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint64), C.c_void_p]),
@@ -106,6 +111,8 @@ EXPORTS = {
     "eri_adam8_dequantize": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_uint64, C.c_void_p, C.c_void_p]),
     "eri_adam8_quantize": (C.c_int, [C.c_void_p, C.c_int, C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p]),
     "eri_adamw32_step_multi": (C.c_int, [C.POINTER(AdamW32Row), C.c_uint32, C.POINTER(AdamW32Hyper), C.c_void_p]),
+    "eri_adamw32_step_multi_scaled": (C.c_int, [C.POINTER(AdamW32Row), C.c_uint32, C.POINTER(AdamW32Hyper), C.c_float,
+                                              C.c_void_p, C.c_void_p]),
     "eri_ema_update_multi": (C.c_int, [C.POINTER(EmaRow), C.c_uint32, C.c_float, C.c_void_p]),
     # ---- include/eri_adam8bit.h
     "eri_param_create": (C.c_int, [C.c_void_p, C.c_uint64, C.c_int, C.POINTER(C.c_void_p)]),
@@ -167,6 +174,7 @@ EXPORTS = {
     "eri_adam8bit_fn_step": (C.c_int, [C.c_void_p]),
     "eri_adam8bit_fn_set_lr": (C.c_int, [C.c_void_p, C.c_float]),
     "eri_adam8bit_fn_get_step": (C.c_uint64, [C.c_void_p]),
+    "eri_adam8bit_fn_table_stats": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "eri_adam8bit_fn_memory_stats": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "eri_adam8bit_fn_state_numel": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_uint64)]),
     "eri_adam8bit_fn_get_state_fp32": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p]),

@@ -128,6 +128,8 @@ int launch_grad_sumsq(const DevTensor *rows, uint32_t n_rows, uint32_t total_ful
                       double *partial, uint32_t grid, void *stream);
 int launch_grad_norm_finish(const double *partial, uint32_t n, float max_norm, float denom_eps, float *out,
                             void *stream);
+/* Clears `bytes` bytes at `p`; both multiples of 16. */
+int launch_fill_zero(void *p, size_t bytes, void *stream);
 int launch_state_init(uint8_t *m, uint8_t *v, float *absmax_m, float *absmax_v, uint64_t numel, void *stream);
 int launch_dequantize(const uint8_t *codes, const float *absmax, int signed_map, uint64_t numel, float *out,
                       const void *lds_image, void *stream);
@@ -143,12 +145,15 @@ struct ElemRow {
     void *e;        /* AdamW: fp32 master copy of p, or null */
     uint64_t numel;
     uint32_t full_start; /* full 2048-element blocks in the rows before this one */
-    uint32_t pad;
+    float scale;         /* AdamW: per-layer multiplier of the gradients (used by the scaled step only) */
 };
 static_assert(sizeof(ElemRow) == 56, "ElemRow must stay 56 bytes");
 
+/* scaled: every gradient is first multiplied by (grad_scale * row.scale) * (*dev_scale, 1 if null), as the 8-bit
+ * step does with ERI_ADAM8_FLAG_GRAD_SCALE. */
 int launch_adamw32(const ElemRow *rows, uint32_t n_rows, uint32_t total_full_blocks, int dtype_tag,
-                   const EriAdamW32Hyper &h, uint32_t grid, void *stream);
+                   const EriAdamW32Hyper &h, bool scaled, float grad_scale, const float *dev_scale, uint32_t grid,
+                   void *stream);
 int launch_ema(const ElemRow *rows, uint32_t n_rows, uint32_t total_full_blocks, int dtype_tag, float decay,
                uint32_t grid, void *stream);
 

@@ -184,11 +184,55 @@ __device__ __forceinline__ uint32_t code_bsearch(float x, const float *mid) {
 // the update of one element
 // ------------------------------------------------------------------------------------------
 
+/* The step's scalars as the kernels use them: the caller's EriAdam8Hyper plus, for the functional update
+ * (mode L2), the two constants of its folded fast chain.  That update is
+ *     lr * (m / bc1) / (sqrt(v / bc2) + eps)  =  (lr * sqrt(bc2) / bc1) * m / (sqrt(v) + eps * sqrt(bc2)),
+ * and the right-hand side needs neither bias correction per element.  Both constants are formed in f64 from the
+ * fp32 scalars the exact chain uses and rounded once. */
+struct StepHyper : EriAdam8Hyper {
+    float l2_step, l2_eps;
+    /* The fast chain's error bounds assume a step constant of at most one (so that a normal update means a normal
+     * m / denominator) and an eps that swallows the root of a second moment in the denormal range, which the
+     * hardware square root does not see.  A launch with other scalars recomputes every element. */
+    bool l2_all_exact;
+};
+template <int MODE>
+__device__ __forceinline__ StepHyper make_step_hyper(const EriAdam8Hyper &h) {
+    StepHyper s;
+    static_cast<EriAdam8Hyper &>(s) = h;
+    s.l2_step = 0.0f;
+    s.l2_eps = 0.0f;
+    s.l2_all_exact = false;
+    if (MODE == ERI_ADAM8_MODE_L2) {
+        const double root = __builtin_sqrt((double)h.bc2);
+        s.l2_step = (float)((double)h.step_size * root / (double)h.bc1);
+        s.l2_eps = (float)((double)h.eps * root);
+        s.l2_all_exact = !(__builtin_fabsf(s.l2_step) <= 1.0f) || !(s.l2_eps >= 0x1p-36f);
+    }
+    return s;
+}
+
+/* Wave-wide mask of the lanes whose x falls into one of the classes of `classes` (the bits of v_cmp_class_f32):
+ * one instruction, where the compiler spells a test for NaN, infinity and denormals as three comparisons. */
+__device__ __forceinline__ uint64_t class_mask(float x, uint32_t classes) {
+    uint64_t m;
+    asm("v_cmp_class_f32 %0, %1, %2" : "=s"(m) : "v"(x), "v"(classes));
+    return m;
+}
+
+/* The fp32 number halfway between the two bf16 neighbours of x (low half 0x8000): where the rounding of x to
+ * bf16 changes direction.  One v_and_or_b32. */
+__device__ __forceinline__ float bf16_tie_point(float x) {
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(f2u(x)), "s"(0xffff0000u), "v"(0x8000u));
+    return u2f(r);
+}
+
 /* The parameter update from finished moments, one rounded operation per line, with IEEE square root and
  * division: what fp32 parameters always get, and bf16 parameters wherever the fast chain below cannot
  * promise the same bits. */
 template <int MODE, bool WD, bool BF16>
-__device__ __forceinline__ float param_exact(float p, float m, float v, const EriAdam8Hyper &h, const BlockDiv &dbc1,
+__device__ __forceinline__ float param_exact(float p, float m, float v, const StepHyper &h, const BlockDiv &dbc1,
                                              const BlockDiv &dbc2) {
     if (MODE == ERI_ADAM8_MODE_L2) {
         float mh = dbc1.fast ? dbc1.div_fast_unbounded(m) : m / dbc1.a; // adam8bit.rs:170
@@ -245,14 +289,24 @@ __device__ __forceinline__ float param_exact(float p, float m, float v, const Er
  * margin's own arithmetic.
  *
  * The functional update (mode L2) rounds the *update* to bf16 before it subtracts (adam8bit.rs:197-198), and
- * that subtraction is a single exact-input operation, so the same argument applies to the update.  The fast
- * chain multiplies by the rounded reciprocals of the two bias corrections instead of dividing (1.5 * 2^-23
- * each, relative to the exact quotient), takes the hardware square root and reciprocal (2^-23 each) and rounds
- * six times: its lr * (m/bc1) / (sqrt(v/bc2) + eps) is within 7.75 * 2^-23 of the exact chain's, relative, and
- * an update further than 16 * 2^-23 of itself from the tie point of its bf16 interval rounds to the same bf16
- * value on both chains.  About one element in 2,000 is flagged and recomputed, and so is every element with a
- * moment below 2^-100, where the products lose relative accuracy to the denormal grid.
+ * that subtraction is a single exact-input operation, so the same argument applies to the update.  With
+ * u = 2^-24: the exact chain rounds m/bc1 (u), v/bc2 (u, halved by the root), the root (u), the sum with eps (u),
+ * the quotient (u) and the product with lr (u), 5.5 u in all, relative to the real-valued update.  The fast
+ * chain evaluates the folded form (StepHyper): hardware root (2 u), the rounded eps*sqrt(bc2) (u), the sum (u) --
+ * the denominator is within 3 u --, the hardware reciprocal (2 u), its product with m (u), the rounded step
+ * constant (u) and the last product (u): 8 u.  So the two updates differ by less than 13.5 u = 6.75 * 2^-23 of
+ * themselves, which is at most 14 fp32 patterns; an update whose low half is further than kL2TieUlps = 20
+ * patterns from 0x8000 rounds to the same bf16 value on both chains.  41 low halves of 65,536 are flagged and
+ * recomputed (one element in 1,600), and so is every NaN, infinity and update in the denormal range.
  */
+/* v_cmp_class_f32 masks: signalling and quiet NaN, -inf, -denormal, +denormal, +inf. */
+constexpr int kClassDenormal = 0x10 | 0x80;
+constexpr int kClassNanInfDenormal = 0x1 | 0x2 | 0x4 | 0x200 | kClassDenormal;
+/* Mode L2: how close (in fp32 patterns) the low half of the fast chain's update may come to 0x8000 before the
+ * element is recomputed.  The two chains' updates differ by less than 6.75 * 2^-23 of themselves (below), which
+ * is at most 14 patterns. */
+constexpr uint32_t kL2TieUlps = 20;
+
 template <int MODE, bool WD>
 struct ExactMargin {
     float c_r, c_p;
@@ -272,32 +326,51 @@ struct ExactMargin {
     __device__ __forceinline__ bool same_bf16_as_exact(float r, float pn) const {
         // the floor 2^-126 flags everything down among the fp32 denormals, where the bounds above do not hold
         const float margin = __builtin_fmaf(__builtin_fabsf(pn), c_p, __builtin_fmaf(__builtin_fabsf(r), c_r, 0x1p-126f));
-        const float tie = u2f((f2u(pn) & 0xffff0000u) | 0x8000u);
-        return __builtin_fabsf(pn - tie) > margin;
+        return __builtin_fabsf(pn - bf16_tie_point(pn)) > margin;
     }
+};
+
+/* Which lanes must recompute which of their eight elements with param_exact: one wave-wide mask per position,
+ * held in scalar registers.  (As an array of per-lane bools the flags were materialised in vector registers:
+ * three vector instructions per element.)  A position no lane has flagged is skipped altogether. */
+struct Redo8 {
+    uint64_t lanes[8];
+    uint64_t any;
+    __device__ __forceinline__ Redo8() : any(0) {}
+    __device__ __forceinline__ void set(int k, uint64_t flagged) {
+        lanes[k] = flagged;
+        any |= flagged;
+    }
+    /* every active lane recomputes all of its elements */
+    __device__ __forceinline__ void set_all() {
+        const uint64_t active = __builtin_amdgcn_ballot_w64(true);
+        for (int k = 0; k < 8; ++k) lanes[k] = active;
+        any = active;
+    }
+    __device__ __forceinline__ bool mine(int k) const { return __builtin_amdgcn_inverse_ballot_w64(lanes[k]); }
 };
 
 /* t1 = m_old * beta1 and t3 = v_old * beta2 come in already multiplied: a kernel that holds a block's 256
  * possible values of either product in a table of its own forms them once per code instead of once per
  * element (same two rounded multiplications, same bits). */
 template <int MODE, bool EXACT, bool BF16, bool WD, bool GS>
-__device__ __forceinline__ void adam_elem_decayed(float p, float g, float t1, float t3, const EriAdam8Hyper &h,
+__device__ __forceinline__ void adam_elem_decayed(float p, float g, float t1, float t3, const StepHyper &h,
                                                   float gscale, const BlockDiv &dbc1, const BlockDiv &dbc2, float &m,
-                                                  float &v, float &pn, bool &recheck);
+                                                  float &v, float &pn, uint64_t &recheck);
 
 template <int MODE, bool EXACT, bool BF16, bool WD, bool GS>
-__device__ __forceinline__ void adam_elem(float p, float g, float m_old, float v_old, const EriAdam8Hyper &h,
+__device__ __forceinline__ void adam_elem(float p, float g, float m_old, float v_old, const StepHyper &h,
                                           float gscale, const BlockDiv &dbc1, const BlockDiv &dbc2, float &m,
-                                          float &v, float &pn, bool &recheck) {
+                                          float &v, float &pn, uint64_t &recheck) {
     float t1 = m_old * h.beta1; // adam8bit_enhanced.rs:256
     float t3 = v_old * h.beta2; // :260
     adam_elem_decayed<MODE, EXACT, BF16, WD, GS>(p, g, t1, t3, h, gscale, dbc1, dbc2, m, v, pn, recheck);
 }
 
 template <int MODE, bool EXACT, bool BF16, bool WD, bool GS>
-__device__ __forceinline__ void adam_elem_decayed(float p, float g, float t1, float t3, const EriAdam8Hyper &h,
+__device__ __forceinline__ void adam_elem_decayed(float p, float g, float t1, float t3, const StepHyper &h,
                                                   float gscale, const BlockDiv &dbc1, const BlockDiv &dbc2, float &m,
-                                                  float &v, float &pn, bool &recheck) {
+                                                  float &v, float &pn, uint64_t &recheck) {
     if (GS) g = g * gscale;
     if (MODE == ERI_ADAM8_MODE_L2 && WD) { // adam8bit.rs:113-120
         float pw = p * h.weight_decay;
@@ -311,38 +384,34 @@ __device__ __forceinline__ void adam_elem_decayed(float p, float g, float t1, fl
     if (!BF16) { // fp32 parameters: every bit of the exact chain counts
         pn = param_exact<MODE, WD, false>(p, m, v, h, dbc1, dbc2);
     } else if (MODE == ERI_ADAM8_MODE_L2) { // always to the exact chain's bits (the reference rounds the update itself)
-        // fast chain: the two bias corrections as products with the rounded reciprocals, hardware square root
-        // and reciprocal; param_exact redoes whatever the test below cannot vouch for
-        float mh = m * dbc1.ras; // adam8bit.rs:170
-        // :178; the clamp at zero (:181-182) only ever acts on NaN here (v is a sum of non-negative terms), and
-        // NaN fails the comparison below and is redone by the exact chain, clamp included
-        float vh = v * dbc2.ras;
-        float den = __builtin_amdgcn_sqrtf(vh) + h.eps;
-        float upd = mh * __builtin_amdgcn_rcpf(den);
-        float us = upd * h.step_size;
-        const float tie = u2f((f2u(us) & 0xffff0000u) | 0x8000u);
-        recheck |= !(__builtin_fabsf(us - tie) > __builtin_fmaf(__builtin_fabsf(us), 0x1p-19f, 0x1p-126f));
-        // a moment near the denormal range loses relative accuracy in the product (the exact chain's division
-        // rounds on the same grid but not to the same point).  For the second moment that only shows when eps is
-        // too small to swallow its square root.  NaN and infinity fail the comparison above, and so does a
-        // zero update (the margin's floor), so a zero moment needs no exception here.
-        recheck |= __builtin_fabsf(m) < 0x1p-100f;
-        if (h.eps < 0x1p-36f) recheck |= (v < 0x1p-100f) & (v != 0.0f);
-        recheck |= !(dbc1.fast && dbc2.fast);
-        pn = p - bf16_round(us); // :197-205
+        // fast chain: the folded form of the update (StepHyper), hardware square root and reciprocal;
+        // param_exact redoes whatever the tests below cannot vouch for
+        float den = __builtin_amdgcn_sqrtf(v) + h.l2_eps;
+        float r = m * __builtin_amdgcn_rcpf(den);
+        float us = r * h.l2_step;
+        // Both chains round the update to bf16, so they agree unless a rounding boundary of bf16 (an fp32 pattern
+        // whose low half is 0x8000) lies between their updates, and those are at most 14 fp32 patterns apart
+        // (kL2TieUlps covers it with room): flagged are the updates whose low half is that close to 0x8000.
+        const uint32_t moved = f2u(us) + (kL2TieUlps - 0x8000u);
+        recheck |= __builtin_amdgcn_ballot_w64((moved & 0xffffu) <= 2u * kL2TieUlps);
+        // NaN, infinity and updates in the denormal range, where the relative bounds do not hold (a zero
+        // update is a zero moment on both chains and passes).  Launches whose scalars void the bounds altogether
+        // (StepHyper::l2_all_exact) recompute every element: the kernels see to that, not this chain.
+        recheck |= class_mask(us, kClassNanInfDenormal);
+        pn = p - u2f(bf16_pair(0.0f, us)); // adam8bit.rs:197-205: the update rounded to bf16, then subtracted
     } else { // h.eps and h.weight_decay of mode BNB carry sqrt(bc2) and the factor 1 - lr*wd
         float den = __builtin_amdgcn_sqrtf(v) + h.eps;
         float r = m * __builtin_amdgcn_rcpf(den);
         if (MODE == ERI_ADAM8_MODE_BNB) {
             float p0 = __builtin_fmaf(-r, h.step_size, p);
             pn = WD ? p0 * h.weight_decay : p0;
-            if (EXACT) recheck |= !ExactMargin<MODE, WD>(h).same_bf16_as_exact(r, pn);
-            else recheck |= __builtin_fabsf(p0) * 4096.0f < __builtin_fabsf(p);
+            if (EXACT) recheck |= __builtin_amdgcn_ballot_w64(!ExactMargin<MODE, WD>(h).same_bf16_as_exact(r, pn));
+            else recheck |= __builtin_amdgcn_ballot_w64(__builtin_fabsf(p0) * 4096.0f < __builtin_fabsf(p));
         } else {
             float u = WD ? __builtin_fmaf(p, h.weight_decay, r) : r;
             pn = __builtin_fmaf(-u, h.step_size, p);
-            if (EXACT) recheck |= !ExactMargin<MODE, WD>(h).same_bf16_as_exact(r, pn);
-            else recheck |= __builtin_fabsf(pn) * 4096.0f < __builtin_fabsf(p);
+            if (EXACT) recheck |= __builtin_amdgcn_ballot_w64(!ExactMargin<MODE, WD>(h).same_bf16_as_exact(r, pn));
+            else recheck |= __builtin_amdgcn_ballot_w64(__builtin_fabsf(pn) * 4096.0f < __builtin_fabsf(p));
         }
     }
 }
@@ -518,7 +587,7 @@ __device__ __forceinline__ void requant8(const float *mf, const float *vf, const
  * per code (eight per lane) instead of once per element (64 per lane); a wave's LDS operations complete in
  * order, so its reads below see its own writes without a barrier. */
 template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB, bool GBF16 = BF16>
-__device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint32_t lane, const EriAdam8Hyper &h,
+__device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint32_t lane, const StepHyper &h,
                                            float gscale, const BlockDiv &dbc1, const BlockDiv &dbc2, const Lds &L,
                                            float (*mine)[256]) {
     const size_t e0 = (size_t)lb * kBlock;
@@ -567,27 +636,27 @@ __device__ __forceinline__ void full_block(const DevTensor &t, uint32_t lb, uint
             float pv[8], gv[8], pn[8];
             pr[d].unpack(pv);
             gr[d].unpack(gv);
-            // one flag per element: the exact chain then runs for the flagged positions only, and a position
-            // is skipped altogether when no lane of the wave has it flagged
-            bool redo[8];
-            bool any = false;
+            // one flag per element: the exact chain then runs for the flagged positions only
+            Redo8 redo;
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
                 const float t1 = lds_float_at(mine[0], code_offset(mr[d], k));
                 const float t3 = lds_float_at(mine[1], code_offset(vr[d], k));
                 float m, v;
-                redo[k] = false;
-                adam_elem_decayed<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], t1, t3, h, gscale, dbc1, dbc2, m, v, pn[k], redo[k]);
-                any |= redo[k];
+                uint64_t flagged = 0;
+                adam_elem_decayed<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], t1, t3, h, gscale, dbc1, dbc2, m, v, pn[k], flagged);
+                redo.set(k, flagged);
                 mf[c * 8 + k] = m;
                 vf[c * 8 + k] = v;
                 lm = fmaxf(lm, __builtin_fabsf(m));
                 lv = fmaxf(lv, __builtin_fabsf(v));
             }
-            if (any) {
+            if (BF16 && MODE == ERI_ADAM8_MODE_L2 && h.l2_all_exact) redo.set_all();
+            if (BF16 && redo.any) {
 #pragma unroll
                 for (int k = 0; k < 8; ++k)
-                    if (redo[k]) pn[k] = param_exact<MODE, WD, BF16>(pv[k], mf[c * 8 + k], vf[c * 8 + k], h, dbc1, dbc2);
+                    if (redo.lanes[k] && redo.mine(k))
+                        pn[k] = param_exact<MODE, WD, BF16>(pv[k], mf[c * 8 + k], vf[c * 8 + k], h, dbc1, dbc2);
             }
             store8<BF16>(p, o, pn);
         }
@@ -634,7 +703,7 @@ __device__ __forceinline__ float load1(const void *base, size_t i) {
 
 template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB, bool GBF16 = BF16>
 __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint32_t n, uint32_t lane,
-                                        const EriAdam8Hyper &h, float gscale, const BlockDiv &dbc1,
+                                        const StepHyper &h, float gscale, const BlockDiv &dbc1,
                                         const BlockDiv &dbc2, const Lds &L) {
     const size_t e0 = (size_t)lb * kBlock;
     ERI_GLOBAL uint8_t *mc = as_global(t.m);
@@ -668,7 +737,7 @@ __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
                     float m, v, pn;
-                    bool unused = false;
+                    uint64_t unused = 0;
                     adam_elem<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], L.map_s[byte_of(mr, k)] * a_m,
                                                          L.map_u[byte_of(vr, k)] * a_v, h, gscale, dbc1, dbc2, m, v, pn, unused);
                     lm = fmaxf(lm, __builtin_fabsf(m));
@@ -691,12 +760,12 @@ __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint
                 float pv[8], gv[8], pn[8], m[8], v[8];
                 pr.unpack(pv);
                 gr.unpack(gv);
-                bool cancel = false;
+                uint64_t cancel = (BF16 && MODE == ERI_ADAM8_MODE_L2 && h.l2_all_exact) ? ~0ull : 0ull;
 #pragma unroll
                 for (int k = 0; k < 8; ++k)
                     adam_elem<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], L.map_s[byte_of(mr, k)] * a_m,
                                                          L.map_u[byte_of(vr, k)] * a_v, h, gscale, dbc1, dbc2, m[k], v[k], pn[k], cancel);
-                if (cancel) {
+                if (BF16 && __builtin_amdgcn_inverse_ballot_w64(cancel)) { // a lane with a flagged element redoes its eight
 #pragma unroll
                     for (int k = 0; k < 8; ++k) pn[k] = param_exact<MODE, WD, BF16>(pv[k], m[k], v[k], h, dbc1, dbc2);
                 }
@@ -716,7 +785,7 @@ __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint
     for (uint32_t i = lane; i < n; i += kWave) {
         const size_t e = e0 + i;
         float m, v, pn;
-        bool unused = false;
+        uint64_t unused = 0;
         adam_elem<MODE, EXACT, BF16, WD, GS>(load1<BF16>(t.p_in, e), load1<GBF16>(t.g, e), L.map_s[mc[e]] * a_m,
                                              L.map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn, unused);
         lm = fmaxf(lm, __builtin_fabsf(m));
@@ -728,11 +797,11 @@ __device__ __forceinline__ void tail_block(const DevTensor &t, uint32_t lb, uint
     for (uint32_t i = lane; i < n; i += kWave) {
         const size_t e = e0 + i;
         float m, v, pn;
-        bool cancel = false;
+        uint64_t cancel = (BF16 && MODE == ERI_ADAM8_MODE_L2 && h.l2_all_exact) ? ~0ull : 0ull;
         const float p_old = load1<BF16>(t.p_in, e);
         adam_elem<MODE, EXACT, BF16, WD, GS>(p_old, load1<GBF16>(t.g, e), L.map_s[mc[e]] * a_m,
                                              L.map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn, cancel);
-        if (cancel) pn = param_exact<MODE, WD, BF16>(p_old, m, v, h, dbc1, dbc2);
+        if (BF16 && __builtin_amdgcn_inverse_ballot_w64(cancel)) pn = param_exact<MODE, WD, BF16>(p_old, m, v, h, dbc1, dbc2);
         const float xm = dm.div_slow(m);
         const float xv = dv.div_slow(v);
         uint32_t cm = KEYTAB ? code_signed_key(xm, L.key_s) : code_bsearch(xm, L.mid_s);

@@ -92,6 +92,22 @@ __global__ void state_init_kernel(uint8_t *m, uint8_t *v, float *am, float *av, 
     }
 }
 
+__global__ void fill_zero_kernel(uint4 *p, uint64_t words) {
+    const uint64_t n = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < words; i += n) p[i] = uint4{0u, 0u, 0u, 0u};
+}
+
+int launch_fill_zero(void *p, size_t bytes, void *stream) {
+    if (bytes == 0) return 0;
+    if ((((uintptr_t)p) | bytes) & 15u) return (int)hipErrorInvalidValue;
+    const uint64_t words = bytes / 16;
+    uint64_t grid = (words + 255) / 256;
+    if (grid > 8192) grid = 8192;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((uint32_t)grid), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<uint4 *>(p), words);
+    return (int)hipGetLastError();
+}
+
 int launch_state_init(uint8_t *m, uint8_t *v, float *absmax_m, float *absmax_v, uint64_t numel, void *stream) {
     const uint64_t nblocks = (numel + kBlock - 1) / kBlock;
     uint64_t grid = (numel + 255) / 256;
@@ -319,10 +335,11 @@ __device__ __forceinline__ double wave_sum_f64(double x) {
 
 template <bool BF16, int MODE, bool WD, bool GS>
 __global__ __launch_bounds__(256) void quant_error_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
-                                                          uint32_t total_blocks, EriAdam8Hyper h,
+                                                          uint32_t total_blocks, EriAdam8Hyper h_in,
                                                           const float *__restrict__ lds_image,
                                                           const float *__restrict__ dev_scale,
                                                           double *__restrict__ err /* [2 * n_rows] */, bool grad_f32) {
+    const StepHyper h = make_step_hyper<MODE>(h_in);
     __shared__ float tab[1024]; // signed map, unsigned map, signed midpoints, unsigned midpoints
     for (uint32_t i = threadIdx.x; i < 1024; i += blockDim.x) tab[i] = lds_image[i];
     __syncthreads();
@@ -359,7 +376,7 @@ __global__ __launch_bounds__(256) void quant_error_kernel(const DevTensor *__res
         for (uint32_t i = lane; i < n; i += kWave) {
             const size_t e = e0 + i;
             float m, v, pn;
-            bool unused = false; // the exact chain never sets it
+            uint64_t unused = 0; // the exact chain never sets it
             const float gr = (BF16 && !grad_f32) ? load1<true>(t.g, e) : load1<false>(t.g, e);
             adam_elem<MODE, true, BF16, WD, GS>(load1<BF16>(t.p_in, e), gr, map_s[mc[e]] * a_m,
                                                 map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn, unused);
@@ -373,7 +390,7 @@ __global__ __launch_bounds__(256) void quant_error_kernel(const DevTensor *__res
         for (uint32_t i = lane; i < n; i += kWave) {
             const size_t e = e0 + i;
             float m, v, pn;
-            bool unused = false; // the exact chain never sets it
+            uint64_t unused = 0; // the exact chain never sets it
             const float gr = (BF16 && !grad_f32) ? load1<true>(t.g, e) : load1<false>(t.g, e);
             adam_elem<MODE, true, BF16, WD, GS>(load1<BF16>(t.p_in, e), gr, map_s[mc[e]] * a_m,
                                                 map_u[vc[e]] * a_v, h, gscale, dbc1, dbc2, m, v, pn, unused);
@@ -446,9 +463,9 @@ __device__ __forceinline__ void store1(void *base, size_t i, float x) {
 /* One full block of the 32-bit step.  MASTER: the parameter value comes from, and goes back to, an fp32
  * master copy; the tensor itself only receives the rounded result (mixed precision,
  * src/kernels/fused_adam.cu:151-193, with the arithmetic of adamw.rs). */
-template <bool BF16, bool MASTER>
+template <bool BF16, bool MASTER, bool GS>
 __device__ __forceinline__ void adamw32_block(const ElemRow &t, size_t e0, uint32_t lane, const EriAdamW32Hyper &h,
-                                              float omb1, float omb2, float neg_lr) {
+                                              float omb1, float omb2, float neg_lr, float gscale) {
     char *p = static_cast<char *>(t.a) + e0 * (BF16 ? 2 : 4);
     const char *g = static_cast<const char *>(t.b) + e0 * (BF16 ? 2 : 4);
     float *m = static_cast<float *>(t.c) + e0;
@@ -475,7 +492,7 @@ __device__ __forceinline__ void adamw32_block(const ElemRow &t, size_t e0, uint3
         mr[c].unpack(mv);
         vr[c].unpack(vv);
 #pragma unroll
-        for (int k = 0; k < 8; ++k) adamw32_elem(pv[k], gv[k], mv[k], vv[k], h, omb1, omb2, neg_lr, pn[k]);
+        for (int k = 0; k < 8; ++k) adamw32_elem(pv[k], GS ? gv[k] * gscale : gv[k], mv[k], vv[k], h, omb1, omb2, neg_lr, pn[k]);
         store8<BF16>(p, o, pn);
         if (MASTER) store8<false>(w, o, pn);
         store8<false>(m, o, mv);
@@ -483,9 +500,12 @@ __device__ __forceinline__ void adamw32_block(const ElemRow &t, size_t e0, uint3
     }
 }
 
-template <bool BF16>
+template <bool BF16, bool GS>
 __global__ __launch_bounds__(256) void adamw32_kernel(const ElemRow *__restrict__ rows, uint32_t n_rows,
-                                                      uint32_t total_blocks, EriAdamW32Hyper h, uint32_t chunks) {
+                                                      uint32_t total_blocks, EriAdamW32Hyper h, float grad_scale,
+                                                      const float *__restrict__ dev_scale, uint32_t chunks) {
+    // the clip factor left on the device by the gradient-norm pass (1.0 when there is none)
+    const float tscale = (GS && dev_scale) ? *dev_scale : 1.0f;
     const uint32_t lane = threadIdx.x & (kWave - 1);
     const uint32_t waves_per_wg = blockDim.x / kWave;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
@@ -498,10 +518,12 @@ __global__ __launch_bounds__(256) void adamw32_kernel(const ElemRow *__restrict_
         ERI_GLOBAL float *mp = as_global(static_cast<float *>(t.c));
         ERI_GLOBAL float *vp = as_global(static_cast<float *>(t.d));
         ERI_GLOBAL float *wp = as_global(static_cast<float *>(t.e)); // fp32 master copy, or null
+        const float gscale = GS ? (grad_scale * t.scale) * tscale : 1.0f; // the order of the 8-bit step's factors
         for (uint32_t i = lane; i < n; i += kWave) {
             float m = mp[e0 + i], v = vp[e0 + i], pn;
             const float pf = wp ? wp[e0 + i] : load1<BF16>(t.a, e0 + i);
-            adamw32_elem(pf, load1<BF16>(t.b, e0 + i), m, v, h, omb1, omb2, neg_lr, pn);
+            const float gf = load1<BF16>(t.b, e0 + i);
+            adamw32_elem(pf, GS ? gf * gscale : gf, m, v, h, omb1, omb2, neg_lr, pn);
             mp[e0 + i] = m;
             vp[e0 + i] = v;
             if (wp) wp[e0 + i] = pn;
@@ -514,8 +536,9 @@ __global__ __launch_bounds__(256) void adamw32_kernel(const ElemRow *__restrict_
     for (uint32_t blk = walk.first; blk < walk.end; blk += walk.stride) {
         seek_row(rows, n_rows, blk, ti, t, t_end);
         const size_t e0 = (size_t)(blk - t.full_start) * kBlock;
-        if (t.e) adamw32_block<BF16, true>(t, e0, lane, h, omb1, omb2, neg_lr);
-        else adamw32_block<BF16, false>(t, e0, lane, h, omb1, omb2, neg_lr);
+        const float gscale = GS ? (grad_scale * t.scale) * tscale : 1.0f;
+        if (t.e) adamw32_block<BF16, true, GS>(t, e0, lane, h, omb1, omb2, neg_lr, gscale);
+        else adamw32_block<BF16, false, GS>(t, e0, lane, h, omb1, omb2, neg_lr, gscale);
     }
 }
 
@@ -568,12 +591,18 @@ __global__ __launch_bounds__(256) void ema_kernel(const ElemRow *__restrict__ ro
 }
 
 int launch_adamw32(const ElemRow *rows, uint32_t n_rows, uint32_t total_blocks, int dtype_tag,
-                   const EriAdamW32Hyper &h, uint32_t grid, void *stream) {
+                   const EriAdamW32Hyper &h, bool scaled, float grad_scale, const float *dev_scale, uint32_t grid,
+                   void *stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dtype_tag == ERI_DTYPE_F32)
-        hipLaunchKernelGGL(adamw32_kernel<false>, dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, h, chunks_for(grid));
-    else
-        hipLaunchKernelGGL(adamw32_kernel<true>, dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, h, chunks_for(grid));
+#define ERI_GO(B, G) hipLaunchKernelGGL((adamw32_kernel<B, G>), dim3(grid), dim3(256), 0, s, rows, n_rows, total_blocks, h, grad_scale, dev_scale, chunks_for(grid))
+    if (dtype_tag == ERI_DTYPE_F32) {
+        if (scaled) ERI_GO(false, true);
+        else ERI_GO(false, false);
+    } else {
+        if (scaled) ERI_GO(true, true);
+        else ERI_GO(true, false);
+    }
+#undef ERI_GO
     return (int)hipGetLastError();
 }
 

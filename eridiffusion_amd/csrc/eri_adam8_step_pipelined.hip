@@ -99,11 +99,12 @@ struct RawBlock {
 template <int MODE, bool EXACT, bool WD, bool GS, bool EMA>
 __global__ __launch_bounds__(kPipeThreads) void ERI_PIPE_KERNEL(const DevTensor *__restrict__ rows,
                                                                    uint32_t n_rows, uint32_t total_blocks,
-                                                                   EriAdam8Hyper h,
+                                                                   EriAdam8Hyper h_in,
                                                                    const uint4 *__restrict__ lds_image,
                                                                    const float *__restrict__ dev_scale,
                                                                    uint32_t chunks) {
     ERI_LDS_IMAGE;
+    const StepHyper h = make_step_hyper<MODE>(h_in);
     // Where the next block's loads go out.  The instantiations of the reference's own update request each quarter
     // of the next block as soon as the same quarter of this one has been consumed (its registers are free from
     // then on), so every load has a whole block's time to arrive; measured 1-4 % faster on 2.6 B parameters,
@@ -228,27 +229,27 @@ __global__ __launch_bounds__(kPipeThreads) void ERI_PIPE_KERNEL(const DevTensor 
                 gv[4] = u2f(gb.x); gv[5] = u2f(gb.y); gv[6] = u2f(gb.z); gv[7] = u2f(gb.w);
             }
             // one flag per element: flagged elements are put right quarter by quarter (before the shadow uses
-            // them), the exact chain runs for the flagged positions only, and a position is skipped when no
-            // lane of the wave has it flagged
-            bool redo[8];
-            bool any = false;
+            // them), and the exact chain runs for the flagged positions only
+            Redo8 redo;
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
                 const float t1 = lds_float_at(mine[0], code_offset(raw.m[c], k));
                 const float t3 = lds_float_at(mine[1], code_offset(raw.v[c], k));
                 float m, v;
-                redo[k] = false;
-                adam_elem_decayed<MODE, EXACT, kParamBf16, WD, GS>(pv[k], gv[k], t1, t3, h, gscale, dbc1, dbc2, m, v, pn[k], redo[k]);
-                any |= redo[k];
+                uint64_t flagged = 0;
+                adam_elem_decayed<MODE, EXACT, kParamBf16, WD, GS>(pv[k], gv[k], t1, t3, h, gscale, dbc1, dbc2, m, v, pn[k], flagged);
+                redo.set(k, flagged);
                 mf[c * 8 + k] = m;
                 vf[c * 8 + k] = v;
                 lm = fmaxf(lm, __builtin_fabsf(m));
                 lv = fmaxf(lv, __builtin_fabsf(v));
             }
-            if (kParamBf16 && any) {
+            if (kParamBf16 && MODE == ERI_ADAM8_MODE_L2 && h.l2_all_exact) redo.set_all();
+            if (kParamBf16 && redo.any) {
 #pragma unroll
                 for (int k = 0; k < 8; ++k)
-                    if (redo[k]) pn[k] = param_exact<MODE, WD, true>(pv[k], mf[c * 8 + k], vf[c * 8 + k], h, dbc1, dbc2);
+                    if (redo.lanes[k] && redo.mine(k))
+                        pn[k] = param_exact<MODE, WD, true>(pv[k], mf[c * 8 + k], vf[c * 8 + k], h, dbc1, dbc2);
             }
             if (kParamBf16) {
                 pw[c].x = bf16_pair(pn[0], pn[1]);

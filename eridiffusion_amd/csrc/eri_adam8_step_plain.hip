@@ -19,11 +19,12 @@ constexpr uint32_t plain_threads(int mode) { return mode == ERI_ADAM8_MODE_L2 ? 
 
 template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB, bool GBF16>
 __global__ __launch_bounds__(plain_threads(MODE)) void adam8_step_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
-                                                          uint32_t total_blocks, EriAdam8Hyper h,
+                                                          uint32_t total_blocks, EriAdam8Hyper h_in,
                                                           const uint4 *__restrict__ lds_image,
                                                           const float *__restrict__ dev_scale, uint32_t chunks) {
     ERI_LDS_IMAGE;
     __shared__ float decayed[16][2][256]; // per wave: the values its block's state codes stand for, decayed
+    const StepHyper h = make_step_hyper<MODE>(h_in);
     // clip factor left on the device by the gradient-norm pass (1.0 when there is none)
     const float tscale = (GS && dev_scale) ? *dev_scale : 1.0f;
     // the binary search needs the maps and midpoints only (4 KB); the slot tables are the other 96 KB

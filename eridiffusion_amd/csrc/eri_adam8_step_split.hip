@@ -16,10 +16,11 @@ namespace eri {
 
 template <bool BF16, bool GBF16, int MODE, bool EXACT, bool WD, bool GS>
 __global__ __launch_bounds__(1024) void adam8_step_split_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
-                                                                uint32_t total_blocks, EriAdam8Hyper h,
+                                                                uint32_t total_blocks, EriAdam8Hyper h_in,
                                                                 const uint4 *__restrict__ lds_image,
                                                                 const float *__restrict__ dev_scale) {
     ERI_LDS_IMAGE;
+    const StepHyper h = make_step_hyper<MODE>(h_in);
     __shared__ float wave_maxima[2][4][8]; // [parity of the iteration][team][4 x first, 4 x second moment]
     // per wave: (MAP[c] * absmax) * beta for the 2 x 256 codes of the block at hand, formed once per code
     // (8 multiplications per lane) instead of once per element (16 per lane)
@@ -112,22 +113,22 @@ __global__ __launch_bounds__(1024) void adam8_step_split_kernel(const DevTensor 
                 reinterpret_cast<f32x4 *>(mine[0])[lane] = ds;
                 reinterpret_cast<f32x4 *>(mine[1])[lane] = du;
             }
-            bool redo[8]; // per element: the exact chain runs for the flagged positions only
-            bool any = false;
+            Redo8 redo; // per element: the exact chain runs for the flagged positions only
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
                 const float t1 = lds_float_at(mine[0], code_offset(q.mr, k));
                 const float t3 = lds_float_at(mine[1], code_offset(q.vr, k));
-                redo[k] = false;
-                adam_elem_decayed<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], t1, t3, h, gscale, dbc1, dbc2, m[k], v[k], pn[k], redo[k]);
-                any |= redo[k];
+                uint64_t flagged = 0;
+                adam_elem_decayed<MODE, EXACT, BF16, WD, GS>(pv[k], gv[k], t1, t3, h, gscale, dbc1, dbc2, m[k], v[k], pn[k], flagged);
+                redo.set(k, flagged);
                 nam = fmaxf(nam, __builtin_fabsf(m[k]));
                 nav = fmaxf(nav, __builtin_fabsf(v[k]));
             }
-            if (any) {
+            if (BF16 && MODE == ERI_ADAM8_MODE_L2 && h.l2_all_exact) redo.set_all();
+            if (BF16 && redo.any) {
 #pragma unroll
                 for (int k = 0; k < 8; ++k)
-                    if (redo[k]) pn[k] = param_exact<MODE, WD, BF16>(pv[k], m[k], v[k], h, dbc1, dbc2);
+                    if (redo.lanes[k] && redo.mine(k)) pn[k] = param_exact<MODE, WD, BF16>(pv[k], m[k], v[k], h, dbc1, dbc2);
             }
             store8<BF16>(p, o, pn);
             wave_max2(nam, nav);

@@ -43,22 +43,25 @@ int fail(int code, const std::string &msg) {
 /* uint8 codes and per-block absmax of both moments, in one device allocation or one piece of a memory pool. */
 struct State8 {
     void *base = nullptr;
-    bool pooled = false; // the piece belongs to a pool and goes back with it
+    EriHipPool *pool = nullptr; // the pool the piece came from and goes back to (not owned), or null
+    uint64_t total = 0;         // bytes of the piece
     uint8_t *m = nullptr, *v = nullptr;
     float *absmax_m = nullptr, *absmax_v = nullptr;
     uint64_t numel = 0;
 
-    int allocate(uint64_t n, void *stream, EriHipPool *pool = nullptr, uint32_t lane = 0) {
+    int allocate(uint64_t n, void *stream, EriHipPool *from = nullptr, uint32_t lane = 0) {
         release();
         const uint64_t nb = blocks_of(n);
         const uint64_t o_v = align256(n), o_am = o_v + align256(n), o_av = o_am + align256(nb * 4);
-        const uint64_t total = o_av + align256(nb * 4);
+        const uint64_t bytes = o_av + align256(nb * 4);
         int dev = 0;
         int rc = eri_hip_get_device(&dev);
         if (rc) return rc;
-        rc = pool ? eri_hip_pool_alloc_zeroed(pool, lane, total, &base) : eri_hip_malloc_zeroed(dev, total, &base);
+        // out of a pool the piece is cleared on the optimizer's stream (state_init below overwrites it anyway)
+        rc = from ? eri_hip_pool_alloc_zeroed_async(from, lane, bytes, stream, &base) : eri_hip_malloc_zeroed(dev, bytes, &base);
         if (rc) return rc;
-        pooled = pool != nullptr;
+        pool = from;
+        total = bytes;
         char *b = static_cast<char *>(base);
         m = reinterpret_cast<uint8_t *>(b);
         v = reinterpret_cast<uint8_t *>(b + o_v);
@@ -68,10 +71,14 @@ struct State8 {
         // the state of a zeros tensor (adam8bit_enhanced.rs:179-197)
         return eri_adam8_state_init(m, v, absmax_m, absmax_v, n, stream);
     }
+    /* A pooled piece goes back to its pool, where the next state of the same size takes it (loading a checkpoint
+     * replaces every state by one of its size).  The pool must outlive the states it backs. */
     void release() {
-        if (base && !pooled) eri_hip_free(base);
+        if (base && pool) eri_hip_pool_release(pool, base, total);
+        else if (base) eri_hip_free(base);
         base = nullptr;
-        pooled = false;
+        pool = nullptr;
+        total = 0;
         m = v = nullptr;
         absmax_m = absmax_v = nullptr;
         numel = 0;
@@ -404,6 +411,9 @@ struct EriAdam8bit {
     EriAdam8Table *table = nullptr;
     std::vector<uint32_t> table_ids;         // parameter indices the table was built for
     std::vector<EriAdam8Tensor> table_rows;  // rows as last uploaded
+    EriAdam8Table *grad_table = nullptr;     // gradients of the tensors kept in 32-bit moments, for the global norm
+    std::vector<EriAdam8Tensor> grad_rows;
+    EriAdam8Table *norm_table = nullptr;     // the table that holds the last norm: table or grad_table (not owned twice)
 };
 
 /* One named state of the functional flavour with its own one-row launch table: updates of many
@@ -431,10 +441,20 @@ struct EriAdam8bitFn {
     std::vector<EriAdam8Tensor> pending;     // rows in call order
     std::vector<std::pair<const std::string *, FnState *>> pending_who;
     std::vector<std::pair<const std::string *, FnState *>> last_order; // names of the last flush, in order
-    EriAdam8Table *table = nullptr;          // launch table of the last flush
-    std::vector<EriAdam8Tensor> table_rows;
+    // Launch tables of the last two distinct sets of rows.  update() returns a new tensor per call
+    // (adam8bit.rs:205-207), so the pointers of one flush differ from those of the flush before; a trainer
+    // that drops the old tensor as it takes the new one gets the old addresses back from its allocator, and
+    // the row sets alternate between two.  Two tables then serve every flush without an upload.
+    struct TableSlot {
+        EriAdam8Table *table = nullptr;
+        std::vector<EriAdam8Tensor> rows; // as last uploaded
+        uint64_t used = 0;                // flush counter of the last use
+    } slots[2];
+    uint64_t flushes = 0;
+    uint64_t uploads = 0; // flushes that had to create or re-upload a table
     ~EriAdam8bitFn() {
-        if (table) eri_adam8_table_destroy(table);
+        for (auto &sl : slots)
+            if (sl.table) eri_adam8_table_destroy(sl.table);
     }
 };
 
@@ -534,6 +554,7 @@ int eri_adam8bit_new(EriParameter *const *params, uint32_t n, const EriAdam8bitC
 int eri_adam8bit_destroy(EriAdam8bit *o) {
     if (!o) return 0;
     if (o->table) eri_adam8_table_destroy(o->table);
+    if (o->grad_table) eri_adam8_table_destroy(o->grad_table);
     for (auto *p : o->params) eri_param_release(p);
     delete o;
     return 0;
@@ -602,6 +623,8 @@ static int adam8bit_step_impl(EriAdam8bit *o, uint32_t *skipped) {
             r.v = o->states32[i]->v;
             r.numel = p->numel;
             r.dtype_tag = p->dtype;
+            r.grad_scale = o->param_scale[i];
+            scaled = scaled || o->param_scale[i] != 1.0f;
             rows32.push_back(r);
             continue;
         }
@@ -665,14 +688,69 @@ static int adam8bit_step_impl(EriAdam8bit *o, uint32_t *skipped) {
             if (in_table) ++k;
         }
     }
-    if (!rows32.empty()) { // refused before anything is launched
-        for (uint32_t i = 0; i < o->params.size(); ++i) scaled = scaled || (o->states32[i] && o->param_scale[i] != 1.0f);
-        if (scaled || clip)
-            return fail(ERI_ERR_ARG, "InvalidOperation: min_8bit_size cannot be combined with gradient scaling or clipping inside the step");
-        if (o->mode != ERI_ADAM8_MODE_ERI)
-            return fail(ERI_ERR_ARG, "InvalidOperation: min_8bit_size needs mode ERI");
-    }
+    if (!rows32.empty() && o->mode != ERI_ADAM8_MODE_ERI) // refused before anything is launched
+        return fail(ERI_ERR_ARG, "InvalidOperation: min_8bit_size needs mode ERI");
+    // Everything that can be refused comes before the first launch: both launch tables are built or refreshed
+    // here, so that a step that fails on them has changed nothing.
     int rc = 0;
+    if (!rows.empty()) {
+        if (!o->table || ids != o->table_ids) {
+            if (o->table) eri_adam8_table_destroy(o->table);
+            o->table = nullptr;
+            o->norm_table = nullptr; // whichever table held the last norm, its result may have lived in this one
+            rc = eri_adam8_table_create(rows.data(), (uint32_t)rows.size(), o->stream, &o->table);
+            if (rc) return rc;
+            o->table_ids = ids;
+            o->table_rows = rows;
+            o->have_qerr = false;
+        } else if (std::memcmp(rows.data(), o->table_rows.data(), rows.size() * sizeof(EriAdam8Tensor)) != 0) {
+            rc = eri_adam8_table_update(o->table, rows.data(), (uint32_t)rows.size(), o->stream);
+            if (rc) return rc;
+            o->table_rows = rows;
+        }
+    }
+    // The tensors kept in 32-bit moments are clipped by the same global norm as the rest
+    // (pipeline_flux_lora_1024.rs:691-697 clips every trainable gradient, then steps): their gradients go into
+    // a gradient-only table that is normed together with the 8-bit table.
+    if (clip && !rows32.empty()) {
+        std::vector<EriAdam8Tensor> grows(rows32.size());
+        uint64_t gstart = 0;
+        for (size_t k = 0; k < rows32.size(); ++k) {
+            EriAdam8Tensor &g = grows[k];
+            std::memset(&g, 0, sizeof g);
+            g.p = rows32[k].p;
+            g.g = rows32[k].g;
+            g.numel = rows32[k].numel;
+            g.dtype_tag = rows32[k].dtype_tag;
+            g.block_start = gstart;
+            g.grad_scale = 1.0f;
+            gstart += blocks_of(g.numel);
+        }
+        bool same = o->grad_table && o->grad_rows.size() == grows.size();
+        for (size_t k = 0; same && k < grows.size(); ++k)
+            same = grows[k].numel == o->grad_rows[k].numel && grows[k].dtype_tag == o->grad_rows[k].dtype_tag;
+        if (!same) {
+            if (o->grad_table) eri_adam8_table_destroy(o->grad_table);
+            o->grad_table = nullptr;
+            o->norm_table = nullptr;
+            o->grad_rows.clear();
+            rc = eri_adam8_grad_table_create(grows.data(), (uint32_t)grows.size(), o->stream, &o->grad_table);
+            if (rc) return rc;
+            o->grad_rows = grows;
+        } else if (std::memcmp(grows.data(), o->grad_rows.data(), grows.size() * sizeof(EriAdam8Tensor)) != 0) {
+            rc = eri_adam8_table_update(o->grad_table, grows.data(), (uint32_t)grows.size(), o->stream);
+            if (rc) return rc;
+            o->grad_rows = grows;
+        }
+    }
+    if (clip) { // one norm over every gradient of this step
+        if (!rows.empty() && !rows32.empty())
+            rc = eri_adam8_grad_norm_joint(o->table, o->grad_table, o->max_grad_norm, o->clip_denom_eps, o->stream);
+        else
+            rc = eri_adam8_grad_norm(rows.empty() ? o->grad_table : o->table, o->max_grad_norm, o->clip_denom_eps, o->stream);
+        if (rc) return rc;
+        o->norm_table = rows.empty() ? o->grad_table : o->table;
+    }
     if (!rows32.empty()) {
         // The reference's update with fp32 moments: the 32-bit step computes
         // p + ((m/(sqrt(v)+eps)) + p*wd) * (-lr), which with lr = the bias-corrected step size is
@@ -686,27 +764,19 @@ static int adam8bit_step_impl(EriAdam8bit *o, uint32_t *skipped) {
         h32.beta2 = h8.beta2;
         h32.eps = h8.eps;
         h32.weight_decay = h8.weight_decay > 0.0f ? h8.weight_decay : 0.0f; // :267: decay only if positive
-        rc = eri_adamw32_step_multi(rows32.data(), (uint32_t)rows32.size(), &h32, o->stream);
+        if (scaled || clip) { // the factors the 8-bit rows get inside their kernel, in the same order
+            const float *dev_scale = nullptr;
+            if (clip) {
+                rc = eri_adam8_grad_norm_scale_ptr(o->norm_table, &dev_scale);
+                if (rc) return rc;
+            }
+            rc = eri_adamw32_step_multi_scaled(rows32.data(), (uint32_t)rows32.size(), &h32, o->grad_scale, dev_scale, o->stream);
+        } else {
+            rc = eri_adamw32_step_multi(rows32.data(), (uint32_t)rows32.size(), &h32, o->stream);
+        }
         if (rc) return rc;
     }
     if (rows.empty()) return adam8bit_ema_rest(o, ema_others, ema_new, ema_decay);
-    if (!o->table || ids != o->table_ids) {
-        if (o->table) eri_adam8_table_destroy(o->table);
-        o->table = nullptr;
-        rc = eri_adam8_table_create(rows.data(), (uint32_t)rows.size(), o->stream, &o->table);
-        if (rc) return rc;
-        o->table_ids = ids;
-        o->table_rows = rows;
-        o->have_qerr = false;
-    } else if (std::memcmp(rows.data(), o->table_rows.data(), rows.size() * sizeof(EriAdam8Tensor)) != 0) {
-        rc = eri_adam8_table_update(o->table, rows.data(), (uint32_t)rows.size(), o->stream);
-        if (rc) return rc;
-        o->table_rows = rows;
-    }
-    if (clip) {
-        rc = eri_adam8_grad_norm(o->table, o->max_grad_norm, o->clip_denom_eps, o->stream);
-        if (rc) return rc;
-    }
     EriAdam8Hyper h;
     uint32_t flags = o->flags | ((scaled || clip) ? (uint32_t)ERI_ADAM8_FLAG_GRAD_SCALE : 0u) |
                      (clip ? (uint32_t)ERI_ADAM8_FLAG_CLIP_FROM_TABLE : 0u);
@@ -783,14 +853,14 @@ int eri_adam8bit_set_max_grad_norm(EriAdam8bit *o, float max_norm, float denom_e
 
 int eri_adam8bit_last_grad_norm(EriAdam8bit *o, float *norm, float *scale) {
     if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
-    if (!o->table) return fail(ERI_ERR_ARG, "no step has run yet");
-    return eri_adam8_grad_norm_read(o->table, norm, scale, o->stream);
+    if (!o->norm_table) return fail(ERI_ERR_ARG, "no step with gradient clipping has run yet");
+    return eri_adam8_grad_norm_read(o->norm_table, norm, scale, o->stream);
 }
 
 int eri_adam8bit_last_nonfinite_grads(EriAdam8bit *o, uint64_t *count) {
     if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
-    if (!o->table) return fail(ERI_ERR_ARG, "no step has run yet");
-    return eri_adam8_grad_nonfinite_read(o->table, count, o->stream);
+    if (!o->norm_table) return fail(ERI_ERR_ARG, "no step with gradient clipping has run yet");
+    return eri_adam8_grad_nonfinite_read(o->norm_table, count, o->stream);
 }
 
 int eri_adam8bit_track_quantization_error(EriAdam8bit *o, int enabled) {
@@ -1024,6 +1094,7 @@ int eri_adam8bit_load_state(EriAdam8bit *o, const char *path) {
     if (o->table) { // state pointers changed
         eri_adam8_table_destroy(o->table);
         o->table = nullptr;
+        o->norm_table = nullptr;
         o->table_ids.clear();
     }
     return 0;
@@ -1202,6 +1273,7 @@ extern "C" int eri_adam8bit_load_legacy_state(EriAdam8bit *o, const char *path) 
     if (o->table) {
         eri_adam8_table_destroy(o->table);
         o->table = nullptr;
+        o->norm_table = nullptr;
         o->table_ids.clear();
     }
     return 0;
@@ -1294,8 +1366,9 @@ int fn_hyper(const EriAdam8bitFn *o, EriAdam8Hyper *h) {
                                 ERI_ADAM8_FLAG_EXACT_PARAM, h);
 }
 
-/* One launch over every queued row.  The launch table of the last flush is kept: the same tensors with
- * new pointers cost one small upload, the same pointers cost nothing. */
+/* One launch over every queued row.  The launch tables of the last two distinct row sets are kept: rows that
+ * equal one of them cost nothing, the same tensors with new pointers cost one small upload into the table
+ * that was used longer ago. */
 int fn_flush(EriAdam8bitFn *o) {
     if (o->pending.empty()) return 0;
     std::vector<EriAdam8Tensor> rows;
@@ -1311,22 +1384,43 @@ int fn_flush(EriAdam8bitFn *o) {
     EriAdam8Hyper h;
     int rc = fn_hyper(o, &h);
     if (rc) return rc;
-    bool same = o->table && o->table_rows.size() == rows.size();
-    for (size_t i = 0; same && i < rows.size(); ++i)
-        same = rows[i].numel == o->table_rows[i].numel && rows[i].dtype_tag == o->table_rows[i].dtype_tag &&
-               rows[i].grad_f32 == o->table_rows[i].grad_f32;
-    if (!same) {
-        if (o->table) eri_adam8_table_destroy(o->table);
-        o->table = nullptr;
-        o->table_rows.clear();
-        rc = eri_adam8_table_create(rows.data(), (uint32_t)rows.size(), o->stream, &o->table);
-    } else if (std::memcmp(rows.data(), o->table_rows.data(), rows.size() * sizeof(EriAdam8Tensor)) != 0) {
-        rc = eri_adam8_table_update(o->table, rows.data(), (uint32_t)rows.size(), o->stream);
+    o->flushes += 1;
+    const size_t bytes = rows.size() * sizeof(EriAdam8Tensor);
+    // the table used longer ago first: that is the one an alternating trainer comes back to
+    const int older = o->slots[0].used <= o->slots[1].used ? 0 : 1;
+    EriAdam8bitFn::TableSlot *hit = nullptr;
+    for (int k : {older, 1 - older}) {
+        auto &sl = o->slots[k];
+        if (sl.table && sl.rows.size() == rows.size() && std::memcmp(rows.data(), sl.rows.data(), bytes) == 0) {
+            hit = &sl;
+            break;
+        }
     }
-    if (rc) return rc;
-    o->table_rows.swap(rows);
+    if (!hit) {
+        auto &sl = o->slots[older];
+        bool same = sl.table && sl.rows.size() == rows.size();
+        for (size_t i = 0; same && i < rows.size(); ++i)
+            same = rows[i].numel == sl.rows[i].numel && rows[i].dtype_tag == sl.rows[i].dtype_tag &&
+                   rows[i].grad_f32 == sl.rows[i].grad_f32;
+        if (!same) {
+            if (sl.table) eri_adam8_table_destroy(sl.table);
+            sl.table = nullptr;
+            sl.rows.clear();
+            rc = eri_adam8_table_create(rows.data(), (uint32_t)rows.size(), o->stream, &sl.table);
+        } else {
+            rc = eri_adam8_table_update(sl.table, rows.data(), (uint32_t)rows.size(), o->stream);
+        }
+        if (rc) {
+            sl.rows.clear(); // whatever the table holds now, it is not a set to come back to
+            return rc;
+        }
+        sl.rows.swap(rows);
+        o->uploads += 1;
+        hit = &sl;
+    }
+    hit->used = o->flushes;
     o->last_order.swap(who);
-    return eri_adam8_step_table(o->table, &h, o->stream);
+    return eri_adam8_step_table(hit->table, &h, o->stream);
 }
 
 int fn_enqueue(EriAdam8bitFn *o, const char *name, const void *param, const void *grad, uint64_t numel, int dtype_tag,
@@ -1390,12 +1484,35 @@ int eri_adam8bit_fn_update_many(EriAdam8bitFn *o, const char *const *names, cons
                                 const int32_t *grad_dtype_tags, void *const *outs, uint32_t n) {
     if (!o || !names || !params || !grads || !numels || !dtype_tags || !outs)
         return fail(ERI_ERR_NULL, "update_many with NULL argument");
-    int rc = fn_flush(o); // rows queued by earlier update() calls keep their place in the order of updates
+    // 1. every row is checked before anything runs: arguments, and the size of a state that exists already
+    for (uint32_t i = 0; i < n; ++i) {
+        int rc = fn_check_update(names[i], params[i], grads[i], numels[i], dtype_tags[i],
+                                 grad_dtype_tags ? grad_dtype_tags[i] : dtype_tags[i], outs[i]);
+        if (rc) return rc;
+        auto it = o->states.find(std::string_view(names[i]));
+        if (it != o->states.end() && it->second->numel != numels[i])
+            return fail(ERI_ERR_ARG, std::string("state of '") + names[i] + "' has a different size");
+    }
+    // 2. states of new names; a failure takes back the ones this call made
+    std::vector<std::string> made;
+    for (uint32_t i = 0; i < n; ++i) {
+        if (o->states.find(std::string_view(names[i])) != o->states.end()) continue;
+        std::unique_ptr<FnState> s(new FnState());
+        int rc = s->allocate(numels[i], o->stream, o->state_pool, o->state_lane);
+        if (rc) {
+            for (auto &name : made) o->states.erase(name);
+            return rc;
+        }
+        made.emplace_back(names[i]);
+        o->states.emplace(names[i], std::move(s));
+    }
+    // 3. rows queued by earlier update() calls keep their place in the order of updates
+    int rc = fn_flush(o);
     if (rc) return rc;
     for (uint32_t i = 0; i < n; ++i) {
         rc = fn_enqueue(o, names[i], params[i], grads[i], numels[i], dtype_tags[i],
                         grad_dtype_tags ? grad_dtype_tags[i] : dtype_tags[i], outs[i]);
-        if (rc) { // nothing of a refused call runs
+        if (rc) { // only a launch can fail here (a name that repeats flushes the rows before it)
             o->pending.clear();
             o->pending_who.clear();
             o->generation += 1;
@@ -1403,6 +1520,13 @@ int eri_adam8bit_fn_update_many(EriAdam8bitFn *o, const char *const *names, cons
         }
     }
     return fn_flush(o);
+}
+
+int eri_adam8bit_fn_table_stats(const EriAdam8bitFn *o, uint64_t *flushes, uint64_t *uploads) {
+    if (!o) return fail(ERI_ERR_NULL, "optimizer is NULL");
+    if (flushes) *flushes = o->flushes;
+    if (uploads) *uploads = o->uploads;
+    return 0;
 }
 
 int eri_adam8bit_fn_set_state_pool(EriAdam8bitFn *o, EriHipPool *pool, uint32_t lane) {

@@ -290,7 +290,9 @@ struct EriAdam8Table {
     bool ordered_valid = false;
     double *partial = nullptr; // one sum of squares per wave of the norm pass, per group
     float *norm_out = nullptr; // device: {norm, clip factor, 64-bit count}, owned by the table
-    float *norm_last = nullptr; // where the last norm pass left its result: norm_out, or the caller's buffer
+    float *norm_last = nullptr; // where the last norm pass left its result: norm_out, the caller's buffer, or the
+                                // norm_out of the table this one was normed together with
+    bool grads_only = false;    // rows carry gradients only: the table serves the norm pass and nothing else
     uint32_t n_partial = 0;
     double *qerr = nullptr;    // device: per row {sum |m - deq m|, sum |v - deq v|}, groups back to back
     bool qerr_valid = false;
@@ -303,14 +305,14 @@ int layout_of(const EriAdam8Tensor &r) {
     return r.grad_f32 ? eri::kLayoutBF16GradF32 : eri::kLayoutBF16;
 }
 
-int validate_rows(const EriAdam8Tensor *rows, uint32_t n) {
+int validate_rows(const EriAdam8Tensor *rows, uint32_t n, bool grads_only = false) {
     if (!rows) return fail(ERI_ERR_NULL, "rows is NULL");
     if (n == 0) return fail(ERI_ERR_ARG, "launch table has no rows");
     uint64_t running = 0;
     char buf[160];
     for (uint32_t i = 0; i < n; ++i) {
         const EriAdam8Tensor &r = rows[i];
-        if (!r.p || !r.g || !r.m || !r.v || !r.absmax_m || !r.absmax_v) {
+        if (grads_only ? !r.g : (!r.p || !r.g || !r.m || !r.v || !r.absmax_m || !r.absmax_v)) {
             std::snprintf(buf, sizeof buf, "row %u: NULL pointer", i);
             return fail(ERI_ERR_NULL, buf);
         }
@@ -499,9 +501,35 @@ struct EriHipPool {
     int device = 0;
     char *base = nullptr;
     size_t lane_bytes = 0;
-    std::vector<size_t> used; // per lane
+    std::vector<size_t> used; // per lane: bytes handed out from the lane's start upwards
+    struct Piece {
+        size_t offset, bytes; // inside the lane
+    };
+    std::vector<std::vector<Piece>> released; // per lane: pieces given back below the lane's top
     std::mutex lock;
 };
+
+namespace {
+
+/* Takes `need` bytes (a multiple of 256) out of `lane`: a released piece of exactly that size if there is one,
+ * else the next bytes above the lane's top. */
+char *pool_take(EriHipPool *pool, uint32_t lane, size_t need) {
+    auto &back = pool->released[lane];
+    for (size_t i = 0; i < back.size(); ++i) {
+        if (back[i].bytes == need) {
+            char *p = pool->base + (size_t)lane * pool->lane_bytes + back[i].offset;
+            back[i] = back.back();
+            back.pop_back();
+            return p;
+        }
+    }
+    if (need > pool->lane_bytes - pool->used[lane]) return nullptr;
+    char *p = pool->base + (size_t)lane * pool->lane_bytes + pool->used[lane];
+    pool->used[lane] += need;
+    return p;
+}
+
+} // namespace
 
 extern "C" {
 
@@ -537,6 +565,7 @@ int eri_hip_pool_create(int device, size_t bytes, uint32_t lanes, EriHipPool **o
     pool->base = static_cast<char *>(p);
     pool->lane_bytes = lane_bytes;
     pool->used.assign(lanes, 0);
+    pool->released.assign(lanes, {});
     *out = pool;
     return 0;
 }
@@ -549,19 +578,79 @@ int eri_hip_pool_alloc_zeroed(EriHipPool *pool, uint32_t lane, size_t bytes, voi
     char *p = nullptr;
     {
         std::lock_guard<std::mutex> g(pool->lock);
-        lane %= (uint32_t)pool->used.size();
-        if (need > pool->lane_bytes - pool->used[lane])
-            return fail(ERI_ERR_ARG, "memory pool: the lane is full");
-        p = pool->base + (size_t)lane * pool->lane_bytes + pool->used[lane];
-        pool->used[lane] += need;
+        p = pool_take(pool, lane % (uint32_t)pool->used.size(), need);
     }
+    if (!p) return fail(ERI_ERR_ARG, "memory pool: the lane is full");
     int prev = 0;
     ERI_HIP(hipGetDevice(&prev));
     if (prev != pool->device) ERI_HIP(hipSetDevice(pool->device));
     const hipError_t e = hipMemset(p, 0, bytes);
     if (prev != pool->device) (void)hipSetDevice(prev);
-    if (e != hipSuccess) return hip_fail(e, "hipMemset");
+    if (e != hipSuccess) {
+        (void)eri_hip_pool_release(pool, p, bytes);
+        return hip_fail(e, "hipMemset");
+    }
     *out = p;
+    return 0;
+}
+
+int eri_hip_pool_alloc_zeroed_async(EriHipPool *pool, uint32_t lane, size_t bytes, void *stream, void **out) {
+    if (!pool || !out) return fail(ERI_ERR_NULL, "pool or out is NULL");
+    *out = nullptr;
+    if (bytes == 0) return fail(ERI_ERR_EMPTY, "pool allocation of zero bytes");
+    const size_t need = (bytes + 255) / 256 * 256;
+    char *p = nullptr;
+    {
+        std::lock_guard<std::mutex> g(pool->lock);
+        p = pool_take(pool, lane % (uint32_t)pool->used.size(), need);
+    }
+    if (!p) return fail(ERI_ERR_ARG, "memory pool: the lane is full");
+    int prev = 0;
+    ERI_HIP(hipGetDevice(&prev));
+    if (prev != pool->device) ERI_HIP(hipSetDevice(pool->device));
+    // pieces are 256-byte aligned and so is `need`: the whole piece is cleared, with a kernel (a memset node in
+    // a captured graph is not reliable on this stack, and the runtime's synchronous memset blocks the host)
+    const int rc = eri::launch_fill_zero(p, need, stream);
+    if (prev != pool->device) (void)hipSetDevice(prev);
+    if (rc) {
+        (void)eri_hip_pool_release(pool, p, bytes);
+        return hip_fail((hipError_t)rc, "fill kernel");
+    }
+    *out = p;
+    return 0;
+}
+
+int eri_hip_pool_release(EriHipPool *pool, void *ptr, size_t bytes) {
+    if (!pool) return fail(ERI_ERR_NULL, "pool is NULL");
+    if (!ptr) return 0;
+    const size_t need = (bytes + 255) / 256 * 256;
+    char *p = static_cast<char *>(ptr);
+    std::lock_guard<std::mutex> g(pool->lock);
+    const size_t lanes = pool->used.size();
+    if (bytes == 0 || p < pool->base || p >= pool->base + pool->lane_bytes * lanes)
+        return fail(ERI_ERR_ARG, "memory pool: release of a piece that is not the pool's");
+    const size_t lane = (size_t)(p - pool->base) / pool->lane_bytes;
+    const size_t offset = (size_t)(p - pool->base) % pool->lane_bytes;
+    if (offset % 256 != 0 || offset + need > pool->used[lane])
+        return fail(ERI_ERR_ARG, "memory pool: release of a piece that is not the pool's");
+    if (offset + need == pool->used[lane]) { // the top piece: the lane shrinks, and so it does past released pieces below it
+        pool->used[lane] = offset;
+        auto &back = pool->released[lane];
+        for (bool again = true; again;) {
+            again = false;
+            for (size_t i = 0; i < back.size(); ++i) {
+                if (back[i].offset + back[i].bytes == pool->used[lane]) {
+                    pool->used[lane] = back[i].offset;
+                    back[i] = back.back();
+                    back.pop_back();
+                    again = true;
+                    break;
+                }
+            }
+        }
+    } else {
+        pool->released[lane].push_back({offset, need});
+    }
     return 0;
 }
 
@@ -583,6 +672,7 @@ int eri_hip_pool_reset(EriHipPool *pool) {
     if (!pool) return fail(ERI_ERR_NULL, "pool is NULL");
     std::lock_guard<std::mutex> g(pool->lock);
     for (auto &u : pool->used) u = 0;
+    for (auto &r : pool->released) r.clear();
     return 0;
 }
 
@@ -730,16 +820,17 @@ int eri_adam8_state_init(uint8_t *m, uint8_t *v, float *absmax_m, float *absmax_
     return 0;
 }
 
-int eri_adam8_table_create(const EriAdam8Tensor *rows, uint32_t n, void *stream, EriAdam8Table **out) {
+static int table_create(const EriAdam8Tensor *rows, uint32_t n, bool grads_only, void *stream, EriAdam8Table **out) {
     if (!out) return fail(ERI_ERR_NULL, "out is NULL");
     *out = nullptr;
-    int rc = validate_rows(rows, n);
+    int rc = validate_rows(rows, n, grads_only);
     if (rc) return rc;
     DeviceCtx *ctx = nullptr;
     rc = get_ctx(&ctx);
     if (rc) return rc;
     EriAdam8Table *t = new EriAdam8Table();
     t->n = n;
+    t->grads_only = grads_only;
     (void)hipGetDevice(&t->device);
     for (int li = 0; li < eri::kLayouts; ++li) t->groups[li].dtype = li; // a Layout
     t->numel.resize(n);
@@ -781,9 +872,17 @@ int eri_adam8_table_create(const EriAdam8Tensor *rows, uint32_t n, void *stream,
     return 0;
 }
 
+int eri_adam8_table_create(const EriAdam8Tensor *rows, uint32_t n, void *stream, EriAdam8Table **out) {
+    return table_create(rows, n, false, stream, out);
+}
+
+int eri_adam8_grad_table_create(const EriAdam8Tensor *rows, uint32_t n, void *stream, EriAdam8Table **out) {
+    return table_create(rows, n, true, stream, out);
+}
+
 int eri_adam8_table_update(EriAdam8Table *t, const EriAdam8Tensor *rows, uint32_t n, void *stream) {
     if (!t) return fail(ERI_ERR_NULL, "table is NULL");
-    int rc = validate_rows(rows, n);
+    int rc = validate_rows(rows, n, t->grads_only);
     if (rc) return rc;
     if (n != t->n) return fail(ERI_ERR_ARG, "table_update: row count differs from the table's");
     for (uint32_t i = 0; i < n; ++i)
@@ -812,6 +911,7 @@ int eri_adam8_table_info(const EriAdam8Table *t, uint64_t *total_numel, uint64_t
 
 int eri_adam8_step_table(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream) {
     if (!t || !h) return fail(ERI_ERR_NULL, "table or hyper is NULL");
+    if (t->grads_only) return fail(ERI_ERR_ARG, "a gradient-only table serves eri_adam8_grad_norm only");
     if (h->mode != ERI_ADAM8_MODE_ERI && h->mode != ERI_ADAM8_MODE_L2 && h->mode != ERI_ADAM8_MODE_BNB)
         return fail(ERI_ERR_ARG, "unknown mode");
     if ((h->flags & ERI_ADAM8_FLAG_EMA) && !(h->ema_decay >= 0.0f && h->ema_decay <= 1.0f))
@@ -829,6 +929,7 @@ int eri_adam8_step_table(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream)
     }
     rc = order_after_upload(t, stream);
     if (rc) return rc;
+    std::vector<EriEmaTensor> ema_rest;
     for (auto &g : t->groups) {
         if (g.n == 0) continue;
         // One wavefront per block.  A small table gets smaller workgroups so that its blocks still
@@ -854,8 +955,7 @@ int eri_adam8_step_table(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream)
         rc = eri::launch_step(g.dev, g.n, g.total_blocks, g.dtype, hh, ctx->image, dev_scale, grid, waves_per_wg * eri::kWave, ctx->cus, stream);
         if (rc) return hip_fail((hipError_t)rc, "adam8 step launch");
         if ((hh.flags & ERI_ADAM8_FLAG_EMA) && !eri::step_fuses_ema(g.total_blocks, g.dtype, hh, ctx->cus)) {
-            // not the kernel that carries the EMA: the plain sweep over this group's shadows, right behind the step
-            std::vector<EriEmaTensor> er;
+            // not the kernel that carries the EMA: this group's shadows join the plain sweep that follows the step
             for (uint32_t j = 0; j < g.n; ++j) {
                 const eri::DevTensor &d = g.pinned[j];
                 if (!d.shadow) continue;
@@ -865,31 +965,37 @@ int eri_adam8_step_table(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream)
                 e.numel = d.numel;
                 e.dtype_tag = eri::layout_param_bf16(g.dtype) ? ERI_DTYPE_BF16 : ERI_DTYPE_F32;
                 e.reserved = 0;
-                er.push_back(e);
-            }
-            if (!er.empty()) {
-                rc = eri_ema_update_multi(er.data(), (uint32_t)er.size(), hh.ema_decay, stream);
-                if (rc) return rc;
+                ema_rest.push_back(e);
             }
         }
+    }
+    if (!ema_rest.empty()) { // one sweep for all groups that did not carry their EMA, right behind the step
+        rc = eri_ema_update_multi(ema_rest.data(), (uint32_t)ema_rest.size(), h->ema_decay, stream);
+        if (rc) return rc;
     }
     return 0;
 }
 
-/* The two launches of the gradient-norm pass.  `partial` holds room for `pairs` {sum, count} pairs. */
-static int grad_norm_launch(EriAdam8Table *t, DeviceCtx *ctx, float max_norm, float denom_eps, double *partial,
-                            uint32_t pairs, float *result, void *stream) {
+/* The launches of the gradient-norm pass over one table, or over two as if they were one (`also` may be null):
+ * a sum-of-squares launch per group of rows, then one launch that adds the per-wave partial sums of all of them.
+ * `partial` holds room for `pairs` {sum, count} pairs. */
+static int grad_norm_launch(EriAdam8Table *t, EriAdam8Table *also, DeviceCtx *ctx, float max_norm, float denom_eps,
+                            double *partial, uint32_t pairs, float *result, void *stream) {
     const uint32_t wpw = (uint32_t)eri::kNormWaves;
     const uint32_t grid_cap = ctx->cus * eri::kNormWavesPerCu / wpw; // persistent
-    uint32_t grids[eri::kLayouts] = {0, 0, 0}, need = 0;
-    for (int gi = 0; gi < eri::kLayouts; ++gi) {
-        const auto &g = t->groups[gi];
-        if (g.n == 0) continue;
-        const uint32_t work = g.total_blocks > g.n ? g.total_blocks : g.n;
-        uint32_t grid = (work + wpw - 1) / wpw;
-        if (grid > grid_cap) grid = grid_cap;
-        grids[gi] = grid;
-        need += grid * wpw;
+    EriAdam8Table *tables[2] = {t, also};
+    uint32_t grids[2][eri::kLayouts] = {{0, 0, 0}, {0, 0, 0}}, need = 0;
+    for (int ti = 0; ti < 2; ++ti) {
+        if (!tables[ti]) continue;
+        for (int gi = 0; gi < eri::kLayouts; ++gi) {
+            const auto &g = tables[ti]->groups[gi];
+            if (g.n == 0) continue;
+            const uint32_t work = g.total_blocks > g.n ? g.total_blocks : g.n;
+            uint32_t grid = (work + wpw - 1) / wpw;
+            if (grid > grid_cap) grid = grid_cap;
+            grids[ti][gi] = grid;
+            need += grid * wpw;
+        }
     }
     if (need > pairs) {
         char buf[160];
@@ -897,33 +1003,55 @@ static int grad_norm_launch(EriAdam8Table *t, DeviceCtx *ctx, float max_norm, fl
                       need, pairs);
         return fail(ERI_ERR_TOO_LARGE, buf);
     }
-    int rc = order_after_upload(t, stream);
-    if (rc) return rc;
     uint32_t off = 0;
-    for (int gi = 0; gi < eri::kLayouts; ++gi) {
-        auto &g = t->groups[gi];
-        if (g.n == 0) continue;
-        rc = eri::launch_grad_sumsq(g.dev, g.n, g.total_blocks, eri::layout_grad_bf16(g.dtype), partial + 2 * off, grids[gi], stream);
-        if (rc) return hip_fail((hipError_t)rc, "gradient sum-of-squares launch");
-        off += grids[gi] * wpw;
+    for (int ti = 0; ti < 2; ++ti) {
+        if (!tables[ti]) continue;
+        int rc = order_after_upload(tables[ti], stream);
+        if (rc) return rc;
+        for (int gi = 0; gi < eri::kLayouts; ++gi) {
+            auto &g = tables[ti]->groups[gi];
+            if (g.n == 0) continue;
+            rc = eri::launch_grad_sumsq(g.dev, g.n, g.total_blocks, eri::layout_grad_bf16(g.dtype), partial + 2 * off, grids[ti][gi], stream);
+            if (rc) return hip_fail((hipError_t)rc, "gradient sum-of-squares launch");
+            off += grids[ti][gi] * wpw;
+        }
     }
     t->n_partial = off;
-    rc = eri::launch_grad_norm_finish(partial, off, max_norm, denom_eps, result, stream);
+    int rc = eri::launch_grad_norm_finish(partial, off, max_norm, denom_eps, result, stream);
     if (rc) return hip_fail((hipError_t)rc, "gradient norm launch");
     t->norm_last = result;
+    if (also) also->norm_last = result;
     return 0;
 }
 
-int eri_adam8_grad_norm(EriAdam8Table *t, float max_norm, float denom_eps, void *stream) {
+static int grad_norm(EriAdam8Table *t, EriAdam8Table *also, float max_norm, float denom_eps, void *stream) {
     if (!t) return fail(ERI_ERR_NULL, "table is NULL");
+    if (also && also->device != t->device) return fail(ERI_ERR_ARG, "the two tables belong to different devices");
     DeviceCtx *ctx = nullptr;
     int rc = get_ctx_on(t->device, &ctx);
     if (rc) return rc;
-    // one group per layout at most, and per wave a sum of squares and a count
-    const uint32_t pairs = eri::kLayouts * ctx->cus * eri::kNormWavesPerCu;
+    // per table one group per layout at most, and per wave a sum of squares and a count; room for two tables
+    const uint32_t pairs = 2 * eri::kLayouts * ctx->cus * eri::kNormWavesPerCu;
     if (!t->partial) ERI_HIP(hipMalloc((void **)&t->partial, sizeof(double) * 2 * pairs));
     if (!t->norm_out) ERI_HIP(hipMalloc((void **)&t->norm_out, sizeof(float) * 4)); // norm, scale, 64-bit count
-    return grad_norm_launch(t, ctx, max_norm, denom_eps, t->partial, pairs, t->norm_out, stream);
+    return grad_norm_launch(t, also, ctx, max_norm, denom_eps, t->partial, pairs, t->norm_out, stream);
+}
+
+int eri_adam8_grad_norm(EriAdam8Table *t, float max_norm, float denom_eps, void *stream) {
+    return grad_norm(t, nullptr, max_norm, denom_eps, stream);
+}
+
+int eri_adam8_grad_norm_joint(EriAdam8Table *t, EriAdam8Table *also, float max_norm, float denom_eps, void *stream) {
+    if (!also) return fail(ERI_ERR_NULL, "the second table is NULL");
+    if (also == t) return fail(ERI_ERR_ARG, "the two tables are the same");
+    return grad_norm(t, also, max_norm, denom_eps, stream);
+}
+
+int eri_adam8_grad_norm_scale_ptr(const EriAdam8Table *t, const float **dev_scale) {
+    if (!t || !dev_scale) return fail(ERI_ERR_NULL, "table or dev_scale is NULL");
+    if (!t->norm_last) return fail(ERI_ERR_ARG, "no gradient norm has been computed for this table");
+    *dev_scale = t->norm_last + 1;
+    return 0;
 }
 
 int eri_adam8_grad_norm_static(EriAdam8Table *t, float max_norm, float denom_eps, void *result, void *stream) {
@@ -932,9 +1060,14 @@ int eri_adam8_grad_norm_static(EriAdam8Table *t, float max_norm, float denom_eps
     int dev = -1;
     ERI_HIP(hipGetDevice(&dev));
     if (dev != t->device) return fail(ERI_ERR_ARG, "the table belongs to another device than the current one");
-    DeviceCtx *ctx = &g_ctx[dev]; // made ready, scratch address included, when the table was created
-    if (!ctx->ready || !ctx->scratch_ptr) return fail(ERI_ERR_INTERNAL, "the library was not initialised on this device");
-    return grad_norm_launch(t, ctx, max_norm, denom_eps, ctx->scratch_ptr, kNormScratchPairs, static_cast<float *>(result), stream);
+    // the device's context was made ready, scratch address included, when the table was created; it is read under
+    // the lock that guards its creation, and nothing is created here
+    DeviceCtx *ctx = &g_ctx[dev];
+    {
+        std::lock_guard<std::mutex> lk(g_ctx_mu);
+        if (!ctx->ready || !ctx->scratch_ptr) return fail(ERI_ERR_INTERNAL, "the library was not initialised on this device");
+    }
+    return grad_norm_launch(t, nullptr, ctx, max_norm, denom_eps, ctx->scratch_ptr, kNormScratchPairs, static_cast<float *>(result), stream);
 }
 
 int eri_adam8_grad_norm_read(EriAdam8Table *t, float *norm, float *scale, void *stream) {
@@ -960,6 +1093,7 @@ int eri_adam8_grad_nonfinite_read(EriAdam8Table *t, uint64_t *count, void *strea
 
 int eri_adam8_quant_error(EriAdam8Table *t, const EriAdam8Hyper *h, void *stream) {
     if (!t || !h) return fail(ERI_ERR_NULL, "table or hyper is NULL");
+    if (t->grads_only) return fail(ERI_ERR_ARG, "a gradient-only table serves eri_adam8_grad_norm only");
     if (h->mode != ERI_ADAM8_MODE_ERI && h->mode != ERI_ADAM8_MODE_L2)
         return fail(ERI_ERR_ARG, "the quantisation error pass knows the modes ERI and L2");
     DeviceCtx *ctx = nullptr;
@@ -1071,53 +1205,95 @@ int eri_adam8_quantize(const float *x, int signed_map, uint64_t numel, uint8_t *
 
 namespace {
 
-/* Device copy of a row table that changes rarely: re-uploaded only when the rows differ from the
- * last call, through a pinned mirror whose previous copy is waited for before it is overwritten. */
+/* Device copies of the row tables of the plain sweeps, kept per calling thread.  An optimizer step can sweep
+ * several row sets in turn (the shadows of the groups that do not carry the EMA inside the step kernel, then the
+ * parameters outside the 8-bit table), the same sets step after step, so the last four distinct sets are kept:
+ * rows found in one of them are not uploaded again.  A set is uploaded through its own pinned mirror, whose
+ * previous copy is waited for before it is overwritten; a set that is used on another stream than the one it
+ * was uploaded on is ordered after the upload by an event wait on that stream. */
 struct ElemCache {
     struct Group {
-        std::vector<eri::ElemRow> rows;
         eri::ElemRow *dev = nullptr, *pinned = nullptr;
-        uint32_t cap = 0, total_blocks = 0;
+        uint32_t cap = 0, n = 0;
     };
-    Group groups[2]; // F32, BF16
-    hipEvent_t ev = nullptr;
-    bool pending = false;
+    struct Slot {
+        Group groups[2]; // F32, BF16
+        hipEvent_t ev = nullptr;
+        bool pending = false;
+        void *stream = nullptr; // of the last upload
+        uint64_t used = 0;
+        void drop() {
+            if (pending && ev) (void)hipEventSynchronize(ev);
+            pending = false;
+            for (auto &g : groups) {
+                if (g.dev) (void)hipFree(g.dev);
+                if (g.pinned) (void)hipHostFree(g.pinned);
+                g.dev = g.pinned = nullptr;
+                g.cap = g.n = 0;
+            }
+            if (ev) (void)hipEventDestroy(ev);
+            ev = nullptr;
+            used = 0;
+        }
+    };
+    static constexpr int kSlots = 4;
+    Slot slots[kSlots];
+    std::vector<eri::ElemRow> rows[2]; // the rows of the call at hand: F32, BF16
+    uint64_t tick = 0;
     int device = -1;
     ~ElemCache() {
-        for (auto &g : groups) {
-            if (g.dev) (void)hipFree(g.dev);
-            if (g.pinned) (void)hipHostFree(g.pinned);
+        for (auto &sl : slots) sl.drop();
+    }
+    bool holds(const Slot &sl) const {
+        for (int gi = 0; gi < 2; ++gi) {
+            const uint32_t n = (uint32_t)rows[gi].size();
+            if (sl.groups[gi].n != n) return false;
+            if (n && std::memcmp(sl.groups[gi].pinned, rows[gi].data(), n * sizeof(eri::ElemRow)) != 0) return false;
         }
-        if (ev) (void)hipEventDestroy(ev);
+        return sl.used != 0;
     }
     int sync(void *stream, uint32_t cus, int (*launch)(const eri::ElemRow *, uint32_t, uint32_t, int, uint32_t, void *, const void *),
              const void *extra) {
         int dev = 0;
         ERI_HIP(hipGetDevice(&dev));
         if (dev != device) { // the thread moved to another device: nothing cached is an address there
-            if (pending) (void)hipEventSynchronize(ev);
-            pending = false;
-            for (auto &g : groups) {
-                if (g.dev) (void)hipFree(g.dev);
-                if (g.pinned) (void)hipHostFree(g.pinned);
-                g.dev = g.pinned = nullptr;
-                g.cap = 0;
-            }
-            if (ev) (void)hipEventDestroy(ev);
-            ev = nullptr;
+            for (auto &sl : slots) sl.drop();
             device = dev;
         }
-        if (!ev) ERI_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
-        for (int gi = 0; gi < 2; ++gi) {
-            Group &g = groups[gi];
-            const uint32_t n = (uint32_t)g.rows.size();
-            if (n == 0) continue;
-            bool same = g.cap >= n && std::memcmp(g.pinned, g.rows.data(), n * sizeof(eri::ElemRow)) == 0;
-            if (!same) {
-                if (pending) {
-                    ERI_HIP(hipEventSynchronize(ev));
-                    pending = false;
+        Slot *sl = nullptr;
+        for (auto &c : slots)
+            if (holds(c)) sl = &c;
+        if (sl) {
+            if (sl->pending && hipEventQuery(sl->ev) == hipSuccess) sl->pending = false;
+            (void)hipGetLastError(); // hipErrorNotReady of the query is not an error
+            if (sl->pending && stream != sl->stream) { // uploaded on another stream and perhaps still on its way
+                hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+                if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &cs) != hipSuccess) {
+                    (void)hipGetLastError();
+                    cs = hipStreamCaptureStatusNone;
                 }
+                if (cs == hipStreamCaptureStatusActive) { // a capture cannot wait for an event from outside it
+                    ERI_HIP(hipEventSynchronize(sl->ev));
+                    sl->pending = false;
+                } else {
+                    ERI_HIP(hipStreamWaitEvent(static_cast<hipStream_t>(stream), sl->ev, 0));
+                }
+            }
+        } else {
+            sl = &slots[0];
+            for (auto &c : slots)
+                if (c.used < sl->used) sl = &c;
+            if (!sl->ev) ERI_HIP(hipEventCreateWithFlags(&sl->ev, hipEventDisableTiming));
+            if (sl->pending) { // the mirror may still be the source of the slot's last copy
+                ERI_HIP(hipEventSynchronize(sl->ev));
+                sl->pending = false;
+            }
+            sl->used = 0; // not a set to come back to until the upload below is complete
+            for (int gi = 0; gi < 2; ++gi) {
+                Group &g = sl->groups[gi];
+                const uint32_t n = (uint32_t)rows[gi].size();
+                g.n = 0;
+                if (n == 0) continue;
                 if (g.cap < n) {
                     if (g.dev) (void)hipFree(g.dev);
                     if (g.pinned) (void)hipHostFree(g.pinned);
@@ -1128,13 +1304,21 @@ struct ElemCache {
                     ERI_HIP(hipHostMalloc((void **)&g.pinned, sizeof(eri::ElemRow) * cap, hipHostMallocDefault));
                     g.cap = cap;
                 }
-                std::memcpy(g.pinned, g.rows.data(), n * sizeof(eri::ElemRow));
+                std::memcpy(g.pinned, rows[gi].data(), n * sizeof(eri::ElemRow));
                 ERI_HIP(hipMemcpyAsync(g.dev, g.pinned, n * sizeof(eri::ElemRow), hipMemcpyHostToDevice,
                                        static_cast<hipStream_t>(stream)));
-                ERI_HIP(hipEventRecord(ev, static_cast<hipStream_t>(stream)));
-                pending = true;
+                g.n = n;
             }
-            const eri::ElemRow &last = g.rows.back();
+            ERI_HIP(hipEventRecord(sl->ev, static_cast<hipStream_t>(stream)));
+            sl->pending = true;
+            sl->stream = stream;
+        }
+        sl->used = ++tick;
+        for (int gi = 0; gi < 2; ++gi) {
+            const Group &g = sl->groups[gi];
+            const uint32_t n = g.n;
+            if (n == 0) continue;
+            const eri::ElemRow &last = rows[gi].back();
             const uint32_t total = last.full_start + (uint32_t)(last.numel / eri::kBlock);
             const uint32_t work = total > n ? total : n;
             uint32_t grid = (work + 3) / 4;
@@ -1157,8 +1341,15 @@ int check_elem(const void *a, const void *b, uint64_t numel, int dtype, uint32_t
     return 0;
 }
 
+struct AdamW32Extra {
+    EriAdamW32Hyper h;
+    bool scaled;            // gradients are multiplied by (grad_scale * row scale) * (*dev_scale)
+    float grad_scale;
+    const float *dev_scale; // device, or null for 1
+};
 int adamw32_launch(const eri::ElemRow *rows, uint32_t n, uint32_t total, int dtype, uint32_t grid, void *stream, const void *extra) {
-    return eri::launch_adamw32(rows, n, total, dtype, *static_cast<const EriAdamW32Hyper *>(extra), grid, stream);
+    const AdamW32Extra &x = *static_cast<const AdamW32Extra *>(extra);
+    return eri::launch_adamw32(rows, n, total, dtype, x.h, x.scaled, x.grad_scale, x.dev_scale, grid, stream);
 }
 int ema_launch(const eri::ElemRow *rows, uint32_t n, uint32_t total, int dtype, uint32_t grid, void *stream, const void *extra) {
     return eri::launch_ema(rows, n, total, dtype, *static_cast<const float *>(extra), grid, stream);
@@ -1168,13 +1359,14 @@ int ema_launch(const eri::ElemRow *rows, uint32_t n, uint32_t total, int dtype, 
 
 extern "C" {
 
-int eri_adamw32_step_multi(const EriAdamW32Tensor *rows, uint32_t n, const EriAdamW32Hyper *hyper, void *stream) {
+static int adamw32_step(const EriAdamW32Tensor *rows, uint32_t n, const EriAdamW32Hyper *hyper, bool scaled, float grad_scale,
+                        const float *dev_scale, void *stream) {
     if (!rows || !hyper) return fail(ERI_ERR_NULL, "rows or hyper is NULL");
     if (n == 0) return fail(ERI_ERR_ARG, "no rows");
     thread_local ElemCache cache;
     DeviceCtx *ctx = nullptr;
     int rc = get_ctx(&ctx);
-    for (auto &g : cache.groups) g.rows.clear();
+    for (auto &g : cache.rows) g.clear();
     uint64_t blocks = 0;
     uint32_t starts[2] = {0, 0};
     for (uint32_t i = 0; i < n; ++i) {
@@ -1186,12 +1378,27 @@ int eri_adamw32_step_multi(const EriAdamW32Tensor *rows, uint32_t n, const EriAd
         const int gi = r.dtype_tag == ERI_DTYPE_F32 ? 0 : 1;
         eri::ElemRow d;
         if ((uintptr_t)r.master & 15u) return fail(ERI_ERR_ALIGN, "master pointer must be 16-byte aligned");
-        d.a = r.p; d.b = r.g; d.c = r.m; d.d = r.v; d.e = r.master; d.numel = r.numel; d.full_start = starts[gi]; d.pad = 0;
+        d.a = r.p; d.b = r.g; d.c = r.m; d.d = r.v; d.e = r.master; d.numel = r.numel; d.full_start = starts[gi];
+        d.scale = r.grad_scale == 0.0f ? 1.0f : r.grad_scale; // a zeroed row: no multiplier
         starts[gi] += (uint32_t)(r.numel / eri::kBlock);
-        cache.groups[gi].rows.push_back(d);
+        cache.rows[gi].push_back(d);
     }
     if (rc) return rc;
-    return cache.sync(stream, ctx->cus, adamw32_launch, hyper);
+    AdamW32Extra x;
+    x.h = *hyper;
+    x.scaled = scaled;
+    x.grad_scale = grad_scale;
+    x.dev_scale = dev_scale;
+    return cache.sync(stream, ctx->cus, adamw32_launch, &x);
+}
+
+int eri_adamw32_step_multi(const EriAdamW32Tensor *rows, uint32_t n, const EriAdamW32Hyper *hyper, void *stream) {
+    return adamw32_step(rows, n, hyper, false, 1.0f, nullptr, stream);
+}
+
+int eri_adamw32_step_multi_scaled(const EriAdamW32Tensor *rows, uint32_t n, const EriAdamW32Hyper *hyper, float grad_scale,
+                                  const float *dev_scale, void *stream) {
+    return adamw32_step(rows, n, hyper, true, grad_scale, dev_scale, stream);
 }
 
 int eri_ema_update_multi(const EriEmaTensor *rows, uint32_t n, float decay, void *stream) {
@@ -1200,7 +1407,7 @@ int eri_ema_update_multi(const EriEmaTensor *rows, uint32_t n, float decay, void
     thread_local ElemCache cache;
     DeviceCtx *ctx = nullptr;
     int rc = get_ctx(&ctx);
-    for (auto &g : cache.groups) g.rows.clear();
+    for (auto &g : cache.rows) g.clear();
     uint64_t blocks = 0;
     uint32_t starts[2] = {0, 0};
     for (uint32_t i = 0; i < n; ++i) {
@@ -1209,9 +1416,9 @@ int eri_ema_update_multi(const EriEmaTensor *rows, uint32_t n, float decay, void
         if (e) return e;
         const int gi = r.dtype_tag == ERI_DTYPE_F32 ? 0 : 1;
         eri::ElemRow d;
-        d.a = r.shadow; d.b = r.p; d.c = nullptr; d.d = nullptr; d.e = nullptr; d.numel = r.numel; d.full_start = starts[gi]; d.pad = 0;
+        d.a = r.shadow; d.b = r.p; d.c = nullptr; d.d = nullptr; d.e = nullptr; d.numel = r.numel; d.full_start = starts[gi]; d.scale = 0.0f;
         starts[gi] += (uint32_t)(r.numel / eri::kBlock);
-        cache.groups[gi].rows.push_back(d);
+        cache.rows[gi].push_back(d);
     }
     if (rc) return rc;
     return cache.sync(stream, ctx->cus, ema_launch, &decay);

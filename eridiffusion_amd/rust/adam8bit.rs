@@ -54,6 +54,16 @@ impl DevicePool {
         check(unsafe { sys::eri_hip_pool_alloc_zeroed(self.pool, lane, bytes, &mut p) }, "eri_hip_pool_alloc_zeroed")?;
         Ok(p as *mut u8)
     }
+    /// The same, cleared by a kernel on `stream` (no host wait; usable under stream capture).
+    pub fn alloc_zeroed_on(&self, lane: u32, bytes: usize, stream: *mut c_void) -> Result<*mut u8> {
+        let mut p: *mut c_void = std::ptr::null_mut();
+        check(unsafe { sys::eri_hip_pool_alloc_zeroed_async(self.pool, lane, bytes, stream, &mut p) }, "eri_hip_pool_alloc_zeroed_async")?;
+        Ok(p as *mut u8)
+    }
+    /// Gives one piece back (`bytes` as requested); the next request of that size in its lane takes it.
+    pub fn release(&self, ptr: *mut u8, bytes: usize) -> Result<()> {
+        check(unsafe { sys::eri_hip_pool_release(self.pool, ptr as *mut c_void, bytes) }, "eri_hip_pool_release")
+    }
     pub fn reset(&self) -> Result<()> {
         check(unsafe { sys::eri_hip_pool_reset(self.pool) }, "eri_hip_pool_reset")
     }

@@ -46,7 +46,7 @@ pub struct EriAdam8bitConfig {
 
 #[repr(C)]
 #[derive(Clone, Copy)]
-pub struct EriAdamW32Tensor { pub p: *mut c_void, pub g: *const c_void, pub m: *mut f32, pub v: *mut f32, pub master: *mut f32, pub numel: u64, pub dtype_tag: i32, pub reserved: i32 }
+pub struct EriAdamW32Tensor { pub p: *mut c_void, pub g: *const c_void, pub m: *mut f32, pub v: *mut f32, pub master: *mut f32, pub numel: u64, pub dtype_tag: i32, pub grad_scale: f32 }
 #[repr(C)]
 #[derive(Clone, Copy)]
 pub struct EriAdamW32Hyper { pub lr: f32, pub beta1: f32, pub beta2: f32, pub eps: f32, pub weight_decay: f32 }
@@ -85,6 +85,8 @@ extern "C" {
     pub fn eri_hip_mem_info(free_bytes: *mut usize, total_bytes: *mut usize) -> c_int;
     pub fn eri_hip_pool_create(device: c_int, bytes: usize, lanes: u32, out: *mut *mut EriHipPool) -> c_int;
     pub fn eri_hip_pool_alloc_zeroed(pool: *mut EriHipPool, lane: u32, bytes: usize, out: *mut *mut c_void) -> c_int;
+    pub fn eri_hip_pool_alloc_zeroed_async(pool: *mut EriHipPool, lane: u32, bytes: usize, stream: *mut c_void, out: *mut *mut c_void) -> c_int;
+    pub fn eri_hip_pool_release(pool: *mut EriHipPool, ptr: *mut c_void, bytes: usize) -> c_int;
     pub fn eri_hip_pool_info(pool: *const EriHipPool, lanes: *mut u32, lane_bytes: *mut usize) -> c_int;
     pub fn eri_hip_pool_lane_used(pool: *const EriHipPool, lane: u32, used_bytes: *mut usize) -> c_int;
     pub fn eri_hip_pool_reset(pool: *mut EriHipPool) -> c_int;
@@ -101,6 +103,9 @@ extern "C" {
     pub fn eri_adam8_table_info(table: *const EriAdam8Table, total_numel: *mut u64, total_blocks: *mut u64) -> c_int;
     pub fn eri_adam8_step_table(table: *mut EriAdam8Table, hyper: *const EriAdam8Hyper, stream: *mut c_void) -> c_int;
     pub fn eri_adam8_grad_norm(table: *mut EriAdam8Table, max_norm: f32, denom_eps: f32, stream: *mut c_void) -> c_int;
+    pub fn eri_adam8_grad_table_create(rows: *const EriAdam8Tensor, n: u32, stream: *mut c_void, out: *mut *mut EriAdam8Table) -> c_int;
+    pub fn eri_adam8_grad_norm_joint(table: *mut EriAdam8Table, also: *mut EriAdam8Table, max_norm: f32, denom_eps: f32, stream: *mut c_void) -> c_int;
+    pub fn eri_adam8_grad_norm_scale_ptr(table: *const EriAdam8Table, dev_scale: *mut *const f32) -> c_int;
     pub fn eri_adam8_grad_norm_static(table: *mut EriAdam8Table, max_norm: f32, denom_eps: f32, result: *mut c_void, stream: *mut c_void) -> c_int;
     pub fn eri_adam8_grad_norm_read(table: *mut EriAdam8Table, norm: *mut f32, scale: *mut f32, stream: *mut c_void) -> c_int;
     pub fn eri_adam8_grad_nonfinite_read(table: *mut EriAdam8Table, count: *mut u64, stream: *mut c_void) -> c_int;
@@ -111,6 +116,7 @@ extern "C" {
     pub fn eri_adam8_quantize(x: *const f32, signed_map: c_int, numel: u64, codes: *mut u8, absmax: *mut f32, stream: *mut c_void) -> c_int;
     // 32-bit sibling and EMA sweep
     pub fn eri_adamw32_step_multi(rows: *const EriAdamW32Tensor, n: u32, hyper: *const EriAdamW32Hyper, stream: *mut c_void) -> c_int;
+    pub fn eri_adamw32_step_multi_scaled(rows: *const EriAdamW32Tensor, n: u32, hyper: *const EriAdamW32Hyper, grad_scale: f32, dev_scale: *const f32, stream: *mut c_void) -> c_int;
     pub fn eri_ema_update_multi(rows: *const EriEmaTensor, n: u32, decay: f32, stream: *mut c_void) -> c_int;
     // optimizer objects
     pub fn eri_param_create(data: *mut c_void, numel: u64, dtype_tag: c_int, out: *mut *mut EriParameter) -> c_int;
@@ -169,6 +175,7 @@ extern "C" {
     pub fn eri_adam8bit_fn_step(opt: *mut EriAdam8bitFn) -> c_int;
     pub fn eri_adam8bit_fn_set_lr(opt: *mut EriAdam8bitFn, lr: f32) -> c_int;
     pub fn eri_adam8bit_fn_get_step(opt: *const EriAdam8bitFn) -> u64;
+    pub fn eri_adam8bit_fn_table_stats(opt: *const EriAdam8bitFn, flushes: *mut u64, uploads: *mut u64) -> c_int;
     pub fn eri_adam8bit_fn_memory_stats(opt: *const EriAdam8bitFn, num_params: *mut u64, bytes: *mut u64) -> c_int;
     pub fn eri_adam8bit_fn_state_numel(opt: *const EriAdam8bitFn, name: *const c_char, numel: *mut u64) -> c_int;
     pub fn eri_adam8bit_fn_get_state_fp32(opt: *mut EriAdam8bitFn, name: *const c_char, m_out: *mut f32, v_out: *mut f32) -> c_int;

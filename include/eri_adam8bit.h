@@ -84,17 +84,21 @@ int eri_adam8bit_attach_ema(EriAdam8bit *opt, EriEmaModel *ema, const char *cons
 /* States that do not exist yet (they are created at the first step that meets their parameter) come out of
  * `lane` of a memory pool (eri_hip_pool_create, include/eri_optim8.h) instead of allocations of their own:
  * a lane 32 GiB or more away from the parameters' makes every later step 10-17 % faster on tables that do not
- * span that much by themselves.  The pool is not owned and must outlive the optimizer; NULL goes back to
- * separate allocations.  No counterpart in the reference, whose states are host vectors. */
+ * span that much by themselves.  The pool is not owned and must outlive the optimizer (a state that is replaced
+ * or destroyed gives its piece back with eri_hip_pool_release, so loading a checkpoint into an optimizer that
+ * has stepped does not grow the lane beyond two sets of states); NULL goes back to separate allocations.  No
+ * counterpart in the reference, whose states are host vectors. */
 int eri_adam8bit_set_state_pool(EriAdam8bit *opt, EriHipPool *pool, uint32_t lane);
 /* min_8bit_size (pipeline_flux_lora_1024.rs:451, the policy of the library the state format comes from):
  * from the next step on, a parameter with fewer than `numel` elements that has no 8-bit state yet keeps
  * fp32 moments instead and takes the same update, adam8bit_enhanced.rs:252-275, without the quantiser --
  * one extra launch of the 32-bit step (eri_adamw32_step_multi) over all such parameters, with the
  * bias-corrected step size as its learning rate.  0 (the default) keeps every parameter in the 8-bit
- * format.  Such parameters need gradients of their own dtype, mode ERI, and no gradient scaling or clipping
- * inside the step (a step that would combine them is refused before anything runs).  save_state / load_state
- * carry the fp32 moments as `optimizer.param_N.m32` / `.v32`. */
+ * format.  Such parameters need gradients of their own dtype and mode ERI (a step in another mode is refused
+ * before anything runs).  The loss scale, the per-parameter multipliers and the clip factor reach them as they
+ * reach the 8-bit parameters, and the global norm behind the clip factor covers the gradients of both kinds
+ * (the trainer that sets min_8bit_size clips every trainable gradient, pipeline_flux_lora_1024.rs:691-697).
+ * save_state / load_state carry the fp32 moments as `optimizer.param_N.m32` / `.v32`. */
 int eri_adam8bit_set_min_8bit_size(EriAdam8bit *opt, uint64_t numel);
 /* Device pointers of one parameter's fp32 moments (NULL if it has none). */
 int eri_adam8bit_state32_ptrs(const EriAdam8bit *opt, uint32_t index, float **m, float **v);
@@ -151,14 +155,22 @@ int eri_adam8bit_fn_set_state_pool(EriAdam8bitFn *opt, EriHipPool *pool, uint32_
  * pipeline_flux_lora_sequential.rs:749-794), eri_adam8bit_fn_flush, set_lr, state read or destroy.  Until
  * then `out` is not written and `param` / `grad` must stay alive and unchanged -- a caller that reads the
  * returned tensor, or frees the gradient, before step() must not enable it.  A second update of the same
- * name flushes the first.  The launch table is kept between flushes: the same tensors at new addresses
- * cost one small upload, at the same addresses nothing.  The hundreds of launches of a LoRA step become one. */
+ * name flushes the first.  The launch tables of the last two distinct sets of rows are kept between flushes:
+ * update() returns a new tensor per call (adam8bit.rs:205-207), so a trainer's rows alternate between two
+ * sets of addresses, and from the third flush on nothing is uploaded; the same tensors at addresses not seen
+ * in the last two flushes cost one small upload.  The hundreds of launches of a LoRA step become one. */
 int eri_adam8bit_fn_set_batching(EriAdam8bitFn *opt, int enabled);
 int eri_adam8bit_fn_flush(EriAdam8bitFn *opt);
+/* How many launches over queued rows have run, and how many of them had to build or re-upload a launch table
+ * first (the others found their rows in one of the two tables kept).  Either pointer may be NULL. */
+int eri_adam8bit_fn_table_stats(const EriAdam8bitFn *opt, uint64_t *flushes, uint64_t *uploads);
 /* n updates in one call and one launch, whatever the batching setting: update(names[i], params[i], grads[i])
  * -> outs[i] for every i (update_params_8bit, adam8bit.rs:333-345, without its loop of launches).
  * grad_dtype_tags may be NULL (every gradient has the dtype of its parameter).  Rows queued earlier run
- * first.  If any row is refused nothing of the call runs. */
+ * first.  Every row is validated, and the states of names not seen before are created, before anything of
+ * the call is launched: if a row is refused or a state cannot be allocated, nothing of the call runs and no
+ * state of the call stays behind.  A name that repeats within the call splits it there: the rows up to the
+ * repetition are one launch, the rest the next (two updates of one tensor are two steps of its state). */
 int eri_adam8bit_fn_update_many(EriAdam8bitFn *opt, const char *const *names, const void *const *params,
                                 const void *const *grads, const uint64_t *numels, const int32_t *dtype_tags,
                                 const int32_t *grad_dtype_tags, void *const *outs, uint32_t n);

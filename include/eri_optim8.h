@@ -89,11 +89,22 @@ int eri_hip_mem_info(size_t *free_bytes, size_t *total_bytes);
  * fall into different lanes by themselves.
  * bytes = 0 takes nine tenths of the free device memory; lanes = 0 makes as many lanes of exactly 48 GiB as fit
  * into `bytes` (a smaller pool is a single lane).
- * Pieces are not returned one by one: eri_hip_pool_reset empties every lane, eri_hip_pool_destroy frees the
- * allocation.  Calls on one pool may come from several threads. */
+ * eri_hip_pool_release gives one piece back: the top piece of a lane lowers the lane's fill level, any other is
+ * kept and handed out again to the next request of exactly its size in that lane (optimizer states that are
+ * replaced, e.g. by loading a checkpoint, have the size of the ones they replace).  eri_hip_pool_reset empties
+ * every lane, eri_hip_pool_destroy frees the allocation.  Calls on one pool may come from several threads. */
 typedef struct EriHipPool EriHipPool;
 int eri_hip_pool_create(int device, size_t bytes, uint32_t lanes, EriHipPool **out);
-int eri_hip_pool_alloc_zeroed(EriHipPool *pool, uint32_t lane, size_t bytes, void **out); /* lane counts modulo the pool's lanes */
+/* lane counts modulo the pool's lanes.  The piece is cleared by the runtime's synchronous memset: it is zero,
+ * for work on any stream, when the call returns. */
+int eri_hip_pool_alloc_zeroed(EriHipPool *pool, uint32_t lane, size_t bytes, void **out);
+/* The same, cleared by a small kernel on `stream` instead: the host does not wait, the call may sit inside a
+ * stream capture, and the piece is zero for whatever follows it on that stream (work on another stream has to be
+ * ordered after it by the caller). */
+int eri_hip_pool_alloc_zeroed_async(EriHipPool *pool, uint32_t lane, size_t bytes, void *stream, void **out);
+/* Gives back a piece with the byte count it was requested with.  The caller orders the release after the last
+ * use of the piece (the next owner clears it on its own stream or through the synchronous memset). */
+int eri_hip_pool_release(EriHipPool *pool, void *ptr, size_t bytes);
 int eri_hip_pool_info(const EriHipPool *pool, uint32_t *lanes, size_t *lane_bytes);
 int eri_hip_pool_lane_used(const EriHipPool *pool, uint32_t lane, size_t *used_bytes);
 int eri_hip_pool_reset(EriHipPool *pool);
@@ -189,8 +200,9 @@ typedef struct EriAdam8Tensor {
                              Adam8bit::update(name, param, grad) -> new tensor (adam8bit.rs:101-208) without a copy */
     int32_t grad_f32;     /* non-zero with BF16 parameters: g holds F32 elements, which enter the arithmetic
                              unrounded -- the reference casts every gradient to F32 and never rounds it
-                             (adam8bit_enhanced.rs:231-235, adam8bit.rs:110).  Such rows run on the
-                             four-waves-per-block kernel whatever the flags say.  Must be 0 for F32 parameters */
+                             (adam8bit_enhanced.rs:231-235, adam8bit.rs:110).  Such rows form a group of their
+                             own with its own launch; the same three kernels serve it (by table size).
+                             Must be 0 for F32 parameters */
     int32_t reserved;     /* 0 */
     void *ema_shadow;     /* NULL, or the EMA shadow of this parameter (dtype of p, numel elements, 16-byte aligned):
                              updated by steps that carry ERI_ADAM8_FLAG_EMA */
@@ -232,6 +244,19 @@ int eri_adam8_step_table(EriAdam8Table *table, const EriAdam8Hyper *hyper, void 
  * clip_grads_global_norm_fp32_tensors (crates/training/src/optimizer.rs:58-85).  A following step with
  * ERI_ADAM8_FLAG_CLIP_FROM_TABLE applies the factor inside the kernel instead of rewriting gradients. */
 int eri_adam8_grad_norm(EriAdam8Table *table, float max_norm, float denom_eps, void *stream);
+/* A table of gradients only, for tensors that take part in the global norm but not in the 8-bit step (the short
+ * tensors a trainer keeps in 32-bit moments, pipeline_flux_lora_1024.rs:451, are clipped by the same global
+ * norm, :691-697).  Of each row only g, numel, block_start, dtype_tag and grad_f32 are read.  Such a table can
+ * be updated, normed and destroyed like any other; the step and the statistics pass refuse it. */
+int eri_adam8_grad_table_create(const EriAdam8Tensor *rows, uint32_t n, void *stream, EriAdam8Table **out);
+/* The norm pass over the gradients of two tables as if they were one: one norm, one clip factor, left in
+ * memory owned by `table` and used by both tables from then on (the reads below and
+ * ERI_ADAM8_FLAG_CLIP_FROM_TABLE work on either) until one of them is normed again; `table` must outlive that
+ * use.  The per-block sums are added in the order: groups of `table`, groups of `also`. */
+int eri_adam8_grad_norm_joint(EriAdam8Table *table, EriAdam8Table *also, float max_norm, float denom_eps, void *stream);
+/* Device address of the clip factor the table's last norm pass left (one float), for a kernel outside the
+ * table that has to apply the same factor: eri_adamw32_step_multi_scaled.  Valid until the next norm pass. */
+int eri_adam8_grad_norm_scale_ptr(const EriAdam8Table *table, const float **dev_scale);
 /* The same pass for callers that cannot allocate (code under HIP graph capture, serving loops, harnesses
  * that forbid hipMalloc).  It has no counterpart in the reference.  eri_adam8_grad_norm allocates the
  * per-wave partial sums and the result words on a table's first call; this variant allocates nothing:
@@ -239,8 +264,9 @@ int eri_adam8_grad_norm(EriAdam8Table *table, float max_norm, float denom_eps, v
  * pairs; a table whose pass needs more is refused with ERI_ERR_TOO_LARGE -- none does on a 256-CU
  * MI355X) and the result to `result`, 16 bytes of device memory the caller owns, 8-byte aligned:
  * {float norm, float scale, uint64 count of non-finite elements}.  A following step with
- * ERI_ADAM8_FLAG_CLIP_FROM_TABLE, and the two read calls below, use `result` until the next norm pass
- * of the table, so it must stay valid that long.  All calls on one device share the array: two such
+ * ERI_ADAM8_FLAG_CLIP_FROM_TABLE, and the two read calls below, read `result` until the next norm pass
+ * of the table: the caller keeps it allocated that long (the library holds the bare address and cannot
+ * tell whether it still is).  All calls on one device share the array: two such
  * calls that overlap in time on one device (different streams, different tables) race.  Nothing in
  * the array has to start at zero (every wave of a pass writes its pair before the pair is read). */
 int eri_adam8_grad_norm_static(EriAdam8Table *table, float max_norm, float denom_eps, void *result, void *stream);
@@ -298,7 +324,8 @@ typedef struct EriAdamW32Tensor {
                          src/kernels/fused_adam.cu:151-193, with the arithmetic above */
     uint64_t numel;
     int32_t dtype_tag;
-    int32_t reserved;
+    float grad_scale; /* per-layer multiplier of the gradients, read by eri_adamw32_step_multi_scaled only;
+                         0 (a zeroed row) reads as 1 */
 } EriAdamW32Tensor;
 
 typedef struct EriAdamW32Hyper {
@@ -307,6 +334,13 @@ typedef struct EriAdamW32Hyper {
 
 /* One launch per dtype over all rows; keeps a cached device copy of the rows per calling thread. */
 int eri_adamw32_step_multi(const EriAdamW32Tensor *rows, uint32_t n, const EriAdamW32Hyper *hyper, void *stream);
+/* The same step with every gradient first multiplied by (grad_scale * row.grad_scale) * (*dev_scale), one rounded
+ * fp32 product of the gradient with that factor, the factor formed in this order -- what the 8-bit step does with
+ * ERI_ADAM8_FLAG_GRAD_SCALE and ERI_ADAM8_FLAG_CLIP_FROM_TABLE, so that tensors kept in 32-bit moments are unscaled
+ * and clipped like the rest (clip_gradients then the optimizer, pipeline_flux_lora_1024.rs:691-697).  dev_scale is
+ * device memory (eri_adam8_grad_norm_scale_ptr) or NULL for 1. */
+int eri_adamw32_step_multi_scaled(const EriAdamW32Tensor *rows, uint32_t n, const EriAdamW32Hyper *hyper, float grad_scale,
+                                  const float *dev_scale, void *stream);
 
 /* Exponential moving average of parameters, shadow = decay*shadow + (1-decay)*p in fp32
  * (EMA update, src/trainers/ema_enhanced.rs:79-108), one launch over all rows.

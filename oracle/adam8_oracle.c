@@ -35,10 +35,19 @@
  *                              quantisation search)                                  parity unpinned
  *   eri_oracle_adamw32_step    closed form at step 1, float64 recurrence, the reference's
  *                              own 2x2 test case                                     pinned
+ *   eri_oracle_adamw32_step_scaled   equals the unscaled step on pre-multiplied fp32
+ *                              gradients                                             pinned
  *   eri_oracle_ema_update      float64 closed form; bf16 intermediate rounding of flame-core
  *                              unknown                                               parity unpinned (bf16)
  *   bit-level equality with the reference's own legacy per-tensor linear format
  *   (adam8bit.rs:211-241, flame-core's to_dtype(U8)/round semantics are absent)     parity unpinned
+ *
+ * The bias corrections of mode L2 are 1 - beta^s with an integer s; the reference forms the power with Rust's
+ * f64::powi (adam8bit.rs:164-175), this file with C's pow(beta, (double)s).  Both are f64 results that are
+ * then rounded to f32, but powi multiplies repeatedly while pow is correctly rounded, so the two can differ in
+ * the last f64 bit before that cast, and in rare cases in the last f32 bit after it.  A wrong exponent or base
+ * would show at once (closed forms at steps 2, 7 and 40); that last bit cannot be pinned without a Rust
+ * toolchain.
  *
  * Build: see oracle/Makefile (gcc -O2 -ffp-contract=off, no fast-math: every fp32 operation
  * below must round exactly once).
@@ -319,11 +328,12 @@ void eri_oracle_quantize(const float *x, const float *map, uint64_t numel, uint8
 /* master != NULL: mixed precision (src/kernels/fused_adam.cu:151-193): the fp32 master copy is the value
  * that is read and updated, and p receives its rounded value.  Pinned by: the master after any number
  * of steps equals what the fp32 path gives on the same gradients, and p equals the rounded master. */
-void eri_oracle_adamw32_step(void *p, const void *g, float *m, float *v, uint64_t numel, int dtype, float lr,
-                             float beta1, float beta2, float eps, float wd, float *master) {
+static void adamw32_step(void *p, const void *g, float *m, float *v, uint64_t numel, int dtype, float lr,
+                         float beta1, float beta2, float eps, float wd, float *master, int scaled, float gscale) {
     const float omb1 = 1.0f - beta1, omb2 = 1.0f - beta2, neg_lr = -lr;
     for (uint64_t i = 0; i < numel; ++i) {
         float pf = master ? master[i] : load_elem(p, i, dtype), gr = load_elem(g, i, dtype);
+        if (scaled) gr = gr * gscale; /* one rounded product, as in the 8-bit step (step_elem above) */
         float ms = m[i] * beta1;       /* :35 */
         float gs = gr * omb1;          /* :36 */
         float mn = ms + gs;            /* :37 */
@@ -343,6 +353,21 @@ void eri_oracle_adamw32_step(void *p, const void *g, float *m, float *v, uint64_
         if (dtype == ERI_ORACLE_F32) ((float *)p)[i] = pn;
         else ((uint16_t *)p)[i] = eri_oracle_f32_to_bf16(pn); /* :55 */
     }
+}
+
+void eri_oracle_adamw32_step(void *p, const void *g, float *m, float *v, uint64_t numel, int dtype, float lr,
+                             float beta1, float beta2, float eps, float wd, float *master) {
+    adamw32_step(p, g, m, v, numel, dtype, lr, beta1, beta2, eps, wd, master, 0, 1.0f);
+}
+
+/* The same step on gradients multiplied by `gscale` first: the clip factor of the global norm and the loss-scale
+ * and per-layer multipliers, which the reference applies by rewriting the gradients before the optimizer runs
+ * (clip_gradients, pipeline_flux_lora_sequential.rs:1198-1213; pipeline_flux_lora_1024.rs:691-697).  Pinned by:
+ * equals the unscaled step on gradients multiplied beforehand (fp32 tensors, where that product is not rounded
+ * to the tensor's dtype in between). */
+void eri_oracle_adamw32_step_scaled(void *p, const void *g, float *m, float *v, uint64_t numel, int dtype, float lr,
+                                    float beta1, float beta2, float eps, float wd, float *master, float gscale) {
+    adamw32_step(p, g, m, v, numel, dtype, lr, beta1, beta2, eps, wd, master, 1, gscale);
 }
 
 /* EMA update, src/trainers/ema_enhanced.rs:91-100: shadow = shadow*decay + p*(1 - decay) in fp32,

@@ -56,6 +56,7 @@ def lib():
         L.eri_oracle_dequantize.argtypes = [C.c_void_p] * 3 + [C.c_uint64, C.c_void_p]
         L.eri_oracle_quantize.argtypes = [C.c_void_p] * 2 + [C.c_uint64, C.c_void_p, C.c_void_p]
         L.eri_oracle_adamw32_step.argtypes = [C.c_void_p] * 4 + [C.c_uint64, C.c_int] + [C.c_float] * 5 + [C.c_void_p]
+        L.eri_oracle_adamw32_step_scaled.argtypes = [C.c_void_p] * 4 + [C.c_uint64, C.c_int] + [C.c_float] * 5 + [C.c_void_p, C.c_float]
         L.eri_oracle_ema_update.argtypes = [C.c_void_p] * 2 + [C.c_uint64, C.c_int, C.c_float]
         L.eri_oracle_num_threads.restype = C.c_int
         _lib = L

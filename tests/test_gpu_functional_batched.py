@@ -330,3 +330,95 @@ def test_python_face_batched_functional_and_f32_gradients():
         assert np.array_equal(p.view(torch.int16).cpu().numpy().view(np.uint16).reshape(-1), p_host), k
     for o in (a, b, c, rounded, opt):
         o.close()
+
+
+def test_alternating_output_sets_stop_uploading_after_two_flushes():
+    """update() returns a new tensor per call (adam8bit.rs:205-207), so a trainer's rows alternate between two sets of
+    addresses.  The two launch tables kept serve every flush from the third on without an upload, and the results
+    stay those of the oracle, bit for bit.  A third set of addresses costs one more upload."""
+    import torch
+    L = _L()
+    sizes = [2048 * 3 + 8, 640 * 16, 2048, 4104]
+    n = len(sizes)
+    ps, _ = hs.make_inputs(sizes, True, 991)
+    states = hs.oracle_states(sizes)
+    bufs = [[_dev(p) for p in ps], [_dev(p) for p in ps]]  # the two sets a trainer's allocator hands back in turn
+    g_dev = [_dev(np.zeros(k, np.uint16)) for k in sizes]   # gradient buffers are reused, refilled every step
+    opt = C.c_void_p()
+    stream = torch.cuda.current_stream().cuda_stream
+    L.check(L.lib().eri_adam8bit_fn_with_params(LR, B1, B2, EPS, WD, stream, C.byref(opt)), "with_params")
+    names = (C.c_char_p * n)(*[("w%d" % i).encode() for i in range(n)])
+    numels = (C.c_uint64 * n)(*sizes)
+    tags = (C.c_int32 * n)(*([L.DTYPE_BF16] * n))
+    arr = lambda ts: (C.c_void_p * n)(*[t.data_ptr() for t in ts])
+    flushes, uploads = C.c_uint64(), C.c_uint64()
+    seen = []
+    for step in range(6):
+        gs = hs.fresh_grads(sizes, True, 8100 + step, 1e-3)
+        for d, g in zip(g_dev, gs):
+            d.copy_(_dev(g))
+        src, dst = bufs[step & 1], bufs[1 - (step & 1)]
+        L.check(L.lib().eri_adam8bit_fn_update_many(opt, names, arr(src), arr(g_dev), numels, tags, None, arr(dst), n), "update_many")
+        L.check(L.lib().eri_adam8bit_fn_step(opt), "fn_step")
+        hs.oracle_step(ps, gs, states, (LR, B1, B2, EPS, WD, step), True, oc.MODE_L2)
+        L.check(L.lib().eri_adam8bit_fn_table_stats(opt, C.byref(flushes), C.byref(uploads)), "table_stats")
+        seen.append((flushes.value, uploads.value))
+    assert seen == [(1, 1), (2, 2), (3, 2), (4, 2), (5, 2), (6, 2)]
+    torch.cuda.synchronize()
+    for i in range(n):
+        assert np.array_equal(_bits(bufs[0][i], np.uint16), ps[i])
+    # addresses seen in neither of the last two flushes: one upload, into the table used longer ago
+    third = [torch.empty_like(t) for t in bufs[0]]
+    gs = hs.fresh_grads(sizes, True, 8200, 1e-3)
+    for d, g in zip(g_dev, gs):
+        d.copy_(_dev(g))
+    L.check(L.lib().eri_adam8bit_fn_update_many(opt, names, arr(bufs[0]), arr(g_dev), numels, tags, None, arr(third), n), "update_many")
+    L.check(L.lib().eri_adam8bit_fn_step(opt), "fn_step")
+    hs.oracle_step(ps, gs, states, (LR, B1, B2, EPS, WD, 6), True, oc.MODE_L2)
+    L.check(L.lib().eri_adam8bit_fn_table_stats(opt, C.byref(flushes), C.byref(uploads)), "table_stats")
+    assert (flushes.value, uploads.value) == (7, 3)
+    torch.cuda.synchronize()
+    for i in range(n):
+        assert np.array_equal(_bits(third[i], np.uint16), ps[i])
+    L.check(L.lib().eri_adam8bit_fn_destroy(opt), "destroy")
+
+
+def test_a_refused_update_many_runs_nothing_and_leaves_no_state_behind():
+    """Every row is validated and every new state created before the first launch: a call with one bad row
+    changes no parameter, creates no state and queues nothing, whether the bad row comes first or last, and also
+    when a name repeats before it (which would otherwise split the call into two launches)."""
+    import torch
+    L = _L()
+    sizes = [4096, 2048 + 8, 1024]
+    n = len(sizes)
+    ps, gs = hs.make_inputs(sizes, True, 77)
+    p_dev = [_dev(p) for p in ps]
+    g_dev = [_dev(g) for g in gs]
+    outs = [torch.zeros_like(p) for p in p_dev]
+    opt = C.c_void_p()
+    L.check(L.lib().eri_adam8bit_fn_with_params(LR, B1, B2, EPS, WD, torch.cuda.current_stream().cuda_stream, C.byref(opt)), "with_params")
+    cnt, nbytes = C.c_uint64(), C.c_uint64()
+
+    def call(names, idx, tags=None, numels=None):
+        k = len(idx)
+        return L.lib().eri_adam8bit_fn_update_many(
+            opt, (C.c_char_p * k)(*names), (C.c_void_p * k)(*[p_dev[i].data_ptr() for i in idx]),
+            (C.c_void_p * k)(*[g_dev[i].data_ptr() for i in idx]), (C.c_uint64 * k)(*(numels or [sizes[i] for i in idx])),
+            (C.c_int32 * k)(*(tags or [L.DTYPE_BF16] * k)), None, (C.c_void_p * k)(*[outs[i].data_ptr() for i in idx]), k)
+
+    # a bad dtype tag in the last row
+    assert call([b"a", b"b", b"c"], [0, 1, 2], tags=[L.DTYPE_BF16, L.DTYPE_BF16, 1]) == -4
+    # a repeated name (which splits the call) followed by an empty tensor
+    assert call([b"a", b"a", b"c"], [0, 0, 2], numels=[sizes[0], sizes[0], 0]) == -3
+    L.check(L.lib().eri_adam8bit_fn_step(opt), "fn_step")
+    torch.cuda.synchronize()
+    L.check(L.lib().eri_adam8bit_fn_memory_stats(opt, C.byref(cnt), C.byref(nbytes)), "memory_stats")
+    assert (cnt.value, nbytes.value) == (0, 0)
+    assert all(int(o.count_nonzero()) == 0 for o in outs)
+    # a state that exists with another size: refused before the new name of the same call gets a state
+    L.check(call([b"a"], [0]), "update_many")
+    assert call([b"d", b"a"], [1, 2]) == -6
+    L.check(L.lib().eri_adam8bit_fn_memory_stats(opt, C.byref(cnt), C.byref(nbytes)), "memory_stats")
+    assert cnt.value == 1
+    assert int(outs[1].count_nonzero()) == 0
+    L.check(L.lib().eri_adam8bit_fn_destroy(opt), "destroy")

@@ -8,6 +8,7 @@ import pytest
 
 import harness as hs
 import oracle_c as oc
+from oracle import adam8_numpy as onp
 
 pytestmark = pytest.mark.gpu
 LR, B1, B2, EPS, WD = 1e-3, 0.9, 0.999, 1e-8, 0.01
@@ -396,7 +397,8 @@ def test_legacy_state_longer_than_one_staging_piece(tmp_path):
 def test_min_8bit_size_keeps_short_tensors_in_fp32_moments(tmp_path):
     """Parameters below min_8bit_size take the same update with fp32 moments (one launch of the 32-bit step
     for all of them), the others the 8-bit step; both against their oracles over three steps, then a
-    save / load round trip that carries both kinds of state, and the refusals."""
+    save / load round trip that carries both kinds of state, then two steps with loss scale, per-layer
+    multipliers and clipping by the global norm of all gradients, and the refusal of another mode."""
     import torch
     L = _L()
     sizes = [2048 * 3 + 5, 300, 4095, 4096, 64, 2048 * 2]
@@ -479,13 +481,43 @@ def test_min_8bit_size_keeps_short_tensors_in_fp32_moments(tmp_path):
     assert L.lib().eri_adam8bit_get_step(opt) == 3
     one_step(opt, 4)
     check(opt)
-    # refusals: scaling or clipping inside the step, and mode BNB, cannot be combined with fp32-moment parameters
+    # loss scale, a per-layer multiplier on one tensor of either kind and clipping by the global norm, all inside
+    # the step: the short tensors get the same factors as the 8-bit ones, and the norm covers every gradient
+    # (the trainer that sets min_8bit_size clips all of them: pipeline_flux_lora_1024.rs:451,691-697)
     L.check(L.lib().eri_adam8bit_set_grad_scale(opt, 0.5), "set_grad_scale")
-    assert L.lib().eri_adam8bit_step(opt, None) == -6
-    L.check(L.lib().eri_adam8bit_set_grad_scale(opt, 1.0), "set_grad_scale")
-    L.check(L.lib().eri_adam8bit_set_max_grad_norm(opt, 1.0, 0.0), "set_max_grad_norm")
+    L.check(L.lib().eri_adam8bit_set_param_grad_scale(opt, 1, 0.25), "param_scale")   # a short tensor
+    L.check(L.lib().eri_adam8bit_set_param_grad_scale(opt, 3, 2.0), "param_scale")    # an 8-bit one
+    L.check(L.lib().eri_adam8bit_set_max_grad_norm(opt, 0.01, 0.0), "set_max_grad_norm")
+    per_param = [1.0, 0.25, 1.0, 2.0, 1.0, 1.0]
+    for t in (5, 6):
+        gs = [hs.fresh_grads([n], bf16, 100 * t + i)[0] for i, (n, bf16) in enumerate(zip(sizes, dts))]
+        g_dev = [torch.from_numpy(g.view(np.uint8).copy()).to(dev) for g in gs]
+        keep.append(g_dev)
+        for i in range(len(sizes)):
+            L.check(L.lib().eri_param_set_grad(handles[i], g_dev[i].data_ptr()), "set_grad")
+        L.check(L.lib().eri_adam8bit_step(opt, None), "step")
+        norm, scale = C.c_float(), C.c_float()
+        L.check(L.lib().eri_adam8bit_last_grad_norm(opt, C.byref(norm), C.byref(scale)), "last_grad_norm")
+        g64 = [(onp.bf16_to_f32(g) if bf16 else g).astype(np.float64) for g, bf16 in zip(gs, dts)]
+        want = np.sqrt(sum(float((g * g).sum()) for g in g64))  # over all six gradients, unscaled as stored
+        assert abs(norm.value - want) <= 2e-6 * want
+        assert norm.value > 0.01 and scale.value == np.float32(0.01) / np.float32(norm.value)
+        h = oc.hyper_pack(1e-4, B1, B2, EPS, WD, t)
+        for i, (n, bf16) in enumerate(zip(sizes, dts)):
+            dt = oc.DT_BF16 if bf16 else oc.DT_F32
+            factor = float((np.float32(0.5) * np.float32(per_param[i])) * np.float32(scale.value))
+            if small[i]:
+                oc.lib().eri_oracle_adamw32_step_scaled(oc.ptr(host_p[i]), oc.ptr(gs[i]), oc.ptr(states32[i][0]), oc.ptr(states32[i][1]),
+                                                        n, dt, float(h.step_size), B1, B2, EPS, WD, None, factor)
+            else:
+                hh = oc.hyper_pack(1e-4, B1, B2, EPS, WD, t, grad_scale=factor)
+                assert oc.step_tensor(host_p[i], gs[i], *states8[i], hh, hs.MAPS, dt, 2) == 0
+    check(opt)
+    # the one refusal left: another arithmetic than the reference's own for the 8-bit tensors
+    L.check(L.lib().eri_adam8bit_set_mode(opt, L.MODE_BNB), "set_mode")
     assert L.lib().eri_adam8bit_step(opt, None) == -6
     assert b"min_8bit_size" in L.lib().eri_last_error()
+    assert L.lib().eri_adam8bit_get_step(opt) == 6  # a refused step counts for nothing
     L.lib().eri_adam8bit_destroy(opt)
     for h in handles:
         L.lib().eri_param_release(h)

@@ -134,3 +134,82 @@ def test_functional_optimizer_with_pooled_states_matches_the_oracle():
         assert np.array_equal(got, ps[i])
     del opt
     pool.close()
+
+
+def test_released_pieces_are_handed_out_again():
+    """eri_hip_pool_release: the top piece lowers the lane's fill level (and takes released pieces right below it
+    along), any other piece waits for the next request of exactly its size; the stream-ordered allocation hands out
+    cleared memory; pieces that are not the pool's are refused."""
+    import torch
+    L = _L()
+    pool = _pool(32 * MiB, 2)
+    used = C.c_size_t()
+    a, b, c, d = (C.c_void_p() for _ in range(4))
+    stream = torch.cuda.current_stream().cuda_stream
+    L.check(L.lib().eri_hip_pool_alloc_zeroed(pool, 0, 1000, C.byref(a)), "alloc")
+    L.check(L.lib().eri_hip_pool_alloc_zeroed(pool, 0, 4096, C.byref(b)), "alloc")
+    L.check(L.lib().eri_hip_pool_alloc_zeroed(pool, 0, 300, C.byref(c)), "alloc")
+    L.check(L.lib().eri_hip_pool_lane_used(pool, 0, C.byref(used)), "lane_used")
+    assert used.value == 1024 + 4096 + 512
+    # dirty the middle piece, give it back, ask for its size again on a stream: the same piece, cleared
+    L.check(L.lib().eri_hip_memset_async(b, 0xAB, 4096, stream), "memset")
+    L.check(L.lib().eri_hip_pool_release(pool, b, 4096), "release")
+    L.check(L.lib().eri_hip_pool_lane_used(pool, 0, C.byref(used)), "lane_used")
+    assert used.value == 1024 + 4096 + 512  # not the top piece: the level stays
+    L.check(L.lib().eri_hip_pool_alloc_zeroed_async(pool, 0, 2000, stream, C.byref(d)), "alloc_async")  # another size: from the top
+    assert d.value == a.value + 1024 + 4096 + 512
+    e = C.c_void_p()
+    L.check(L.lib().eri_hip_pool_alloc_zeroed_async(pool, 0, 4000, stream, C.byref(e)), "alloc_async")  # 4000 rounds to 4096
+    assert e.value == b.value
+    host = np.full(4096, 7, np.uint8)
+    L.check(L.lib().eri_hip_memcpy_async(host.ctypes.data, e, 4096, 2, stream), "d2h")
+    L.check(L.lib().eri_hip_stream_sync(stream), "sync")
+    assert not host.any()
+    # top piece back: the level drops to its start; then the piece below it, and the released one under that goes along
+    L.check(L.lib().eri_hip_pool_release(pool, d, 2000), "release")
+    L.check(L.lib().eri_hip_pool_lane_used(pool, 0, C.byref(used)), "lane_used")
+    assert used.value == 1024 + 4096 + 512
+    L.check(L.lib().eri_hip_pool_release(pool, e, 4000), "release")
+    L.check(L.lib().eri_hip_pool_release(pool, c, 300), "release")
+    L.check(L.lib().eri_hip_pool_lane_used(pool, 0, C.byref(used)), "lane_used")
+    assert used.value == 1024
+    # not the pool's, or beyond the lane's level
+    assert L.lib().eri_hip_pool_release(pool, C.c_void_p(a.value + 8 * MiB), 256) == -6
+    assert L.lib().eri_hip_pool_release(pool, C.c_void_p(a.value + 100), 256) == -6
+    assert L.lib().eri_hip_pool_release(pool, None, 256) == 0
+    L.check(L.lib().eri_hip_pool_destroy(pool), "destroy")
+
+
+def test_loading_a_checkpoint_again_does_not_grow_the_state_lane(tmp_path):
+    """States that are replaced go back to the pool and the next load takes them: the lane holds two sets of states
+    after the first load into an optimizer that has stepped, and not a byte more after the second and third."""
+    import torch
+    from eridiffusion_amd.adam8bit import Adam8bit, Adam8bitConfig, DevicePool
+    L = _L()
+    sizes = [2048 * 4 + 16, 5000, 2048]
+    ps, gs = hs.make_inputs(sizes, True, 555)
+    to_t = lambda a: torch.from_numpy(a.view(np.int16)).cuda().view(torch.bfloat16)
+    params = [to_t(p) for p in ps]
+    pool = DevicePool(16 * MiB, 2)
+    opt = Adam8bit(params, Adam8bitConfig(lr=LR, betas=(B1, B2), eps=EPS, weight_decay=WD))
+    opt.set_state_pool(pool, 1)
+    for p, g in zip(params, gs):
+        p.grad = to_t(g)
+    opt.step()
+    torch.cuda.synchronize()
+    used = C.c_size_t()
+    L.check(L.lib().eri_hip_pool_lane_used(pool._pool, 1, C.byref(used)), "lane_used")
+    one_set = used.value
+    assert one_set > 0
+    path = str(tmp_path / "state.safetensors")
+    opt.save_state(path)
+    levels = []
+    for _ in range(3):
+        opt.load_state(path)
+        L.check(L.lib().eri_hip_pool_lane_used(pool._pool, 1, C.byref(used)), "lane_used")
+        levels.append(used.value)
+    assert levels[0] <= 2 * one_set and levels[1] == levels[0] and levels[2] == levels[0]
+    opt.step()  # the loaded states are the ones that step
+    torch.cuda.synchronize()
+    del opt
+    pool.close()

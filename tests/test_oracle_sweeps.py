@@ -126,3 +126,42 @@ def test_adamw32_with_the_bias_corrected_step_size_is_the_8bit_update_without_a_
             q = onp.f32_to_bf16(qn) if bf16 else qn
             assert np.array_equal(m.view(np.uint32), mm.view(np.uint32)) and np.array_equal(v.view(np.uint32), vv.view(np.uint32))
             assert np.array_equal(p.view(np.uint16 if bf16 else np.uint32), q.view(np.uint16 if bf16 else np.uint32)), (bf16, t)
+
+
+def test_adamw32_scaled_equals_the_unscaled_step_on_gradients_multiplied_beforehand():
+    """The scale enters as one rounded fp32 product with the gradient and nowhere else: on fp32 tensors the
+    scaled step equals the plain step on g * scale (formed in fp32), moments and parameters bit for bit, over
+    several steps; on bf16 tensors the product is not rounded to bf16 in between, so it equals the fp32-gradient
+    arithmetic and differs from the step on the bf16-rounded product; and a wrong place for the scale (after
+    the square, or on the update) would fail the first comparison."""
+    rng = np.random.default_rng(5)
+    n, lr, b1, b2, eps, wd = 4099, 3e-4, 0.9, 0.999, 1e-8, 0.01
+    scale = np.float32(0.37)
+    p0 = (rng.standard_normal(n) * 0.05).astype(np.float32)
+    pa, pb = p0.copy(), p0.copy()
+    ma, va, mb, vb = (np.zeros(n, np.float32) for _ in range(4))
+    for t in range(4):
+        g = (rng.standard_normal(n) * 1e-2).astype(np.float32)
+        oc.lib().eri_oracle_adamw32_step_scaled(oc.ptr(pa), oc.ptr(g), oc.ptr(ma), oc.ptr(va), n, oc.DT_F32, lr, b1, b2, eps, wd,
+                                                None, float(scale))
+        gs = (g * scale).astype(np.float32)
+        adamw(pb, gs, mb, vb, oc.DT_F32, lr, b1, b2, eps, wd)
+        assert np.array_equal(pa.view(np.uint32), pb.view(np.uint32))
+        assert np.array_equal(ma.view(np.uint32), mb.view(np.uint32)) and np.array_equal(va.view(np.uint32), vb.view(np.uint32))
+    # scale 1 is the plain step
+    pc, mc, vc = p0.copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    pd, md, vd = p0.copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    g = (rng.standard_normal(n) * 1e-2).astype(np.float32)
+    oc.lib().eri_oracle_adamw32_step_scaled(oc.ptr(pc), oc.ptr(g), oc.ptr(mc), oc.ptr(vc), n, oc.DT_F32, lr, b1, b2, eps, wd, None, 1.0)
+    adamw(pd, g, md, vd, oc.DT_F32, lr, b1, b2, eps, wd)
+    assert np.array_equal(pc.view(np.uint32), pd.view(np.uint32)) and np.array_equal(mc, md) and np.array_equal(vc, vd)
+    # bf16: the product stays fp32 (first moment = (1 - b1) * (g * scale) exactly as fp32 arithmetic gives it)
+    gb = onp.f32_to_bf16(g)
+    pe = onp.f32_to_bf16(p0)
+    me, ve = np.zeros(n, np.float32), np.zeros(n, np.float32)
+    oc.lib().eri_oracle_adamw32_step_scaled(oc.ptr(pe), oc.ptr(gb), oc.ptr(me), oc.ptr(ve), n, oc.DT_BF16, lr, b1, b2, eps, wd,
+                                            None, float(scale))
+    want_m = (onp.bf16_to_f32(gb) * scale).astype(np.float32) * (np.float32(1.0) - np.float32(b1))
+    assert np.array_equal(me.view(np.uint32), want_m.astype(np.float32).view(np.uint32))
+    rounded = onp.bf16_to_f32(onp.f32_to_bf16((onp.bf16_to_f32(gb) * scale).astype(np.float32)))
+    assert not np.array_equal(me, rounded * (np.float32(1.0) - np.float32(b1)))
