@@ -29,7 +29,8 @@ PEAK_HBM_GBPS = 8000.0
 BYTES_PER_PARAM = {"bf16": 2 + 2 + 1 + 1 + 2 + 1 + 1 + 16.0 / 2048, "f32": 4 + 4 + 1 + 1 + 4 + 1 + 1 + 16.0 / 2048}
 # the type the arithmetic of each kernel is carried out in, whatever the parameters are stored as: every one of
 # them widens its inputs to fp32 and rounds each operation to fp32 (the gradient norm adds its fp32 block sums in f64)
-ARITHMETIC = {"adam8": "f32", "adam8_clip": "f32", "adam8_ema": "f32", "grad_norm": "f32", "adamw32": "f32", "ema": "f32"}
+ARITHMETIC = {"adam8": "f32", "adam8_clip": "f32", "adam8_ema": "f32", "grad_norm": "f32", "adamw32": "f32", "ema": "f32",
+              "traffic": "u8"}  # the traffic probe moves bytes and computes nothing
 
 HEADLINE = dict(config="c5_flux12b_full", flags=0, kernel="adam8", mode="eri", api="table", param_dtype="config",
                 grad_dtype="param", alloc="pool")
@@ -44,6 +45,7 @@ ROWS = [
     (dict(config="c4_sdxl_unet_full"), 20, 3),
     (dict(config="c5_flux12b_full", flags=2), 20, 3),
     (dict(config="c5_flux12b_full", mode="l2"), 20, 3),
+    (dict(config="c5_flux12b_full", kernel="traffic"), 20, 3),
     (dict(config="c5_flux12b_full", alloc="tensor"), 20, 3),
 ]
 
@@ -59,7 +61,8 @@ def parse():
     ap.add_argument("--kernel", choices=sorted(ARITHMETIC), default="adam8",
                     help="what one step is: the 8-bit AdamW step (headline), the same preceded by the device-side "
                          "gradient norm, the same with the EMA of the parameters taken inside it, the norm alone, "
-                         "the 32-bit AdamW sibling, or the EMA sweep")
+                         "the 32-bit AdamW sibling, the EMA sweep, or the traffic probe (the step's reads and writes in "
+                         "the step's launch shape with no arithmetic: what the memory system gives that mix of streams)")
     ap.add_argument("--mode", choices=["eri", "l2"], default="eri",
                     help="arithmetic of the table API's step: the list optimizer's (adam8bit_enhanced.rs) or the "
                          "functional update's (adam8bit.rs, what --api functional always runs)")
@@ -432,6 +435,9 @@ def measure(args, torch, separate_events=False):
         if args.kernel == "ema":
             L.check(L.lib().eri_ema_update_multi(rows_e, len(sizes), 0.999, stream), "ema")
             return
+        if args.kernel == "traffic":
+            L.check(L.lib().eri_adam8_traffic_probe(table, stream), "traffic_probe")
+            return
         flags = args.flags
         if args.kernel in ("grad_norm", "adam8_clip"):
             L.check(L.lib().eri_adam8_grad_norm(table, 1.0, 0.0, stream), "grad_norm")
@@ -532,7 +538,7 @@ def measure(args, torch, separate_events=False):
 def row_of(out):
     """The short form of a measurement for the `configs` list."""
     c, r = out["config"], out["roofline"]
-    return {"workload": c["workload"], "api": c["api"], "mode": c["mode"], "flags": c["flags"], "alloc": c["alloc"],
+    return {"workload": c["workload"], "kernel": c["kernel"], "api": c["api"], "mode": c["mode"], "flags": c["flags"], "alloc": c["alloc"],
             "param_dtype": c["param_dtype"], "params": c["params"], "tensors": c["tensors"], "steps": out["steps"],
             "warmup": out["warmup"], "ms_per_step": out["ms_per_step"], "params_per_s": out["value"],
             "kernel_ms": r["kernel_ms"], "kernel_ms_min": r["kernel_ms_min"], "frac": r["frac"],

@@ -84,6 +84,8 @@ EXPORTS = {
     "eri_hip_pool_alloc_zeroed": (C.c_int, [C.c_void_p, C.c_uint32, C.c_size_t, C.POINTER(C.c_void_p)]),
     "eri_hip_pool_alloc_zeroed_async": (C.c_int, [C.c_void_p, C.c_uint32, C.c_size_t, C.c_void_p, C.POINTER(C.c_void_p)]),
     "eri_hip_pool_release": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
+    "eri_hip_pool_retain": (C.c_int, [C.c_void_p]),
+    "eri_hip_pool_unretain": (C.c_int, [C.c_void_p]),
     "eri_hip_pool_info": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint32), C.POINTER(C.c_size_t)]),
     "eri_hip_pool_lane_used": (C.c_int, [C.c_void_p, C.c_uint32, C.POINTER(C.c_size_t)]),
     "eri_hip_pool_reset": (C.c_int, [C.c_void_p]),
@@ -105,6 +107,7 @@ EXPORTS = {
     "eri_adam8_grad_norm_static": (C.c_int, [C.c_void_p, C.c_float, C.c_float, C.c_void_p, C.c_void_p]),
     "eri_adam8_grad_norm_read": (C.c_int, [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_void_p]),
     "eri_adam8_grad_nonfinite_read": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint64), C.c_void_p]),
+    "eri_adam8_traffic_probe": (C.c_int, [C.c_void_p, C.c_void_p]),
     "eri_adam8_quant_error": (C.c_int, [C.c_void_p, C.POINTER(Hyper), C.c_void_p]),
     "eri_adam8_quant_error_read": (C.c_int, [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_void_p]),
     "eri_adam8_step_multi": (C.c_int, [C.POINTER(TensorRow), C.c_uint32, C.POINTER(Hyper), C.c_void_p]),

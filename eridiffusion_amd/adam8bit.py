@@ -230,6 +230,7 @@ class Adam8bitFunctional:
                                                 C.byref(self._opt)), "eri_adam8bit_fn_with_params")
         self._names: List[str] = []
         self._live: List[torch.Tensor] = []
+        self._launched = False
         self._batched = bool(batched)
         if batched:
             check(lib().eri_adam8bit_fn_set_batching(self._opt, 1), "eri_adam8bit_fn_set_batching")
@@ -245,15 +246,23 @@ class Adam8bitFunctional:
 
     def step(self) -> None:
         check(lib().eri_adam8bit_fn_step(self._opt), "eri_adam8bit_fn_step")
-        self._live = []
+        self._launched = True
 
     def flush(self) -> None:
         check(lib().eri_adam8bit_fn_flush(self._opt), "eri_adam8bit_fn_flush")
-        self._live = []
+        self._launched = True
 
     def set_lr(self, lr: float) -> None:
         check(lib().eri_adam8bit_fn_set_lr(self._opt, lr), "eri_adam8bit_fn_set_lr")
-        self._live = []
+        self._launched = True
+
+    def _keep(self, tensors) -> None:
+        """What a launch reads and writes stays referenced until the first update after that launch: the launch is
+        asynchronous (and, batched, still to come), and nothing it touches may go back to the allocator under it."""
+        if self._launched:
+            self._live = []
+            self._launched = False
+        self._live += tensors
 
     def get_step(self) -> int:
         return lib().eri_adam8bit_fn_get_step(self._opt)
@@ -264,8 +273,9 @@ class Adam8bitFunctional:
         out = torch.empty_like(p)
         check(lib().eri_adam8bit_fn_update(self._opt, name.encode(), p.data_ptr(), g.data_ptr(), p.numel(),
                                            _dtype_tag(p), _dtype_tag(g), out.data_ptr()), "eri_adam8bit_fn_update")
-        if self._batched:
-            self._live += [p, g, out]
+        self._keep([p, g, out])
+        if not self._batched:
+            self._launched = True  # ran at once; released when the next update arrives
         if name not in self._names:
             self._names.append(name)
         return out
@@ -284,6 +294,8 @@ class Adam8bitFunctional:
                                                 (C.c_int32 * k)(*[_dtype_tag(p) for p in ps]),
                                                 (C.c_int32 * k)(*[_dtype_tag(g) for g in gs]), arr(outs), k),
               "eri_adam8bit_fn_update_many")
+        self._keep(ps + gs + outs)
+        self._launched = True
         for n in names:
             if n not in self._names:
                 self._names.append(n)

@@ -110,8 +110,8 @@ bool step_fuses_ema(uint32_t total_full_blocks, int layout, const EriAdam8Hyper 
 int launch_step_pipelined(int mode, bool exact, bool wd, bool gs, bool ema, const DevTensor *rows, uint32_t n_rows,
                           uint32_t total_blocks, const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale,
                           uint32_t grid, uint32_t wg, void *stream);
-/* The same kernel for bf16 parameters whose gradients are fp32 (no EMA inside it). */
-int launch_step_pipelined_grad_f32(int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
+/* The same kernel for bf16 parameters whose gradients are fp32. */
+int launch_step_pipelined_grad_f32(int mode, bool exact, bool wd, bool gs, bool ema, const DevTensor *rows, uint32_t n_rows,
                                    uint32_t total_blocks, const EriAdam8Hyper &h, const void *lds_image,
                                    const float *dev_scale, uint32_t grid, uint32_t wg, void *stream);
 /* The same kernel for fp32 parameters (IEEE chain throughout, no EMA inside it). */
@@ -128,6 +128,8 @@ int launch_grad_sumsq(const DevTensor *rows, uint32_t n_rows, uint32_t total_ful
                       double *partial, uint32_t grid, void *stream);
 int launch_grad_norm_finish(const double *partial, uint32_t n, float max_norm, float denom_eps, float *out,
                             void *stream);
+/* Diagnostics: reads and rewrites (unchanged) every full block of a group of bf16 rows as the step does. */
+int launch_traffic_probe(const DevTensor *rows, uint32_t n_rows, uint32_t total_full_blocks, uint32_t grid, void *stream);
 /* Clears `bytes` bytes at `p`; both multiples of 16. */
 int launch_fill_zero(void *p, size_t bytes, void *stream);
 int launch_state_init(uint8_t *m, uint8_t *v, float *absmax_m, float *absmax_v, uint64_t numel, void *stream);

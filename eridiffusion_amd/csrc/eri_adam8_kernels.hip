@@ -7,9 +7,10 @@
 
 namespace eri {
 
-/* The one case in which the EMA runs inside the step kernel: the prefetching kernel in mode ERI. */
+/* The one case in which the EMA runs inside the step kernel: the prefetching kernel in mode ERI, on bf16
+ * parameters (with bf16 or fp32 gradients). */
 bool step_fuses_ema(uint32_t total_blocks, int layout, const EriAdam8Hyper &h, uint32_t compute_units) {
-    if ((h.flags & ERI_ADAM8_FLAG_EMA) == 0 || layout != kLayoutBF16 || h.mode != ERI_ADAM8_MODE_ERI) return false;
+    if ((h.flags & ERI_ADAM8_FLAG_EMA) == 0 || !layout_param_bf16(layout) || h.mode != ERI_ADAM8_MODE_ERI) return false;
     if (h.flags & (ERI_ADAM8_FLAG_BSEARCH | ERI_ADAM8_FLAG_NO_PIPELINE)) return false;
     const bool few = (uint64_t)total_blocks <= (uint64_t)compute_units * (uint64_t)kSplitBlocksPerCu;
     return (h.flags & ERI_ADAM8_FLAG_ONE_WAVE) != 0 || !few;
@@ -48,7 +49,8 @@ int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, i
     if (mixed) {
         const bool wd_m = h.mode == ERI_ADAM8_MODE_BNB ? h.weight_decay != 1.0f : h.weight_decay > 0.0f;
         if ((h.flags & ERI_ADAM8_FLAG_NO_PIPELINE) == 0 && prefetch_pays(total_blocks, h, compute_units))
-            return launch_step_pipelined_grad_f32(h.mode, (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0, wd_m, gs, rows, n_rows,
+            return launch_step_pipelined_grad_f32(h.mode, (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0, wd_m, gs,
+                                                  step_fuses_ema(total_blocks, layout, h, compute_units), rows, n_rows,
                                                   total_blocks, h, lds_image, dev_scale, grid, wg, stream);
         return launch_step_plain_bf16(h.mode, (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0, wd_m, gs, true, true, rows, n_rows,
                                       total_blocks, h, lds_image, dev_scale, grid, wg, stream);
@@ -90,6 +92,62 @@ __global__ void state_init_kernel(uint8_t *m, uint8_t *v, float *am, float *av, 
         am[b] = 0.0f;
         av[b] = 0.0f;
     }
+}
+
+// ------------------------------------------------------------------------------------------
+// diagnostics: the memory traffic of one step over bf16 rows and nothing else
+// ------------------------------------------------------------------------------------------
+
+/* Every full block of the table is read and written as the step kernel reads and writes it -- the launch shape
+ * of the prefetching kernel (one workgroup of 768 threads per compute unit, one range of the block list per die),
+ * 128-bit non-temporal loads of parameters and gradients, 64-bit ones of the two code arrays, the two absmax
+ * words, all of a block's loads in flight before its first store -- with no arithmetic between load and store.
+ * Parameters, codes and absmax are written back with the bits they had (`zero` is 0 at run time, which the
+ * compiler cannot know, so neither the loads of the gradients nor the stores fall away).  What this launch takes
+ * is what the memory system gives the step's mix of four read and three written streams in the placement at
+ * hand; the step kernel cannot be faster than that. */
+__global__ __launch_bounds__(768) void traffic_probe_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
+                                                            uint32_t total_blocks, uint32_t chunks, uint32_t zero) {
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const BlockWalk walk(total_blocks, chunks);
+    const BlockRowMap map(rows, n_rows);
+    uint32_t ti = 0, t_end = 0;
+    DevTensor t;
+    for (uint32_t blk = walk.first; blk < walk.end; blk += walk.stride) {
+        map.seek(rows, blk, ti, t, t_end);
+        const uint32_t lb = blk - t.full_start;
+        const size_t e0 = (size_t)lb * kBlock;
+        ERI_GLOBAL u32x4 *pp = as_global(reinterpret_cast<u32x4 *>(static_cast<char *>(t.p) + e0 * 2));
+        ERI_GLOBAL const u32x4 *gp = as_global(reinterpret_cast<const u32x4 *>(static_cast<const char *>(t.g) + e0 * 2));
+        ERI_GLOBAL u32x2 *mp = as_global(reinterpret_cast<u32x2 *>(t.m + e0));
+        ERI_GLOBAL u32x2 *vp = as_global(reinterpret_cast<u32x2 *>(t.v + e0));
+        u32x4 p[4], g[4];
+        u32x2 m[4], v[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            p[c] = __builtin_nontemporal_load(&pp[c * 64 + lane]);
+            g[c] = __builtin_nontemporal_load(&gp[c * 64 + lane]);
+            m[c] = __builtin_nontemporal_load(&mp[c * 64 + lane]);
+            v[c] = __builtin_nontemporal_load(&vp[c * 64 + lane]);
+        }
+        const uint32_t a_m = f2u(as_global(t.absmax_m)[lb]), a_v = f2u(as_global(t.absmax_v)[lb]);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            __builtin_nontemporal_store(p[c] ^ (g[c] & zero), &pp[c * 64 + lane]);
+            __builtin_nontemporal_store(m[c] ^ zero, &mp[c * 64 + lane]);
+            __builtin_nontemporal_store(v[c] ^ zero, &vp[c * 64 + lane]);
+        }
+        if (lane == 0) {
+            as_global(t.absmax_m)[lb] = u2f(a_m ^ zero);
+            as_global(t.absmax_v)[lb] = u2f(a_v ^ zero);
+        }
+    }
+}
+
+int launch_traffic_probe(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, uint32_t grid, void *stream) {
+    hipLaunchKernelGGL(traffic_probe_kernel, dim3(grid), dim3(768), 0, static_cast<hipStream_t>(stream), rows, n_rows,
+                       total_blocks, chunks_for(grid), 0u);
+    return (int)hipGetLastError();
 }
 
 __global__ void fill_zero_kernel(uint4 *p, uint64_t words) {

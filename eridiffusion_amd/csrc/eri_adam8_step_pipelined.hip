@@ -316,7 +316,7 @@ int launch_pipelined(const DevTensor *rows, uint32_t n_rows, uint32_t total_bloc
 template <int MODE, bool EXACT>
 int launch_flags(bool wd, bool gs, bool ema, const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
                  const void *img, const float *dev_scale, uint32_t grid, uint32_t wg, hipStream_t s) {
-    if constexpr (MODE == ERI_ADAM8_MODE_ERI && kGradBf16) { // (which implies bf16 parameters) // the EMA is built into the reference's own update only
+    if constexpr (MODE == ERI_ADAM8_MODE_ERI && kParamBf16) { // the EMA is built into the reference's own update, on bf16 parameters
         if (ema) {
             if (wd) {
                 if (gs) return launch_pipelined<MODE, EXACT, true, true, true>(rows, n_rows, total_blocks, h, img, dev_scale, grid, wg, s);
@@ -343,10 +343,9 @@ int launch_step_pipelined(int mode, bool exact, bool wd, bool gs, bool ema, cons
                           uint32_t total_blocks, const EriAdam8Hyper &h, const void *img, const float *dev_scale,
                           uint32_t grid, uint32_t wg, void *stream) {
 #elif ERI_PIPE_LAYOUT == 2
-int launch_step_pipelined_grad_f32(int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
+int launch_step_pipelined_grad_f32(int mode, bool exact, bool wd, bool gs, bool ema, const DevTensor *rows, uint32_t n_rows,
                                    uint32_t total_blocks, const EriAdam8Hyper &h, const void *img,
                                    const float *dev_scale, uint32_t grid, uint32_t wg, void *stream) {
-    const bool ema = false; // rows with fp32 gradients get their EMA from the sweep
 #else
 int launch_step_pipelined_f32(int mode, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks,
                               const EriAdam8Hyper &h, const void *img, const float *dev_scale, uint32_t grid,

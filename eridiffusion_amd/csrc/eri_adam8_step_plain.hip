@@ -10,6 +10,7 @@
 #error "compile with -DERI_PLAIN_BF16=0 or 1"
 #endif
 
+
 namespace eri {
 
 /* Threads per workgroup.  The coupled-decay mode holds two more divisions' worth of values per element:
@@ -59,8 +60,8 @@ __global__ __launch_bounds__(plain_threads(MODE)) void adam8_step_kernel(const D
     }
     uint32_t ti = 0, t_end = 0;
     DevTensor t;
-    const BlockWalk walk(total_blocks, chunks);
     const BlockRowMap map(rows, n_rows);
+    const BlockWalk walk(total_blocks, chunks);
     for (uint32_t blk = walk.first; blk < walk.end; blk += walk.stride) {
         map.seek(rows, blk, ti, t, t_end);
         const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;

@@ -60,6 +60,7 @@ struct State8 {
         // out of a pool the piece is cleared on the optimizer's stream (state_init below overwrites it anyway)
         rc = from ? eri_hip_pool_alloc_zeroed_async(from, lane, bytes, stream, &base) : eri_hip_malloc_zeroed(dev, bytes, &base);
         if (rc) return rc;
+        if (from) eri_hip_pool_retain(from); // the piece goes back to it, also if the caller destroys the pool first
         pool = from;
         total = bytes;
         char *b = static_cast<char *>(base);
@@ -72,10 +73,14 @@ struct State8 {
         return eri_adam8_state_init(m, v, absmax_m, absmax_v, n, stream);
     }
     /* A pooled piece goes back to its pool, where the next state of the same size takes it (loading a checkpoint
-     * replaces every state by one of its size).  The pool must outlive the states it backs. */
+     * replaces every state by one of its size).  The state holds the pool (eri_hip_pool_retain) until then. */
     void release() {
-        if (base && pool) eri_hip_pool_release(pool, base, total);
-        else if (base) eri_hip_free(base);
+        if (base && pool) {
+            eri_hip_pool_release(pool, base, total);
+            eri_hip_pool_unretain(pool);
+        } else if (base) {
+            eri_hip_free(base);
+        }
         base = nullptr;
         pool = nullptr;
         total = 0;
@@ -1484,19 +1489,34 @@ int eri_adam8bit_fn_update_many(EriAdam8bitFn *o, const char *const *names, cons
                                 const int32_t *grad_dtype_tags, void *const *outs, uint32_t n) {
     if (!o || !names || !params || !grads || !numels || !dtype_tags || !outs)
         return fail(ERI_ERR_NULL, "update_many with NULL argument");
-    // 1. every row is checked before anything runs: arguments, and the size of a state that exists already
+    // 1. every row is checked before anything runs: arguments, and the size of a state that exists already.
+    //    Trainers update the same names in the same order every step, so the name at position i is usually the
+    //    one the last flush had there and the map is not searched.
+    std::vector<uint32_t> unknown;
     for (uint32_t i = 0; i < n; ++i) {
         int rc = fn_check_update(names[i], params[i], grads[i], numels[i], dtype_tags[i],
                                  grad_dtype_tags ? grad_dtype_tags[i] : dtype_tags[i], outs[i]);
         if (rc) return rc;
-        auto it = o->states.find(std::string_view(names[i]));
-        if (it != o->states.end() && it->second->numel != numels[i])
+        const FnState *known = nullptr;
+        if (i < o->last_order.size() && *o->last_order[i].first == names[i]) {
+            known = o->last_order[i].second;
+        } else {
+            auto it = o->states.find(std::string_view(names[i]));
+            if (it != o->states.end()) known = it->second.get();
+        }
+        if (!known) unknown.push_back(i);
+        else if (known->numel != numels[i])
             return fail(ERI_ERR_ARG, std::string("state of '") + names[i] + "' has a different size");
     }
     // 2. states of new names; a failure takes back the ones this call made
     std::vector<std::string> made;
-    for (uint32_t i = 0; i < n; ++i) {
-        if (o->states.find(std::string_view(names[i])) != o->states.end()) continue;
+    for (uint32_t i : unknown) {
+        auto it = o->states.find(std::string_view(names[i]));
+        if (it != o->states.end()) { // the name came up earlier in this call
+            if (it->second->numel == numels[i]) continue;
+            for (auto &name : made) o->states.erase(name);
+            return fail(ERI_ERR_ARG, std::string("state of '") + names[i] + "' has a different size");
+        }
         std::unique_ptr<FnState> s(new FnState());
         int rc = s->allocate(numels[i], o->stream, o->state_pool, o->state_lane);
         if (rc) {

@@ -507,6 +507,8 @@ struct EriHipPool {
     };
     std::vector<std::vector<Piece>> released; // per lane: pieces given back below the lane's top
     std::mutex lock;
+    int refs = 1;        // the creator's reference plus one per eri_hip_pool_retain (guarded by lock)
+    bool closed = false; // the creator has let go: nothing more is handed out
 };
 
 namespace {
@@ -578,6 +580,7 @@ int eri_hip_pool_alloc_zeroed(EriHipPool *pool, uint32_t lane, size_t bytes, voi
     char *p = nullptr;
     {
         std::lock_guard<std::mutex> g(pool->lock);
+        if (pool->closed) return fail(ERI_ERR_ARG, "memory pool: the pool has been destroyed");
         p = pool_take(pool, lane % (uint32_t)pool->used.size(), need);
     }
     if (!p) return fail(ERI_ERR_ARG, "memory pool: the lane is full");
@@ -602,6 +605,7 @@ int eri_hip_pool_alloc_zeroed_async(EriHipPool *pool, uint32_t lane, size_t byte
     char *p = nullptr;
     {
         std::lock_guard<std::mutex> g(pool->lock);
+        if (pool->closed) return fail(ERI_ERR_ARG, "memory pool: the pool has been destroyed");
         p = pool_take(pool, lane % (uint32_t)pool->used.size(), need);
     }
     if (!p) return fail(ERI_ERR_ARG, "memory pool: the lane is full");
@@ -676,12 +680,36 @@ int eri_hip_pool_reset(EriHipPool *pool) {
     return 0;
 }
 
-int eri_hip_pool_destroy(EriHipPool *pool) {
-    if (!pool) return 0;
+int eri_hip_pool_retain(EriHipPool *pool) {
+    if (!pool) return fail(ERI_ERR_NULL, "pool is NULL");
+    std::lock_guard<std::mutex> g(pool->lock);
+    pool->refs += 1;
+    return 0;
+}
+
+static int pool_unref(EriHipPool *pool, bool creator) {
+    bool last;
+    {
+        std::lock_guard<std::mutex> g(pool->lock);
+        if (creator) pool->closed = true;
+        pool->refs -= 1;
+        last = pool->refs <= 0;
+    }
+    if (!last) return 0;
     const hipError_t e = hipFree(pool->base);
     delete pool;
     if (e != hipSuccess) return hip_fail(e, "hipFree");
     return 0;
+}
+
+int eri_hip_pool_destroy(EriHipPool *pool) {
+    if (!pool) return 0;
+    return pool_unref(pool, true);
+}
+
+int eri_hip_pool_unretain(EriHipPool *pool) {
+    if (!pool) return 0;
+    return pool_unref(pool, false);
 }
 
 void *eri_hip_host_alloc(size_t bytes) {
@@ -1088,6 +1116,21 @@ int eri_adam8_grad_nonfinite_read(EriAdam8Table *t, uint64_t *count, void *strea
     ERI_HIP(hipMemcpyAsync(&host, t->norm_last + 2, sizeof host, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream)));
     ERI_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
     *count = host;
+    return 0;
+}
+
+int eri_adam8_traffic_probe(EriAdam8Table *t, void *stream) {
+    if (!t) return fail(ERI_ERR_NULL, "table is NULL");
+    if (t->grads_only) return fail(ERI_ERR_ARG, "a gradient-only table serves eri_adam8_grad_norm only");
+    DeviceCtx *ctx = nullptr;
+    int rc = get_ctx_on(t->device, &ctx);
+    if (rc) return rc;
+    const auto &g = t->groups[eri::kLayoutBF16];
+    if (g.n == 0 || g.total_blocks == 0) return fail(ERI_ERR_ARG, "the traffic probe needs full blocks of BF16 rows with BF16 gradients");
+    rc = order_after_upload(t, stream);
+    if (rc) return rc;
+    rc = eri::launch_traffic_probe(g.dev, g.n, g.total_blocks, ctx->cus * ctx->wg_per_cu, stream);
+    if (rc) return hip_fail((hipError_t)rc, "traffic probe launch");
     return 0;
 }
 

@@ -314,11 +314,13 @@ impl Adam8bitFunctional {
             sys::eri_adam8bit_fn_update(self.opt, c.as_ptr(), param.cuda_ptr() as *const c_void, g.cuda_ptr() as *const c_void,
                                         numel as u64, dtype_tag(param.dtype())?, g_tag, out.cuda_ptr_mut() as *mut c_void)
         }, "eri_adam8bit_fn_update")?;
-        // the launch is asynchronous (and, batched, still to come): what it reads must not be freed under it
+        // the launch is asynchronous (and, batched, still to come): what it reads and writes must not be freed
+        // under it; released when the first update after the launch arrives
         self.live.push(g);
-        if self.batched {
-            self.live.push(param.clone());
-            self.live.push(out.clone());
+        self.live.push(param.clone());
+        self.live.push(out.clone());
+        if !self.batched {
+            self.launched = true;
         }
         if !self.names.iter().any(|n| n == name) {
             self.names.push(name.to_string());
@@ -392,6 +394,8 @@ impl Adam8bitFunctional {
             tags.push(dtype_tag(param.dtype())?);
             g_tags.push(g_tag);
             self.live.push(g);
+            self.live.push((*param).clone()); // the kernel reads the old parameter in place, without a copy
+            self.live.push(out.clone());
             outs.push(out);
             if !self.names.iter().any(|k| k == name) {
                 self.names.push(name.to_string());

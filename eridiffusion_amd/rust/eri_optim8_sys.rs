@@ -86,6 +86,8 @@ extern "C" {
     pub fn eri_hip_pool_create(device: c_int, bytes: usize, lanes: u32, out: *mut *mut EriHipPool) -> c_int;
     pub fn eri_hip_pool_alloc_zeroed(pool: *mut EriHipPool, lane: u32, bytes: usize, out: *mut *mut c_void) -> c_int;
     pub fn eri_hip_pool_alloc_zeroed_async(pool: *mut EriHipPool, lane: u32, bytes: usize, stream: *mut c_void, out: *mut *mut c_void) -> c_int;
+    pub fn eri_hip_pool_retain(pool: *mut EriHipPool) -> c_int;
+    pub fn eri_hip_pool_unretain(pool: *mut EriHipPool) -> c_int;
     pub fn eri_hip_pool_release(pool: *mut EriHipPool, ptr: *mut c_void, bytes: usize) -> c_int;
     pub fn eri_hip_pool_info(pool: *const EriHipPool, lanes: *mut u32, lane_bytes: *mut usize) -> c_int;
     pub fn eri_hip_pool_lane_used(pool: *const EriHipPool, lane: u32, used_bytes: *mut usize) -> c_int;
@@ -109,6 +111,7 @@ extern "C" {
     pub fn eri_adam8_grad_norm_static(table: *mut EriAdam8Table, max_norm: f32, denom_eps: f32, result: *mut c_void, stream: *mut c_void) -> c_int;
     pub fn eri_adam8_grad_norm_read(table: *mut EriAdam8Table, norm: *mut f32, scale: *mut f32, stream: *mut c_void) -> c_int;
     pub fn eri_adam8_grad_nonfinite_read(table: *mut EriAdam8Table, count: *mut u64, stream: *mut c_void) -> c_int;
+    pub fn eri_adam8_traffic_probe(table: *mut EriAdam8Table, stream: *mut c_void) -> c_int;
     pub fn eri_adam8_quant_error(table: *mut EriAdam8Table, hyper: *const EriAdam8Hyper, stream: *mut c_void) -> c_int;
     pub fn eri_adam8_quant_error_read(table: *mut EriAdam8Table, m_error: *mut f32, v_error: *mut f32, stream: *mut c_void) -> c_int;
     pub fn eri_adam8_step_multi(rows: *const EriAdam8Tensor, n: u32, hyper: *const EriAdam8Hyper, stream: *mut c_void) -> c_int;

@@ -92,7 +92,11 @@ int eri_hip_mem_info(size_t *free_bytes, size_t *total_bytes);
  * eri_hip_pool_release gives one piece back: the top piece of a lane lowers the lane's fill level, any other is
  * kept and handed out again to the next request of exactly its size in that lane (optimizer states that are
  * replaced, e.g. by loading a checkpoint, have the size of the ones they replace).  eri_hip_pool_reset empties
- * every lane, eri_hip_pool_destroy frees the allocation.  Calls on one pool may come from several threads. */
+ * every lane.  eri_hip_pool_destroy ends the creator's use of the pool: nothing more is handed out, and the
+ * allocation is freed at once unless somebody else holds the pool through eri_hip_pool_retain (the optimizers do,
+ * once per state they took from it, so that a state destroyed after the pool still has somewhere to give its
+ * piece back to); then it is freed when the last of them lets go with eri_hip_pool_unretain.  Calls on one pool
+ * may come from several threads. */
 typedef struct EriHipPool EriHipPool;
 int eri_hip_pool_create(int device, size_t bytes, uint32_t lanes, EriHipPool **out);
 /* lane counts modulo the pool's lanes.  The piece is cleared by the runtime's synchronous memset: it is zero,
@@ -109,6 +113,8 @@ int eri_hip_pool_info(const EriHipPool *pool, uint32_t *lanes, size_t *lane_byte
 int eri_hip_pool_lane_used(const EriHipPool *pool, uint32_t lane, size_t *used_bytes);
 int eri_hip_pool_reset(EriHipPool *pool);
 int eri_hip_pool_destroy(EriHipPool *pool);
+int eri_hip_pool_retain(EriHipPool *pool);
+int eri_hip_pool_unretain(EriHipPool *pool);
 
 /* ---------------------------------------------------------------------------------------------
  * The optimizer step.
@@ -287,6 +293,14 @@ int eri_adam8_grad_nonfinite_read(EriAdam8Table *table, uint64_t *count, void *s
  * per-tensor `quantization_error` is the same mean (:93-100).  Diagnostics; costs one read pass. */
 int eri_adam8_quant_error(EriAdam8Table *table, const EriAdam8Hyper *hyper, void *stream);
 int eri_adam8_quant_error_read(EriAdam8Table *table, float *m_error, float *v_error, void *stream);
+
+/* Diagnostics, no counterpart in the reference: one launch that moves the bytes of a step over the table's
+ * BF16 rows (BF16 gradients) and does nothing else -- every full block read as the step kernel reads it and
+ * written back unchanged, in the launch shape of the kernel that takes the largest tables.  Its duration is what
+ * the device's memory system gives the step's mix of read and written streams where the caller has placed them,
+ * the figure a step's duration is to be read against (`bench.py --kernel traffic`).  Partial last blocks are
+ * left out.  No data changes. */
+int eri_adam8_traffic_probe(EriAdam8Table *table, void *stream);
 
 /* Convenience for callers that keep no handle: keeps one cached table per calling thread and
  * re-uploads it only when `rows` changed since that thread's last call. */

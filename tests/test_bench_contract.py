@@ -51,7 +51,9 @@ def test_the_rows_of_the_default_run_cover_every_configuration_and_entry_point()
         if change["config"] in ("c2_sdxl_lora_r16", "c3_flux_lora_r32"):
             assert steps == 100
         assert warmup >= 1
-    assert set(b.ARITHMETIC.values()) == {"f32"}  # every kernel widens to fp32 and rounds each operation to fp32
+    # every kernel widens to fp32 and rounds each operation to fp32; the traffic probe only moves bytes
+    assert {k: v for k, v in b.ARITHMETIC.items() if v != "f32"} == {"traffic": "u8"}
+    assert any(r["config"] == "c5_flux12b_full" and r["kernel"] == "traffic" for r in rows)
 
 
 @pytest.mark.gpu
@@ -69,7 +71,7 @@ def test_the_rows_of_the_small_configurations_carry_their_keys():
         ("c3_flux_lora_r32", "table"), ("c3_flux_lora_r32", "functional")]
     for r in rows:
         assert "error" not in r, r
-        for key in ("workload", "api", "mode", "flags", "alloc", "param_dtype", "params", "tensors", "steps", "warmup",
+        for key in ("workload", "kernel", "api", "mode", "flags", "alloc", "param_dtype", "params", "tensors", "steps", "warmup",
                     "ms_per_step", "params_per_s", "kernel_ms", "kernel_ms_min", "frac", "frac_of_step"):
             assert key in r, key
         assert r["steps"] == 100 and r["ms_per_step"] > 0 and 0 < r["frac"] < 1 and 0 < r["frac_of_step"] < 1

@@ -20,16 +20,21 @@ def _dev(a):
     return torch.from_numpy(np.ascontiguousarray(a).view(np.uint8).reshape(-1).copy()).to("cuda:0")
 
 
-@pytest.mark.parametrize("case", ["bf16-in-the-step-kernel", "bf16-small-table", "bf16-plain-kernel", "f32", "bf16-mode-bnb"])
+@pytest.mark.parametrize("case", ["bf16-in-the-step-kernel", "bf16-f32-grads-in-the-step-kernel", "bf16-small-table",
+                                  "bf16-plain-kernel", "f32", "bf16-mode-bnb"])
 def test_shadows_follow_the_updated_parameters(case):
     import torch
     from eridiffusion_amd import _lib as L
     bf16 = case != "f32"
     mode = L.MODE_BNB if case.endswith("bnb") else L.MODE_ERI
-    extra = {"bf16-in-the-step-kernel": L.FLAG_ONE_WAVE, "bf16-plain-kernel": L.FLAG_NO_PIPELINE}.get(case, 0)
+    extra = {"bf16-in-the-step-kernel": L.FLAG_ONE_WAVE, "bf16-f32-grads-in-the-step-kernel": L.FLAG_ONE_WAVE,
+             "bf16-plain-kernel": L.FLAG_NO_PIPELINE}.get(case, 0)
+    grad_f32 = "f32-grads" in case  # bf16 parameters whose gradients are fp32 and enter the arithmetic unrounded
     sizes = [2048 * 5 + 24, 2048 * 3, 77, 2048 * 2 + 1001, 640]
     has_shadow = [True, False, True, True, True]
     ps, gs = hs.make_inputs(sizes, bf16, 21)
+    if grad_f32:
+        gs = hs.fresh_grads(sizes, False, 299)
     states = hs.oracle_states(sizes)
     gt = hs.GpuTensors(ps, gs, states, bf16)
     rng = np.random.default_rng(4)
@@ -41,17 +46,23 @@ def test_shadows_follow_the_updated_parameters(case):
     rows = gt.rows()
     for r, d, yes in zip(rows, sh_dev, has_shadow):
         r.ema_shadow = d.data_ptr() if yes else None
+        r.grad_f32 = 1 if grad_f32 else 0
     table = C.c_void_p()
     L.check(L.lib().eri_adam8_table_create(rows, len(rows), None, C.byref(table)), "table_create")
     decays = [0.5, 0.999, 0.9]
-    all_g = [gs] + [hs.fresh_grads(sizes, bf16, 300 + k) for k in (1, 2)]
+    all_g = [gs] + [hs.fresh_grads(sizes, bf16 and not grad_f32, 300 + k) for k in (1, 2)]
     for k, d in enumerate(decays):
         if k:
             gt.set_grads(all_g[k])
         h = L.hyper_pack(LR, B1, B2, EPS, WD, k + 1, mode, L.FLAG_EXACT_PARAM | L.FLAG_EMA | extra)
         h.ema_decay = d
         L.check(L.lib().eri_adam8_step_table(table, C.byref(h), None), "step_table")
-        hs.oracle_step(ps, all_g[k], states, (LR, B1, B2, EPS, WD, k + 1), bf16, oc.MODE_BNB if mode == L.MODE_BNB else oc.MODE_ERI)
+        if grad_f32:
+            ho = oc.hyper_pack(LR, B1, B2, EPS, WD, k + 1)
+            for pa, ga, st in zip(ps, all_g[k], states):
+                assert oc.step_tensor(pa, ga, *st, ho, hs.MAPS, oc.DT_BF16, 4, g_dtype=oc.DT_F32) == 0
+        else:
+            hs.oracle_step(ps, all_g[k], states, (LR, B1, B2, EPS, WD, k + 1), bf16, oc.MODE_BNB if mode == L.MODE_BNB else oc.MODE_ERI)
         for i, n in enumerate(sizes):
             if has_shadow[i]:
                 oc.lib().eri_oracle_ema_update(oc.ptr(shadows[i]), oc.ptr(ps[i]), n, oc.DT_BF16 if bf16 else oc.DT_F32, d)

@@ -120,3 +120,74 @@ def test_results_on_the_edge_of_a_bf16_rounding_are_bit_exact(mode, wd, lr, p_st
     stats2 = hs.compare(got_p2, got_st2, ps, states, True, False, "near ties, default arithmetic")
     print("near-tie inputs: default arithmetic one bf16 step off on %d of %d" % (stats2["param_1ulp"], n), flush=True)
     L.lib().eri_adam8_table_destroy(table)
+
+
+def _update_fp32_l2(p16, g16, mc, vc, h):
+    """The functional update's fp32 update term before its rounding to bf16 (adam8bit.rs:113-196, one rounded
+    operation per line), from the state {codes mc, vc; every block's absmax A_M, A_V}."""
+    p = onp.bf16_to_f32(p16)
+    g = onp.bf16_to_f32(g16)
+    with np.errstate(all="ignore"):
+        if h.weight_decay > 0:
+            g = g + p * h.weight_decay
+        m = (hs.MAPS[0][mc] * A_M) * h.beta1 + g * h.omb1
+        v = (hs.MAPS[1][vc] * A_V) * h.beta2 + (g * g) * h.omb2
+        mh = m / h.bc1
+        vh = np.maximum(v / h.bc2, F32(0.0))
+        den = np.sqrt(vh) + h.eps
+        us = (mh / den) * h.step_size
+    return us.astype(F32)
+
+
+@pytest.mark.parametrize("kernels", ["default-kernels", "one-wave", "plain"])
+@pytest.mark.parametrize("wd,lr,step,spread", [(0.01, 1e-4, 7, 3), (0.0, 1e-3, 1, 3), (0.01, 1e-4, 40, 30)])
+def test_functional_updates_on_the_edge_of_a_bf16_rounding_are_bit_exact(wd, lr, step, spread, kernels):
+    """Mode L2 rounds the update itself to bf16 and decides by the low half of its fast chain's update whether the
+    exact chain has to be asked.  Tensors that consist of nothing but updates within `spread` fp32 patterns of a
+    bf16 tie point -- 3: where the two chains' roundings part; 30: on both sides of the edge of the window in
+    which the fast chain is not trusted -- must come out with the oracle's bits on every step kernel."""
+    import torch
+    from eridiffusion_amd import _lib as L
+    extra = {"default-kernels": 0, "one-wave": L.FLAG_ONE_WAVE, "plain": L.FLAG_NO_PIPELINE}[kernels]
+    n = 2048 * 3 + 40
+    key = ("l2", wd, lr, step, spread)
+    if key not in _found:
+        h = oc.hyper_pack(lr, 0.9, 0.999, 1e-8, wd, step, oc.MODE_L2)
+        hh = type("H", (), {k: F32(getattr(h, k)) for k in ("beta1", "beta2", "omb1", "omb2", "eps", "weight_decay", "step_size", "bc1", "bc2")})
+        rng = np.random.default_rng(500 + step)
+        keep, have = [[], [], [], []], 0
+        for _ in range(400):
+            k = 1 << 21
+            p16 = onp.f32_to_bf16((rng.standard_normal(k) * 0.02).astype(F32))
+            g16 = onp.f32_to_bf16((rng.standard_normal(k) * 1e-3).astype(F32))
+            mc = rng.integers(0, 256, k, dtype=np.uint8)
+            vc = rng.integers(0, 256, k, dtype=np.uint8)
+            us = _update_fp32_l2(p16, g16, mc, vc, hh)
+            low = (us.view(np.uint32) & 0xFFFF).astype(np.int32)
+            near = (np.abs(low - 0x8000) <= spread) & np.isfinite(us) & (np.abs(us) > F32(1e-30))
+            for dst, src in zip(keep, (p16, g16, mc, vc)):
+                dst.append(src[near])
+            have += int(near.sum())
+            if have >= n:
+                break
+        _found[key] = tuple(np.concatenate(x)[:n] for x in keep)
+    p16, g16, mc, vc = _found[key]
+    assert p16.size == n, "the search found too few near-tie updates"
+    sizes = [2048 * 2, 2048 + 40]
+    cut = sizes[0]
+    ps = [p16[:cut].copy(), p16[cut:].copy()]
+    gs = [g16[:cut].copy(), g16[cut:].copy()]
+    states = [[mc[:cut].copy(), vc[:cut].copy(), np.full(2, A_M, F32), np.full(2, A_V, F32)],
+              [mc[cut:].copy(), vc[cut:].copy(), np.full(2, A_M, F32), np.full(2, A_V, F32)]]
+    gt = hs.GpuTensors(ps, gs, states, True)
+    rows = gt.rows()
+    table = C.c_void_p()
+    L.check(L.lib().eri_adam8_table_create(rows, len(rows), None, C.byref(table)), "table_create")
+    h = L.hyper_pack(lr, 0.9, 0.999, 1e-8, wd, step, L.MODE_L2, L.FLAG_EXACT_PARAM | extra)
+    L.check(L.lib().eri_adam8_step_table(table, C.byref(h), None), "step_table")
+    torch.cuda.synchronize()
+    hs.oracle_step(ps, gs, states, (lr, 0.9, 0.999, 1e-8, wd, step), True, oc.MODE_L2)
+    got_p, got_st = gt.fetch()
+    stats = hs.compare(got_p, got_st, ps, states, True, True, "near ties, functional update")
+    assert stats["code_mismatch"] == 0
+    L.lib().eri_adam8_table_destroy(table)

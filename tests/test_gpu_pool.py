@@ -181,8 +181,8 @@ def test_released_pieces_are_handed_out_again():
 
 
 def test_loading_a_checkpoint_again_does_not_grow_the_state_lane(tmp_path):
-    """States that are replaced go back to the pool and the next load takes them: the lane holds two sets of states
-    after the first load into an optimizer that has stepped, and not a byte more after the second and third."""
+    """States that are replaced go back to the pool and the next load takes them: however often a checkpoint is
+    loaded into an optimizer that has stepped, the lane never holds more than two sets of states."""
     import torch
     from eridiffusion_amd.adam8bit import Adam8bit, Adam8bitConfig, DevicePool
     L = _L()
@@ -208,8 +208,67 @@ def test_loading_a_checkpoint_again_does_not_grow_the_state_lane(tmp_path):
         opt.load_state(path)
         L.check(L.lib().eri_hip_pool_lane_used(pool._pool, 1, C.byref(used)), "lane_used")
         levels.append(used.value)
-    assert levels[0] <= 2 * one_set and levels[1] == levels[0] and levels[2] == levels[0]
+    # a load builds the new states before it lets the old ones go (a load that fails changes nothing), so the
+    # lane holds two sets at most; each load takes the pieces the load before it gave back
+    assert max(levels) <= 2 * one_set and levels[2] == levels[0]
     opt.step()  # the loaded states are the ones that step
     torch.cuda.synchronize()
-    del opt
+    # the pool's creator lets go first: the states keep the allocation alive and still return their pieces
+    raw = C.c_void_p(pool._pool.value)
     pool.close()
+    assert L.lib().eri_hip_pool_alloc_zeroed(raw, 0, 256, C.byref(C.c_void_p())) == -6  # alive, but hands out nothing more
+    assert b"destroyed" in L.lib().eri_last_error()
+    del opt
+
+
+def test_parameters_and_gradients_in_lane_0_states_in_lane_2():
+    """What a tensor runtime gets by backing its allocator with the pool and choosing the lane by dtype alone (U8 into
+    lane 2, everything else into lane 0): parameters and gradients share a lane, the optimizer's states lie two
+    lanes away.  The step over such a placement is checked against the oracle like any other, and the pieces are
+    cleared on the optimizer's stream."""
+    import torch
+    L = _L()
+    sizes = [2048 * 6 + 40, 4096, 333, 2048 * 3]
+    ps, gs = hs.make_inputs(sizes, True, 8088)
+    states = hs.oracle_states(sizes)
+    stream = torch.cuda.current_stream().cuda_stream
+    pool = _pool(96 * MiB, 3)
+    lanes, lane_bytes = C.c_uint32(), C.c_size_t()
+    L.check(L.lib().eri_hip_pool_info(pool, C.byref(lanes), C.byref(lane_bytes)), "pool_info")
+
+    def place(lane, arr):
+        out = C.c_void_p()
+        L.check(L.lib().eri_hip_pool_alloc_zeroed_async(pool, lane, arr.nbytes, stream, C.byref(out)), "alloc_async")
+        L.check(L.lib().eri_hip_memcpy_async(out, arr.ctypes.data, arr.nbytes, 1, stream), "h2d")
+        return out.value
+
+    rows = (L.TensorRow * len(sizes))()
+    start = 0
+    first = None
+    for i, n in enumerate(sizes):
+        r = rows[i]
+        r.p, r.g = place(0, ps[i]), place(0, gs[i])               # BF16: lane 0
+        r.m, r.v = place(2, states[i][0]), place(2, states[i][1])  # U8: lane 2
+        r.absmax_m, r.absmax_v = place(2, states[i][2]), place(2, states[i][3])
+        r.numel, r.block_start, r.dtype_tag, r.grad_scale = n, start, L.DTYPE_BF16, 1.0
+        start += (n + 2047) // 2048
+        first = first or r.p
+        assert first <= r.p < first + lane_bytes.value and first <= r.g < first + lane_bytes.value
+        assert first + 2 * lane_bytes.value <= r.m < first + 3 * lane_bytes.value
+    L.check(L.lib().eri_hip_stream_sync(stream), "sync")  # the host arrays above were pageable
+    table = C.c_void_p()
+    L.check(L.lib().eri_adam8_table_create(rows, len(rows), stream, C.byref(table)), "table_create")
+    for t in (1, 2):
+        h = L.hyper_pack(LR, B1, B2, EPS, WD, t, L.MODE_ERI, L.FLAG_EXACT_PARAM)
+        L.check(L.lib().eri_adam8_step_table(table, C.byref(h), stream), "step_table")
+        hs.oracle_step(ps, gs, states, (LR, B1, B2, EPS, WD, t), True)
+    L.check(L.lib().eri_hip_stream_sync(stream), "sync")
+    for i, n in enumerate(sizes):
+        for ptr, want in ((rows[i].p, ps[i]), (rows[i].m, states[i][0]), (rows[i].v, states[i][1]),
+                          (rows[i].absmax_m, states[i][2]), (rows[i].absmax_v, states[i][3])):
+            got = np.empty_like(want)
+            L.check(L.lib().eri_hip_memcpy_async(got.ctypes.data, ptr, got.nbytes, 2, stream), "d2h")
+            L.check(L.lib().eri_hip_stream_sync(stream), "sync")
+            assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), i
+    L.lib().eri_adam8_table_destroy(table)
+    L.check(L.lib().eri_hip_pool_destroy(pool), "destroy")

@@ -5,6 +5,7 @@ import ctypes as C
 import numpy as np
 import pytest
 
+import harness as hs
 import oracle_c as oc
 from oracle import adam8_numpy as onp
 
@@ -226,3 +227,40 @@ def test_quantize_dequantize_with_extreme_values():
         assert np.array_equal(codes.cpu().numpy(), wc), signed
         assert np.array_equal(absmax.cpu().numpy().view(np.uint32), wa.view(np.uint32)), signed
         assert _same_bits_nan_aware(back.cpu().numpy(), wb, False), signed
+
+
+def test_traffic_probe_moves_the_bytes_and_changes_none():
+    """eri_adam8_traffic_probe reads and rewrites every full block of the BF16 rows as the step does, with the
+    bits they had: parameters, gradients, codes and absmax are unchanged afterwards (guard bands included), a
+    table without such rows and a gradient-only table are refused."""
+    import ctypes as C
+    import torch
+    from eridiffusion_amd import _lib as L
+    sizes = [2048 * 7 + 99, 2048 * 2, 100, 2048 * 33]
+    ps, gs = hs.make_inputs(sizes, True, 606)
+    states = hs.oracle_states(sizes)
+    hs.oracle_step(ps, gs, states, (1e-4, 0.9, 0.999, 1e-8, 0.01, 1), True)  # states with real contents
+    want_p = [p.copy() for p in ps]
+    gt = hs.GpuTensors(ps, gs, states, True)
+    rows = gt.rows()
+    table = C.c_void_p()
+    L.check(L.lib().eri_adam8_table_create(rows, len(rows), None, C.byref(table)), "table_create")
+    for _ in range(3):
+        L.check(L.lib().eri_adam8_traffic_probe(table, None), "traffic_probe")
+    torch.cuda.synchronize()
+    got_p, got_st = gt.fetch()
+    for i in range(len(sizes)):
+        assert np.array_equal(got_p[i], want_p[i]), i
+        for k in range(4):
+            assert np.array_equal(got_st[i][k].view(np.uint8), states[i][k].view(np.uint8)), (i, k)
+        assert np.array_equal(gt.down(gt.g[i]), gs[i]), i
+    L.lib().eri_adam8_table_destroy(table)
+    # fp32 rows only: nothing for the probe
+    ps32, gs32 = hs.make_inputs([4096], False, 607)
+    gt32 = hs.GpuTensors(ps32, gs32, hs.oracle_states([4096]), False)
+    rows32 = gt32.rows()
+    t32 = C.c_void_p()
+    L.check(L.lib().eri_adam8_table_create(rows32, 1, None, C.byref(t32)), "table_create")
+    assert L.lib().eri_adam8_traffic_probe(t32, None) == -6
+    L.lib().eri_adam8_table_destroy(t32)
+    assert L.lib().eri_adam8_traffic_probe(None, None) == -1
