@@ -384,8 +384,8 @@ def measure(args, torch, separate_events=False):
             obj_params.append(hnd)
         obj_opt = C.c_void_p()
         L.check(L.lib().eri_adam8bit_new(handles, len(sizes), C.byref(cfg), stream, C.byref(obj_opt)), "adam8bit_new")
-        if args.flags:
-            L.check(L.lib().eri_adam8bit_set_flags(obj_opt, args.flags), "set_flags")
+        # the object starts with ERI_ADAM8_FLAG_EXACT_PARAM; the bench times what --flags says, as for the table
+        L.check(L.lib().eri_adam8bit_set_flags(obj_opt, args.flags), "set_flags")
         if alloc == "pool":  # the optimizer's own states out of the state lane
             L.check(L.lib().eri_adam8bit_set_state_pool(obj_opt, Pool.handle, LANE_STATE), "set_state_pool")
     elif args.api != "table":

@@ -87,7 +87,7 @@ class Adam8bitConfig:
 class Adam8bit:
     """`step()` over a list of tensors that carry their gradients in `.grad`."""
 
-    def __init__(self, params: List[torch.Tensor], config: Optional[Adam8bitConfig] = None, flags: int = 0):
+    def __init__(self, params: List[torch.Tensor], config: Optional[Adam8bitConfig] = None, flags: Optional[int] = None):
         config = config or Adam8bitConfig()
         self.params = list(params)
         for p in self.params:
@@ -103,7 +103,7 @@ class Adam8bit:
         self._opt = C.c_void_p()
         check(lib().eri_adam8bit_new(self._handles, len(self.params), C.byref(cfg), _stream_ptr(),
                                      C.byref(self._opt)), "eri_adam8bit_new")
-        if flags:
+        if flags is not None:  # None keeps the library's default, FLAG_EXACT_PARAM; 0 selects the faster arithmetic
             check(lib().eri_adam8bit_set_flags(self._opt, flags), "eri_adam8bit_set_flags")
         if config.min_8bit_size:
             check(lib().eri_adam8bit_set_min_8bit_size(self._opt, config.min_8bit_size), "eri_adam8bit_set_min_8bit_size")

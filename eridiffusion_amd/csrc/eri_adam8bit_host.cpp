@@ -399,7 +399,8 @@ struct EriAdam8bit {
     std::vector<EriParameter *> params;
     double lr = 1e-3, beta1 = 0.9, beta2 = 0.999, eps = 1e-8, wd = 0.01;
     uint64_t step = 0;
-    uint32_t flags = 0;
+    // bf16 parameters come out with the reference's bits unless the caller trades that for the last 0.6-0.9 %
+    uint32_t flags = ERI_ADAM8_FLAG_EXACT_PARAM;
     int mode = ERI_ADAM8_MODE_ERI;
     float grad_scale = 1.0f;
     float max_grad_norm = 0.0f, clip_denom_eps = 0.0f;

@@ -122,7 +122,9 @@ unsafe impl Send for Adam8bit {}
 unsafe impl Sync for Adam8bit {}
 
 impl Adam8bit {
-    /// adam8bit_enhanced.rs:161
+    /// adam8bit_enhanced.rs:161.  The object starts in the arithmetic that reproduces the reference's bf16
+    /// parameters bit for bit (ERI_ADAM8_FLAG_EXACT_PARAM); `eri_adam8bit_set_flags(opt, 0)` trades that for
+    /// under one per cent of step time.
     pub fn new(params: Vec<Parameter>, config: Adam8bitConfig) -> Result<Self> {
         let mut handles = Vec::with_capacity(params.len());
         let mut stream: *mut c_void = std::ptr::null_mut();

@@ -153,11 +153,11 @@ enum {
     ERI_ADAM8_FLAG_EMA = 1u << 6,         /* after the update, every row that has an ema_shadow also gets
                                              shadow = ema_decay*shadow + (1 - ema_decay)*p', the EMA update of
                                              src/trainers/ema_enhanced.rs:91-100 on the parameter as it was just
-                                             stored.  BF16 tables in mode ERI beyond the small-table kernel's
-                                             range do it inside the step kernel (the new parameter is still in
-                                             registers: the separate sweep's read of p is saved); every other
-                                             table runs the EMA sweep right after the step, in the same call.
-                                             Same results either way */
+                                             stored.  Tables of BF16 parameters (BF16 or F32 gradients) in mode
+                                             ERI beyond the small-table kernel's range do it inside the step
+                                             kernel (the new parameter is still in registers: the separate
+                                             sweep's read of p is saved); every other table runs one EMA sweep
+                                             right after the step, in the same call.  Same results either way */
     ERI_ADAM8_FLAG_ONE_WAVE = 1u << 5     /* take the kernel of the largest tables whatever the size: one
                                              wave per block with the next block's loads in flight.  Same
                                              results; lets tests reach every kernel with small inputs */
