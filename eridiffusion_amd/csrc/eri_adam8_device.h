@@ -104,7 +104,7 @@ int launch_step_plain_bf16(int mode, bool exact, bool wd, bool gs, bool keytab, 
 /* Four waves per block, for tables of few blocks; `grid` workgroups of 1024 threads. */
 int launch_step_split(int layout, int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
                       uint32_t total_blocks, const EriAdam8Hyper &h, const void *lds_image, const float *dev_scale,
-                      uint32_t grid, void *stream);
+                      uint32_t grid, uint32_t teams, void *stream);
 /* Whether launch_step would run this group on the prefetching kernel with the EMA update inside it. */
 bool step_fuses_ema(uint32_t total_full_blocks, int layout, const EriAdam8Hyper &h, uint32_t compute_units);
 int launch_step_pipelined(int mode, bool exact, bool wd, bool gs, bool ema, const DevTensor *rows, uint32_t n_rows,

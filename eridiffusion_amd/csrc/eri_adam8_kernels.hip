@@ -39,12 +39,17 @@ int launch_step(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, i
         const bool bnb = h.mode == ERI_ADAM8_MODE_BNB;
         const bool wd_s = bnb ? h.weight_decay != 1.0f : h.weight_decay > 0.0f;
         const bool exact_s = !bf16 || (h.flags & ERI_ADAM8_FLAG_EXACT_PARAM) != 0;
-        uint32_t need = (total_blocks + 3) / 4;
+        // Up to four blocks per workgroup at a time (a team of four waves each), but no more than it takes to
+        // give every compute unit a workgroup: 512 blocks on 256 units run as 256 workgroups of two teams.
+        uint32_t teams = (total_blocks + compute_units - 1) / compute_units;
+        teams = teams < 1 ? 1 : teams > 4 ? 4 : teams;
+        uint32_t need = (total_blocks + teams - 1) / teams;
         const uint32_t for_tails = (n_rows + 15) / 16;
         if (need < for_tails) need = for_tails;
         if (need > compute_units) need = compute_units;
         if (need == 0) need = 1;
-        return launch_step_split(layout, h.mode, exact_s, wd_s, gs, rows, n_rows, total_blocks, h, lds_image, dev_scale, need, stream);
+        return launch_step_split(layout, h.mode, exact_s, wd_s, gs, rows, n_rows, total_blocks, h, lds_image, dev_scale, need,
+                                 teams, stream);
     }
     if (mixed) {
         const bool wd_m = h.mode == ERI_ADAM8_MODE_BNB ? h.weight_decay != 1.0f : h.weight_decay > 0.0f;

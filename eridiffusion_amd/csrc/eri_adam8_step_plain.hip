@@ -22,7 +22,7 @@ template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB, bool G
 __global__ __launch_bounds__(plain_threads(MODE)) void adam8_step_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
                                                           uint32_t total_blocks, EriAdam8Hyper h_in,
                                                           const uint4 *__restrict__ lds_image,
-                                                          const float *__restrict__ dev_scale, uint32_t chunks) {
+                                                          const float *__restrict__ dev_scale) {
     ERI_LDS_IMAGE;
     __shared__ float decayed[16][2][256]; // per wave: the values its block's state codes stand for, decayed
     const StepHyper h = make_step_hyper<MODE>(h_in);
@@ -47,10 +47,20 @@ __global__ __launch_bounds__(plain_threads(MODE)) void adam8_step_kernel(const D
     const uint32_t stride = gridDim.x * waves_per_wg;
     const BlockDiv dbc1(h.bc1), dbc2(h.bc2);
 
-    // partial last blocks first: one per row at most, handed out from the last wave backwards -- the
-    // waves at the end of each range are the ones that get one full block fewer when the blocks do not
-    // divide evenly, so the slower element-wise tail lands where there is slack
-    for (uint32_t r = stride - 1 - wave; r < n_rows; r += stride) {
+    // Full blocks: round k gives wave w block k * stride + w, and the blocks left over when the list does not
+    // divide (fewer than one per wave) go one to each workgroup in turn -- workgroup i takes left-over blocks
+    // i, i + grid, i + 2 grid, ... on its first waves -- so that the short last round runs on every compute
+    // unit instead of filling the first few (2-3 % of the launch on tables of 5-20 blocks per wave).
+    const uint32_t wave_in_wg = threadIdx.x / kWave;
+    const uint32_t rounds = total_blocks / stride;
+    const uint32_t left_first = rounds * stride;
+    const uint32_t left_mine = wave_in_wg * gridDim.x + blockIdx.x;
+    const bool has_left = left_first + left_mine < total_blocks;
+
+    // partial last blocks first: one per row at most, one to each workgroup in turn, from a workgroup's last
+    // wave backwards: those are the waves without a left-over block, so the slower element-wise tail lands
+    // where there is slack
+    for (uint32_t r = blockIdx.x + (waves_per_wg - 1 - wave_in_wg) * gridDim.x; r < n_rows; r += stride) {
         const DevTensor t = rows[r];
         const uint32_t n = (uint32_t)(t.numel % kBlock);
         if (n != 0) {
@@ -61,8 +71,9 @@ __global__ __launch_bounds__(plain_threads(MODE)) void adam8_step_kernel(const D
     uint32_t ti = 0, t_end = 0;
     DevTensor t;
     const BlockRowMap map(rows, n_rows);
-    const BlockWalk walk(total_blocks, chunks);
-    for (uint32_t blk = walk.first; blk < walk.end; blk += walk.stride) {
+    const uint32_t trips = rounds + (has_left ? 1u : 0u);
+    for (uint32_t k = 0; k < trips; ++k) {
+        const uint32_t blk = k < rounds ? k * stride + wave : left_first + left_mine;
         map.seek(rows, blk, ti, t, t_end);
         const float gscale = GS ? (h.grad_scale * t.grad_scale) * tscale : 1.0f;
         full_block<BF16, MODE, EXACT, WD, GS, KEYTAB, GBF16>(t, blk - t.full_start, lane, h, gscale, dbc1, dbc2, L,
@@ -79,11 +90,11 @@ int launch_one(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, co
                const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg, hipStream_t s) {
     auto k = adam8_step_kernel<kBf16, MODE, EXACT, WD, GS, KEYTAB, GBF16>;
     if (wg > plain_threads(MODE)) wg = plain_threads(MODE);
-    // One common window for all dies (the plain grid-stride walk): on the tables this kernel takes, up to 1,024
+    // One common window for all dies (a grid-stride walk): on the tables this kernel takes, up to 1,024
     // blocks per compute unit, it measured 2 % ahead of one range per die with the arrays far apart in device
     // memory and 5 % with them adjacent; the tables of the prefetching kernel want the ranges.
     hipLaunchKernelGGL(k, dim3(grid), dim3(wg), 0, s, rows, n_rows, total_blocks, h,
-                       static_cast<const uint4 *>(lds_image), dev_scale, 1u);
+                       static_cast<const uint4 *>(lds_image), dev_scale);
     return (int)hipGetLastError();
 }
 

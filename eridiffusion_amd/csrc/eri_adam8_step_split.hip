@@ -7,7 +7,8 @@
  * as one wave's trip through one block.  Here a block is cut into four 512-element quarters, one per
  * wave; the block's absmax is the maximum of the four wave maxima (DPP inside the wave, then four floats
  * through LDS and one workgroup barrier), after which every wave requantises its own quarter.  A
- * workgroup is four such teams (1024 threads), so the table image is staged into LDS once per four blocks.
+ * workgroup is four such teams (1024 threads), so the table image is staged into LDS once per four blocks;
+ * a table with fewer blocks than four per compute unit uses `teams` < 4 of them, in more workgroups.
  * Arithmetic, rounding and results are those of the other two kernels.
  */
 #include "eri_adam8_inline.h"
@@ -18,7 +19,7 @@ template <bool BF16, bool GBF16, int MODE, bool EXACT, bool WD, bool GS>
 __global__ __launch_bounds__(1024) void adam8_step_split_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
                                                                 uint32_t total_blocks, EriAdam8Hyper h_in,
                                                                 const uint4 *__restrict__ lds_image,
-                                                                const float *__restrict__ dev_scale) {
+                                                                const float *__restrict__ dev_scale, uint32_t teams) {
     ERI_LDS_IMAGE;
     const StepHyper h = make_step_hyper<MODE>(h_in);
     __shared__ float wave_maxima[2][4][8]; // [parity of the iteration][team][4 x first, 4 x second moment]
@@ -47,7 +48,7 @@ __global__ __launch_bounds__(1024) void adam8_step_split_kernel(const DevTensor 
     const BlockRowMap map(rows, n_rows);
     auto request = [&](uint32_t first) {
         const uint32_t blk = first + team;
-        q.active = blk < total_blocks;
+        q.active = team < teams && blk < total_blocks;
         if (!q.active) return;
         map.seek(rows, blk, ti, q.t, t_end);
         q.lb = blk - q.t.full_start;
@@ -60,7 +61,7 @@ __global__ __launch_bounds__(1024) void adam8_step_split_kernel(const DevTensor 
         q.a_m = as_global(q.t.absmax_m)[q.lb];
         q.a_v = as_global(q.t.absmax_v)[q.lb];
     };
-    request(blockIdx.x * 4);
+    request(blockIdx.x * teams);
 
     for (uint32_t i = threadIdx.x; i < kLdsImageBytes / 16; i += blockDim.x) lds_raw[i] = lds_image[i];
     __syncthreads();
@@ -90,7 +91,7 @@ __global__ __launch_bounds__(1024) void adam8_step_split_kernel(const DevTensor 
 
     uint32_t parity = 0;
     // every wave of the workgroup runs the same number of iterations: the barrier is inside the loop
-    for (uint32_t first = blockIdx.x * 4; first < total_blocks; first += gridDim.x * 4, parity ^= 1) {
+    for (uint32_t first = blockIdx.x * teams; first < total_blocks; first += gridDim.x * teams, parity ^= 1) {
         float m[8], v[8];
         float nam = 0.0f, nav = 0.0f;
         // the quarter at hand; q itself is handed to the next request as soon as its raw words are used up
@@ -139,7 +140,7 @@ __global__ __launch_bounds__(1024) void adam8_step_split_kernel(const DevTensor 
         }
         __syncthreads();
         // the next quarter's loads travel while this one is requantised
-        const uint32_t next = first + gridDim.x * 4;
+        const uint32_t next = first + gridDim.x * teams;
         if (next < total_blocks) request(next);
         else q.active = false;
         if (active) {
@@ -165,11 +166,11 @@ namespace {
 
 template <bool BF16, bool GBF16, int MODE, bool EXACT>
 int launch_flags(bool wd, bool gs, const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
-                 const void *img, const float *dev_scale, uint32_t grid, hipStream_t s) {
+                 const void *img, const float *dev_scale, uint32_t grid, uint32_t teams, hipStream_t s) {
 #define ERI_GO(W, G)                                                                                                     \
     do {                                                                                                                 \
         hipLaunchKernelGGL((adam8_step_split_kernel<BF16, GBF16, MODE, EXACT, W, G>), dim3(grid), dim3(1024), 0, s, rows, n_rows, \
-                           total_blocks, h, static_cast<const uint4 *>(img), dev_scale);                                  \
+                           total_blocks, h, static_cast<const uint4 *>(img), dev_scale, teams);                           \
         return (int)hipGetLastError();                                                                                   \
     } while (0)
     if (wd) { if (gs) ERI_GO(true, true); ERI_GO(true, false); }
@@ -182,9 +183,9 @@ int launch_flags(bool wd, bool gs, const DevTensor *rows, uint32_t n_rows, uint3
 
 int launch_step_split(int layout, int mode, bool exact, bool wd, bool gs, const DevTensor *rows, uint32_t n_rows,
                       uint32_t total_blocks, const EriAdam8Hyper &h, const void *img, const float *dev_scale, uint32_t grid,
-                      void *stream) {
+                      uint32_t teams, void *stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
-#define ERI_ARGS wd, gs, rows, n_rows, total_blocks, h, img, dev_scale, grid, s
+#define ERI_ARGS wd, gs, rows, n_rows, total_blocks, h, img, dev_scale, grid, teams, s
     if (layout == kLayoutF32) { // fp32 parameters always take the IEEE square root and division
         if (mode == ERI_ADAM8_MODE_BNB) return launch_flags<false, false, ERI_ADAM8_MODE_BNB, true>(ERI_ARGS);
         if (mode == ERI_ADAM8_MODE_L2) return launch_flags<false, false, ERI_ADAM8_MODE_L2, true>(ERI_ARGS);
