@@ -80,6 +80,7 @@ EXPORTS = {
     "eri_hip_stream_sync": (C.c_int, [C.c_void_p]),
     "eri_hip_stream_destroy": (C.c_int, [C.c_void_p]),
     "eri_hip_mem_info": (C.c_int, [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
+    "eri_hip_pointer_kind": (C.c_int, [C.c_void_p, C.POINTER(C.c_int)]),
     "eri_hip_pool_create": (C.c_int, [C.c_int, C.c_size_t, C.c_uint32, C.POINTER(C.c_void_p)]),
     "eri_hip_pool_alloc_zeroed": (C.c_int, [C.c_void_p, C.c_uint32, C.c_size_t, C.POINTER(C.c_void_p)]),
     "eri_hip_pool_alloc_zeroed_async": (C.c_int, [C.c_void_p, C.c_uint32, C.c_size_t, C.c_void_p, C.POINTER(C.c_void_p)]),

@@ -773,6 +773,39 @@ int eri_hip_mem_info(size_t *free_bytes, size_t *total_bytes) {
     return 0;
 }
 
+int eri_hip_pointer_kind(const void *p, int *kind) {
+    if (!kind) return fail(ERI_ERR_NULL, "kind is NULL");
+    *kind = ERI_PTR_UNKNOWN;
+    if (!p) return 0;
+    hipPointerAttribute_t a;
+    std::memset(&a, 0, sizeof a);
+    const hipError_t e = hipPointerGetAttributes(&a, p);
+    if (e == hipErrorInvalidValue) { // how older runtimes answer for memory they did not allocate
+        (void)hipGetLastError();
+        return 0;
+    }
+    if (e != hipSuccess) return hip_fail(e, "hipPointerGetAttributes");
+    switch (a.type) {
+    case hipMemoryTypeDevice: case hipMemoryTypeArray: *kind = ERI_PTR_DEVICE; break;
+    case hipMemoryTypeHost: *kind = ERI_PTR_PINNED_HOST; break;
+    case hipMemoryTypeManaged: case hipMemoryTypeUnified: *kind = ERI_PTR_MANAGED; break;
+    default: *kind = ERI_PTR_UNKNOWN; break;
+    }
+    return 0;
+}
+
+/* The checkpoint calls below run a kernel on pointers that come straight from a caller who is often handling
+ * host buffers at that moment; ordinary host memory handed to a kernel is a memory fault of the whole device,
+ * so these calls (none of them is on a step's path) ask the runtime first. */
+static int require_kernel_visible(const void *p, const char *what) {
+    int kind = ERI_PTR_UNKNOWN;
+    const int rc = eri_hip_pointer_kind(p, &kind);
+    if (rc) return rc;
+    if (kind == ERI_PTR_UNKNOWN)
+        return fail(ERI_ERR_ARG, std::string(what) + " is not device, pinned or managed memory: kernels cannot reach it");
+    return 0;
+}
+
 // ---- optimizer ------------------------------------------------------------------------------
 
 int eri_adam8_init(void) {
@@ -1226,6 +1259,9 @@ int eri_adam8_dequantize(const uint8_t *codes, const float *absmax, int signed_m
     DeviceCtx *ctx = nullptr;
     int rc = get_ctx(&ctx);
     if (rc) return rc;
+    if ((rc = require_kernel_visible(codes, "dequantize: codes")) != 0) return rc;
+    if ((rc = require_kernel_visible(absmax, "dequantize: absmax")) != 0) return rc;
+    if ((rc = require_kernel_visible(out, "dequantize: out")) != 0) return rc;
     rc = eri::launch_dequantize(codes, absmax, signed_map, numel, out, ctx->image, stream);
     if (rc) return hip_fail((hipError_t)rc, "dequantize launch");
     return 0;
@@ -1237,6 +1273,9 @@ int eri_adam8_quantize(const float *x, int signed_map, uint64_t numel, uint8_t *
     DeviceCtx *ctx = nullptr;
     int rc = get_ctx(&ctx);
     if (rc) return rc;
+    if ((rc = require_kernel_visible(x, "quantize: x")) != 0) return rc;
+    if ((rc = require_kernel_visible(codes, "quantize: codes")) != 0) return rc;
+    if ((rc = require_kernel_visible(absmax, "quantize: absmax")) != 0) return rc;
     rc = eri::launch_quantize(x, signed_map, numel, codes, absmax, ctx->image, stream);
     if (rc) return hip_fail((hipError_t)rc, "quantize launch");
     return 0;

@@ -83,6 +83,8 @@ extern "C" {
     pub fn eri_hip_stream_sync(stream: *mut c_void) -> c_int;
     pub fn eri_hip_stream_destroy(stream: *mut c_void) -> c_int;
     pub fn eri_hip_mem_info(free_bytes: *mut usize, total_bytes: *mut usize) -> c_int;
+    /// 0 = memory the runtime never allocated, 1 = pinned host, 2 = device, 3 = managed
+    pub fn eri_hip_pointer_kind(p: *const c_void, kind: *mut c_int) -> c_int;
     pub fn eri_hip_pool_create(device: c_int, bytes: usize, lanes: u32, out: *mut *mut EriHipPool) -> c_int;
     pub fn eri_hip_pool_alloc_zeroed(pool: *mut EriHipPool, lane: u32, bytes: usize, out: *mut *mut c_void) -> c_int;
     pub fn eri_hip_pool_alloc_zeroed_async(pool: *mut EriHipPool, lane: u32, bytes: usize, stream: *mut c_void, out: *mut *mut c_void) -> c_int;

@@ -185,7 +185,9 @@ uint64_t eri_adam8bit_fn_get_step(const EriAdam8bitFn *opt);    /* :311-313 */
 /* memory_stats() :253-266: number of named states and their bytes */
 int eri_adam8bit_fn_memory_stats(const EriAdam8bitFn *opt, uint64_t *num_params, uint64_t *bytes);
 /* get_state_as_tensors / load_state_from_tensors :296-329, one name at a time: fp32 moments.
- * `numel` of an unknown name reads 0. */
+ * `numel` of an unknown name reads 0.  m_out / v_out and m / v are DEVICE buffers of numel floats (the
+ * reference hands out and takes device tensors): the conversion runs on the optimizer's stream, and the
+ * buffers are valid in stream order; ordinary host memory is refused (ERI_ERR_ARG). */
 int eri_adam8bit_fn_state_numel(const EriAdam8bitFn *opt, const char *name, uint64_t *numel);
 int eri_adam8bit_fn_get_state_fp32(EriAdam8bitFn *opt, const char *name, float *m_out, float *v_out);
 int eri_adam8bit_fn_load_state_fp32(EriAdam8bitFn *opt, const char *name, const float *m, const float *v,

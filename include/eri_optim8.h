@@ -77,6 +77,13 @@ int eri_hip_stream_create(void **stream);                        /* default prio
 int eri_hip_stream_sync(void *stream);
 int eri_hip_stream_destroy(void *stream);
 int eri_hip_mem_info(size_t *free_bytes, size_t *total_bytes);
+/* What the runtime knows about an address: memory it never allocated (malloc, the stack, a mapped file) is
+ * ERI_PTR_UNKNOWN, and a kernel that touches it faults the device.  The calls that take device pointers from
+ * code which is usually holding host buffers at that moment (eri_adam8_quantize / _dequantize and the
+ * optimizer calls built on them) ask this first and refuse with ERI_ERR_ARG; the step's own calls do not (their
+ * tables hold thousands of pointers and are rebuilt on a trainer's hot path). */
+enum { ERI_PTR_UNKNOWN = 0, ERI_PTR_PINNED_HOST = 1, ERI_PTR_DEVICE = 2, ERI_PTR_MANAGED = 3 };
+int eri_hip_pointer_kind(const void *p, int *kind);
 
 /* A device memory pool with lanes: ONE device allocation cut into `lanes` equal parts, each handing out
  * 256-byte aligned, zero-filled pieces from its start upwards.  It exists for placement.  On MI355X a kernel
@@ -314,7 +321,8 @@ int eri_adam8_table_image(void *out, size_t cap, size_t *bytes, uint32_t offsets
 
 /* Blockwise state <-> fp32, for checkpoints that store unquantised moments
  * (get_state_as_tensors / load_state_from_tensors, src/trainers/adam8bit.rs:296-329).
- * signed_map != 0 selects the first-moment map. */
+ * signed_map != 0 selects the first-moment map.  Every pointer is memory a kernel can reach (device, pinned
+ * host or managed): the conversion runs on the device, on `stream`; ordinary host memory is refused. */
 int eri_adam8_dequantize(const uint8_t *codes, const float *absmax, int signed_map, uint64_t numel,
                          float *out, void *stream);
 int eri_adam8_quantize(const float *x, int signed_map, uint64_t numel, uint8_t *codes, float *absmax,

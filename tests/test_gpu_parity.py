@@ -533,6 +533,17 @@ def test_randomized_extreme_values_against_the_oracle():
         assert stats["code_mismatch"] == 0, case
 
 
+@pytest.mark.parametrize("blocks", [255, 257, 513, 768, 769, 1300])
+def test_tables_around_the_team_counts_of_the_small_table_kernel(blocks):
+    """The four-waves-per-block kernel runs a table of up to one, two, three blocks per compute unit with that many
+    teams per workgroup and anything larger with four; the block counts here sit on both sides of each change (256
+    units).  Three ragged tensors, bf16 and fp32."""
+    a = blocks // 3
+    sizes = [2048 * a + 5, 2048 * (blocks - 2 * a), 2048 * a + 2047]
+    for bf16 in (True, False):
+        run_case(sizes, bf16, 600 + blocks, steps=2, flags=2, label="teams-%d-%s" % (blocks, "bf16" if bf16 else "f32"))
+
+
 def test_five_thousand_small_tensors_in_one_launch():
     """A long launch table: 5,000 tensors of 1 to 6,000 elements (most of them nothing but a partial
     block), both through the table handle and through step_multi."""

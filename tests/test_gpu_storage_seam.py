@@ -108,3 +108,46 @@ def test_table_update_points_the_same_table_at_new_buffers():
     rows[1].numel = 500
     L.check(L.lib().eri_adam8_table_update(table, rows, len(rows), stream), "table_update")
     L.lib().eri_adam8_table_destroy(table)
+
+
+def test_checkpoint_conversions_refuse_memory_a_kernel_cannot_reach():
+    """eri_hip_pointer_kind tells ordinary host memory from pinned host and device memory, and the calls that
+    convert optimizer state to and from fp32 refuse the first kind before any kernel is launched (the refusals
+    are only attempted after the runtime has shown that it tells the kinds apart)."""
+    import torch
+    L = _L()
+    lib = L.lib()
+    n = 2048 * 3 + 17
+    nb = (n + 2047) // 2048
+    dev_x = torch.randn(n, device="cuda:0")
+    dev_codes = torch.empty(n, dtype=torch.uint8, device="cuda:0")
+    dev_absmax = torch.empty(nb, dtype=torch.float32, device="cuda:0")
+    dev_out = torch.empty(n, device="cuda:0")
+    host = np.zeros(n, np.float32)
+    lib.eri_hip_host_alloc.restype = C.c_void_p
+    pinned = lib.eri_hip_host_alloc(4 * n)
+    assert pinned
+
+    def kind(p):
+        k = C.c_int(-1)
+        L.check(lib.eri_hip_pointer_kind(C.c_void_p(p), C.byref(k)), "pointer_kind")
+        return k.value
+
+    assert kind(host.ctypes.data) == 0
+    assert kind(pinned) == 1
+    assert kind(dev_x.data_ptr()) == 2 and kind(dev_x.data_ptr() + 4 * 1000) == 2
+    assert kind(None) == 0
+
+    stream = torch.cuda.current_stream().cuda_stream
+    x, codes, absmax, out = dev_x.data_ptr(), dev_codes.data_ptr(), dev_absmax.data_ptr(), dev_out.data_ptr()
+    L.check(lib.eri_adam8_quantize(x, 1, n, codes, absmax, stream), "quantize")
+    assert lib.eri_adam8_quantize(host.ctypes.data, 1, n, codes, absmax, stream) == -6
+    assert b"not device, pinned or managed memory" in lib.eri_last_error()
+    assert lib.eri_adam8_dequantize(codes, absmax, 1, n, host.ctypes.data, stream) == -6
+    # pinned host memory is reachable: the dequantised values land in it and equal the device copy
+    L.check(lib.eri_adam8_dequantize(codes, absmax, 1, n, out, stream), "dequantize")
+    L.check(lib.eri_adam8_dequantize(codes, absmax, 1, n, pinned, stream), "dequantize to pinned")
+    torch.cuda.synchronize()
+    got = np.frombuffer((C.c_float * n).from_address(pinned), np.float32)
+    assert np.array_equal(got.view(np.uint32), dev_out.cpu().numpy().view(np.uint32))
+    lib.eri_hip_host_free(C.c_void_p(pinned))
