@@ -229,7 +229,8 @@ int eri_adam8_init(void);
 /* The two 256-entry maps (code -> value in [-1, 1] / [0, 1]) the states are expressed in. */
 int eri_adam8_get_maps(float *signed256, float *unsigned256);
 
-/* Codes of 0.0 (127 / 0) and absmax 0: the state of a zeros tensor (adam8bit_enhanced.rs:179-197). */
+/* Codes of 0.0 (127 / 0) and absmax 0: the state of a zeros tensor (adam8bit_enhanced.rs:179-197).
+ * Device pointers, as in a row of the launch table; written by a kernel on `stream`. */
 int eri_adam8_state_init(uint8_t *m, uint8_t *v, float *absmax_m, float *absmax_v, uint64_t numel,
                          void *stream);
 
