@@ -48,11 +48,14 @@ def _step_fp32(p16, g16, mc, vc, h, mode):
 _found = {}
 
 
-def _near_tie_elements(mode, wd, lr, want, seed, p_std):
-    key = (mode, wd, lr, want, seed, p_std)
+DEFAULT_HYP = (0.9, 0.999, 1e-8, 7)  # beta1, beta2, eps, step
+
+
+def _near_tie_elements(mode, wd, lr, want, seed, p_std, hyp=DEFAULT_HYP):
+    key = (mode, wd, lr, want, seed, p_std, hyp)
     if key in _found:
         return _found[key]
-    h = oc.hyper_pack(lr, 0.9, 0.999, 1e-8, wd, 7, mode)
+    h = oc.hyper_pack(lr, hyp[0], hyp[1], hyp[2], wd, hyp[3], mode)
     hh = type("H", (), {k: F32(getattr(h, k)) for k in ("beta1", "beta2", "omb1", "omb2", "eps", "weight_decay", "step_size")})
     rng = np.random.default_rng(seed)
     keep = [[], [], [], []]
@@ -79,12 +82,30 @@ def _near_tie_elements(mode, wd, lr, want, seed, p_std):
 @pytest.mark.parametrize("mode,wd,lr,p_std", [(oc.MODE_ERI, 0.01, 1e-4, 0.02), (oc.MODE_ERI, 0.0, 1e-3, 0.02),
                                              (oc.MODE_BNB, 0.01, 1e-4, 0.02), (oc.MODE_ERI, 0.01, 1e-4, 2e-4)])
 def test_results_on_the_edge_of_a_bf16_rounding_are_bit_exact(mode, wd, lr, p_std, kernels):
+    _run_near_ties(mode, wd, lr, p_std, kernels, DEFAULT_HYP)
+
+
+@pytest.mark.parametrize("kernels", ["default-kernels", "one-wave", "plain"])
+@pytest.mark.parametrize("mode,wd,lr,p_std,hyp", [
+    (oc.MODE_ERI, 0.1, 3e-2, 0.5, (0.5, 0.9, 1e-3, 1)),        # first step, large eps, strong decay
+    (oc.MODE_ERI, 1.0, 0.1, 0.05, (0.0, 0.99, 1e-6, 3)),       # no momentum; a decay of a tenth per step
+    (oc.MODE_ERI, 0.0, 2e-3, 1.0, (0.99, 0.99999, 0.0, 100000)),  # late in a run, eps 0, steps of half a bf16 unit
+    (oc.MODE_BNB, 0.1, 1e-2, 0.1, (0.95, 0.95, 1e-6, 2)),
+])
+def test_near_ties_under_other_hyper_parameters_are_bit_exact(mode, wd, lr, p_std, hyp, kernels):
+    """The margins of the recomputation are functions of the step size and the decay; the same construction
+    away from the default hyper-parameters."""
+    _run_near_ties(mode, wd, lr, p_std, kernels, hyp)
+
+
+def _run_near_ties(mode, wd, lr, p_std, kernels, hyp):
     import torch
     from eridiffusion_amd import _lib as L
     extra = {"default-kernels": 0, "one-wave": L.FLAG_ONE_WAVE, "plain": L.FLAG_NO_PIPELINE}[kernels]
     n = 2048 * 3 + 40
-    p16, g16, mc, vc = _near_tie_elements(mode, wd, lr, n, 11 + mode, p_std)
+    p16, g16, mc, vc = _near_tie_elements(mode, wd, lr, n, 11 + mode, p_std, hyp)
     assert p16.size == n, "the search found too few near-tie elements"
+    b1, b2, eps, t = hyp
     sizes = [2048 * 2, 2048 + 40]
     cut = sizes[0]
 
@@ -101,10 +122,10 @@ def test_results_on_the_edge_of_a_bf16_rounding_are_bit_exact(mode, wd, lr, p_st
     table = C.c_void_p()
     L.check(L.lib().eri_adam8_table_create(rows, len(rows), None, C.byref(table)), "table_create")
     gmode = {oc.MODE_ERI: L.MODE_ERI, oc.MODE_BNB: L.MODE_BNB}[mode]
-    h = L.hyper_pack(lr, 0.9, 0.999, 1e-8, wd, 7, gmode, L.FLAG_EXACT_PARAM | extra)
+    h = L.hyper_pack(lr, b1, b2, eps, wd, t, gmode, L.FLAG_EXACT_PARAM | extra)
     L.check(L.lib().eri_adam8_step_table(table, C.byref(h), None), "step_table")
     torch.cuda.synchronize()
-    hs.oracle_step(ps, gs, states, (lr, 0.9, 0.999, 1e-8, wd, 7), True, mode)
+    hs.oracle_step(ps, gs, states, (lr, b1, b2, eps, wd, t), True, mode)
     got_p, got_st = gt.fetch()
     stats = hs.compare(got_p, got_st, ps, states, True, True, "near ties")
     assert stats["code_mismatch"] == 0
@@ -113,7 +134,7 @@ def test_results_on_the_edge_of_a_bf16_rounding_are_bit_exact(mode, wd, lr, p_st
     gt2 = hs.GpuTensors(*(lambda f: (f[0], gs, f[1]))(fresh()), True)
     rows2 = gt2.rows()
     L.check(L.lib().eri_adam8_table_update(table, rows2, len(rows2), None), "table_update")
-    h0 = L.hyper_pack(lr, 0.9, 0.999, 1e-8, wd, 7, gmode, extra)
+    h0 = L.hyper_pack(lr, b1, b2, eps, wd, t, gmode, extra)
     L.check(L.lib().eri_adam8_step_table(table, C.byref(h0), None), "step_table")
     torch.cuda.synchronize()
     got_p2, got_st2 = gt2.fetch()

@@ -9,6 +9,7 @@ test_gpu_parity.py: 8-bit states and fp32 parameters bit-exact, bf16 parameters 
 ERI_ADAM8_FLAG_EXACT_PARAM and in the functional mode, within one bf16 step otherwise.
 """
 import ctypes as C
+import os
 
 import numpy as np
 import pytest
@@ -19,6 +20,7 @@ import oracle_c as oc
 pytestmark = pytest.mark.gpu
 
 SIZES = [2048 * 9 + 13, 2048 * 4, 777, 2048 * 2 + 2047, 2048 * 23 + 1]
+CASES = int(os.environ.get("ERI_HYPER_CASES", "48"))  # per combination of dtype, mode and kernel; more for a soak
 
 
 def _lib():
@@ -50,7 +52,7 @@ def test_drawn_hyper_parameters_against_the_oracle(bf16, mode, kernels):
     rng = np.random.default_rng(5150 + 10 * mode + bf16)  # the same draws for the three kernels
     stream = torch.cuda.current_stream().cuda_stream
     flips = 0
-    for case in range(48):
+    for case in range(CASES):
         d = _draw(rng)
         flags = 2 if mode == 1 else int(rng.choice([0, 2, 2]))
         exact = (not bf16) or bool(flags & 2)
