@@ -1529,7 +1529,10 @@ int eri_adam8bit_fn_update_many(EriAdam8bitFn *o, const char *const *names, cons
     }
     // 3. rows queued by earlier update() calls keep their place in the order of updates
     int rc = fn_flush(o);
-    if (rc) return rc;
+    if (rc) { // their launch failed: nothing of this call has run, and its new states go
+        for (auto &name : made) o->states.erase(name);
+        return rc;
+    }
     for (uint32_t i = 0; i < n; ++i) {
         rc = fn_enqueue(o, names[i], params[i], grads[i], numels[i], dtype_tags[i],
                         grad_dtype_tags ? grad_dtype_tags[i] : dtype_tags[i], outs[i]);

@@ -637,6 +637,9 @@ int eri_hip_pool_release(EriHipPool *pool, void *ptr, size_t bytes) {
     const size_t offset = (size_t)(p - pool->base) % pool->lane_bytes;
     if (offset % 256 != 0 || offset + need > pool->used[lane])
         return fail(ERI_ERR_ARG, "memory pool: release of a piece that is not the pool's");
+    for (const auto &piece : pool->released[lane]) // a second release would hand the same bytes out twice
+        if (offset < piece.offset + piece.bytes && piece.offset < offset + need)
+            return fail(ERI_ERR_ARG, "memory pool: the piece, or a part of it, has been released already");
     if (offset + need == pool->used[lane]) { // the top piece: the lane shrinks, and so it does past released pieces below it
         pool->used[lane] = offset;
         auto &back = pool->released[lane];

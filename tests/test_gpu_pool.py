@@ -173,6 +173,17 @@ def test_released_pieces_are_handed_out_again():
     L.check(L.lib().eri_hip_pool_release(pool, c, 300), "release")
     L.check(L.lib().eri_hip_pool_lane_used(pool, 0, C.byref(used)), "lane_used")
     assert used.value == 1024
+    # a piece given back twice would be handed out twice: refused while it waits below the lane's level
+    f, g = C.c_void_p(), C.c_void_p()
+    L.check(L.lib().eri_hip_pool_alloc_zeroed(pool, 0, 4096, C.byref(f)), "alloc")
+    L.check(L.lib().eri_hip_pool_alloc_zeroed(pool, 0, 256, C.byref(g)), "alloc")
+    L.check(L.lib().eri_hip_pool_release(pool, f, 4096), "release")
+    assert L.lib().eri_hip_pool_release(pool, f, 4096) == -6
+    assert b"released already" in L.lib().eri_last_error()
+    assert L.lib().eri_hip_pool_release(pool, C.c_void_p(f.value + 1024), 256) == -6  # a part of it
+    L.check(L.lib().eri_hip_pool_release(pool, g, 256), "release")
+    L.check(L.lib().eri_hip_pool_lane_used(pool, 0, C.byref(used)), "lane_used")
+    assert used.value == 1024
     # not the pool's, or beyond the lane's level
     assert L.lib().eri_hip_pool_release(pool, C.c_void_p(a.value + 8 * MiB), 256) == -6
     assert L.lib().eri_hip_pool_release(pool, C.c_void_p(a.value + 100), 256) == -6
