@@ -40,9 +40,12 @@ ROWS = [
     (dict(config="c1_flat_fp32"), 100, 10),
     (dict(config="c2_sdxl_lora_r16"), 100, 10),
     (dict(config="c2_sdxl_lora_r16", api="functional"), 100, 10),
+    (dict(config="c2_sdxl_lora_r16", kernel="traffic"), 100, 10),
     (dict(config="c3_flux_lora_r32"), 100, 10),
     (dict(config="c3_flux_lora_r32", api="functional"), 100, 10),
+    (dict(config="c3_flux_lora_r32", kernel="traffic"), 100, 10),
     (dict(config="c4_sdxl_unet_full"), 20, 3),
+    (dict(config="c4_sdxl_unet_full", kernel="traffic"), 20, 3),
     (dict(config="c5_flux12b_full", flags=2), 20, 3),
     (dict(config="c5_flux12b_full", mode="l2"), 20, 3),
     (dict(config="c5_flux12b_full", kernel="traffic"), 20, 3),
