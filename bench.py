@@ -582,7 +582,7 @@ def main():
                 continue
             row = row_of(o)
             small = W.total_params(tens) <= (1 << 28)
-            if args.cpu_sample > 0 and small and a.api == "table" and a.mode == "eri" and a.flags == 0:
+            if args.cpu_sample > 0 and small and a.kernel == "adam8" and a.api == "table" and a.mode == "eri" and a.flags == 0:
                 cb = cpu_baseline(tens, b16, 1 << 62, hy, single_thread=False)  # the whole configuration
                 row["cpu_params_per_s"], row["cpu_sample"] = cb["value"], cb["sample"]
             rows.append(row)
