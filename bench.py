@@ -47,6 +47,7 @@ ROWS = [
     (dict(config="c4_sdxl_unet_full"), 20, 3),
     (dict(config="c4_sdxl_unet_full", kernel="traffic"), 20, 3),
     (dict(config="c5_flux12b_full", flags=2), 20, 3),
+    (dict(config="c5_flux12b_full", flags=2, api="object"), 20, 3),  # the list optimizer as a trainer gets it
     (dict(config="c5_flux12b_full", mode="l2"), 20, 3),
     (dict(config="c5_flux12b_full", kernel="traffic"), 20, 3),
     (dict(config="c5_flux12b_full", alloc="tensor"), 20, 3),
@@ -302,9 +303,9 @@ def measure(args, torch, separate_events=False):
         lanes, lane_bytes = C.c_uint32(), C.c_size_t()
         L.check(L.lib().eri_hip_pool_info(Pool.handle, C.byref(lanes), C.byref(lane_bytes)), "eri_hip_pool_info")
         state_bytes = 2 * n_params + 8 * n_blocks + 1024 * len(sizes)
-        if args.api == "object":
-            state_bytes *= 2  # the optimizer's own states beside the (unused) flat ones
         widest = max(n_params * max(esz, gsz) + 256 * len(sizes), state_bytes)
+        if args.api != "table":  # the flat states, unused by the optimizer objects, share the last lane
+            widest = max(widest, state_bytes + (0 if args.api == "object" else n_params * esz + 256 * len(sizes)))
         if lanes.value < 4 or widest > lane_bytes.value:
             print("bench.py: the lane pool has %d lanes of %.1f GiB, too few or too narrow for this workload; the "
                   "flat buffers become allocations of their own (--alloc arena)" % (lanes.value, lane_bytes.value / 2**30),
@@ -315,10 +316,13 @@ def measure(args, torch, separate_events=False):
     LANE_PARAM, LANE_GRAD, LANE_STATE, LANE_OTHER = 0, 1, 2, 3  # the pool's lanes, one per kind of tensor
     a_p = Alloc(torch, [n * esz for n in sizes], LANE_PARAM)
     a_g = Alloc(torch, [n * gsz for n in sizes], LANE_GRAD)
-    a_m = Alloc(torch, sizes, LANE_STATE)
-    a_v = Alloc(torch, sizes, LANE_STATE)
-    a_am = Alloc(torch, [((n + 2047) // 2048) * 4 for n in sizes], LANE_STATE)
-    a_av = Alloc(torch, [((n + 2047) // 2048) * 4 for n in sizes], LANE_STATE)
+    # The optimizer objects allocate their states themselves, out of the state lane, as they would under a trainer;
+    # the flat state arrays (which only the table API steps) then stay out of that lane.
+    flat_lane = LANE_STATE if args.api == "table" else LANE_OTHER
+    a_m = Alloc(torch, sizes, flat_lane)
+    a_v = Alloc(torch, sizes, flat_lane)
+    a_am = Alloc(torch, [((n + 2047) // 2048) * 4 for n in sizes], flat_lane)
+    a_av = Alloc(torch, [((n + 2047) // 2048) * 4 for n in sizes], flat_lane)
     tdt = torch.bfloat16 if bf16 else torch.float32
     gen = torch.Generator(device="cuda:0")
     gen.manual_seed(0xE21D + 5)

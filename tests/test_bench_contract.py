@@ -40,11 +40,12 @@ def test_the_rows_of_the_default_run_cover_every_configuration_and_entry_point()
     from eridiffusion_amd import workloads as W
     rows = [dict(b.HEADLINE, **change) for change, _, _ in b.ROWS]
     for r in rows:
-        assert r["config"] in W.CONFIGS and r["api"] in ("table", "functional") and r["alloc"] in ("pool", "tensor")
+        assert r["config"] in W.CONFIGS and r["api"] in ("table", "functional", "object") and r["alloc"] in ("pool", "tensor")
     table = {r["config"] for r in rows if r["api"] == "table" and r["flags"] == 0 and r["alloc"] == "pool" and r["mode"] == "eri"}
     assert table | {b.HEADLINE["config"]} == set(W.CONFIGS)
     assert {r["config"] for r in rows if r["api"] == "functional"} == {"c2_sdxl_lora_r16", "c3_flux_lora_r32"}
-    assert any(r["config"] == "c5_flux12b_full" and r["flags"] == 2 for r in rows)
+    assert any(r["config"] == "c5_flux12b_full" and r["flags"] == 2 and r["api"] == "table" for r in rows)
+    assert any(r["config"] == "c5_flux12b_full" and r["flags"] == 2 and r["api"] == "object" for r in rows)
     assert any(r["config"] == "c5_flux12b_full" and r["alloc"] == "tensor" for r in rows)
     assert any(r["config"] == "c5_flux12b_full" and r["mode"] == "l2" for r in rows)
     for change, steps, warmup in b.ROWS:
