@@ -147,15 +147,12 @@ def test_legacy_state_file_errors(tmp_path):
     L.lib().eri_adam8bit_destroy(opt)
 
 
-def test_state_file_parsers_survive_random_corruption(tmp_path):
-    """Six hundred random mutations (truncations, byte flips, overwritten length fields, spliced garbage)
-    of a valid safetensors state and of a valid bincode state: every one must come back with a return
-    code -- refused with -6, or passed on to the device upload, which fails without a GPU -- and never
-    crash the process or leave a half-loaded optimizer."""
+def mutated_state_files(count, seed=1234, numel=4096):
+    """`count` random mutations (truncations, byte flips, overwritten length fields, spliced garbage), in turn of
+    a valid safetensors state and of a valid bincode state of two parameters of `numel` elements: (is_safetensors,
+    bytes) pairs."""
     import json
     import random
-    numel = 4096
-    opt, handles = _optimizer(n_params=2, numel=numel)
     nb = (numel + 2047) // 2048
     tensors, payload = {}, b""
     for i in range(2):
@@ -169,7 +166,7 @@ def test_state_file_parsers_survive_random_corruption(tmp_path):
     good_st = struct.pack("<Q", len(hdr)) + hdr + payload
     good_bc = _bincode_state(7, 2e-4, {"param_0": ([1] * numel, 0.5, 0, [numel], 0.0), "param_1": ([3] * numel, 0.1, 2, [64, 64], 0.0)},
                              {"param_0": ([2] * numel, 0.25, -1, [numel], 0.0), "param_1": ([4] * numel, 0.2, 0, [numel], 0.0)})
-    rnd = random.Random(1234)
+    rnd = random.Random(seed)
 
     def mutate(blob):
         b = bytearray(blob)
@@ -189,11 +186,20 @@ def test_state_file_parsers_survive_random_corruption(tmp_path):
             return bytes(b[:at]) + bytes(rnd.randrange(256) for _ in range(rnd.randrange(1, 64))) + bytes(b[at:])
         return bytes(b) + bytes(rnd.randrange(1, 9))
 
+    for k in range(count):
+        use_st = k % 2 == 0
+        yield use_st, mutate(good_st if use_st else good_bc)
+
+
+def test_state_file_parsers_survive_random_corruption(tmp_path):
+    """Six hundred random mutations of a valid safetensors state and of a valid bincode state: every one must
+    come back with a return code -- refused with -6, or passed on to the device upload, which fails without a
+    GPU -- and never crash the process or leave a half-loaded optimizer."""
+    opt, handles = _optimizer(n_params=2, numel=4096)
     path = tmp_path / "fuzz.bin"
     refused = 0
-    for k in range(600):
-        use_st = k % 2 == 0
-        path.write_bytes(mutate(good_st if use_st else good_bc))
+    for use_st, blob in mutated_state_files(600):
+        path.write_bytes(blob)
         fn = L.lib().eri_adam8bit_load_state if use_st else L.lib().eri_adam8bit_load_legacy_state
         rc = fn(opt, str(path).encode())
         if rc == -6:
