@@ -5,7 +5,7 @@
  * there and are never reached), and this program drives the code that handles untrusted bytes and caller
  * mistakes: the state-file parsers over a directory of mutated files, row validation, the functional
  * optimizer's queue, the pool's book-keeping arguments.  Every call must come back with a return code.
- * Test infrastructure: built by tests/Makefile (target san_host), run by tests/test_host_sanitizers.py.
+ * Test infrastructure: built by tests/san_host.mk, run by tests/test_host_sanitizers.py.
  *
  * usage: san_host <directory with NNN.st (safetensors) and NNN.bc (bincode) files> <count>
  */
