@@ -235,8 +235,11 @@ template <int MODE, bool WD, bool BF16>
 __device__ __forceinline__ float param_exact(float p, float m, float v, const StepHyper &h, const BlockDiv &dbc1,
                                              const BlockDiv &dbc2) {
     if (MODE == ERI_ADAM8_MODE_L2) {
-        float mh = dbc1.fast ? dbc1.div_fast_unbounded(m) : m / dbc1.a; // adam8bit.rs:170
-        float vh = dbc2.fast ? dbc2.div_fast_unbounded(v) : v / dbc2.a; // :178
+        // bf16 parameters come here for one element in 1,600 (the fast chain's near-ties): the plain IEEE
+        // division, so that the kernel need not hold the two prepared divisors; fp32 parameters come here
+        // with every element and take the prepared form (same bits)
+        float mh = BF16 ? m / h.bc1 : dbc1.fast ? dbc1.div_fast_unbounded(m) : m / dbc1.a; // adam8bit.rs:170
+        float vh = BF16 ? v / h.bc2 : dbc2.fast ? dbc2.div_fast_unbounded(v) : v / dbc2.a; // :178
         vh = fmaxf(vh, 0.0f);                                           // :181-182
         float den = sqrtf(vh) + h.eps;                                  // :187
         float upd = mh / den;

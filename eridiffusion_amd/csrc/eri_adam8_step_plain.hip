@@ -13,13 +13,15 @@
 
 namespace eri {
 
-/* Threads per workgroup.  The coupled-decay mode holds two more divisions' worth of values per element:
- * with the 128 registers a 1024-thread workgroup leaves each lane it spilled 28-68 bytes, with 768
- * threads (170 registers) it does not. */
-constexpr uint32_t plain_threads(int mode) { return mode == ERI_ADAM8_MODE_L2 ? 768 : 1024; }
+/* Threads per workgroup: sixteen waves per compute unit where the instantiation fits the 128 registers that
+ * leaves each lane, twelve (170 registers) where it would spill: the coupled-decay mode with a gradient scale,
+ * with fp32 gradients or with the binary search (12-30 spilled registers at sixteen waves). */
+constexpr uint32_t plain_threads(int mode, bool gs, bool keytab, bool gbf16) {
+    return (mode == ERI_ADAM8_MODE_L2 && (gs || !keytab || !gbf16)) ? 768 : 1024;
+}
 
 template <bool BF16, int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB, bool GBF16>
-__global__ __launch_bounds__(plain_threads(MODE)) void adam8_step_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
+__global__ __launch_bounds__(plain_threads(MODE, GS, KEYTAB, GBF16)) void adam8_step_kernel(const DevTensor *__restrict__ rows, uint32_t n_rows,
                                                           uint32_t total_blocks, EriAdam8Hyper h_in,
                                                           const uint4 *__restrict__ lds_image,
                                                           const float *__restrict__ dev_scale) {
@@ -89,7 +91,7 @@ template <int MODE, bool EXACT, bool WD, bool GS, bool KEYTAB, bool GBF16>
 int launch_one(const DevTensor *rows, uint32_t n_rows, uint32_t total_blocks, const EriAdam8Hyper &h,
                const void *lds_image, const float *dev_scale, uint32_t grid, uint32_t wg, hipStream_t s) {
     auto k = adam8_step_kernel<kBf16, MODE, EXACT, WD, GS, KEYTAB, GBF16>;
-    if (wg > plain_threads(MODE)) wg = plain_threads(MODE);
+    if (wg > plain_threads(MODE, GS, KEYTAB, GBF16)) wg = plain_threads(MODE, GS, KEYTAB, GBF16);
     // One common window for all dies (a grid-stride walk): on the tables this kernel takes, up to 1,024
     // blocks per compute unit, it measured 2 % ahead of one range per die with the arrays far apart in device
     // memory and 5 % with them adjacent; the tables of the prefetching kernel want the ranges.
