@@ -51,6 +51,12 @@ ROWS = [
     (dict(config="c5_flux12b_full", mode="l2"), 20, 3),
     (dict(config="c5_flux12b_full", kernel="traffic"), 20, 3),
     (dict(config="c5_flux12b_full", alloc="tensor"), 20, 3),
+    # the sweeps that sit beside the step in a training iteration
+    (dict(config="c5_flux12b_full", kernel="grad_norm"), 20, 3),
+    (dict(config="c5_flux12b_full", kernel="adam8_clip"), 20, 3),
+    (dict(config="c5_flux12b_full", kernel="adam8_ema"), 20, 3),
+    (dict(config="c5_flux12b_full", kernel="ema"), 20, 3),
+    (dict(config="c4_sdxl_unet_full", kernel="adamw32"), 20, 3),
 ]
 
 
