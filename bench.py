@@ -352,7 +352,7 @@ def measure(args, torch, separate_events=False):
     extra = []
     if args.kernel == "adamw32":
         a_m32 = Alloc(torch, [4 * n for n in sizes], LANE_STATE)
-        a_v32 = Alloc(torch, [4 * n for n in sizes], LANE_STATE)
+        a_v32 = Alloc(torch, [4 * n for n in sizes], LANE_OTHER)  # 32-bit moments are the bulk of the written bytes: a lane each
         extra += [a_m32, a_v32]
         rows32 = (L.AdamW32Row * len(sizes))()
         for i, n in enumerate(sizes):
